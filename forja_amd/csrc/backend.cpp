@@ -1,0 +1,1495 @@
+// Host side of libforja_hip: allocation registry, operand validation (the checks of
+// crates/forja-core/src/ops.rs:1300-2378 for the ops on the ragged forward step), kernel
+// selection and the C ABI declared in include/forja_hip.h.
+#include <algorithm>
+#include <chrono>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <new>
+#include <thread>
+#include <unordered_map>
+#include <vector>
+
+#include "fast_kernels.hpp"
+#include "kernels.hpp"
+
+namespace fh {
+
+namespace {
+
+struct Allocation {
+  char *ptr = nullptr;
+  uint64_t bytes = 0;
+  bool readonly = false;
+};
+
+struct Program {
+  uint32_t kind = 0;  // 0 map, 1 row
+  std::vector<fh_inst> insts;
+  std::vector<uint32_t> pairs;  // (slot, value)
+  uint32_t n_inputs = 0;
+  uint32_t n_outputs = 0;
+  uint32_t n_reduce = 0;
+  // Device instruction arrays keyed by the u32-ness mask of the bound inputs.
+  std::map<uint32_t, DInst *> typed;
+};
+
+bool is_float(uint32_t dtype) { return dtype == FH_F32 || dtype == FH_F16 || dtype == FH_BF16; }
+bool is_half(uint32_t dtype) { return dtype == FH_F16 || dtype == FH_BF16; }
+
+uint64_t element_count(const fh_tensor &t) {
+  uint64_t count = 1;
+  for (uint32_t axis = 0; axis < t.rank; ++axis) count *= t.shape[axis];
+  return count;
+}
+
+// Layout::is_contiguous (crates/forja-core/src/layout.rs:292-309): extent-1 axes are ignored.
+bool is_contiguous(const fh_tensor &t) {
+  uint64_t expected = 1;
+  for (int axis = (int)t.rank - 1; axis >= 0; --axis) {
+    if (t.shape[axis] == 1) continue;
+    if (t.stride[axis] != expected) return false;
+    expected *= t.shape[axis];
+  }
+  return true;
+}
+
+bool shape_is(const fh_tensor &t, std::initializer_list<uint32_t> shape) {
+  if (t.rank != shape.size()) return false;
+  uint32_t axis = 0;
+  for (uint32_t extent : shape)
+    if (t.shape[axis++] != extent) return false;
+  return true;
+}
+
+}  // namespace
+
+}  // namespace fh
+
+using namespace fh;
+
+struct fh_submission {
+  fh_backend *backend = nullptr;
+  uint64_t serial = 0;
+  uint32_t count = 0;
+  std::vector<uint32_t> ops;
+  ErrorSlot *device_errors = nullptr;
+  ErrorSlot *host_errors = nullptr;  // pinned
+  hipEvent_t start = nullptr, end = nullptr;
+  bool waited = false;
+  fh_status result = FH_OK;
+  fh_error error{};
+  uint64_t gpu_ns = 0;
+};
+
+struct fh_backend {
+  std::mutex mutex;
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipDeviceProp_t props{};
+  std::unordered_map<uint64_t, Allocation> allocations;
+  std::unordered_map<uint64_t, Program> programs;
+  uint64_t next_id = 1;
+  uint64_t next_serial = 1;
+  uint64_t used_bytes = 0;
+  char *workspace = nullptr;
+  uint64_t workspace_bytes = 0;
+  // profiling
+  bool profiling = false;
+  struct Timed {
+    hipEvent_t start, end;
+    uint32_t kernel_class;
+  };
+  std::vector<Timed> timed;
+  std::vector<hipEvent_t> event_pool;
+  uint64_t class_ns[FH_KC_COUNT] = {0, 0, 0, 0};
+  uint64_t class_launches[FH_KC_COUNT] = {0, 0, 0, 0};
+
+  char *ensure_workspace(uint64_t bytes) {
+    if (bytes <= workspace_bytes) return workspace;
+    (void)hipStreamSynchronize(stream);
+    if (workspace) (void)hipFree(workspace);
+    workspace = nullptr;
+    workspace_bytes = 0;
+    uint64_t want = std::max<uint64_t>(bytes, 64ull << 20);
+    void *ptr = nullptr;
+    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
+    workspace = (char *)ptr;
+    workspace_bytes = want;
+    return workspace;
+  }
+};
+
+namespace {
+
+#define FH_REQUIRE(cond)              \
+  do {                                \
+    if (!(cond)) return FH_INVALID_INPUT; \
+  } while (0)
+
+// Resolves a tensor to a device view after checking identity and that the touched span fits the
+// allocation (AllocationRegistry::validate, backend.rs:315-339; Layout::new, layout.rs:203-227).
+fh_status make_view(fh_backend *b, const fh_tensor &t, bool writable, View *out) {
+  auto it = b->allocations.find(t.buffer);
+  FH_REQUIRE(it != b->allocations.end());
+  FH_REQUIRE(t.rank <= FH_MAX_RANK && t.dtype <= FH_U32);
+  if (writable) FH_REQUIRE(!it->second.readonly);
+  uint64_t span = t.offset;
+  bool empty = false;
+  for (uint32_t axis = 0; axis < t.rank; ++axis) {
+    if (t.shape[axis] == 0) {
+      empty = true;
+      break;
+    }
+    uint64_t reach = (uint64_t)(t.shape[axis] - 1) * t.stride[axis];
+    FH_REQUIRE(t.stride[axis] == 0 || reach / t.stride[axis] == (uint64_t)(t.shape[axis] - 1));
+    FH_REQUIRE(span + reach >= span);
+    span += reach;
+  }
+  if (!empty) {
+    uint64_t size = dtype_size(t.dtype);
+    FH_REQUIRE(span < (1ull << 60));
+    FH_REQUIRE((span + 1) * size <= it->second.bytes);
+  } else {
+    FH_REQUIRE(t.offset * dtype_size(t.dtype) <= it->second.bytes);
+  }
+  out->base = it->second.ptr;
+  out->dtype = t.dtype;
+  out->rank = t.rank;
+  for (uint32_t axis = 0; axis < FH_MAX_RANK; ++axis) {
+    out->shape[axis] = axis < t.rank ? t.shape[axis] : 1;
+    out->stride[axis] = axis < t.rank ? t.stride[axis] : 0;
+  }
+  out->offset = t.offset;
+  return FH_OK;
+}
+
+View null_view() {
+  View v{};
+  v.base = nullptr;
+  return v;
+}
+
+// ---------------------------------------------------------------- scalar programs
+
+// Type inference and the structural rules of Program::validate
+// (crates/forja-core/src/program.rs): SSA order, typed operands, reductions only in row
+// programs and at most four, f32 outputs.  `u32_mask` bit i = input slot i is bound to a u32
+// tensor.  Produces the typed device instructions.
+fh_status type_program(const Program &p, uint32_t u32_mask, uint32_t rank,
+                       std::vector<DInst> *out) {
+  std::vector<uint8_t> types(p.insts.size());
+  out->resize(p.insts.size());
+  uint32_t reductions = 0;
+  for (size_t i = 0; i < p.insts.size(); ++i) {
+    const fh_inst &in = p.insts[i];
+    DInst d{};
+    d.kind = (uint8_t)in.kind;
+    d.op = (uint8_t)in.op;
+    d.a = in.a;
+    d.b = in.b;
+    d.c = in.c;
+    auto operand_ok = [&](uint32_t v) { return (size_t)v < i; };
+    switch (in.kind) {
+    case 0:
+      FH_REQUIRE(in.a < kMaxProgramInputs && in.a < p.n_inputs);
+      types[i] = (u32_mask >> in.a) & 1u ? 1 : 0;
+      break;
+    case 1: types[i] = 0; break;
+    case 2:
+    case 3:
+      FH_REQUIRE(in.op < rank);
+      types[i] = 1;
+      break;
+    case 4:
+      FH_REQUIRE(in.op <= 13 && operand_ok(in.a) && types[in.a] == 0);
+      types[i] = 0;
+      break;
+    case 5: {
+      FH_REQUIRE(in.op <= 12 && operand_ok(in.a) && operand_ok(in.b));
+      uint8_t ta = types[in.a], tb = types[in.b];
+      FH_REQUIRE(ta == tb && ta != 2);
+      if (ta == 1) FH_REQUIRE(in.op != 3 && in.op != 6);
+      d.ty = ta;
+      types[i] = in.op >= 7 ? 2 : ta;
+      break;
+    }
+    case 6:
+      FH_REQUIRE(operand_ok(in.a) && operand_ok(in.b) && operand_ok(in.c));
+      FH_REQUIRE(types[in.a] == 2 && types[in.b] == types[in.c]);
+      types[i] = types[in.b];
+      break;
+    case 7:
+      FH_REQUIRE(in.op <= 2 && operand_ok(in.a));
+      d.ty = types[in.a];
+      types[i] = (uint8_t)in.op;
+      break;
+    case 8:
+      FH_REQUIRE(p.kind == 1 && in.op <= 2 && operand_ok(in.a) && types[in.a] == 0);
+      FH_REQUIRE(++reductions <= kMaxReductions);
+      types[i] = 0;
+      break;
+    default: return FH_INVALID_INPUT;
+    }
+    if (in.kind == 4) d.ty = 0;
+    (*out)[i] = d;
+  }
+  for (size_t pair = 0; pair + 1 < p.pairs.size(); pair += 2) {
+    FH_REQUIRE(p.pairs[pair] < p.n_outputs && p.pairs[pair + 1] < p.insts.size());
+    FH_REQUIRE(types[p.pairs[pair + 1]] == 0);
+  }
+  return FH_OK;
+}
+
+// Binds a prepared program to tensors (BoundProgram, program.rs:759-857): every input and output
+// has exactly the iteration shape; inputs float or u32; outputs float.
+fh_status bind_program(fh_backend *b, Program &p, const fh_tensor *inputs, uint32_t n_inputs,
+                       const View *input_views, const fh_tensor *outputs, uint32_t n_outputs,
+                       const View *output_views, const uint32_t *shape, uint32_t rank,
+                       ProgramArgs *args) {
+  FH_REQUIRE(n_inputs == p.n_inputs && n_outputs == p.n_outputs);
+  FH_REQUIRE(rank >= 1 && rank <= FH_MAX_RANK);
+  uint32_t mask = 0;
+  for (uint32_t i = 0; i < n_inputs; ++i) {
+    FH_REQUIRE(inputs[i].rank == rank);
+    for (uint32_t axis = 0; axis < rank; ++axis) FH_REQUIRE(inputs[i].shape[axis] == shape[axis]);
+    FH_REQUIRE(is_float(inputs[i].dtype) || inputs[i].dtype == FH_U32);
+    if (inputs[i].dtype == FH_U32) mask |= 1u << i;
+  }
+  for (uint32_t i = 0; i < n_outputs; ++i) {
+    FH_REQUIRE(outputs[i].rank == rank && is_float(outputs[i].dtype));
+    for (uint32_t axis = 0; axis < rank; ++axis) FH_REQUIRE(outputs[i].shape[axis] == shape[axis]);
+  }
+  auto cached = p.typed.find(mask | (rank << 16));
+  DInst *device = nullptr;
+  if (cached == p.typed.end()) {
+    std::vector<DInst> typed;
+    fh_status status = type_program(p, mask, rank, &typed);
+    if (status != FH_OK) return status;
+    void *ptr = nullptr;
+    if (hipMalloc(&ptr, typed.size() * sizeof(DInst)) != hipSuccess) return FH_ALLOCATION_FAILED;
+    if (hipMemcpy(ptr, typed.data(), typed.size() * sizeof(DInst), hipMemcpyHostToDevice) !=
+        hipSuccess)
+      return FH_DEVICE_EXECUTION_FAILED;
+    device = (DInst *)ptr;
+    p.typed[mask | (rank << 16)] = device;
+  } else {
+    device = cached->second;
+  }
+  memset(args, 0, sizeof(*args));
+  args->insts = device;
+  args->n_insts = (uint32_t)p.insts.size();
+  args->n_inputs = n_inputs;
+  args->rank = rank;
+  for (uint32_t axis = 0; axis < FH_MAX_RANK; ++axis) args->shape[axis] = axis < rank ? shape[axis] : 1;
+  args->n_pairs = (uint32_t)(p.pairs.size() / 2);
+  FH_REQUIRE(args->n_pairs <= kMaxProgramOutputs);
+  for (uint32_t pair = 0; pair < args->n_pairs; ++pair) {
+    args->out_slot[pair] = p.pairs[2 * pair];
+    args->out_value[pair] = p.pairs[2 * pair + 1];
+  }
+  args->n_reduce = 0;
+  for (uint32_t i = 0; i < p.insts.size(); ++i)
+    if (p.insts[i].kind == 8) args->reduce_at[args->n_reduce++] = i;
+  for (uint32_t i = 0; i < n_inputs; ++i) args->inputs[i] = input_views[i];
+  for (uint32_t i = 0; i < n_outputs; ++i) args->outputs[i] = output_views[i];
+  return FH_OK;
+}
+
+// ---------------------------------------------------------------- per-op planning
+
+struct Planned {
+  const fh_dispatch *d;
+  View in[FH_MAX_INPUTS];
+  View out[FH_MAX_OUTPUTS];
+};
+
+fh_tensor f32_like(const fh_tensor &t) {
+  // A contiguous f32 tensor of the same shape (buffer filled in by the caller's view).
+  fh_tensor r = t;
+  r.dtype = FH_F32;
+  uint64_t stride = 1;
+  for (int axis = (int)t.rank - 1; axis >= 0; --axis) {
+    r.stride[axis] = stride;
+    stride *= t.shape[axis];
+  }
+  r.offset = 0;
+  return r;
+}
+
+View contiguous_view(char *base, uint32_t dtype, const fh_tensor &like) {
+  View v{};
+  v.base = base;
+  v.dtype = dtype;
+  v.rank = like.rank;
+  uint64_t stride = 1;
+  for (uint32_t axis = 0; axis < FH_MAX_RANK; ++axis) {
+    v.shape[axis] = 1;
+    v.stride[axis] = 0;
+  }
+  for (int axis = (int)like.rank - 1; axis >= 0; --axis) {
+    v.shape[axis] = like.shape[axis];
+    v.stride[axis] = stride;
+    stride *= like.shape[axis];
+  }
+  v.offset = 0;
+  return v;
+}
+
+// check_quantized_weights (ops.rs:1798-1842 and check_quantized_expert_weights): packed u32
+// [.., N, K*bits/32], scales/biases half [.., N, K/group], same dtype.
+fh_status check_quant_triple(const fh_tensor &packed, const fh_tensor &scales,
+                             const fh_tensor &biases, uint32_t rank, uint32_t inner,
+                             uint32_t bits, uint32_t group, uint32_t *columns,
+                             uint32_t *experts) {
+  FH_REQUIRE(bits == 4 || bits == 8);
+  FH_REQUIRE(group == 32 || group == 64 || group == 128);
+  FH_REQUIRE(inner != 0 && inner % group == 0);
+  FH_REQUIRE(packed.dtype == FH_U32 && packed.rank == rank);
+  FH_REQUIRE(is_half(scales.dtype) && biases.dtype == scales.dtype);
+  FH_REQUIRE(scales.rank == rank && biases.rank == rank);
+  uint32_t n = packed.shape[rank - 2];
+  FH_REQUIRE((uint64_t)packed.shape[rank - 1] * 32 == (uint64_t)inner * bits);
+  for (const fh_tensor *t : {&scales, &biases}) {
+    FH_REQUIRE(t->shape[rank - 2] == n && t->shape[rank - 1] == inner / group);
+    if (rank == 3) FH_REQUIRE(t->shape[0] == packed.shape[0]);
+  }
+  *columns = n;
+  if (experts) *experts = rank == 3 ? packed.shape[0] : 1;
+  return FH_OK;
+}
+
+fh_status run_epilogue(fh_backend *b, const Planned &pl, uint32_t primitive_inputs,
+                       char *accumulators, uint32_t accumulator_count) {
+  const fh_dispatch &d = *pl.d;
+  auto it = b->programs.find(d.epilogue);
+  FH_REQUIRE(it != b->programs.end());
+  Program &p = it->second;
+  FH_REQUIRE(p.kind == 0);
+  FH_REQUIRE(d.accumulator_count == accumulator_count);
+  FH_REQUIRE(primitive_inputs + d.n_extras == d.n_inputs);
+  uint32_t n_inputs = accumulator_count + d.n_extras;
+  FH_REQUIRE(n_inputs <= kMaxProgramInputs);
+  fh_tensor tensors[kMaxProgramInputs];
+  View views[kMaxProgramInputs];
+  const fh_tensor &out = d.outputs[0];
+  uint64_t elements = element_count(out);
+  for (uint32_t i = 0; i < accumulator_count; ++i) {
+    tensors[i] = f32_like(out);
+    views[i] = contiguous_view(accumulators + (uint64_t)i * elements * 4, FH_F32, out);
+  }
+  for (uint32_t i = 0; i < d.n_extras; ++i) {
+    tensors[accumulator_count + i] = d.inputs[primitive_inputs + i];
+    views[accumulator_count + i] = pl.in[primitive_inputs + i];
+  }
+  ProgramArgs args;
+  fh_status status = bind_program(b, p, tensors, n_inputs, views, &out, 1, &pl.out[0], out.shape,
+                                  out.rank, &args);
+  if (status != FH_OK) return status;
+  launch_program(b->stream, args, false, elements);
+  return FH_OK;
+}
+
+fh_status plan_copy(fh_backend *b, const Planned &pl, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_inputs == 1 && d.n_outputs == 1);
+  const fh_tensor &in = d.inputs[0], &out = d.outputs[0];
+  FH_REQUIRE(in.rank == out.rank);
+  for (uint32_t axis = 0; axis < in.rank; ++axis) FH_REQUIRE(in.shape[axis] == out.shape[axis]);
+  bool in_int = in.dtype == FH_I32 || in.dtype == FH_U32;
+  bool out_int = out.dtype == FH_I32 || out.dtype == FH_U32;
+  FH_REQUIRE(in_int == out_int);
+  if (in_int) FH_REQUIRE(in.dtype == out.dtype);
+  if (execute) launch_copy(b->stream, pl.in[0], pl.out[0], element_count(out));
+  return FH_OK;
+}
+
+fh_status plan_program(fh_backend *b, const Planned &pl, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  auto it = b->programs.find(d.program);
+  FH_REQUIRE(it != b->programs.end());
+  FH_REQUIRE(d.n_outputs >= 1 && d.n_outputs <= kMaxProgramOutputs);
+  FH_REQUIRE(d.n_inputs <= kMaxProgramInputs);
+  const fh_tensor &first = d.outputs[0];
+  ProgramArgs args;
+  fh_status status = bind_program(b, it->second, d.inputs, d.n_inputs, pl.in, d.outputs,
+                                  d.n_outputs, pl.out, first.shape, first.rank, &args);
+  if (status != FH_OK) return status;
+  uint64_t elements = element_count(first);
+  if (it->second.kind == 1) FH_REQUIRE(first.shape[first.rank - 1] != 0);
+  if (execute) {
+    if (try_fast_program(b->stream, it->second.kind == 1, args, elements)) return FH_OK;
+    launch_program(b->stream, args, it->second.kind == 1, elements);
+  }
+  return FH_OK;
+}
+
+fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  uint32_t primitive = 4;
+  FH_REQUIRE(d.n_outputs == 1 && d.n_inputs == primitive + (d.epilogue ? d.n_extras : 0));
+  const fh_tensor &x = d.inputs[0], &out = d.outputs[0];
+  FH_REQUIRE(is_float(x.dtype) && out.dtype == x.dtype);
+  FH_REQUIRE(x.rank == 2 && out.rank == 2);
+  uint32_t rows = x.shape[0], inner = x.shape[1], columns = 0;
+  fh_status status = check_quant_triple(d.inputs[1], d.inputs[2], d.inputs[3], 2, inner, d.bits,
+                                        d.group_size, &columns, nullptr);
+  if (status != FH_OK) return status;
+  FH_REQUIRE(shape_is(out, {rows, columns}));
+  if (!execute) return FH_OK;
+  if (rows == 0 || columns == 0) return FH_OK;
+  if (!d.epilogue) {
+    QmmProblem problem{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows, inner, columns,
+                       d.bits, d.group_size};
+    if (try_fast_quant_matmul(b->stream, problem)) return FH_OK;
+    launch_quant_matmul_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows,
+                                inner, columns, d.bits, d.group_size);
+    return FH_OK;
+  }
+  uint64_t elements = (uint64_t)rows * columns;
+  char *acc = b->ensure_workspace(elements * 4);
+  if (!acc) return FH_ALLOCATION_FAILED;
+  View acc_view = contiguous_view(acc, FH_F32, out);
+  QmmProblem problem{pl.in[0], pl.in[1], pl.in[2], pl.in[3], acc_view, rows, inner, columns,
+                     d.bits, d.group_size};
+  if (!try_fast_quant_matmul(b->stream, problem))
+    launch_quant_matmul_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], acc_view, rows,
+                                inner, columns, d.bits, d.group_size);
+  return run_epilogue(b, pl, primitive, acc, 1);
+}
+
+fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_outputs == 1);
+  uint32_t extras = d.epilogue ? d.n_extras : 0;
+  FH_REQUIRE(d.n_inputs >= extras);
+  uint32_t primitive = d.n_inputs - extras;
+  FH_REQUIRE(primitive == 5 || primitive == 6 || primitive == 8);
+  const fh_tensor &x = d.inputs[0], &out = d.outputs[0];
+  FH_REQUIRE(is_float(x.dtype) && out.dtype == x.dtype);
+  uint32_t columns = 0, experts = 0;
+  if (primitive == 6) {
+    // check_gather_quant_weighted_sum (ops.rs:1884-1931)
+    const fh_tensor &idx = d.inputs[4], &w = d.inputs[5];
+    FH_REQUIRE(x.rank == 3 && x.shape[1] != 0);
+    FH_REQUIRE(w.dtype == x.dtype && idx.dtype == FH_U32);
+    uint32_t rows = x.shape[0], routes = x.shape[1], inner = x.shape[2];
+    fh_status status = check_quant_triple(d.inputs[1], d.inputs[2], d.inputs[3], 3, inner, d.bits,
+                                          d.group_size, &columns, &experts);
+    if (status != FH_OK) return status;
+    FH_REQUIRE(shape_is(idx, {rows, routes}) && shape_is(w, {rows, routes}));
+    FH_REQUIRE(shape_is(out, {rows, columns}));
+    FH_REQUIRE(experts <= 4096);
+    if (!execute || rows == 0 || columns == 0) return FH_OK;
+    bool fuse_residual = false;
+    GatherProblem problem{};
+    problem.x = pl.in[0];
+    problem.packed[0] = pl.in[1];
+    problem.scales[0] = pl.in[2];
+    problem.biases[0] = pl.in[3];
+    problem.indices = pl.in[4];
+    problem.weights = pl.in[5];
+    problem.rows = rows;
+    problem.k = routes;
+    problem.inner = inner;
+    problem.experts = experts;
+    problem.columns = columns;
+    problem.bits = d.bits;
+    problem.group = d.group_size;
+    if (!d.epilogue) {
+      problem.out = pl.out[0];
+      if (try_fast_gather_weighted(b, problem, nullptr, error)) return FH_OK;
+      launch_gather_weighted_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4],
+                                     pl.in[5], pl.out[0], rows, routes, inner, experts, columns,
+                                     d.bits, d.group_size, error);
+      return FH_OK;
+    }
+    // Recognised epilogue: out = accumulator + extra (the MoE residual add).
+    auto prog = b->programs.find(d.epilogue);
+    FH_REQUIRE(prog != b->programs.end());
+    fuse_residual = d.accumulator_count == 1 && extras == 1 && is_add_epilogue(prog->second.insts,
+                                                                               prog->second.pairs);
+    if (fuse_residual) {
+      const fh_tensor &residual = d.inputs[primitive];
+      FH_REQUIRE(shape_is(residual, {rows, columns}) && is_float(residual.dtype));
+      problem.out = pl.out[0];
+      if (try_fast_gather_weighted(b, problem, &pl.in[primitive], error)) return FH_OK;
+    }
+    uint64_t elements = (uint64_t)rows * columns;
+    char *acc = b->ensure_workspace(elements * 4);
+    if (!acc) return FH_ALLOCATION_FAILED;
+    View acc_view = contiguous_view(acc, FH_F32, out);
+    launch_gather_weighted_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4],
+                                   pl.in[5], acc_view, rows, routes, inner, experts, columns,
+                                   d.bits, d.group_size, error);
+    return run_epilogue(b, pl, primitive, acc, 1);
+  }
+  // check_gather_quant_projection (ops.rs:1933-1992), once or twice.
+  const fh_tensor &idx = d.inputs[primitive - 1];
+  FH_REQUIRE(x.rank == 2 && idx.dtype == FH_U32 && idx.rank == 2);
+  uint32_t rows = x.shape[0], inner = x.shape[1], k = idx.shape[1];
+  FH_REQUIRE(idx.shape[0] == rows);
+  fh_status status = check_quant_triple(d.inputs[1], d.inputs[2], d.inputs[3], 3, inner, d.bits,
+                                        d.group_size, &columns, &experts);
+  if (status != FH_OK) return status;
+  if (primitive == 8) {
+    uint32_t columns2 = 0, experts2 = 0;
+    status = check_quant_triple(d.inputs[4], d.inputs[5], d.inputs[6], 3, inner, d.bits,
+                                d.group_size, &columns2, &experts2);
+    if (status != FH_OK) return status;
+    FH_REQUIRE(columns2 == columns && experts2 == experts);
+    FH_REQUIRE(d.epilogue != 0 && d.accumulator_count == 2);
+  }
+  FH_REQUIRE(shape_is(out, {rows, k, columns}));
+  FH_REQUIRE(experts <= 4096);
+  if (!execute || rows == 0 || columns == 0 || k == 0) return FH_OK;
+  GatherProblem problem{};
+  problem.x = pl.in[0];
+  problem.packed[0] = pl.in[1];
+  problem.scales[0] = pl.in[2];
+  problem.biases[0] = pl.in[3];
+  if (primitive == 8) {
+    problem.packed[1] = pl.in[4];
+    problem.scales[1] = pl.in[5];
+    problem.biases[1] = pl.in[6];
+  }
+  problem.indices = pl.in[primitive - 1];
+  problem.out = pl.out[0];
+  problem.rows = rows;
+  problem.k = k;
+  problem.inner = inner;
+  problem.experts = experts;
+  problem.columns = columns;
+  problem.bits = d.bits;
+  problem.group = d.group_size;
+  if (!d.epilogue) {
+    if (try_fast_gather_projection(b, problem, 1, false, error)) return FH_OK;
+    launch_gather_projection_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3],
+                                     pl.in[primitive - 1], pl.out[0], rows, inner, experts,
+                                     columns, k, d.bits, d.group_size, error);
+    return FH_OK;
+  }
+  auto prog = b->programs.find(d.epilogue);
+  FH_REQUIRE(prog != b->programs.end());
+  if (primitive == 8 && extras == 0 &&
+      is_swiglu_epilogue(prog->second.insts, prog->second.pairs) &&
+      try_fast_gather_projection(b, problem, 2, true, error))
+    return FH_OK;
+  uint32_t accumulators = primitive == 8 ? 2 : 1;
+  FH_REQUIRE(d.accumulator_count == accumulators);
+  uint64_t elements = (uint64_t)rows * k * columns;
+  char *acc = b->ensure_workspace(elements * 4 * accumulators);
+  if (!acc) return FH_ALLOCATION_FAILED;
+  View acc0 = contiguous_view(acc, FH_F32, out);
+  launch_gather_projection_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3],
+                                   pl.in[primitive - 1], acc0, rows, inner, experts, columns, k,
+                                   d.bits, d.group_size, error);
+  if (primitive == 8) {
+    View acc1 = contiguous_view(acc + elements * 4, FH_F32, out);
+    launch_gather_projection_generic(b->stream, pl.in[0], pl.in[4], pl.in[5], pl.in[6], pl.in[7],
+                                     acc1, rows, inner, experts, columns, k, d.bits, d.group_size,
+                                     error);
+  }
+  return run_epilogue(b, pl, primitive, acc, accumulators);
+}
+
+fh_status plan_top_k(fh_backend *b, const Planned &pl, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_inputs == 1 && d.n_outputs == 2);
+  const fh_tensor &in = d.inputs[0];
+  FH_REQUIRE(is_float(in.dtype) && d.outputs[0].dtype == in.dtype && d.outputs[1].dtype == FH_U32);
+  FH_REQUIRE(in.rank >= 1 && in.rank <= 2);
+  uint32_t width = in.shape[in.rank - 1];
+  FH_REQUIRE(d.k != 0 && d.k <= width && d.k <= 256);
+  uint32_t rows = in.rank == 2 ? in.shape[0] : 1;
+  for (uint32_t o = 0; o < 2; ++o) {
+    FH_REQUIRE(d.outputs[o].rank == in.rank);
+    if (in.rank == 2) FH_REQUIRE(d.outputs[o].shape[0] == rows);
+    FH_REQUIRE(d.outputs[o].shape[in.rank - 1] == d.k);
+  }
+  if (!execute) return FH_OK;
+  View in_v = pl.in[0], val_v = pl.out[0], idx_v = pl.out[1];
+  if (in.rank == 1) {
+    for (View *v : {&in_v, &val_v, &idx_v}) {
+      v->stride[1] = v->stride[0];
+      v->shape[1] = v->shape[0];
+      v->stride[0] = 0;
+      v->shape[0] = 1;
+      v->rank = 2;
+    }
+  }
+  launch_top_k(b->stream, in_v, val_v, idx_v, rows, width, d.k, d.normalize != 0);
+  return FH_OK;
+}
+
+fh_status plan_argmax(fh_backend *b, const Planned &pl, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_inputs == 1 && d.n_outputs == 1);
+  const fh_tensor &in = d.inputs[0], &out = d.outputs[0];
+  FH_REQUIRE(is_float(in.dtype) && out.dtype == FH_U32);
+  FH_REQUIRE(in.rank >= 1 && in.rank <= 2 && in.shape[in.rank - 1] != 0);
+  uint32_t rows = in.rank == 2 ? in.shape[0] : 1;
+  FH_REQUIRE(element_count(out) == rows);
+  if (!execute) return FH_OK;
+  View in_v = pl.in[0];
+  if (in.rank == 1) {
+    in_v.stride[1] = in_v.stride[0];
+    in_v.shape[1] = in_v.shape[0];
+    in_v.stride[0] = 0;
+    in_v.shape[0] = 1;
+    in_v.rank = 2;
+  }
+  launch_argmax(b->stream, in_v, pl.out[0], rows, in.shape[in.rank - 1]);
+  return FH_OK;
+}
+
+fh_status plan_quant_embed(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_inputs == 4 && d.n_outputs == 1);
+  const fh_tensor &packed = d.inputs[0], &ids = d.inputs[3], &out = d.outputs[0];
+  FH_REQUIRE(d.bits == 4 || d.bits == 8);
+  FH_REQUIRE(packed.rank == 2 && packed.dtype == FH_U32 && ids.dtype == FH_U32);
+  uint32_t vocab = packed.shape[0], packed_width = packed.shape[1];
+  uint64_t width64 = (uint64_t)packed_width * (32u / d.bits);
+  FH_REQUIRE(width64 <= 0xffffffffull);
+  uint32_t width = (uint32_t)width64, columns = 0;
+  fh_status status = check_quant_triple(packed, d.inputs[1], d.inputs[2], 2, width, d.bits,
+                                        d.group_size, &columns, nullptr);
+  if (status != FH_OK) return status;
+  FH_REQUIRE(is_float(out.dtype) && out.rank == ids.rank + 1);
+  for (uint32_t axis = 0; axis < ids.rank; ++axis) FH_REQUIRE(out.shape[axis] == ids.shape[axis]);
+  FH_REQUIRE(out.shape[out.rank - 1] == width);
+  if (execute)
+    launch_quant_embed(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0],
+                       (uint32_t)element_count(ids), vocab, packed_width, d.bits, d.group_size,
+                       error);
+  return FH_OK;
+}
+
+fh_status plan_matmul(fh_backend *b, const Planned &pl, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  uint32_t primitive = 2;
+  FH_REQUIRE(d.n_outputs == 1 && d.n_inputs == primitive + (d.epilogue ? d.n_extras : 0));
+  const fh_tensor &l = d.inputs[0], &r = d.inputs[1], &out = d.outputs[0];
+  FH_REQUIRE(is_float(l.dtype) && is_float(r.dtype) && is_float(out.dtype));
+  FH_REQUIRE((l.rank == 2 || l.rank == 3) && r.rank == l.rank && out.rank == l.rank);
+  uint32_t rank = l.rank;
+  uint32_t batches = rank == 3 ? l.shape[0] : 1;
+  uint32_t rows = l.shape[rank - 2], inner = l.shape[rank - 1], columns = r.shape[rank - 1];
+  FH_REQUIRE(r.shape[rank - 2] == inner && inner != 0);
+  if (rank == 3) FH_REQUIRE(r.shape[0] == batches && out.shape[0] == batches);
+  FH_REQUIRE(out.shape[rank - 2] == rows && out.shape[rank - 1] == columns);
+  if (!execute) return FH_OK;
+  if (!d.epilogue) {
+    launch_matmul(b->stream, pl.in[0], pl.in[1], pl.out[0], batches, rows, inner, columns);
+    return FH_OK;
+  }
+  uint64_t elements = element_count(out);
+  char *acc = b->ensure_workspace(elements * 4);
+  if (!acc) return FH_ALLOCATION_FAILED;
+  View acc_view = contiguous_view(acc, FH_F32, out);
+  launch_matmul(b->stream, pl.in[0], pl.in[1], acc_view, batches, rows, inner, columns);
+  return run_epilogue(b, pl, primitive, acc, 1);
+}
+
+fh_status plan_rms_norm(fh_backend *b, const Planned &pl, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_inputs == 2 && d.n_outputs == 1);
+  const fh_tensor &in = d.inputs[0], &w = d.inputs[1], &out = d.outputs[0];
+  FH_REQUIRE(is_float(in.dtype) && is_float(w.dtype) && is_float(out.dtype));
+  FH_REQUIRE(in.rank >= 1 && w.rank == 1 && w.shape[0] == in.shape[in.rank - 1] && w.shape[0] != 0);
+  FH_REQUIRE(out.rank == in.rank);
+  for (uint32_t axis = 0; axis < in.rank; ++axis) FH_REQUIRE(in.shape[axis] == out.shape[axis]);
+  FH_REQUIRE(std::isfinite(d.eps) && d.eps >= 0.0f);
+  if (execute)
+    launch_rms_norm(b->stream, pl.in[0], pl.in[1], pl.out[0],
+                    (uint32_t)(element_count(in) / w.shape[0]), w.shape[0], d.eps);
+  return FH_OK;
+}
+
+fh_status plan_rope(fh_backend *b, const Planned &pl, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_inputs == 2 && d.n_outputs == 1);
+  const fh_tensor &in = d.inputs[0], &pos = d.inputs[1], &out = d.outputs[0];
+  FH_REQUIRE(is_float(in.dtype) && is_float(out.dtype) && pos.dtype == FH_U32);
+  FH_REQUIRE(in.rank == 3 && out.rank == 3 && pos.rank == 1 && pos.shape[0] == in.shape[0]);
+  for (uint32_t axis = 0; axis < 3; ++axis) FH_REQUIRE(in.shape[axis] == out.shape[axis]);
+  FH_REQUIRE(in.shape[2] % 2 == 0 && std::isfinite(d.theta) && d.theta > 0.0f);
+  if (execute)
+    launch_rope(b->stream, pl.in[0], pl.in[1], pl.out[0], in.shape[0], in.shape[1], in.shape[2],
+                d.theta);
+  return FH_OK;
+}
+
+// check_paged_copy (ops.rs:1369-1441).
+fh_status plan_paged_copy(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE((d.n_inputs == 3 || d.n_inputs == 4) && d.n_outputs == 1);
+  bool into = d.direction == 0;
+  FH_REQUIRE(d.direction <= 1);
+  const fh_tensor &ordinary = into ? d.inputs[0] : d.outputs[0];
+  const fh_tensor &pool = into ? d.outputs[0] : d.inputs[0];
+  for (uint32_t i = 1; i < d.n_inputs; ++i) FH_REQUIRE(is_contiguous(d.inputs[i]));
+  FH_REQUIRE(is_contiguous(pool));
+  FH_REQUIRE(is_float(ordinary.dtype) && is_float(pool.dtype));
+  FH_REQUIRE(ordinary.rank >= 2 && pool.rank == 3);
+  uint64_t elements = 1;
+  for (uint32_t axis = 1; axis < ordinary.rank; ++axis) elements *= ordinary.shape[axis];
+  uint32_t tokens = ordinary.shape[0];
+  FH_REQUIRE(elements <= 0xffffffffull && (uint64_t)tokens * elements <= 0xffffffffull);
+  const fh_tensor &table = d.inputs[1], &gens = d.inputs[2];
+  FH_REQUIRE(table.dtype == FH_U32 && table.rank == 2 && table.shape[1] == 2);
+  FH_REQUIRE(gens.dtype == FH_U32 && shape_is(gens, {pool.shape[0]}));
+  if (d.n_inputs == 4) FH_REQUIRE(d.inputs[3].dtype == FH_U32 && shape_is(d.inputs[3], {1}));
+  uint64_t capacity = (uint64_t)table.shape[0] * d.page_tokens;
+  FH_REQUIRE(d.page_tokens != 0 && pool.shape[1] == d.page_tokens && pool.shape[2] == elements);
+  FH_REQUIRE((uint64_t)d.start + tokens <= capacity);
+  if (execute) {
+    const View &ordinary_v = into ? pl.in[0] : pl.out[0];
+    const View &pool_v = into ? pl.out[0] : pl.in[0];
+    launch_paged_copy(b->stream, ordinary_v, pool_v, pl.in[1], pl.in[2],
+                      d.n_inputs == 4 ? pl.in[3] : null_view(), into, tokens, (uint32_t)elements,
+                      d.start, d.page_tokens, pool.shape[0], table.shape[0], error);
+  }
+  return FH_OK;
+}
+
+// check_paged_sdpa (ops.rs:2281-2359) on (q, key pool, value pool, table, generations, activity?).
+fh_status check_paged_attention(const fh_tensor &q, const fh_tensor &kp, const fh_tensor &vp,
+                                const fh_tensor &table, const fh_tensor &gens,
+                                const fh_tensor *activity, const fh_tensor &out, float scale,
+                                bool causal, uint32_t q_start, uint32_t key_length,
+                                uint32_t page_tokens) {
+  FH_REQUIRE(is_contiguous(kp) && is_contiguous(vp) && is_contiguous(table) && is_contiguous(gens));
+  if (activity) FH_REQUIRE(is_contiguous(*activity));
+  FH_REQUIRE(is_float(q.dtype) && is_float(kp.dtype) && vp.dtype == kp.dtype && is_float(out.dtype));
+  FH_REQUIRE(std::isfinite(scale) && page_tokens != 0 && key_length != 0);
+  FH_REQUIRE(q.rank == 3 && kp.rank == 4 && vp.rank == 4 && out.rank == 3);
+  FH_REQUIRE(table.dtype == FH_U32 && table.rank == 2 && table.shape[1] == 2);
+  FH_REQUIRE(gens.dtype == FH_U32 && shape_is(gens, {kp.shape[0]}));
+  if (activity) FH_REQUIRE(activity->dtype == FH_U32 && shape_is(*activity, {1}));
+  uint64_t capacity = (uint64_t)table.shape[0] * page_tokens;
+  FH_REQUIRE(kp.shape[1] == page_tokens && vp.shape[1] == page_tokens);
+  FH_REQUIRE(vp.shape[0] == kp.shape[0] && vp.shape[2] == kp.shape[2]);
+  FH_REQUIRE(kp.shape[3] == q.shape[2] && kp.shape[2] != 0 && q.shape[0] % kp.shape[2] == 0);
+  FH_REQUIRE(q.shape[0] != 0 && key_length <= capacity);
+  if (causal) FH_REQUIRE((uint64_t)q_start + q.shape[1] <= key_length);
+  FH_REQUIRE(shape_is(out, {q.shape[0], q.shape[1], vp.shape[3]}));
+  FH_REQUIRE(q.shape[2] <= 512 && vp.shape[3] <= 256);
+  return FH_OK;
+}
+
+fh_status plan_paged_sdpa(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE((d.n_inputs == 5 || d.n_inputs == 6) && d.n_outputs == 1);
+  const fh_tensor *activity = d.n_inputs == 6 ? &d.inputs[5] : nullptr;
+  fh_status status =
+      check_paged_attention(d.inputs[0], d.inputs[1], d.inputs[2], d.inputs[3], d.inputs[4],
+                            activity, d.outputs[0], d.scale, d.causal != 0, d.q_start,
+                            d.key_length, d.page_tokens);
+  if (status != FH_OK) return status;
+  if (!execute) return FH_OK;
+  const fh_tensor &q = d.inputs[0], &kp = d.inputs[1], &vp = d.inputs[2];
+  LaneAttention lane{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4],
+                     activity ? pl.in[5] : null_view(), pl.out[0], q.shape[0], q.shape[1],
+                     kp.shape[2], q.shape[2], vp.shape[3], d.key_length, d.q_start, d.scale,
+                     d.causal != 0, d.page_tokens, kp.shape[0], d.inputs[3].shape[0]};
+  if (try_fast_lane_attention(b, lane, error)) return FH_OK;
+  launch_paged_sdpa_generic(b->stream, lane.q, lane.key_pool, lane.value_pool, lane.table,
+                            lane.generations, lane.activity, lane.out, lane.query_heads,
+                            lane.query_length, lane.kv_heads, lane.width, lane.value_width,
+                            lane.key_length, lane.query_start, lane.scale, lane.causal,
+                            lane.page_tokens, lane.physical_pages, lane.logical_pages, error);
+  return FH_OK;
+}
+
+// check_paged_append (ops.rs:2236-2278): inputs (q, k_new, v_new, table, generations, activity?),
+// outputs (attention, key pool, value pool).
+fh_status plan_paged_append(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE((d.n_inputs == 5 || d.n_inputs == 6) && d.n_outputs == 3);
+  FH_REQUIRE(d.q_start != 0xffffffffu);
+  const fh_tensor *activity = d.n_inputs == 6 ? &d.inputs[5] : nullptr;
+  const fh_tensor &q = d.inputs[0], &kp = d.outputs[1], &vp = d.outputs[2];
+  fh_status status = check_paged_attention(q, kp, vp, d.inputs[3], d.inputs[4], activity,
+                                           d.outputs[0], d.scale, true, d.q_start, d.q_start + 1,
+                                           d.page_tokens);
+  if (status != FH_OK) return status;
+  FH_REQUIRE(kp.shape[3] == vp.shape[3] && q.shape[1] == 1);
+  FH_REQUIRE(kp.buffer != vp.buffer);
+  for (uint32_t index : {1u, 2u}) {
+    const fh_tensor &pool = d.outputs[index];
+    FH_REQUIRE(d.inputs[index].dtype == q.dtype);
+    FH_REQUIRE(shape_is(d.inputs[index], {1, pool.shape[2], pool.shape[3]}));
+  }
+  if (!execute) return FH_OK;
+  // Store both planes, then attend through them (lib.rs:262-306).
+  View act = activity ? pl.in[5] : null_view();
+  for (uint32_t index : {1u, 2u}) {
+    const fh_tensor &pool = d.outputs[index];
+    launch_paged_copy(b->stream, pl.in[index], pl.out[index], pl.in[3], pl.in[4], act, true, 1,
+                      pool.shape[2] * pool.shape[3], d.q_start, d.page_tokens, pool.shape[0],
+                      d.inputs[3].shape[0], error);
+  }
+  LaneAttention lane{pl.in[0], pl.out[1], pl.out[2], pl.in[3], pl.in[4], act, pl.out[0],
+                     q.shape[0], 1, kp.shape[2], q.shape[2], vp.shape[3], d.q_start + 1,
+                     d.q_start, d.scale, true, d.page_tokens, kp.shape[0], d.inputs[3].shape[0]};
+  if (try_fast_lane_attention(b, lane, error)) return FH_OK;
+  launch_paged_sdpa_generic(b->stream, lane.q, lane.key_pool, lane.value_pool, lane.table,
+                            lane.generations, lane.activity, lane.out, lane.query_heads, 1,
+                            lane.kv_heads, lane.width, lane.value_width, lane.key_length,
+                            lane.query_start, lane.scale, true, lane.page_tokens,
+                            lane.physical_pages, lane.logical_pages, error);
+  return FH_OK;
+}
+
+fh_status plan_ragged(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE((d.n_inputs == 7 || d.n_inputs == 8) && d.n_outputs == 3);
+  const fh_tensor &q = d.inputs[0], &kn = d.inputs[1], &vn = d.inputs[2], &tables = d.inputs[3],
+                  &gens = d.inputs[4], &cu = d.inputs[5], &starts = d.inputs[6];
+  const fh_tensor &out = d.outputs[0], &kp = d.outputs[1], &vp = d.outputs[2];
+  for (uint32_t i = 3; i < d.n_inputs; ++i)
+    FH_REQUIRE(is_contiguous(d.inputs[i]) && d.inputs[i].dtype == FH_U32);
+  FH_REQUIRE(is_contiguous(kp) && is_contiguous(vp) && kp.buffer != vp.buffer);
+  FH_REQUIRE(is_float(q.dtype) && kn.dtype == q.dtype && vn.dtype == q.dtype);
+  FH_REQUIRE(is_float(kp.dtype) && vp.dtype == kp.dtype && is_float(out.dtype));
+  FH_REQUIRE(q.rank == 3 && kn.rank == 3 && vn.rank == 3 && out.rank == 3);
+  FH_REQUIRE(kp.rank == 4 && vp.rank == 4 && tables.rank == 3 && tables.shape[2] == 2);
+  uint32_t tokens = q.shape[0], lanes = tables.shape[0];
+  FH_REQUIRE(lanes != 0 && shape_is(cu, {lanes + 1}) && shape_is(starts, {lanes}));
+  if (d.n_inputs == 8) FH_REQUIRE(shape_is(d.inputs[7], {lanes}));
+  FH_REQUIRE(shape_is(gens, {kp.shape[0]}));
+  FH_REQUIRE(std::isfinite(d.scale) && d.page_tokens != 0);
+  FH_REQUIRE(kp.shape[1] == d.page_tokens && vp.shape[1] == d.page_tokens);
+  FH_REQUIRE(vp.shape[0] == kp.shape[0] && vp.shape[2] == kp.shape[2]);
+  FH_REQUIRE(kp.shape[2] != 0 && q.shape[1] % kp.shape[2] == 0 && q.shape[1] != 0);
+  FH_REQUIRE(kp.shape[3] == q.shape[2]);
+  FH_REQUIRE(shape_is(kn, {tokens, kp.shape[2], kp.shape[3]}));
+  FH_REQUIRE(shape_is(vn, {tokens, vp.shape[2], vp.shape[3]}));
+  FH_REQUIRE(shape_is(out, {tokens, q.shape[1], vp.shape[3]}));
+  FH_REQUIRE(q.shape[2] <= 512 && vp.shape[3] <= 256);
+  if (!execute || tokens == 0) return FH_OK;
+  RaggedAttention problem{};
+  problem.q = pl.in[0];
+  problem.k_new = pl.in[1];
+  problem.v_new = pl.in[2];
+  problem.tables = pl.in[3];
+  problem.generations = pl.in[4];
+  problem.cu_seqlens = pl.in[5];
+  problem.q_starts = pl.in[6];
+  problem.activity = d.n_inputs == 8 ? pl.in[7] : null_view();
+  problem.out = pl.out[0];
+  problem.key_pool = pl.out[1];
+  problem.value_pool = pl.out[2];
+  problem.tokens = tokens;
+  problem.lanes = lanes;
+  problem.query_heads = q.shape[1];
+  problem.kv_heads = kp.shape[2];
+  problem.width = q.shape[2];
+  problem.value_width = vp.shape[3];
+  problem.page_tokens = d.page_tokens;
+  problem.physical_pages = kp.shape[0];
+  problem.table_pages = tables.shape[1];
+  problem.scale = d.scale;
+  if (!run_ragged_attention(b, problem, error)) return FH_ALLOCATION_FAILED;
+  return FH_OK;
+}
+
+fh_status plan_route_pack(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_inputs == 1 && d.n_outputs == 4);
+  const fh_tensor &idx = d.inputs[0];
+  FH_REQUIRE(idx.dtype == FH_U32 && idx.rank == 2);
+  for (uint32_t o = 0; o < 4; ++o)
+    FH_REQUIRE(d.outputs[o].dtype == FH_U32 && is_contiguous(d.outputs[o]));
+  uint32_t experts = d.outputs[0].shape[0];
+  FH_REQUIRE(d.outputs[0].rank == 1 && experts != 0 && experts <= 4096);
+  FH_REQUIRE(shape_is(d.outputs[1], {experts + 1}));
+  uint64_t routes = (uint64_t)idx.shape[0] * idx.shape[1];
+  FH_REQUIRE(routes <= (1u << 24) && shape_is(d.outputs[2], {(uint32_t)routes}));
+  FH_REQUIRE(d.outputs[3].rank == 2 && d.outputs[3].shape[1] == 3 && d.k != 0);
+  uint32_t max_blocks = d.outputs[3].shape[0];
+  FH_REQUIRE(max_blocks >= experts + routes / d.k);
+  if (!execute) return FH_OK;
+  char *ws = b->ensure_workspace(256);
+  if (!ws) return FH_ALLOCATION_FAILED;
+  auto ptr = [](const View &v) { return (uint32_t *)v.base + v.offset; };
+  launch_route_pack(b->stream, pl.in[0], idx.shape[0], idx.shape[1], experts, d.k, ptr(pl.out[0]),
+                    ptr(pl.out[1]), ptr(pl.out[2]), ptr(pl.out[3]), max_blocks, (uint32_t *)ws,
+                    error);
+  return FH_OK;
+}
+
+fh_status plan_fill(fh_backend *b, const Planned &pl, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  FH_REQUIRE(d.n_inputs == 0 && d.n_outputs == 1 && d.k <= 2);
+  const fh_tensor &out = d.outputs[0];
+  FH_REQUIRE(is_contiguous(out));
+  if (d.k == 0)
+    FH_REQUIRE(out.dtype == FH_U32);
+  else
+    FH_REQUIRE(is_float(out.dtype));
+  if (execute) {
+    uint64_t seed = (uint64_t)d.q_start | ((uint64_t)d.key_length << 32);
+    launch_fill_seeded(b->stream, pl.out[0], element_count(out), d.k, seed, d.start, d.direction,
+                       d.scale, d.eps);
+  }
+  return FH_OK;
+}
+
+uint32_t kernel_class_of(uint32_t op) {
+  switch (op) {
+  case FH_OP_QUANT_MATMUL: return FH_KC_QMM;
+  case FH_OP_GATHER_QUANT_MATMUL: return FH_KC_MOE;
+  case FH_OP_PAGED_SDPA:
+  case FH_OP_PAGED_SDPA_APPEND:
+  case FH_OP_PAGED_ATTENTION_RAGGED: return FH_KC_ATTENTION;
+  default: return FH_KC_OTHER;
+  }
+}
+
+// Validates one dispatch and, when `execute`, enqueues it.
+fh_status process(fh_backend *b, const fh_dispatch &d, ErrorSlot *error, bool execute) {
+  FH_REQUIRE(d.n_inputs <= FH_MAX_INPUTS && d.n_outputs <= FH_MAX_OUTPUTS && d.n_outputs >= 1);
+  Planned pl;
+  pl.d = &d;
+  for (uint32_t i = 0; i < d.n_inputs; ++i) {
+    fh_status status = make_view(b, d.inputs[i], false, &pl.in[i]);
+    if (status != FH_OK) return status;
+  }
+  for (uint32_t i = 0; i < d.n_outputs; ++i) {
+    fh_status status = make_view(b, d.outputs[i], true, &pl.out[i]);
+    if (status != FH_OK) return status;
+  }
+  // Outputs must not alias inputs or each other (check_common, ops.rs:1300-1344): conservative
+  // whole-span test per allocation.
+  auto span_of = [](const fh_tensor &t, uint64_t *lo, uint64_t *hi) {
+    uint64_t reach = t.offset;
+    for (uint32_t axis = 0; axis < t.rank; ++axis) {
+      if (t.shape[axis] == 0) {
+        *lo = *hi = 0;
+        return;
+      }
+      reach += (uint64_t)(t.shape[axis] - 1) * t.stride[axis];
+    }
+    *lo = t.offset * dtype_size(t.dtype);
+    *hi = (reach + 1) * dtype_size(t.dtype);
+  };
+  for (uint32_t o = 0; o < d.n_outputs; ++o) {
+    uint64_t olo, ohi;
+    span_of(d.outputs[o], &olo, &ohi);
+    if (olo == ohi) continue;
+    for (uint32_t i = 0; i < d.n_inputs; ++i) {
+      if (d.inputs[i].buffer != d.outputs[o].buffer) continue;
+      uint64_t ilo, ihi;
+      span_of(d.inputs[i], &ilo, &ihi);
+      FH_REQUIRE(ihi <= olo || ohi <= ilo);
+    }
+    for (uint32_t other = o + 1; other < d.n_outputs; ++other) {
+      if (d.outputs[other].buffer != d.outputs[o].buffer) continue;
+      uint64_t ilo, ihi;
+      span_of(d.outputs[other], &ilo, &ihi);
+      FH_REQUIRE(ihi <= olo || ohi <= ilo);
+    }
+  }
+  switch (d.op) {
+  case FH_OP_PROGRAM: return plan_program(b, pl, execute);
+  case FH_OP_COPY: return plan_copy(b, pl, execute);
+  case FH_OP_PAGED_COPY: return plan_paged_copy(b, pl, error, execute);
+  case FH_OP_RMS_NORM: return plan_rms_norm(b, pl, execute);
+  case FH_OP_ARGMAX: return plan_argmax(b, pl, execute);
+  case FH_OP_TOP_K: return plan_top_k(b, pl, execute);
+  case FH_OP_ROPE: return plan_rope(b, pl, execute);
+  case FH_OP_QUANT_EMBED: return plan_quant_embed(b, pl, error, execute);
+  case FH_OP_MATMUL: return plan_matmul(b, pl, execute);
+  case FH_OP_QUANT_MATMUL: return plan_quant_matmul(b, pl, error, execute);
+  case FH_OP_GATHER_QUANT_MATMUL: return plan_gather(b, pl, error, execute);
+  case FH_OP_PAGED_SDPA_APPEND: return plan_paged_append(b, pl, error, execute);
+  case FH_OP_PAGED_SDPA: return plan_paged_sdpa(b, pl, error, execute);
+  case FH_OP_PAGED_ATTENTION_RAGGED: return plan_ragged(b, pl, error, execute);
+  case FH_OP_ROUTE_PACK: return plan_route_pack(b, pl, error, execute);
+  case FH_OP_FILL_SEEDED: return plan_fill(b, pl, execute);
+  default: return FH_UNSUPPORTED_OPERATION;
+  }
+}
+
+hipEvent_t take_event(fh_backend *b) {
+  if (!b->event_pool.empty()) {
+    hipEvent_t e = b->event_pool.back();
+    b->event_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+
+void drain_profile(fh_backend *b) {
+  for (auto &t : b->timed) {
+    float ms = 0.0f;
+    if (hipEventElapsedTime(&ms, t.start, t.end) == hipSuccess) {
+      b->class_ns[t.kernel_class] += (uint64_t)((double)ms * 1e6);
+      b->class_launches[t.kernel_class] += 1;
+    }
+    b->event_pool.push_back(t.start);
+    b->event_pool.push_back(t.end);
+  }
+  b->timed.clear();
+}
+
+}  // namespace
+
+// ================================================================== C ABI
+
+extern "C" {
+
+const char *fh_version(void) { return "forja-hip 0.1 (gfx950)"; }
+
+fh_status fh_create(int device, fh_backend **out) {
+  if (!out) return FH_INVALID_INPUT;
+  *out = nullptr;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count)
+    return FH_DEVICE_EXECUTION_FAILED;
+  fh_backend *b = new (std::nothrow) fh_backend();
+  if (!b) return FH_ALLOCATION_FAILED;
+  b->device = device;
+  if (hipSetDevice(device) != hipSuccess || hipGetDeviceProperties(&b->props, device) != hipSuccess ||
+      hipStreamCreate(&b->stream) != hipSuccess) {
+    delete b;
+    return FH_DEVICE_EXECUTION_FAILED;
+  }
+  *out = b;
+  return FH_OK;
+}
+
+void fh_destroy(fh_backend *b) {
+  if (!b) return;
+  {
+    std::lock_guard<std::mutex> lock(b->mutex);
+    (void)hipSetDevice(b->device);
+    (void)hipStreamSynchronize(b->stream);
+    for (auto &entry : b->allocations) (void)hipFree(entry.second.ptr);
+    for (auto &entry : b->programs)
+      for (auto &typed : entry.second.typed) (void)hipFree(typed.second);
+    if (b->workspace) (void)hipFree(b->workspace);
+    for (auto &t : b->timed) {
+      (void)hipEventDestroy(t.start);
+      (void)hipEventDestroy(t.end);
+    }
+    for (auto e : b->event_pool) (void)hipEventDestroy(e);
+    (void)hipStreamDestroy(b->stream);
+  }
+  delete b;
+}
+
+static fh_status alloc_locked(fh_backend *b, uint64_t bytes, bool readonly, fh_buffer *out) {
+  void *ptr = nullptr;
+  uint64_t want = bytes == 0 ? 256 : bytes;
+  if (hipMalloc(&ptr, want) != hipSuccess) return FH_ALLOCATION_FAILED;
+  if (hipMemsetAsync(ptr, 0, want, b->stream) != hipSuccess) {
+    (void)hipFree(ptr);
+    return FH_DEVICE_EXECUTION_FAILED;
+  }
+  uint64_t id = b->next_id++;
+  b->allocations[id] = Allocation{(char *)ptr, bytes, readonly};
+  b->used_bytes += bytes;
+  *out = id;
+  return FH_OK;
+}
+
+fh_status fh_alloc(fh_backend *b, uint64_t bytes, fh_buffer *out) {
+  if (!b || !out) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  return alloc_locked(b, bytes, false, out);
+}
+
+fh_status fh_release(fh_backend *b, fh_buffer buffer) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  auto it = b->allocations.find(buffer);
+  if (it == b->allocations.end()) return FH_INVALID_INPUT;
+  (void)hipSetDevice(b->device);
+  (void)hipStreamSynchronize(b->stream);
+  (void)hipFree(it->second.ptr);
+  b->used_bytes -= it->second.bytes;
+  b->allocations.erase(it);
+  return FH_OK;
+}
+
+fh_status fh_import(fh_backend *b, const void *bytes, uint64_t len, fh_buffer *out) {
+  if (!b || !out || (!bytes && len)) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  fh_status status = alloc_locked(b, len, true, out);
+  if (status != FH_OK) return status;
+  if (len && hipMemcpyAsync(b->allocations[*out].ptr, bytes, len, hipMemcpyHostToDevice,
+                            b->stream) != hipSuccess)
+    return FH_DEVICE_EXECUTION_FAILED;
+  if (hipStreamSynchronize(b->stream) != hipSuccess) return FH_DEVICE_EXECUTION_FAILED;
+  return FH_OK;
+}
+
+fh_status fh_write(fh_backend *b, fh_buffer buffer, uint64_t byte_offset, const void *bytes,
+                   uint64_t len) {
+  if (!b || (!bytes && len)) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  auto it = b->allocations.find(buffer);
+  if (it == b->allocations.end() || it->second.readonly) return FH_INVALID_INPUT;
+  if (byte_offset > it->second.bytes || len > it->second.bytes - byte_offset)
+    return FH_INVALID_INPUT;
+  if (len == 0) return FH_OK;
+  (void)hipSetDevice(b->device);
+  if (hipMemcpyAsync(it->second.ptr + byte_offset, bytes, len, hipMemcpyHostToDevice, b->stream) !=
+      hipSuccess)
+    return FH_DEVICE_EXECUTION_FAILED;
+  // The caller's bytes may be reused as soon as this returns.
+  if (hipStreamSynchronize(b->stream) != hipSuccess) return FH_DEVICE_EXECUTION_FAILED;
+  return FH_OK;
+}
+
+fh_status fh_read(fh_backend *b, fh_buffer buffer, uint64_t byte_offset, void *bytes,
+                  uint64_t len) {
+  if (!b || (!bytes && len)) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  auto it = b->allocations.find(buffer);
+  if (it == b->allocations.end()) return FH_INVALID_INPUT;
+  if (byte_offset > it->second.bytes || len > it->second.bytes - byte_offset)
+    return FH_INVALID_INPUT;
+  if (len == 0) return FH_OK;
+  (void)hipSetDevice(b->device);
+  if (hipMemcpyAsync(bytes, it->second.ptr + byte_offset, len, hipMemcpyDeviceToHost, b->stream) !=
+      hipSuccess)
+    return FH_DEVICE_EXECUTION_FAILED;
+  if (hipStreamSynchronize(b->stream) != hipSuccess) return FH_DEVICE_EXECUTION_FAILED;
+  return FH_OK;
+}
+
+fh_status fh_read_tensor(fh_backend *b, const fh_tensor *tensor, void *bytes, uint64_t len) {
+  if (!b || !tensor || (!bytes && len)) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  View view;
+  fh_status status = make_view(b, *tensor, false, &view);
+  if (status != FH_OK) return status;
+  uint64_t elements = element_count(*tensor);
+  uint64_t size = dtype_size(tensor->dtype);
+  if (len != elements * size) return FH_INVALID_INPUT;
+  if (elements == 0) return FH_OK;
+  char *staging = b->ensure_workspace(elements * size);
+  if (!staging) return FH_ALLOCATION_FAILED;
+  // Gather on the device as a same-dtype copy into contiguous staging.
+  View flat = contiguous_view(staging, tensor->dtype, *tensor);
+  View source = view;
+  if (tensor->dtype == FH_I32) {
+    source.dtype = FH_U32;
+    flat.dtype = FH_U32;
+  }
+  if (is_float(tensor->dtype) && tensor->dtype != FH_F32) {
+    // 16-bit payloads are moved as raw bits by viewing them as u16 pairs is not possible with
+    // arbitrary strides; the float path round-trips exactly (f16/bf16 -> f32 -> same dtype).
+  }
+  launch_copy(b->stream, source, flat, elements);
+  if (hipMemcpyAsync(bytes, staging, elements * size, hipMemcpyDeviceToHost, b->stream) !=
+      hipSuccess)
+    return FH_DEVICE_EXECUTION_FAILED;
+  if (hipStreamSynchronize(b->stream) != hipSuccess) return FH_DEVICE_EXECUTION_FAILED;
+  return FH_OK;
+}
+
+fh_status fh_prepare_program(fh_backend *b, uint32_t kind, const fh_inst *insts, uint32_t n_insts,
+                             const uint32_t *outputs, uint32_t n_pairs, fh_program *out) {
+  if (!b || !insts || !outputs || !out) return FH_INVALID_INPUT;
+  if (kind > 1 || n_insts == 0 || n_insts > 256 || n_pairs == 0 || n_pairs > kMaxProgramOutputs)
+    return FH_INVALID_INPUT;
+  Program p;
+  p.kind = kind;
+  p.insts.assign(insts, insts + n_insts);
+  p.pairs.assign(outputs, outputs + 2 * n_pairs);
+  uint32_t max_input = 0, max_output = 0;
+  bool any_input = false;
+  for (const fh_inst &inst : p.insts) {
+    if (inst.kind > 8) return FH_INVALID_INPUT;
+    if (inst.kind == 0) {
+      if (inst.a >= kMaxProgramInputs) return FH_INVALID_INPUT;
+      max_input = std::max(max_input, inst.a);
+      any_input = true;
+    }
+    if (inst.kind == 8) {
+      if (kind != 1) return FH_INVALID_INPUT;
+      p.n_reduce += 1;
+    }
+  }
+  if (p.n_reduce > kMaxReductions) return FH_INVALID_INPUT;
+  std::vector<bool> seen(kMaxProgramOutputs, false);
+  for (uint32_t pair = 0; pair < n_pairs; ++pair) {
+    uint32_t slot = outputs[2 * pair];
+    if (slot >= kMaxProgramOutputs || seen[slot] || outputs[2 * pair + 1] >= n_insts)
+      return FH_INVALID_INPUT;
+    seen[slot] = true;
+    max_output = std::max(max_output, slot);
+  }
+  p.n_inputs = any_input ? max_input + 1 : 0;
+  p.n_outputs = max_output + 1;
+  for (uint32_t slot = 0; slot < p.n_outputs; ++slot)
+    if (!seen[slot]) return FH_INVALID_INPUT;
+  // Structural check with every input assumed f32; u32 bindings are re-typed at dispatch.
+  std::vector<DInst> typed;
+  fh_status status = type_program(p, 0, FH_MAX_RANK, &typed);
+  if (status != FH_OK) {
+    // A program whose integer inputs make the all-f32 typing fail is still legal; defer.
+    bool uses_index_math = false;
+    for (const fh_inst &inst : p.insts)
+      if (inst.kind == 0) uses_index_math = true;
+    if (!uses_index_math) return status;
+  }
+  std::lock_guard<std::mutex> lock(b->mutex);
+  uint64_t id = b->next_id++;
+  b->programs[id] = std::move(p);
+  *out = id;
+  return FH_OK;
+}
+
+fh_status fh_release_program(fh_backend *b, fh_program program) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  auto it = b->programs.find(program);
+  if (it == b->programs.end()) return FH_INVALID_INPUT;
+  (void)hipSetDevice(b->device);
+  (void)hipStreamSynchronize(b->stream);
+  for (auto &typed : it->second.typed) (void)hipFree(typed.second);
+  b->programs.erase(it);
+  return FH_OK;
+}
+
+fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count,
+                    fh_submission **out) {
+  if (!b || !out || (!dispatches && count)) return FH_INVALID_INPUT;
+  *out = nullptr;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  // Validate the whole list before anything is enqueued (lib.rs:1423-1432).
+  for (uint32_t i = 0; i < count; ++i) {
+    fh_status status = process(b, dispatches[i], nullptr, false);
+    if (status != FH_OK) return status;
+  }
+  fh_submission *s = new (std::nothrow) fh_submission();
+  if (!s) return FH_ALLOCATION_FAILED;
+  s->backend = b;
+  s->serial = b->next_serial++;
+  s->count = count;
+  s->ops.resize(count);
+  uint32_t slots = count == 0 ? 1 : count;
+  void *dev = nullptr, *host = nullptr;
+  if (hipMalloc(&dev, slots * sizeof(ErrorSlot)) != hipSuccess ||
+      hipHostMalloc(&host, slots * sizeof(ErrorSlot), hipHostMallocDefault) != hipSuccess ||
+      hipEventCreate(&s->start) != hipSuccess || hipEventCreate(&s->end) != hipSuccess) {
+    if (dev) (void)hipFree(dev);
+    if (host) (void)hipHostFree(host);
+    delete s;
+    return FH_ALLOCATION_FAILED;
+  }
+  s->device_errors = (ErrorSlot *)dev;
+  s->host_errors = (ErrorSlot *)host;
+  launch_init_errors(b->stream, s->device_errors, slots);
+  (void)hipEventRecord(s->start, b->stream);
+  fh_status status = FH_OK;
+  for (uint32_t i = 0; i < count && status == FH_OK; ++i) {
+    s->ops[i] = dispatches[i].op;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    if (b->profiling) {
+      t0 = take_event(b);
+      t1 = take_event(b);
+      (void)hipEventRecord(t0, b->stream);
+    }
+    status = process(b, dispatches[i], &s->device_errors[i], true);
+    if (b->profiling) {
+      (void)hipEventRecord(t1, b->stream);
+      b->timed.push_back({t0, t1, kernel_class_of(dispatches[i].op)});
+    }
+  }
+  (void)hipEventRecord(s->end, b->stream);
+  (void)hipMemcpyAsync(s->host_errors, s->device_errors, slots * sizeof(ErrorSlot),
+                       hipMemcpyDeviceToHost, b->stream);
+  if (status != FH_OK) {
+    (void)hipStreamSynchronize(b->stream);
+    (void)hipFree(s->device_errors);
+    (void)hipHostFree(s->host_errors);
+    (void)hipEventDestroy(s->start);
+    (void)hipEventDestroy(s->end);
+    delete s;
+    return status;
+  }
+  hipError_t launch_error = hipGetLastError();
+  if (launch_error != hipSuccess) {
+    s->result = FH_DEVICE_EXECUTION_FAILED;
+    s->error.code = FH_DEVICE_EXECUTION_FAILED;
+    s->error.submission = s->serial;
+    s->error.value = (uint32_t)launch_error;
+  }
+  *out = s;
+  return FH_OK;
+}
+
+fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
+  if (!s) return FH_INVALID_INPUT;
+  fh_backend *b = s->backend;
+  if (!s->waited) {
+    // The trailing async copy of the error slots is the last work of the submission; a pinned
+    // target makes stream synchronisation the completion point.
+    if (timeout_ns != 0) {
+      auto deadline = std::chrono::steady_clock::now() + std::chrono::nanoseconds(timeout_ns);
+      for (;;) {
+        hipError_t q;
+        {
+          std::lock_guard<std::mutex> lock(b->mutex);
+          (void)hipSetDevice(b->device);
+          q = hipStreamQuery(b->stream);
+        }
+        if (q == hipSuccess) break;
+        if (q != hipErrorNotReady) {
+          s->result = FH_DEVICE_EXECUTION_FAILED;
+          break;
+        }
+        if (std::chrono::steady_clock::now() >= deadline) {
+          if (error) {
+            memset(error, 0, sizeof(*error));
+            error->code = FH_TIMEOUT;
+            error->submission = s->serial;
+          }
+          return FH_TIMEOUT;
+        }
+        std::this_thread::sleep_for(std::chrono::microseconds(50));
+      }
+    }
+    std::lock_guard<std::mutex> lock(b->mutex);
+    (void)hipSetDevice(b->device);
+    hipError_t sync = hipStreamSynchronize(b->stream);
+    s->waited = true;
+    if (sync != hipSuccess) {
+      s->result = FH_DEVICE_EXECUTION_FAILED;
+      s->error.code = FH_DEVICE_EXECUTION_FAILED;
+      s->error.submission = s->serial;
+      s->error.value = (uint32_t)sync;
+    } else if (s->result == FH_OK) {
+      float ms = 0.0f;
+      if (hipEventElapsedTime(&ms, s->start, s->end) == hipSuccess)
+        s->gpu_ns = (uint64_t)((double)ms * 1e6);
+      for (uint32_t i = 0; i < s->count; ++i) {
+        if (!s->host_errors[i].flag) continue;
+        uint32_t op = s->ops[i];
+        bool index_error = op == FH_OP_GATHER_QUANT_MATMUL || op == FH_OP_QUANT_EMBED ||
+                           op == FH_OP_ROUTE_PACK;
+        s->result = index_error ? FH_INDEX_OUT_OF_RANGE : FH_DEVICE_ERROR_FLAG;
+        s->error.code = s->result;
+        s->error.dispatch = i;
+        s->error.submission = s->serial;
+        s->error.operation = op;
+        s->error.flag = s->host_errors[i].flag;
+        s->error.value = s->host_errors[i].value;
+        break;
+      }
+    }
+    if (b->profiling) drain_profile(b);
+  }
+  if (error) {
+    *error = s->error;
+    error->code = s->result;
+    error->submission = s->serial;
+  }
+  return s->result;
+}
+
+uint64_t fh_gpu_time_ns(fh_submission *s) { return s ? s->gpu_ns : 0; }
+
+void fh_submission_free(fh_submission *s) {
+  if (!s) return;
+  fh_backend *b = s->backend;
+  {
+    std::lock_guard<std::mutex> lock(b->mutex);
+    (void)hipSetDevice(b->device);
+    if (!s->waited) (void)hipStreamSynchronize(b->stream);
+    (void)hipFree(s->device_errors);
+    (void)hipHostFree(s->host_errors);
+    (void)hipEventDestroy(s->start);
+    (void)hipEventDestroy(s->end);
+  }
+  delete s;
+}
+
+fh_status fh_device_info_get(fh_backend *b, fh_device_info *out) {
+  if (!b || !out) return FH_INVALID_INPUT;
+  memset(out, 0, sizeof(*out));
+  snprintf(out->family, sizeof(out->family), "%s", b->props.gcnArchName);
+  out->total_memory = b->props.totalGlobalMem;
+  out->lds_bytes = b->props.sharedMemPerBlock;
+  out->compute_units = (uint32_t)b->props.multiProcessorCount;
+  out->wavefront = (uint32_t)b->props.warpSize;
+  return FH_OK;
+}
+
+fh_status fh_memory_usage(fh_backend *b, uint64_t *bytes) {
+  if (!b || !bytes) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  *bytes = b->used_bytes + b->workspace_bytes;
+  return FH_OK;
+}
+
+fh_status fh_synchronize(fh_backend *b) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  if (hipStreamSynchronize(b->stream) != hipSuccess) return FH_DEVICE_EXECUTION_FAILED;
+  if (b->profiling) drain_profile(b);
+  return FH_OK;
+}
+
+fh_status fh_profile_enable(fh_backend *b, int enabled) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  (void)hipStreamSynchronize(b->stream);
+  drain_profile(b);
+  b->profiling = enabled != 0;
+  return FH_OK;
+}
+
+fh_status fh_profile_reset(fh_backend *b) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  (void)hipStreamSynchronize(b->stream);
+  drain_profile(b);
+  for (int c = 0; c < FH_KC_COUNT; ++c) {
+    b->class_ns[c] = 0;
+    b->class_launches[c] = 0;
+  }
+  return FH_OK;
+}
+
+fh_status fh_profile_read(fh_backend *b, uint32_t kernel_class, uint64_t *nanoseconds,
+                          uint64_t *launches) {
+  if (!b || kernel_class >= FH_KC_COUNT || !nanoseconds || !launches) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  (void)hipStreamSynchronize(b->stream);
+  drain_profile(b);
+  *nanoseconds = b->class_ns[kernel_class];
+  *launches = b->class_launches[kernel_class];
+  return FH_OK;
+}
+
+}  // extern "C"
+
+namespace fh {
+char *backend_workspace(fh_backend *backend, uint64_t bytes) { return backend->ensure_workspace(bytes); }
+hipStream_t backend_stream(fh_backend *backend) { return backend->stream; }
+uint32_t backend_compute_units(fh_backend *backend) {
+  return (uint32_t)backend->props.multiProcessorCount;
+}
+}  // namespace fh

@@ -1,0 +1,67 @@
+// Specialised gfx950 kernels for the hot shapes of the ragged forward step.  Each `try_fast_*`
+// inspects the operand layouts and either enqueues the specialised kernel and returns true, or
+// returns false so the caller falls back to the strided generic kernel.
+#pragma once
+
+#include <vector>
+
+#include "kernels.hpp"
+
+struct fh_backend;
+
+namespace fh {
+
+// Implemented in backend.cpp.
+char *backend_workspace(fh_backend *backend, uint64_t bytes);
+hipStream_t backend_stream(fh_backend *backend);
+uint32_t backend_compute_units(fh_backend *backend);
+
+struct QmmProblem {
+  View x, packed, scales, biases, out;
+  uint32_t rows, inner, columns, bits, group;
+};
+bool try_fast_quant_matmul(hipStream_t stream, const QmmProblem &problem);
+
+struct GatherProblem {
+  View x;           // projection: [R,K]; weighted sum: [R,k,K]
+  View packed[2], scales[2], biases[2];
+  View indices;     // [R,k]
+  View weights;     // weighted sum only: [R,k]
+  View out;         // projection: [R,k,N]; weighted sum: [R,N]
+  uint32_t rows, k, inner, experts, columns, bits, group;
+};
+// projections = 1 (plain) or 2 (gate/up pair); swiglu = fuse silu(acc0)*acc1.
+bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &problem, int projections,
+                                bool swiglu, ErrorSlot *error);
+// residual may be null; otherwise out = residual + sum.
+bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &problem,
+                              const View *residual, ErrorSlot *error);
+
+struct LaneAttention {
+  View q, key_pool, value_pool, table, generations, activity, out;
+  uint32_t query_heads, query_length, kv_heads, width, value_width, key_length, query_start;
+  float scale;
+  bool causal;
+  uint32_t page_tokens, physical_pages, logical_pages;
+};
+bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, ErrorSlot *error);
+
+struct RaggedAttention {
+  View q, k_new, v_new, tables, generations, cu_seqlens, q_starts, activity;
+  View out, key_pool, value_pool;
+  uint32_t tokens, lanes, query_heads, kv_heads, width, value_width, page_tokens, physical_pages,
+      table_pages;
+  float scale;
+};
+// Always handles the problem (specialised kernel when the layout allows, generic otherwise);
+// false only when workspace allocation fails.
+bool run_ragged_attention(fh_backend *backend, const RaggedAttention &problem, ErrorSlot *error);
+
+bool try_fast_program(hipStream_t stream, bool row, const ProgramArgs &args, uint64_t elements);
+
+// Epilogue recognisers: `acc + extra` and `silu(acc0) * acc1` in the instruction orders the SDK
+// emits (crates/forja-sdk/src/nn/blocks.rs:406-416) and commuted variants.
+bool is_add_epilogue(const std::vector<fh_inst> &insts, const std::vector<uint32_t> &pairs);
+bool is_swiglu_epilogue(const std::vector<fh_inst> &insts, const std::vector<uint32_t> &pairs);
+
+}  // namespace fh

@@ -1,0 +1,93 @@
+// Host-callable launchers for every kernel in libforja_hip.  Each launcher assumes the caller
+// (backend.cpp) has already validated operand shapes; none allocates or synchronises.
+#pragma once
+
+#include "common.hpp"
+
+namespace fh {
+
+// Device form of one Program IR instruction: the host validator resolves operand types so the
+// interpreter needs no dynamic typing.  ty = value type of operand `a` (0 f32, 1 u32, 2 bool).
+struct DInst {
+  uint8_t kind, op, ty, pad;
+  uint32_t a, b, c;
+};
+
+constexpr int kMaxProgramInputs = 8;
+constexpr int kMaxProgramOutputs = 4;
+constexpr int kMaxReductions = 4;
+
+struct ProgramArgs {
+  const DInst *insts;
+  uint32_t n_insts;
+  uint32_t n_inputs;
+  uint32_t n_pairs;
+  uint32_t rank;
+  uint32_t shape[FH_MAX_RANK];
+  uint32_t out_slot[kMaxProgramOutputs];
+  uint32_t out_value[kMaxProgramOutputs];
+  uint32_t n_reduce;
+  uint32_t reduce_at[kMaxReductions];
+  View inputs[kMaxProgramInputs];
+  View outputs[kMaxProgramOutputs];
+};
+
+// ---- generic_ops.hip: strided, any-dtype kernels that follow the reference loop order ----
+void launch_copy(hipStream_t s, const View &in, const View &out, uint64_t elements);
+void launch_program(hipStream_t s, const ProgramArgs &args, bool row, uint64_t elements);
+void launch_quant_matmul_generic(hipStream_t s, const View &x, const View &packed,
+                                 const View &scales, const View &biases, const View &out,
+                                 uint32_t rows, uint32_t inner, uint32_t columns, uint32_t bits,
+                                 uint32_t group);
+// projection: out [R,k,N]; `experts` bounds the ids; bad routes give zero rows + error.
+void launch_gather_projection_generic(hipStream_t s, const View &x, const View &packed,
+                                      const View &scales, const View &biases, const View &indices,
+                                      const View &out, uint32_t rows, uint32_t inner,
+                                      uint32_t experts, uint32_t columns, uint32_t k,
+                                      uint32_t bits, uint32_t group, ErrorSlot *error);
+void launch_gather_weighted_generic(hipStream_t s, const View &x, const View &packed,
+                                    const View &scales, const View &biases, const View &indices,
+                                    const View &weights, const View &out, uint32_t rows,
+                                    uint32_t routes, uint32_t inner, uint32_t experts,
+                                    uint32_t columns, uint32_t bits, uint32_t group,
+                                    ErrorSlot *error);
+void launch_top_k(hipStream_t s, const View &in, const View &values, const View &indices,
+                  uint32_t rows, uint32_t width, uint32_t k, bool normalize);
+void launch_argmax(hipStream_t s, const View &in, const View &out, uint32_t rows, uint32_t width);
+void launch_quant_embed(hipStream_t s, const View &packed, const View &scales,
+                        const View &biases, const View &ids, const View &out, uint32_t id_count,
+                        uint32_t vocab, uint32_t packed_width, uint32_t bits, uint32_t group,
+                        ErrorSlot *error);
+void launch_matmul(hipStream_t s, const View &left, const View &right, const View &out,
+                   uint32_t batches, uint32_t rows, uint32_t inner, uint32_t columns);
+void launch_rms_norm(hipStream_t s, const View &in, const View &weight, const View &out,
+                     uint32_t rows, uint32_t width, float eps);
+void launch_rope(hipStream_t s, const View &in, const View &positions, const View &out,
+                 uint32_t rows, uint32_t heads, uint32_t width, float theta);
+// ordinary [T, elements] <-> pool [P, pt, elements]; table [Lp,2]; activity may have base null.
+void launch_paged_copy(hipStream_t s, const View &ordinary, const View &pool, const View &table,
+                       const View &generations, const View &activity, bool into_pages,
+                       uint32_t tokens, uint32_t elements, uint32_t start, uint32_t page_tokens,
+                       uint32_t physical_pages, uint32_t logical_pages, ErrorSlot *error);
+// Generic paged attention for one lane: q [Hq,Sq,D] view, out [Hq,Sq,Dv] view.
+void launch_paged_sdpa_generic(hipStream_t s, const View &q, const View &key_pool,
+                               const View &value_pool, const View &table,
+                               const View &generations, const View &activity, const View &out,
+                               uint32_t query_heads, uint32_t query_length, uint32_t kv_heads,
+                               uint32_t width, uint32_t value_width, uint32_t key_length,
+                               uint32_t query_start, float scale, bool causal,
+                               uint32_t page_tokens, uint32_t physical_pages,
+                               uint32_t logical_pages, ErrorSlot *error);
+void launch_fill_seeded(hipStream_t s, const View &out, uint64_t elements, uint32_t kind,
+                        uint64_t seed, uint64_t stream, uint64_t first, float lo, float hi);
+void launch_fill_u32(hipStream_t s, uint32_t *ptr, uint64_t count, uint32_t value);
+void launch_init_errors(hipStream_t s, ErrorSlot *slots, uint32_t count);
+
+// ---- moe.hip ----
+// counts [E], offsets [E+1], sorted_routes [R*k], blocks [max_blocks,3], n_blocks [1].
+void launch_route_pack(hipStream_t s, const View &indices, uint32_t rows, uint32_t k,
+                       uint32_t experts, uint32_t tile_rows, uint32_t *counts, uint32_t *offsets,
+                       uint32_t *sorted_routes, uint32_t *blocks, uint32_t max_blocks,
+                       uint32_t *n_blocks, ErrorSlot *error);
+
+}  // namespace fh

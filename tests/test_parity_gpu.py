@@ -1,0 +1,667 @@
+"""Differential tests: the HIP library (through the C ABI) against the CPU oracle on identical
+seeded bytes, in the manner of crates/forja-metal/tests/*.rs (CpuBackend = reference,
+candidate = device backend).  Integer results are bit-exact; float results meet the elementwise
+rel 1e-2 / abs 1e-2 bar and the reference's normwise bound for the dtype."""
+import math
+
+import numpy as np
+import pytest
+
+from forja_amd import programs
+from forja_amd.core import (BackendError, BinOp, CommandList, DType, Inst, Op, Program,
+                            ProgramBuilder, ProgramKind, RedOp, Slice, Status, UnOp, ValueType,
+                            INTO_PAGES, OUT_OF_PAGES)
+from oracle import cpu_backend as orc
+from tests.helpers import (Quantised, assert_close, from_f32, normal_bf16, to_f32, upload,
+                           upload_raw)
+from tests.test_oracle_golden import paged_case, top_k_case
+
+pytestmark = pytest.mark.gpu
+
+
+def run(backend, commands):
+    backend.submit(commands).wait()
+
+
+def compare(cpu, hip, cpu_tensor, hip_tensor, **kw):
+    dtype = cpu_tensor.dtype
+    a, b = cpu.read(cpu_tensor), hip.read(hip_tensor)
+    if dtype in (DType.U32, DType.I32):
+        assert a == b
+    else:
+        assert_close(to_f32(b, dtype), to_f32(a, dtype), dtype, **kw)
+
+
+def differential(cpu, hip, build, expect_error=None, **kw):
+    """build(backend) -> (commands, [outputs]); runs on both and compares every output."""
+    results = []
+    for backend in (cpu, hip):
+        commands, outputs = build(backend)
+        error = None
+        try:
+            run(backend, commands)
+        except BackendError as e:
+            error = e
+        results.append((outputs, error))
+    (cpu_out, cpu_err), (hip_out, hip_err) = results
+    if expect_error is None:
+        assert cpu_err is None and hip_err is None, (cpu_err, hip_err)
+    else:
+        assert cpu_err is not None and hip_err is not None
+        assert hip_err.status in expect_error
+    for a, b in zip(cpu_out, hip_out):
+        compare(cpu, hip, a, b, **kw)
+    return results
+
+
+# ------------------------------------------------------------------ device info / storage
+
+def test_device_is_gfx950_and_storage_round_trips(hip):
+    info = hip.device_info()
+    assert info["family"].startswith("gfx950"), info
+    assert info["wavefront"] == 64
+    t = hip.alloc(DType.U32, (5, 7))
+    assert hip.read(t) == bytes(5 * 7 * 4)                      # zero-initialised
+    data = np.arange(35, dtype=np.uint32)
+    hip.write(t, data.tobytes())
+    assert np.frombuffer(hip.read(t), np.uint32).tolist() == data.tolist()
+    view = t.slice([Slice(1, 2, 2), Slice(0, 3, 3)]).permute([1, 0])
+    assert np.frombuffer(hip.read(view), np.uint32).tolist() == data.reshape(5, 7)[1::2, 0::3][:2, :3].T.ravel().tolist()
+    with pytest.raises(BackendError):
+        hip.write(view, bytes(24))                              # non-contiguous write refused
+    hip.release(t)
+    with pytest.raises(BackendError):
+        hip.read(t)                                             # released allocation
+
+
+def test_submit_refuses_foreign_tensors_and_bad_shapes(hip):
+    x = hip.alloc(DType.BF16, (4, 64))
+    out = hip.alloc(DType.BF16, (4, 8))
+    packed = hip.alloc(DType.U32, (8, 8))
+    scales, biases = hip.alloc(DType.BF16, (8, 1)), hip.alloc(DType.BF16, (8, 1))
+    wrong = hip.alloc(DType.BF16, (4, 9))
+    commands = CommandList()
+    commands.dispatch(Op.quant_matmul(4, 64), [x, packed, scales, biases], wrong)
+    with pytest.raises(BackendError) as info:
+        hip.submit(commands)
+    assert info.value.status == Status.INVALID_INPUT
+    hip.release(scales)
+    commands = CommandList()
+    commands.dispatch(Op.quant_matmul(4, 64), [x, packed, scales, biases], out)
+    with pytest.raises(BackendError):
+        hip.submit(commands)
+
+
+def test_seeded_fill_matches_the_host_generator_bit_for_bit(cpu, hip):
+    def build(backend):
+        words = backend.alloc(DType.U32, (3, 1000))
+        uniform = backend.alloc(DType.BF16, (777,))
+        normal = backend.alloc(DType.BF16, (5, 999))
+        normal32 = backend.alloc(DType.F32, (4096,))
+        commands = CommandList()
+        commands.dispatch(Op.fill_seeded(0, 0x1234_5678_9abc, 3, first=17), [], words)
+        commands.dispatch(Op.fill_seeded(1, 99, 4, lo=0.001, hi=0.02), [], uniform)
+        commands.dispatch(Op.fill_seeded(2, 99, 5, first=1 << 20), [], normal)
+        commands.dispatch(Op.fill_seeded(2, 7, 6), [], normal32)
+        return commands, [words, uniform, normal, normal32]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    for a, b in zip(cpu_out, hip_out):
+        assert cpu.read(a) == hip.read(b)
+
+
+# ------------------------------------------------------------------ quantised matmul
+
+QMM_CASES = [
+    # rows, N, K, bits, group, activation dtype
+    (1, 64, 64, 4, 64, DType.F32),
+    (7, 48, 128, 4, 64, DType.BF16),
+    (33, 40, 256, 4, 64, DType.BF16),
+    (4, 4096, 1024, 4, 64, DType.BF16),     # C0 stacked qkv
+    (4, 1024, 3072, 4, 64, DType.BF16),     # C0 down
+    (128, 160, 2048, 4, 64, DType.BF16),    # C3 row count, narrow N
+    (128, 128, 2048, 8, 64, DType.BF16),    # router (q8 in the reference engine)
+    (5, 24, 256, 4, 32, DType.F16),
+    (3, 24, 256, 8, 128, DType.F32),
+    (40, 72, 192, 4, 64, DType.BF16),
+]
+
+
+@pytest.mark.parametrize("rows,n,k,bits,group,dtype", QMM_CASES)
+def test_quant_matmul(cpu, hip, rows, n, k, bits, group, dtype):
+    weights = Quantised(21, 100 + n + k, (n, k), bits=bits, group=group)
+    x_values = normal_bf16(21, 7, (rows, k))
+
+    def build(backend):
+        x = upload(backend, x_values, dtype)
+        packed, scales, biases = weights.upload(backend)
+        out = backend.alloc(dtype, (rows, n))
+        commands = CommandList()
+        commands.dispatch(Op.quant_matmul(bits, group), [x, packed, scales, biases], out)
+        return commands, [out]
+    differential(cpu, hip, build)
+
+
+def test_quant_matmul_on_strided_views_with_bias_epilogue(cpu, hip):
+    """Every operand sliced with step 2 (crates/forja-metal/tests/quant_matmul/shared.rs:95-107)
+    plus a fused epilogue that adds a broadcast bias."""
+    rows, n, k = 6, 32, 128
+    weights = Quantised(22, 5, (2 * n, 2 * k), bits=4, group=64)
+    x_values = normal_bf16(22, 8, (2 * rows, 2 * k))
+    bias_values = normal_bf16(22, 9, (n,))
+
+    def build(backend):
+        x = upload(backend, x_values, DType.BF16).slice([Slice(0, rows, 2), Slice(0, k)])
+        packed, scales, biases = weights.upload(backend)
+        packed = packed.slice([Slice(1, n, 2), Slice(0, k // 8)])
+        scales = scales.slice([Slice(1, n, 2), Slice(0, k // 64)])
+        biases = biases.slice([Slice(1, n, 2), Slice(0, k // 64)])
+        big = backend.alloc(DType.BF16, (rows, 2 * n))
+        out = big.slice([Slice(0, rows), Slice(1, n, 2)])
+        bias = upload(backend, bias_values, DType.BF16).broadcast((rows, n))
+        epilogue = backend.prepare_epilogue(programs.add_elements())
+        commands = CommandList()
+        commands.dispatch_epilogue(Op.quant_matmul(4, 64), [x, packed, scales, biases], out, epilogue, [bias])
+        return commands, [big]
+    differential(cpu, hip, build)
+
+
+# ------------------------------------------------------------------ routed projections
+
+def routed_case(seed, rows, k, experts, n, inner, bad=()):
+    rng = np.random.default_rng(seed)
+    indices = np.stack([rng.permutation(experts)[:k] for _ in range(rows)]).astype(np.uint32)
+    for (r, s, value) in bad:
+        indices[r, s] = value
+    return indices
+
+
+@pytest.mark.parametrize("rows,k,experts,n,inner", [(24, 4, 16, 128, 128), (256, 8, 128, 64, 128),
+                                                   (5, 2, 3, 64, 64), (40, 8, 8, 192, 256)])
+def test_gather_projection_pair_and_weighted_sum(cpu, hip, rows, k, experts, n, inner):
+    gate = Quantised(31, 1, (n, inner), experts=experts)
+    up = Quantised(31, 11, (n, inner), experts=experts)
+    down = Quantised(31, 21, (inner, n), experts=experts)
+    indices = routed_case(31, rows, k, experts, n, inner)
+    x_values = normal_bf16(31, 40, (rows, inner))
+    logits = orc.fill_normal_f32(31, 41, rows * k).reshape(rows, k)
+    w_values = np.exp(logits) / np.exp(logits).sum(axis=1, keepdims=True)
+    residual_values = normal_bf16(31, 42, (rows, inner))
+
+    def build(backend):
+        x = upload(backend, x_values, DType.BF16)
+        idx = upload(backend, indices, DType.U32)
+        g, u, d = gate.upload(backend), up.upload(backend), down.upload(backend)
+        plain = backend.alloc(DType.BF16, (rows, k, n))
+        activated = backend.alloc(DType.BF16, (rows, k, n))
+        combined = backend.alloc(DType.BF16, (rows, inner))
+        summed = backend.alloc(DType.BF16, (rows, inner))
+        weights = upload(backend, w_values, DType.BF16)
+        residual = upload(backend, residual_values, DType.BF16)
+        swiglu = backend.prepare_epilogue(programs.silu_mul_elements())
+        add = backend.prepare_epilogue(programs.add_elements())
+        commands = CommandList()
+        commands.dispatch(Op.gather_quant_matmul(4, 64), [x, *g, idx], plain)
+        commands.dispatch_epilogue(Op.gather_quant_matmul(4, 64), [x, *g, *u, idx], activated, swiglu, [])
+        commands.dispatch_epilogue(Op.gather_quant_matmul(4, 64), [activated, *d, idx, weights], combined,
+                                   add, [residual])
+        commands.dispatch(Op.gather_quant_matmul(4, 64), [activated, *d, idx, weights], summed)
+        return commands, [plain, activated, combined, summed]
+    differential(cpu, hip, build)
+
+
+def test_gather_reports_lowest_bad_expert_and_zeroes_its_rows(cpu, hip):
+    """lib.rs:2929-2950, crates/forja-metal/tests/gather_quant_matmul.rs:644-764"""
+    rows, k, experts, n, inner = 6, 3, 4, 32, 64
+    gate = Quantised(32, 1, (n, inner), experts=experts)
+    indices = routed_case(32, rows, k, experts, n, inner, bad=[(1, 2, 99), (4, 0, 7)])
+    x_values = normal_bf16(32, 40, (rows, inner))
+
+    def build(backend):
+        x = upload(backend, x_values, DType.BF16)
+        idx = upload(backend, indices, DType.U32)
+        out = upload(backend, np.full((rows, k, n), 3.0), DType.BF16)
+        commands = CommandList()
+        commands.dispatch(Op.gather_quant_matmul(4, 64), [x, *gate.upload(backend), idx], out)
+        return commands, [out]
+    results = differential(cpu, hip, build, expect_error={Status.INDEX_OUT_OF_RANGE, Status.DEVICE_ERROR_FLAG})
+    (cpu_out, cpu_err), (hip_out, hip_err) = results
+    assert cpu_err.index == 7 and hip_err.index == 7
+    values = to_f32(hip.read(hip_out[0]), DType.BF16).reshape(rows, k, n)
+    assert not values[1, 2].any() and not values[4, 0].any() and values[0, 0].any()
+
+
+def test_gather_with_an_unrecognised_epilogue_uses_the_interpreter(cpu, hip):
+    rows, k, experts, n, inner = 8, 2, 4, 32, 64
+    gate, up = Quantised(33, 1, (n, inner), experts=experts), Quantised(33, 2, (n, inner), experts=experts)
+    indices = routed_case(33, rows, k, experts, n, inner)
+    x_values = normal_bf16(33, 3, (rows, inner))
+    program = Program(ProgramKind.MAP, [
+        Inst.input(0), Inst.input(1), Inst.unary(UnOp.TANH, 0), Inst.binary(BinOp.MAX, 1, 2),
+        Inst.const(0.5), Inst.binary(BinOp.MUL, 3, 4)], [(0, 5)])
+
+    def build(backend):
+        x = upload(backend, x_values, DType.F32)
+        idx = upload(backend, indices, DType.U32)
+        out = backend.alloc(DType.F32, (rows, k, n))
+        commands = CommandList()
+        commands.dispatch_epilogue(Op.gather_quant_matmul(4, 64),
+                                   [x, *gate.upload(backend), *up.upload(backend), idx], out,
+                                   backend.prepare_epilogue(program), [])
+        return commands, [out]
+    differential(cpu, hip, build, rel=1e-4, abs_=1e-4, norm_tol=1e-4)
+
+
+@pytest.mark.parametrize("rows,k,experts,tile", [(256, 8, 128, 16), (128, 8, 128, 32), (7, 3, 5, 2),
+                                                (1, 1, 1, 1), (300, 8, 128, 32), (64, 2, 200, 8)])
+def test_route_pack_is_bit_exact(cpu, hip, rows, k, experts, tile):
+    rng = np.random.default_rng(rows * 31 + k)
+    indices = rng.integers(0, experts, (rows, k)).astype(np.uint32)
+
+    def build(backend):
+        idx = upload(backend, indices, DType.U32)
+        max_blocks = experts + rows * k // tile + 1
+        outs = [backend.alloc(DType.U32, (experts,)), backend.alloc(DType.U32, (experts + 1,)),
+                backend.alloc(DType.U32, (rows * k,)), backend.alloc(DType.U32, (max_blocks, 3))]
+        commands = CommandList()
+        commands.dispatch_many(Op.route_pack(tile), [idx], outs)
+        return commands, outs
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    flat = indices.ravel().astype(np.int64)
+    order = np.argsort(flat, kind="stable")
+    assert np.frombuffer(hip.read(hip_out[2]), np.uint32).tolist() == order.tolist()
+
+
+def test_route_pack_skips_bad_routes_and_reports_the_lowest(cpu, hip):
+    indices = np.array([[0, 9, 2], [7, 1, 1], [2, 2, 50]], dtype=np.uint32)
+
+    def build(backend):
+        idx = upload(backend, indices, DType.U32)
+        outs = [backend.alloc(DType.U32, (3,)), backend.alloc(DType.U32, (4,)),
+                backend.alloc(DType.U32, (9,)), backend.alloc(DType.U32, (8, 3))]
+        commands = CommandList()
+        commands.dispatch_many(Op.route_pack(2), [idx], outs)
+        return commands, outs[:2]
+    results = differential(cpu, hip, build, expect_error={Status.INDEX_OUT_OF_RANGE})
+    assert results[1][1].index == 7
+
+
+# ------------------------------------------------------------------ selection
+
+@pytest.mark.parametrize("width,k", [(1, 1), (64, 8), (128, 8), (2050, 64)])
+def test_top_k_edge_widths_ties_and_nans(cpu, hip, width, k):
+    values = top_k_case(width)
+
+    def build(backend):
+        x = upload_raw(backend, values, DType.F32, (1, width))
+        outs = [backend.alloc(DType.F32, (1, k)), backend.alloc(DType.U32, (1, k))]
+        commands = CommandList()
+        commands.dispatch_many(Op.top_k(k, False), [x], outs)
+        return commands, outs
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    assert cpu.read(cpu_out[0]) == hip.read(hip_out[0])       # values copied bit for bit
+
+
+@pytest.mark.parametrize("dtype", [DType.BF16, DType.F32])
+def test_router_top_k_is_bit_exact_in_order_and_close_in_weight(cpu, hip, dtype):
+    logits = orc.fill_normal_f32(41, 1, 256 * 128).reshape(256, 128)
+
+    def build(backend):
+        x = upload(backend, logits, dtype)
+        outs = [backend.alloc(dtype, (256, 8)), backend.alloc(DType.U32, (256, 8))]
+        commands = CommandList()
+        commands.dispatch_many(Op.top_k(8, True), [x], outs)
+        return commands, outs
+    differential(cpu, hip, build)
+
+
+def test_argmax_ties_and_vocabulary_width(cpu, hip):
+    rng = np.random.default_rng(3)
+    logits = rng.standard_normal((4, 151936)).astype(np.float32)
+    logits[1, 77] = logits[1, 150000] = 99.0            # tie: highest index wins
+    logits[2, 5] = np.inf
+    logits[3, 100] = np.nan                             # +NaN is the maximum under total order
+    small = np.array([[1.0, 9.0, 2.0, 9.0, 3.0]], dtype=np.float32)
+
+    def build(backend):
+        a, b = upload(backend, logits, DType.BF16), upload(backend, small, DType.F32)
+        outs = [backend.alloc(DType.U32, (4,)), backend.alloc(DType.U32, (1,))]
+        commands = CommandList()
+        commands.dispatch(Op.argmax(), [a], outs[0])
+        commands.dispatch(Op.argmax(), [b], outs[1])
+        return commands, outs
+    (_, _), (hip_out, _) = differential(cpu, hip, build)
+    assert np.frombuffer(hip.read(hip_out[1]), np.uint32).tolist() == [3]
+    assert np.frombuffer(hip.read(hip_out[0]), np.uint32).tolist()[1:] == [150000, 5, 100]
+
+
+# ------------------------------------------------------------------ paged storage
+
+def test_paged_copy_round_trip_with_conversion(cpu, hip):
+    values = np.arange(21, dtype=np.float32) / 8.0
+
+    def build(backend):
+        source = upload(backend, values.reshape(7, 3), DType.F32)
+        pool = backend.alloc(DType.F16, (3, 4, 3))
+        table = upload(backend, np.array([[2, 5], [0, 7]]), DType.U32)
+        generations = upload(backend, np.array([7, 0, 5]), DType.U32)
+        output = backend.alloc(DType.F32, (7, 3))
+        commands = CommandList()
+        commands.dispatch(Op.paged_copy(INTO_PAGES, 1, 4), [source, table, generations], pool)
+        commands.dispatch(Op.paged_copy(OUT_OF_PAGES, 1, 4), [pool, table, generations], output)
+        return commands, [pool, output]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    assert cpu.read(cpu_out[0]) == hip.read(hip_out[0]) and cpu.read(cpu_out[1]) == hip.read(hip_out[1])
+
+
+def test_paged_copy_refuses_stale_entries_without_writing(hip):
+    """crates/forja-metal/tests/paged.rs:239-277: rejected rows are not written, others are."""
+    source = upload(hip, np.arange(16, dtype=np.float32).reshape(8, 2) + 1.0, DType.F32)
+    pool = hip.alloc(DType.F32, (3, 4, 2))
+    generations = upload(hip, np.array([7, 8, 9]), DType.U32)
+    table = upload(hip, np.array([[1, 8], [2, 1]]), DType.U32)     # second entry is stale
+    commands = CommandList()
+    commands.dispatch(Op.paged_copy(INTO_PAGES, 0, 4), [source, table, generations], pool)
+    with pytest.raises(BackendError) as info:
+        run(hip, commands)
+    assert info.value.status == Status.DEVICE_ERROR_FLAG and info.value.index == 1
+    values = to_f32(hip.read(pool), DType.F32).reshape(3, 4, 2)
+    assert values[1].ravel().tolist() == list(np.arange(8) + 1.0) and not values[2].any()
+
+
+PAGED_CASES = [
+    # hq, hkv, sq, key_length, q_start, causal, pool dtype, page_tokens
+    (16, 8, 1, 18, 17, True, DType.BF16, 16),
+    (16, 8, 1, 65, 64, True, DType.BF16, 16),
+    (16, 8, 1, 131, 130, True, DType.BF16, 16),
+    (16, 8, 1, 512, 511, True, DType.BF16, 16),
+    (32, 4, 1, 1000, 999, True, DType.BF16, 16),
+    (32, 4, 1, 300, 299, True, DType.BF16, 64),
+    (4, 2, 5, 37, 32, True, DType.BF16, 16),
+    (4, 4, 3, 33, 0, False, DType.F16, 16),
+    (2, 1, 4, 20, 16, True, DType.F32, 4),
+]
+
+
+@pytest.mark.parametrize("hq,hkv,sq,key_length,q_start,causal,dtype,pt", PAGED_CASES)
+def test_paged_sdpa(cpu, hip, hq, hkv, sq, key_length, q_start, causal, dtype, pt):
+    scale = 1.0 / math.sqrt(128)
+
+    def build(backend):
+        t, _ = paged_case(backend, hq, hkv, sq, key_length, pt, q_start, pool_dtype=dtype)
+        commands = CommandList()
+        commands.dispatch(Op.paged_sdpa(scale, causal, q_start, key_length, pt),
+                          [t["q"], t["keys"], t["values"], t["table"], t["generations"]], t["out"])
+        return commands, [t["out"]]
+    differential(cpu, hip, build)
+
+
+def test_paged_sdpa_through_a_permuted_query_view(cpu, hip):
+    """Engines pass q as a permuted [Hq,Sq,D] view of [Sq,Hq,D] storage and read the output the
+    same way (crates/forja-host/src/lib.rs:6223-6333)."""
+    hq, hkv, sq, key_length, q_start = 8, 2, 3, 40, 37
+    scale = 0.1
+
+    def build(backend):
+        t, host = paged_case(backend, hq, hkv, sq, key_length, 16, q_start)
+        stored_q = upload(backend, np.transpose(host["q"], (1, 0, 2)), DType.BF16)
+        stored_out = backend.alloc(DType.BF16, (sq, hq, 128))
+        commands = CommandList()
+        commands.dispatch(Op.paged_sdpa(scale, True, q_start, key_length, 16),
+                          [stored_q.permute([1, 0, 2]), t["keys"], t["values"], t["table"], t["generations"]],
+                          stored_out.permute([1, 0, 2]))
+        return commands, [stored_out]
+    differential(cpu, hip, build)
+
+
+def test_paged_append_then_attend(cpu, hip):
+    hq, hkv, q_start = 16, 8, 130
+    scale = 1.0 / math.sqrt(128)
+    k_new = normal_bf16(51, 1, (1, hkv, 128))
+    v_new = normal_bf16(51, 2, (1, hkv, 128))
+
+    def build(backend):
+        t, _ = paged_case(backend, hq, hkv, 1, q_start + 1, 16, q_start)
+        kn, vn = upload(backend, k_new, DType.BF16), upload(backend, v_new, DType.BF16)
+        commands = CommandList()
+        commands.dispatch_many(Op.paged_sdpa_append(scale, q_start, 16),
+                               [t["q"], kn, vn, t["table"], t["generations"]],
+                               [t["out"], t["keys"], t["values"]])
+        return commands, [t["out"]]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+
+
+def test_inactive_lane_is_zero_and_touches_nothing(hip):
+    query = upload(hip, np.ones((2, 1, 4)), DType.F32)
+    key = upload(hip, np.ones((1, 1, 4)), DType.F32)
+    value = upload(hip, np.ones((1, 1, 4)), DType.F32)
+    table = upload(hip, np.array([[0, 0xffffffff]]), DType.U32)
+    generations = upload(hip, np.array([1]), DType.U32)
+    activity = upload(hip, np.array([0]), DType.U32)
+    key_pages, value_pages = hip.alloc(DType.F32, (1, 4, 1, 4)), hip.alloc(DType.F32, (1, 4, 1, 4))
+    output = upload(hip, np.full((2, 1, 4), 5.0), DType.F32)
+    commands = CommandList()
+    commands.dispatch_many(Op.paged_sdpa_append(1.0, 0, 4), [query, key, value, table, generations, activity],
+                           [output, key_pages, value_pages])
+    run(hip, commands)
+    assert not any(hip.read(output)) and not any(hip.read(key_pages)) and not any(hip.read(value_pages))
+
+
+def test_stale_generation_is_reported_and_never_dereferenced(hip):
+    t, _ = paged_case(hip, 4, 2, 1, 40, 16, 39)
+    generations = np.frombuffer(hip.read(t["generations"]), np.uint32).copy()
+    table = np.frombuffer(hip.read(t["table"]), np.uint32).reshape(-1, 2)
+    generations[table[1, 0]] += 1                       # logical page 1 is now stale
+    hip.write(t["generations"], generations.tobytes())
+    commands = CommandList()
+    commands.dispatch(Op.paged_sdpa(0.1, True, 39, 40, 16),
+                      [t["q"], t["keys"], t["values"], t["table"], t["generations"]], t["out"])
+    with pytest.raises(BackendError) as info:
+        run(hip, commands)
+    assert info.value.status == Status.DEVICE_ERROR_FLAG and info.value.index == 1
+    assert not any(hip.read(t["out"]))
+
+
+# ------------------------------------------------------------------ ragged batch
+
+def ragged_case(backend, contexts, counts, hq, hkv, pt, seed, activity=None, dtype=DType.BF16,
+                corrupt=None):
+    """Lanes with `contexts[l]` tokens already cached and `counts[l]` new queries each.  Shuffled
+    physical pages shared by all lanes, generations 11+page, poisoned table tails."""
+    width = 128
+    lanes = len(contexts)
+    pages_needed = [(c + n + pt - 1) // pt for c, n in zip(contexts, counts)]
+    table_pages = max(pages_needed) + 2
+    physical = sum(pages_needed) + 5
+    rng = np.random.default_rng(seed)
+    free = list(rng.permutation(physical))
+    tables = np.zeros((lanes, table_pages, 2), np.uint32)
+    tables[:, :, 1] = 0xffffffff
+    for lane, need in enumerate(pages_needed):
+        for logical in range(need):
+            page = free.pop()
+            tables[lane, logical] = (page, 11 + page)
+    if corrupt is not None:
+        lane, logical = corrupt
+        tables[lane, logical, 1] += 1
+    pool_k = orc.bf16_to_f32(orc.fill_normal_bf16(seed, 1, physical * pt * hkv * width))
+    pool_v = orc.bf16_to_f32(orc.fill_normal_bf16(seed, 2, physical * pt * hkv * width))
+    total = sum(counts)
+    cu = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+    tensors = dict(
+        q=upload(backend, normal_bf16(seed, 3, (total, hq, width)), dtype),
+        k_new=upload(backend, normal_bf16(seed, 4, (total, hkv, width)), dtype),
+        v_new=upload(backend, normal_bf16(seed, 5, (total, hkv, width)), dtype),
+        tables=upload(backend, tables, DType.U32),
+        generations=upload(backend, 11 + np.arange(physical), DType.U32),
+        cu=upload(backend, cu, DType.U32),
+        starts=upload(backend, np.array(contexts), DType.U32),
+        out=backend.alloc(dtype, (total, hq, width)),
+        keys=upload(backend, pool_k.reshape(physical, pt, hkv, width), dtype),
+        values=upload(backend, pool_v.reshape(physical, pt, hkv, width), dtype))
+    inputs = [tensors[n] for n in ("q", "k_new", "v_new", "tables", "generations", "cu", "starts")]
+    if activity is not None:
+        inputs.append(upload(backend, np.array(activity), DType.U32))
+    return tensors, inputs
+
+
+RAGGED_CASES = [
+    # contexts, new tokens per lane, hq, hkv, page_tokens
+    ([17, 64, 130, 511], [1, 1, 1, 1], 16, 8, 16),                 # BASELINE config 0
+    ([300, 1, 2047, 700, 15, 16, 0], [1, 1, 1, 1, 1, 1, 1], 32, 4, 16),
+    ([40, 0, 100], [1, 5, 3], 8, 2, 16),                           # decode + prefill chunks
+    ([100, 257], [1, 1], 32, 4, 64),                               # engine page size
+]
+
+
+@pytest.mark.parametrize("contexts,counts,hq,hkv,pt", RAGGED_CASES)
+def test_ragged_attention_equals_the_per_lane_sequence(cpu, hip, contexts, counts, hq, hkv, pt):
+    scale = 1.0 / math.sqrt(128)
+
+    def build(backend):
+        t, inputs = ragged_case(backend, contexts, counts, hq, hkv, pt, seed=61)
+        commands = CommandList()
+        commands.dispatch_many(Op.paged_attention_ragged(scale, pt), inputs, [t["out"], t["keys"], t["values"]])
+        return commands, [t["out"], t["keys"], t["values"]]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    # block-table gather and append placement are pure addressing: pools must match bit for bit
+    assert cpu.read(cpu_out[1]) == hip.read(hip_out[1]) and cpu.read(cpu_out[2]) == hip.read(hip_out[2])
+
+
+def test_ragged_attention_skips_inactive_lanes(cpu, hip):
+    def build(backend):
+        t, inputs = ragged_case(backend, [33, 70, 5], [1, 1, 1], 8, 4, 16, seed=62, activity=[1, 0, 1])
+        commands = CommandList()
+        commands.dispatch_many(Op.paged_attention_ragged(0.09, 16), inputs, [t["out"], t["keys"], t["values"]])
+        return commands, [t["out"], t["keys"], t["values"]]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    assert cpu.read(cpu_out[1]) == hip.read(hip_out[1])
+    assert not to_f32(hip.read(hip_out[0]), DType.BF16).reshape(3, -1)[1].any()
+
+
+def test_ragged_attention_reports_a_stale_page(hip):
+    t, inputs = ragged_case(hip, [33, 70, 5], [1, 1, 1], 8, 4, 16, seed=63, corrupt=(1, 2))
+    commands = CommandList()
+    commands.dispatch_many(Op.paged_attention_ragged(0.09, 16), inputs, [t["out"], t["keys"], t["values"]])
+    with pytest.raises(BackendError) as info:
+        run(hip, commands)
+    assert info.value.status == Status.DEVICE_ERROR_FLAG and info.value.index == 2
+    out = to_f32(hip.read(t["out"]), DType.BF16).reshape(3, -1)
+    assert not out[1].any() and out[0].any() and out[2].any()
+
+
+# ------------------------------------------------------------------ programs and glue
+
+def test_engine_row_programs(cpu, hip):
+    rows, hidden, heads, half = 6, 1024, 24, 64
+    x_values = normal_bf16(71, 1, (rows, hidden))
+    u_values = normal_bf16(71, 2, (rows, hidden))
+    w_values = 1.0 + 0.1 * normal_bf16(71, 3, (hidden,))
+    qk_values = normal_bf16(71, 4, (rows, heads, 2 * half))
+    norm_values = 1.0 + 0.1 * normal_bf16(71, 5, (heads, 2 * half))
+    positions = np.array([0, 1, 17, 511, 4095, 32767], dtype=np.float32)
+
+    def build(backend):
+        x, u = upload(backend, x_values, DType.BF16), upload(backend, u_values, DType.BF16)
+        w = upload(backend, w_values, DType.BF16).broadcast((rows, hidden))
+        normed = backend.alloc(DType.BF16, (rows, hidden))
+        hidden_out, normed2 = backend.alloc(DType.BF16, (rows, hidden)), backend.alloc(DType.BF16, (rows, hidden))
+        qk = upload(backend, qk_values, DType.BF16)
+        norm = upload(backend, norm_values, DType.BF16).broadcast((rows, heads, 2 * half))
+        pos = upload(backend, positions, DType.F32).reshape((rows, 1, 1)).broadcast((rows, heads, half))
+        rotated = backend.alloc(DType.BF16, (rows, heads, 2 * half))
+        commands = CommandList()
+        commands.dispatch_kernel(backend.prepare_program(programs.rms_norm_rows(1e-6)), [x, w], [normed])
+        commands.dispatch_kernel(backend.prepare_program(programs.residual_norm_rows(1e-6)), [x, u, w],
+                                 [hidden_out, normed2])
+        commands.dispatch_kernel(
+            backend.prepare_program(programs.qk_norm_rope_rows(128.0, 1e-6, 1e6)),
+            [qk.narrow(2, 0, half), qk.narrow(2, half, half), norm.narrow(2, 0, half),
+             norm.narrow(2, half, half), pos],
+            [rotated.narrow(2, 0, half), rotated.narrow(2, half, half)])
+        return commands, [normed, hidden_out, normed2, rotated]
+    differential(cpu, hip, build, abs_=2e-2)
+
+
+def test_map_programs_casts_index_select(cpu, hip):
+    values = np.array([[-1.5, 3.7, np.nan, 5e9, 0.25, -0.0, 7.0, 1e-3]], dtype=np.float32).repeat(3, axis=0)
+    b = ProgramBuilder(ProgramKind.MAP)
+    v, w = b.input(0), b.input(1)
+    as_u32 = b.cast(ValueType.U32, v)
+    b.output(0, b.cast(ValueType.F32, as_u32))
+    column = b.cast(ValueType.F32, b.index(1))
+    big = b.binary(BinOp.GT, column, b.const(3.5))
+    b.output(1, b.select(big, b.binary(BinOp.MAX, v, b.const(0.0)), b.unary(UnOp.ABS, v)))
+    b.output(2, b.cast(ValueType.F32, b.binary(BinOp.ADD, w, b.extent(1))))
+    program = b.finish()
+
+    def build(backend):
+        x = upload_raw(backend, values, DType.F32, values.shape)
+        ids = upload(backend, np.arange(24).reshape(3, 8), DType.U32)
+        outs = [backend.alloc(DType.F32, values.shape) for _ in range(3)]
+        commands = CommandList()
+        commands.dispatch_kernel(backend.prepare_program(program), [x, ids], outs)
+        return commands, outs
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    for a, b_ in zip(cpu_out, hip_out):
+        assert cpu.read(a) == hip.read(b_)
+
+
+def test_softmax_row_program_with_max_and_sum_reductions(cpu, hip):
+    b = ProgramBuilder(ProgramKind.ROW)
+    x = b.input(0)
+    e = b.unary(UnOp.EXP, b.sub(x, b.reduce(RedOp.MAX, x)))
+    b.output(0, b.div(e, b.reduce(RedOp.SUM, e)))
+    program = b.finish()
+    values = orc.fill_normal_f32(72, 1, 5 * 700).reshape(5, 700)
+
+    def build(backend):
+        x = upload(backend, values, DType.F32)
+        out = backend.alloc(DType.F32, (5, 700))
+        commands = CommandList()
+        commands.dispatch_kernel(backend.prepare_program(program), [x], [out])
+        return commands, [out]
+    differential(cpu, hip, build, rel=1e-4, abs_=1e-6, norm_tol=1e-5)
+
+
+def test_quant_embed_copy_matmul_rms_norm_rope(cpu, hip):
+    table = Quantised(81, 1, (300, 128))
+    ids_values = np.array([[5, 299, 0], [17, 100, 3]], dtype=np.uint32)
+    experts_values = normal_bf16(81, 2, (6, 32, 4))
+    weights_values = normal_bf16(81, 3, (6, 4, 1))
+    x_values = normal_bf16(81, 4, (7, 16, 128))
+
+    def build(backend):
+        ids = upload(backend, ids_values, DType.U32)
+        embedded = backend.alloc(DType.BF16, (2, 3, 128))
+        experts = upload(backend, experts_values, DType.BF16)
+        weights = upload(backend, weights_values, DType.BF16)
+        combined = backend.alloc(DType.BF16, (6, 32, 1))
+        x = upload(backend, x_values, DType.BF16)
+        copied = backend.alloc(DType.F32, (16, 7, 128))
+        normed = backend.alloc(DType.BF16, (7, 16, 128))
+        w = upload(backend, np.linspace(0.5, 1.5, 128), DType.F32)
+        roped = backend.alloc(DType.BF16, (7, 16, 128))
+        pos = upload(backend, np.array([0, 1, 2, 100, 1000, 20000, 32767]), DType.U32)
+        commands = CommandList()
+        commands.dispatch(Op.quant_embed(4, 64), [*table.upload(backend), ids], embedded)
+        commands.dispatch(Op.matmul(), [experts, weights], combined)     # MoE combine shape
+        commands.dispatch(Op.copy(), [x.permute([1, 0, 2])], copied)
+        commands.dispatch(Op.rms_norm(1e-6), [x, w], normed)
+        commands.dispatch(Op.rope(1e6), [x, pos], roped)
+        return commands, [embedded, combined, copied, normed, roped]
+    differential(cpu, hip, build, abs_=2e-2)
+
+
+def test_quant_embed_zeroes_bad_rows_and_reports_the_lowest_bad_id(cpu, hip):
+    """lib.rs:3020-3037 for the quantised table"""
+    table = Quantised(82, 1, (300, 128))
+    ids_values = np.array([5, 1000, 0, 999], dtype=np.uint32)
+
+    def build(backend):
+        ids = upload(backend, ids_values, DType.U32)
+        embedded = upload(backend, np.ones((4, 128)), DType.BF16)
+        commands = CommandList()
+        commands.dispatch(Op.quant_embed(4, 64), [*table.upload(backend), ids], embedded)
+        return commands, [embedded]
+    results = differential(cpu, hip, build, expect_error={Status.INDEX_OUT_OF_RANGE})
+    assert results[0][1].index == 999 and results[1][1].index == 999

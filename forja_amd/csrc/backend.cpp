@@ -9,6 +9,7 @@
 #include <map>
 #include <mutex>
 #include <new>
+#include <set>
 #include <thread>
 #include <unordered_map>
 #include <vector>
@@ -105,6 +106,7 @@ struct fh_backend {
   };
   std::vector<Timed> timed;
   std::vector<hipEvent_t> event_pool;
+  std::set<fh_submission *> submissions;  // live submissions owning device resources
   uint64_t class_ns[FH_KC_COUNT] = {0, 0, 0, 0};
   uint64_t class_launches[FH_KC_COUNT] = {0, 0, 0, 0};
 
@@ -124,6 +126,16 @@ struct fh_backend {
 };
 
 namespace {
+
+// Backends that are still alive.  A submission may outlive its backend (a host-language object
+// finalised late); it must then release only its own host memory.
+std::mutex g_live_mutex;
+std::set<fh_backend *> g_live_backends;
+
+bool backend_alive(fh_backend *b) {
+  std::lock_guard<std::mutex> lock(g_live_mutex);
+  return g_live_backends.count(b) != 0;
+}
 
 #define FH_REQUIRE(cond)              \
   do {                                \
@@ -165,6 +177,57 @@ fh_status make_view(fh_backend *b, const fh_tensor &t, bool writable, View *out)
   }
   out->offset = t.offset;
   return FH_OK;
+}
+
+// byte_ranges_overlap (crates/forja-core/src/layout.rs:496-560): a conservative span test refined
+// by a lattice proof for the common case of two boxes cut from one parent layout (identical
+// strides that divide each other): there the offsets decompose into parent coordinates uniquely
+// and the boxes overlap iff their intervals overlap on every axis.
+bool may_overlap(const fh_tensor &a, const fh_tensor &b) {
+  if (a.buffer != b.buffer) return false;
+  auto span_of = [](const fh_tensor &t, uint64_t *lo, uint64_t *hi) {
+    uint64_t reach = t.offset;
+    for (uint32_t axis = 0; axis < t.rank; ++axis) {
+      if (t.shape[axis] == 0) {
+        *lo = *hi = 0;
+        return;
+      }
+      reach += (uint64_t)(t.shape[axis] - 1) * t.stride[axis];
+    }
+    *lo = t.offset * dtype_size(t.dtype);
+    *hi = (reach + 1) * dtype_size(t.dtype);
+  };
+  uint64_t alo, ahi, blo, bhi;
+  span_of(a, &alo, &ahi);
+  span_of(b, &blo, &bhi);
+  if (alo == ahi || blo == bhi) return false;
+  if (ahi <= blo || bhi <= alo) return false;
+  if (a.rank != b.rank || dtype_size(a.dtype) != dtype_size(b.dtype) || a.rank == 0) return true;
+  // Axes sorted by descending stride; identical strides required.
+  uint32_t order[FH_MAX_RANK];
+  for (uint32_t i = 0; i < a.rank; ++i) {
+    if (a.stride[i] != b.stride[i] || a.stride[i] == 0) return true;
+    order[i] = i;
+  }
+  std::sort(order, order + a.rank, [&](uint32_t l, uint32_t r) { return a.stride[l] > a.stride[r]; });
+  uint64_t ra = a.offset, rb = b.offset;
+  bool disjoint = false;
+  for (uint32_t n = 0; n < a.rank; ++n) {
+    uint32_t axis = order[n];
+    uint64_t stride = a.stride[axis];
+    uint64_t pa = ra / stride, pb = rb / stride;
+    ra %= stride;
+    rb %= stride;
+    if (n > 0) {
+      uint64_t outer = a.stride[order[n - 1]];
+      if (outer % stride != 0) return true;
+      uint64_t extent = outer / stride;
+      if (pa + a.shape[axis] > extent || pb + b.shape[axis] > extent) return true;
+    }
+    if (pa + a.shape[axis] <= pb || pb + b.shape[axis] <= pa) disjoint = true;
+  }
+  if (ra != 0 || rb != 0) return true;
+  return !disjoint;
 }
 
 View null_view() {
@@ -965,36 +1028,11 @@ fh_status process(fh_backend *b, const fh_dispatch &d, ErrorSlot *error, bool ex
     fh_status status = make_view(b, d.outputs[i], true, &pl.out[i]);
     if (status != FH_OK) return status;
   }
-  // Outputs must not alias inputs or each other (check_common, ops.rs:1300-1344): conservative
-  // whole-span test per allocation.
-  auto span_of = [](const fh_tensor &t, uint64_t *lo, uint64_t *hi) {
-    uint64_t reach = t.offset;
-    for (uint32_t axis = 0; axis < t.rank; ++axis) {
-      if (t.shape[axis] == 0) {
-        *lo = *hi = 0;
-        return;
-      }
-      reach += (uint64_t)(t.shape[axis] - 1) * t.stride[axis];
-    }
-    *lo = t.offset * dtype_size(t.dtype);
-    *hi = (reach + 1) * dtype_size(t.dtype);
-  };
+  // Outputs must not alias inputs or each other (check_common, ops.rs:1300-1344).
   for (uint32_t o = 0; o < d.n_outputs; ++o) {
-    uint64_t olo, ohi;
-    span_of(d.outputs[o], &olo, &ohi);
-    if (olo == ohi) continue;
-    for (uint32_t i = 0; i < d.n_inputs; ++i) {
-      if (d.inputs[i].buffer != d.outputs[o].buffer) continue;
-      uint64_t ilo, ihi;
-      span_of(d.inputs[i], &ilo, &ihi);
-      FH_REQUIRE(ihi <= olo || ohi <= ilo);
-    }
-    for (uint32_t other = o + 1; other < d.n_outputs; ++other) {
-      if (d.outputs[other].buffer != d.outputs[o].buffer) continue;
-      uint64_t ilo, ihi;
-      span_of(d.outputs[other], &ilo, &ihi);
-      FH_REQUIRE(ihi <= olo || ohi <= ilo);
-    }
+    for (uint32_t i = 0; i < d.n_inputs; ++i) FH_REQUIRE(!may_overlap(d.outputs[o], d.inputs[i]));
+    for (uint32_t other = o + 1; other < d.n_outputs; ++other)
+      FH_REQUIRE(!may_overlap(d.outputs[o], d.outputs[other]));
   }
   switch (d.op) {
   case FH_OP_PROGRAM: return plan_program(b, pl, execute);
@@ -1063,6 +1101,10 @@ fh_status fh_create(int device, fh_backend **out) {
     delete b;
     return FH_DEVICE_EXECUTION_FAILED;
   }
+  {
+    std::lock_guard<std::mutex> lock(g_live_mutex);
+    g_live_backends.insert(b);
+  }
   *out = b;
   return FH_OK;
 }
@@ -1070,9 +1112,22 @@ fh_status fh_create(int device, fh_backend **out) {
 void fh_destroy(fh_backend *b) {
   if (!b) return;
   {
+    std::lock_guard<std::mutex> lock(g_live_mutex);
+    if (!g_live_backends.erase(b)) return;
+  }
+  {
     std::lock_guard<std::mutex> lock(b->mutex);
     (void)hipSetDevice(b->device);
     (void)hipStreamSynchronize(b->stream);
+    for (fh_submission *s : b->submissions) {
+      (void)hipFree(s->device_errors);
+      (void)hipHostFree(s->host_errors);
+      (void)hipEventDestroy(s->start);
+      (void)hipEventDestroy(s->end);
+      s->device_errors = nullptr;
+      s->host_errors = nullptr;
+    }
+    b->submissions.clear();
     for (auto &entry : b->allocations) (void)hipFree(entry.second.ptr);
     for (auto &entry : b->programs)
       for (auto &typed : entry.second.typed) (void)hipFree(typed.second);
@@ -1332,6 +1387,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
     s->error.submission = s->serial;
     s->error.value = (uint32_t)launch_error;
   }
+  b->submissions.insert(s);
   *out = s;
   return FH_OK;
 }
@@ -1339,6 +1395,11 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
 fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
   if (!s) return FH_INVALID_INPUT;
   fh_backend *b = s->backend;
+  if (!s->waited && !backend_alive(b)) {
+    // fh_destroy drained the stream, but the error record went with the backend.
+    s->waited = true;
+    s->result = FH_EXECUTION_FAILED;
+  }
   if (!s->waited) {
     // The trailing async copy of the error slots is the last work of the submission; a pinned
     // target makes stream synchronisation the completion point.
@@ -1410,10 +1471,17 @@ uint64_t fh_gpu_time_ns(fh_submission *s) { return s ? s->gpu_ns : 0; }
 void fh_submission_free(fh_submission *s) {
   if (!s) return;
   fh_backend *b = s->backend;
+  std::lock_guard<std::mutex> live(g_live_mutex);
+  if (g_live_backends.count(b) == 0) {
+    // The device context went with the backend; only the host record remains.
+    delete s;
+    return;
+  }
   {
     std::lock_guard<std::mutex> lock(b->mutex);
     (void)hipSetDevice(b->device);
     if (!s->waited) (void)hipStreamSynchronize(b->stream);
+    b->submissions.erase(s);
     (void)hipFree(s->device_errors);
     (void)hipHostFree(s->host_errors);
     (void)hipEventDestroy(s->start);

@@ -168,15 +168,428 @@ __global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *er
   }
 }
 
+
+// ---------------------------------------------------------------- bf16, D = Dv = 128 fast path
+//
+// Split-KV decode-style attention on the matrix cores.  One wave owns (split, token, kv head):
+// it streams its span of the lane's K/V pages once, 32 tokens at a time.
+//   S^T = K . Q^T : v_mfma_f32_16x16x32_bf16, M = 16 tokens, N = the kv head's query heads padded
+//                   to 16, K = 32 of the 128 head-dim elements per step (4 steps)
+//   O^T = V^T . P^T: M = 16 of the 128 value columns (8 tiles), N = heads, K = 32 tokens
+// K rows go straight from global memory into the A-operand layout (each lane reads 64
+// contiguous bytes of one token row).  V needs its token axis on the contraction side, so the
+// 32x128 tile is staged in LDS with coalesced 16-byte loads and read back column-wise.  The
+// score accumulators already sit in the B-operand layout of the second product, so P never
+// leaves registers.  Softmax runs in the exp2 domain with one running maximum per head.
+// HBM-bound: each K/V byte is read exactly once; partial (m, l, O) per split are merged by
+// ragged_reduce_kernel.
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr uint32_t kSplitTokens = 256;   // target tokens per split
+constexpr uint32_t kTile = 32;           // tokens per inner step
+constexpr uint32_t kVPitch = 264;        // bytes per staged V row: 256 + 8 keeps the four lane
+                                         // groups of a transposed read on disjoint banks
+
+struct FastRagged {
+  const uint16_t *q, *key_pool, *value_pool;
+  uint16_t *out;
+  const uint32_t *tables, *generations, *cu, *starts, *activity;
+  float *partial_o;    // [T, S, Hq, 128]
+  float2 *partial_ml;  // [T, S, Hq]
+  uint32_t *bad;       // [T]
+  uint64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h;
+  uint32_t tokens, lanes, query_heads, kv_heads, group, page_tokens, physical_pages, table_pages,
+      max_splits;
+  float scale_log2;
+  // Single-lane form (Op::PagedSdpa / Op::PagedSdpaAppend): cu == nullptr, every token belongs
+  // to lane 0 whose first query sits at `one_start`; `fixed_attended` != 0 disables the causal
+  // limit (every row attends exactly that many keys).
+  uint32_t one_start, fixed_attended;
+};
+
+struct SplitPlan {
+  uint32_t lane, attended, chunk, splits;
+  bool live;
+};
+
+// Work decomposition shared by the attention and the reduce kernels.
+__device__ inline SplitPlan plan_token(const FastRagged &p, uint32_t token) {
+  SplitPlan plan{0, 0, 0, 0, false};
+  uint64_t attended;
+  if (p.cu == nullptr) {
+    if (p.activity && p.activity[0] == 0) return plan;
+    attended = p.fixed_attended ? p.fixed_attended : (uint64_t)p.one_start + token + 1;
+  } else {
+    if (token < p.cu[0] || token >= p.cu[p.lanes]) return plan;
+    plan.lane = find_lane(p.cu, p.lanes, token);
+    if (p.activity && p.activity[plan.lane] == 0) return plan;
+    attended = (uint64_t)p.starts[plan.lane] + (token - p.cu[plan.lane]) + 1;
+  }
+  uint64_t capacity = (uint64_t)p.table_pages * p.page_tokens;
+  plan.live = true;
+  if (attended > capacity) {
+    plan.attended = 0;  // reported as a bad page by the caller
+    return plan;
+  }
+  plan.attended = (uint32_t)attended;
+  uint32_t want = (plan.attended + kSplitTokens - 1) / kSplitTokens;
+  if (want > p.max_splits) want = p.max_splits;
+  uint32_t chunk = (plan.attended + want - 1) / want;
+  plan.chunk = (chunk + kTile - 1) / kTile * kTile;
+  plan.splits = (plan.attended + plan.chunk - 1) / plan.chunk;
+  return plan;
+}
+
+__device__ inline uint32_t pack_bf16(float lo, float hi) {
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+__global__ __launch_bounds__(64) void ragged_attention_mfma_kernel(FastRagged p, ErrorSlot *error) {
+  __shared__ __attribute__((aligned(16))) unsigned char v_tile[kTile * kVPitch];
+  const uint32_t lane = threadIdx.x, hl = lane & 15, g = lane >> 4;
+  const uint32_t split = blockIdx.x, token = blockIdx.y, kv_head = blockIdx.z;
+  const SplitPlan plan = plan_token(p, token);
+  if (!plan.live) return;
+  if (plan.attended == 0) {
+    if (split == 0 && kv_head == 0 && lane == 0) {
+      report_error(error, p.table_pages);
+      p.bad[token] = 1;
+    }
+    return;
+  }
+  if (split >= plan.splits) return;
+  const uint32_t begin = split * plan.chunk;
+  const uint32_t end = min(plan.attended, begin + plan.chunk);
+  const uint32_t pt = p.page_tokens;
+  const uint32_t *table = p.tables + (uint64_t)plan.lane * p.table_pages * 2;
+
+  // Query operand: head hl of this kv head's group (zero rows beyond the group).
+  uint4 q_reg[4];
+  {
+    const uint32_t head = kv_head * p.group + hl;
+    const uint16_t *q_row = p.q + (uint64_t)token * p.q_stride_t + (uint64_t)head * p.q_stride_h;
+    for (int step = 0; step < 4; ++step) {
+      q_reg[step] = make_uint4(0, 0, 0, 0);
+      if (hl < p.group) q_reg[step] = *(const uint4 *)(q_row + 32 * g + 8 * step);
+    }
+  }
+  f32x4 o[8];
+  for (int mt = 0; mt < 8; ++mt) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -__builtin_inff(), l_run = 0.0f;
+
+  const uint32_t first_page = begin / pt, last_page = (end - 1) / pt;
+  for (uint32_t page0 = first_page; page0 <= last_page; page0 += 64) {
+    // Authenticate up to 64 table entries at once; nothing is dereferenced through a bad one.
+    uint32_t my_page = page0 + lane, physical = 0;
+    bool mine = my_page <= last_page, ok = true;
+    if (mine) {
+      uint32_t page = table[2 * (uint64_t)my_page], generation = table[2 * (uint64_t)my_page + 1];
+      ok = page < p.physical_pages && p.generations[page] == generation;
+      physical = page;
+    }
+    unsigned long long bad_mask = __ballot(mine && !ok);
+    if (bad_mask) {
+      if (lane == (uint32_t)__ffsll((long long)bad_mask) - 1) {
+        report_error(error, my_page);
+        p.bad[token] = 1;
+      }
+      return;
+    }
+    const uint32_t tok_lo = max(begin, page0 * pt);
+    const uint64_t tok_hi64 = min((uint64_t)end, ((uint64_t)page0 + 64) * pt);
+    const uint32_t tok_hi = (uint32_t)tok_hi64;
+    for (uint32_t tile0 = tok_lo; tile0 < tok_hi; tile0 += kTile) {
+      // Pool row of the first token of each 16-token half (a half never straddles a page).
+      uint64_t row0[2] = {0, 0};
+      for (int sub = 0; sub < 2; ++sub) {
+        uint32_t tok0 = tile0 + 16 * sub;
+        if (tok0 < end) {
+          uint32_t page = __shfl(physical, (int)(tok0 / pt - page0), 64);
+          row0[sub] = (uint64_t)page * pt + tok0 % pt;
+        }
+      }
+      // K: lane (token hl, group g) reads 64 contiguous bytes of its token row.
+      uint4 k_reg[2][4];
+      for (int sub = 0; sub < 2; ++sub) {
+        uint32_t tok = tile0 + 16 * sub + hl;
+        const uint16_t *k_row =
+            p.key_pool + ((row0[sub] + hl) * p.kv_heads + kv_head) * 128 + 32 * g;
+        for (int step = 0; step < 4; ++step) {
+          k_reg[sub][step] = make_uint4(0, 0, 0, 0);
+          if (tok < end) k_reg[sub][step] = *(const uint4 *)(k_row + 8 * step);
+        }
+      }
+      // V: coalesced 16-byte loads of the 32x128 tile (zeros past the end: unused pool slots may
+      // hold anything, and 0 * NaN would poison the product).
+      uint4 v_reg[8];
+      for (int j = 0; j < 8; ++j) {
+        uint32_t piece = lane + 64 * j, row = piece >> 4, col = piece & 15;
+        uint32_t tok = tile0 + row;
+        v_reg[j] = make_uint4(0, 0, 0, 0);
+        if (tok < end)
+          v_reg[j] = *(const uint4 *)(p.value_pool +
+                                      ((row0[row >> 4] + (row & 15)) * p.kv_heads + kv_head) * 128 +
+                                      8 * col);
+      }
+      __syncthreads();  // previous tile's transposed reads are done
+      for (int j = 0; j < 8; ++j) {
+        uint32_t piece = lane + 64 * j, row = piece >> 4, col = piece & 15;
+        uint2 *dst = (uint2 *)(v_tile + row * kVPitch + col * 16);
+        dst[0] = make_uint2(v_reg[j].x, v_reg[j].y);
+        dst[1] = make_uint2(v_reg[j].z, v_reg[j].w);
+      }
+      // Scores.
+      float s_val[8];
+      for (int sub = 0; sub < 2; ++sub) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int step = 0; step < 4; ++step)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(bf16x8, k_reg[sub][step]), __builtin_bit_cast(bf16x8, q_reg[step]),
+              acc, 0, 0, 0);
+        for (int j = 0; j < 4; ++j) {
+          uint32_t tok = tile0 + 16 * sub + 4 * g + j;
+          s_val[4 * sub + j] = tok < end ? acc[j] * p.scale_log2 : -__builtin_inff();
+        }
+      }
+      float tile_max = s_val[0];
+      for (int i = 1; i < 8; ++i) tile_max = fmaxf(tile_max, s_val[i]);
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+      float m_new = fmaxf(m_run, tile_max);
+      float alpha = exp2f(m_run - m_new);
+      float p_val[8], p_sum = 0.0f;
+      for (int i = 0; i < 8; ++i) {
+        p_val[i] = exp2f(s_val[i] - m_new);
+        p_sum += p_val[i];
+      }
+      l_run = l_run * alpha + p_sum;
+      m_run = m_new;
+      uint4 p_reg = make_uint4(pack_bf16(p_val[0], p_val[1]), pack_bf16(p_val[2], p_val[3]),
+                               pack_bf16(p_val[4], p_val[5]), pack_bf16(p_val[6], p_val[7]));
+      for (int mt = 0; mt < 8; ++mt)
+        for (int j = 0; j < 4; ++j) o[mt][j] *= alpha;
+      __syncthreads();  // V tile visible
+      // O^T += V^T . P^T ; contraction slot i of lane group g is token (i<4 ? 4g+i : 16+4g+i-4).
+      const uint16_t *v_lds = (const uint16_t *)v_tile;
+      for (int mt = 0; mt < 8; ++mt) {
+        uint32_t a_words[4];
+        for (int pair = 0; pair < 4; ++pair) {
+          uint32_t i0 = 2 * pair, i1 = 2 * pair + 1;
+          uint32_t r0 = (i0 < 4 ? 4 * g + i0 : 16 + 4 * g + i0 - 4);
+          uint32_t r1 = (i1 < 4 ? 4 * g + i1 : 16 + 4 * g + i1 - 4);
+          uint32_t lo = v_lds[r0 * (kVPitch / 2) + 16 * mt + hl];
+          uint32_t hi = v_lds[r1 * (kVPitch / 2) + 16 * mt + hl];
+          a_words[pair] = lo | (hi << 16);
+        }
+        uint4 a_reg = make_uint4(a_words[0], a_words[1], a_words[2], a_words[3]);
+        o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_reg),
+                                                       __builtin_bit_cast(bf16x8, p_reg), o[mt], 0,
+                                                       0, 0);
+      }
+    }
+  }
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (hl >= p.group) return;
+  const uint32_t head = kv_head * p.group + hl;
+  if (plan.splits == 1) {
+    float inv = 1.0f / l_run;
+    uint16_t *out_row = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
+    for (int mt = 0; mt < 8; ++mt) {
+      uint2 packed = make_uint2(pack_bf16(o[mt][0] * inv, o[mt][1] * inv),
+                                pack_bf16(o[mt][2] * inv, o[mt][3] * inv));
+      *(uint2 *)(out_row + 16 * mt + 4 * g) = packed;
+    }
+    return;
+  }
+  uint64_t item = ((uint64_t)token * p.max_splits + split) * p.query_heads + head;
+  float *po = p.partial_o + item * 128;
+  for (int mt = 0; mt < 8; ++mt)
+    *(float4 *)(po + 16 * mt + 4 * g) = make_float4(o[mt][0], o[mt][1], o[mt][2], o[mt][3]);
+  if (g == 0) p.partial_ml[item] = make_float2(m_run, l_run);
+}
+
+// Merges the per-split partials of one token: out = sum_s O_s 2^(m_s-M) / sum_s l_s 2^(m_s-M).
+// Also writes the zero rows of inactive lanes, uncovered tokens and tokens whose page table was
+// refused.
+__global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
+  const uint32_t token = blockIdx.x;
+  const SplitPlan plan = plan_token(p, token);
+  const bool zero = !plan.live || plan.attended == 0 || p.bad[token] != 0;
+  if (!zero && plan.splits == 1) return;
+  const uint32_t work = p.query_heads * 32;  // 4 value columns per thread
+  for (uint32_t item = threadIdx.x; item < work; item += blockDim.x) {
+    uint32_t head = item >> 5, column = (item & 31) * 4;
+    uint16_t *dst = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
+    if (zero) {
+      *(uint2 *)dst = make_uint2(0, 0);
+      continue;
+    }
+    uint64_t base = (uint64_t)token * p.max_splits * p.query_heads + head;
+    float m_all = -__builtin_inff();
+    for (uint32_t s = 0; s < plan.splits; ++s)
+      m_all = fmaxf(m_all, p.partial_ml[base + (uint64_t)s * p.query_heads].x);
+    float l_all = 0.0f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t s = 0; s < plan.splits; ++s) {
+      uint64_t at = base + (uint64_t)s * p.query_heads;
+      float2 ml = p.partial_ml[at];
+      float w = exp2f(ml.x - m_all);
+      l_all += ml.y * w;
+      float4 part = *(const float4 *)(p.partial_o + at * 128 + column);
+      acc.x += part.x * w;
+      acc.y += part.y * w;
+      acc.z += part.z * w;
+      acc.w += part.w * w;
+    }
+    float inv = 1.0f / l_all;
+    *(uint2 *)dst = make_uint2(pack_bf16(acc.x * inv, acc.y * inv), pack_bf16(acc.z * inv, acc.w * inv));
+  }
+}
+
+__global__ void clear_flags_kernel(uint32_t *flags, uint32_t count) {
+  uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) flags[i] = 0;
+}
+
+bool fast_ragged_eligible(const RaggedAttention &p) {
+  auto bf16 = [](const View &v) { return v.dtype == FH_BF16; };
+  if (!bf16(p.q) || !bf16(p.k_new) || !bf16(p.v_new) || !bf16(p.out) || !bf16(p.key_pool) ||
+      !bf16(p.value_pool))
+    return false;
+  if (p.width != 128 || p.value_width != 128 || p.page_tokens % 16 != 0) return false;
+  uint32_t group = p.query_heads / p.kv_heads;
+  if (group > 16) return false;
+  // innermost axis contiguous, 16-byte aligned rows
+  if (p.q.stride[2] != 1 || p.out.stride[2] != 1) return false;
+  if (p.q.stride[0] % 8 || p.q.stride[1] % 8 || p.q.offset % 8) return false;
+  if (p.out.stride[0] % 4 || p.out.stride[1] % 4 || p.out.offset % 4) return false;
+  if (p.key_pool.offset % 8 || p.value_pool.offset % 8) return false;
+  return true;
+}
+
 }  // namespace
 
-bool try_fast_lane_attention(fh_backend *, const LaneAttention &, ErrorSlot *) { return false; }
+namespace {
+
+uint32_t splits_for(uint32_t tokens) {
+  uint32_t max_splits = 16384u / (tokens ? tokens : 1);
+  if (max_splits > 64) max_splits = 64;
+  if (max_splits < 1) max_splits = 1;
+  return max_splits;
+}
+
+// Carves flags / (m,l) / O partial storage for `tokens` out of the backend workspace.
+bool carve_partials(fh_backend *backend, FastRagged *f) {
+  uint64_t items = (uint64_t)f->tokens * f->max_splits * f->query_heads;
+  uint64_t flags_bytes = ((uint64_t)f->tokens * 4 + 255) / 256 * 256;
+  uint64_t ml_bytes = (items * sizeof(float2) + 255) / 256 * 256;
+  uint64_t o_bytes = items * 128 * sizeof(float);
+  char *ws = backend_workspace(backend, flags_bytes + ml_bytes + o_bytes);
+  if (!ws) return false;
+  f->bad = (uint32_t *)ws;
+  f->partial_ml = (float2 *)(ws + flags_bytes);
+  f->partial_o = (float *)(ws + flags_bytes + ml_bytes);
+  return true;
+}
+
+void launch_fast(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
+  ragged_attention_mfma_kernel<<<dim3(f.max_splits, f.tokens, f.kv_heads), 64, 0, stream>>>(f, error);
+  ragged_reduce_kernel<<<dim3(f.tokens), 256, 0, stream>>>(f);
+}
+
+}  // namespace
+
+bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, ErrorSlot *error) {
+  auto bf16 = [](const View &v) { return v.dtype == FH_BF16; };
+  if (!bf16(lane.q) || !bf16(lane.out) || !bf16(lane.key_pool) || !bf16(lane.value_pool))
+    return false;
+  if (lane.width != 128 || lane.value_width != 128 || lane.page_tokens % 16 != 0) return false;
+  uint32_t group = lane.query_heads / lane.kv_heads;
+  if (group > 16 || lane.query_length == 0) return false;
+  if (lane.q.stride[2] != 1 || lane.out.stride[2] != 1) return false;
+  if (lane.q.stride[0] % 8 || lane.q.stride[1] % 8 || lane.q.offset % 8) return false;
+  if (lane.out.stride[0] % 4 || lane.out.stride[1] % 4 || lane.out.offset % 4) return false;
+  if (lane.key_pool.offset % 8 || lane.value_pool.offset % 8) return false;
+  FastRagged f{};
+  f.tokens = lane.query_length;
+  f.lanes = 1;
+  f.query_heads = lane.query_heads;
+  f.kv_heads = lane.kv_heads;
+  f.group = group;
+  f.page_tokens = lane.page_tokens;
+  f.physical_pages = lane.physical_pages;
+  f.table_pages = lane.logical_pages;
+  f.max_splits = splits_for(f.tokens);
+  f.scale_log2 = lane.scale * 1.4426950408889634f;
+  f.one_start = lane.query_start;
+  f.fixed_attended = lane.causal ? 0 : lane.key_length;
+  if (!carve_partials(backend, &f)) return false;
+  f.q = (const uint16_t *)lane.q.base + lane.q.offset;
+  f.out = (uint16_t *)lane.out.base + lane.out.offset;
+  f.key_pool = (const uint16_t *)lane.key_pool.base + lane.key_pool.offset;
+  f.value_pool = (const uint16_t *)lane.value_pool.base + lane.value_pool.offset;
+  f.tables = (const uint32_t *)lane.table.base + lane.table.offset;
+  f.generations = (const uint32_t *)lane.generations.base + lane.generations.offset;
+  f.cu = nullptr;
+  f.starts = nullptr;
+  f.activity =
+      lane.activity.base ? (const uint32_t *)lane.activity.base + lane.activity.offset : nullptr;
+  // q / out are [Hq, Sq, D] views: the token axis is axis 1.
+  f.q_stride_t = lane.q.stride[1];
+  f.q_stride_h = lane.q.stride[0];
+  f.out_stride_t = lane.out.stride[1];
+  f.out_stride_h = lane.out.stride[0];
+  hipStream_t stream = backend_stream(backend);
+  clear_flags_kernel<<<dim3((f.tokens + 255) / 256), 256, 0, stream>>>(f.bad, f.tokens);
+  launch_fast(stream, f, error);
+  return true;
+}
 
 bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSlot *error) {
   hipStream_t stream = backend_stream(backend);
+  const bool fast = fast_ragged_eligible(p);
+  FastRagged f{};
+  if (fast) {
+    f.tokens = p.tokens;
+    f.query_heads = p.query_heads;
+    f.max_splits = splits_for(p.tokens);
+    if (!carve_partials(backend, &f)) return false;
+    f.q = (const uint16_t *)p.q.base + p.q.offset;
+    f.out = (uint16_t *)p.out.base + p.out.offset;
+    f.key_pool = (const uint16_t *)p.key_pool.base + p.key_pool.offset;
+    f.value_pool = (const uint16_t *)p.value_pool.base + p.value_pool.offset;
+    f.tables = (const uint32_t *)p.tables.base + p.tables.offset;
+    f.generations = (const uint32_t *)p.generations.base + p.generations.offset;
+    f.cu = (const uint32_t *)p.cu_seqlens.base + p.cu_seqlens.offset;
+    f.starts = (const uint32_t *)p.q_starts.base + p.q_starts.offset;
+    f.activity = p.activity.base ? (const uint32_t *)p.activity.base + p.activity.offset : nullptr;
+    f.q_stride_t = p.q.stride[0];
+    f.q_stride_h = p.q.stride[1];
+    f.out_stride_t = p.out.stride[0];
+    f.out_stride_h = p.out.stride[1];
+    f.tokens = p.tokens;
+    f.lanes = p.lanes;
+    f.query_heads = p.query_heads;
+    f.kv_heads = p.kv_heads;
+    f.group = p.query_heads / p.kv_heads;
+    f.page_tokens = p.page_tokens;
+    f.physical_pages = p.physical_pages;
+    f.table_pages = p.table_pages;
+    f.scale_log2 = p.scale * 1.4426950408889634f;
+    clear_flags_kernel<<<dim3((p.tokens + 255) / 256), 256, 0, stream>>>(f.bad, p.tokens);
+  }
   uint64_t append_work =
       (uint64_t)p.tokens * (p.kv_heads * p.width + p.kv_heads * p.value_width);
   ragged_append_kernel<<<dim3((unsigned)((append_work + 255) / 256)), 256, 0, stream>>>(p, error);
+  if (fast) {
+    launch_fast(stream, f, error);
+    return true;
+  }
   uint32_t blocks = p.tokens * p.query_heads;
   if (p.value_width <= 64)
     ragged_attention_generic_kernel<64><<<dim3(blocks), 64, 0, stream>>>(p, error);

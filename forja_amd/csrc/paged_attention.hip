@@ -4,6 +4,8 @@
 // the lane's new K/V rows were stored at its q_start (execute_paged_append,
 // crates/forja-cpu/src/lib.rs:262-306).  Pools are [P, page_tokens, Hkv, D]; a table entry is
 // (physical page, generation) and is valid iff page < P and generations[page] == generation.
+#include <cstdlib>
+
 #include "fast_kernels.hpp"
 
 namespace fh {
@@ -171,27 +173,34 @@ __global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *er
 
 // ---------------------------------------------------------------- bf16, D = Dv = 128 fast path
 //
-// Split-KV decode-style attention on the matrix cores.  One wave owns (split, token, kv head):
-// it streams its span of the lane's K/V pages once, 32 tokens at a time.
+// Split-KV decode-style attention on the matrix cores, registers only.  One wave owns
+// (token, split, kv head): it streams its span of the lane's K/V pages once, 32 tokens per step.
 //   S^T = K . Q^T : v_mfma_f32_16x16x32_bf16, M = 16 tokens, N = the kv head's query heads padded
 //                   to 16, K = 32 of the 128 head-dim elements per step (4 steps)
-//   O^T = V^T . P^T: M = 16 of the 128 value columns (8 tiles), N = heads, K = 32 tokens
-// K rows go straight from global memory into the A-operand layout (each lane reads 64
-// contiguous bytes of one token row).  V needs its token axis on the contraction side, so the
-// 32x128 tile is staged in LDS with coalesced 16-byte loads and read back column-wise.  The
-// score accumulators already sit in the B-operand layout of the second product, so P never
-// leaves registers.  Softmax runs in the exp2 domain with one running maximum per head.
-// HBM-bound: each K/V byte is read exactly once; partial (m, l, O) per split are merged by
-// ragged_reduce_kernel.
+//   O^T = V^T . P^T: M = 16 value columns (8 tiles), N = heads, K = 32 tokens
+// Operand layouts are chosen so that every global load is a 16-byte piece of a 256-byte K or V
+// row and nothing is staged through LDS:
+//   * K: lane (token t, group g) reads bytes [64 step + 16 g, +16) of row t - the A operand.
+//   * V: MFMA row m of value tile mt is value column 8 m + mt, so lane (m, g) needs columns
+//     [8m, 8m+8) - one 16-byte piece - of the 8 tokens in its contraction slots; an 8x8 in-register
+//     transpose (v_perm) turns the 8 pieces into the 8 tiles' A operands.
+//   * P: the score accumulators of lane (head h, group g) are exactly the B operand of the second
+//     product (contraction slot i of group g = token 4g+i of the first half, 16+4g+i-4 of the
+//     second), so probabilities never leave registers.
+// Softmax runs in the exp2 domain with one running maximum per head.  HBM-bound: every K/V byte
+// is read once; per-split partial (m, l, O) are merged by ragged_reduce_kernel.
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr uint32_t kSplitTokens = 256;   // target tokens per split
-constexpr uint32_t kTile = 32;           // tokens per inner step
-constexpr uint32_t kVPitch = 264;        // bytes per staged V row: 256 + 8 keeps the four lane
-                                         // groups of a transposed read on disjoint banks
+constexpr uint32_t kMinSplitTokens = 128, kMaxSplitTokens = 1024;  // split length bounds
+constexpr uint32_t kTargetItems = 1024;  // (token, split) items wanted per launch
+constexpr uint32_t kTile = 32;          // tokens per inner step
+
+struct TokenPlan {
+  uint32_t lane, attended, chunk, splits;  // splits == 0: token produces zeros
+};
 
 struct FastRagged {
   const uint16_t *q, *key_pool, *value_pool;
@@ -200,9 +209,12 @@ struct FastRagged {
   float *partial_o;    // [T, S, Hq, 128]
   float2 *partial_ml;  // [T, S, Hq]
   uint32_t *bad;       // [T]
+  TokenPlan *plans;    // [T]
+  uint2 *items;        // [T * S] (token, split) of every live split, compacted
+  uint32_t *item_count;
   uint64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h;
   uint32_t tokens, lanes, query_heads, kv_heads, group, page_tokens, physical_pages, table_pages,
-      max_splits;
+      max_splits, split_tokens;
   float scale_log2;
   // Single-lane form (Op::PagedSdpa / Op::PagedSdpaAppend): cu == nullptr, every token belongs
   // to lane 0 whose first query sits at `one_start`; `fixed_attended` != 0 disables the causal
@@ -210,14 +222,10 @@ struct FastRagged {
   uint32_t one_start, fixed_attended;
 };
 
-struct SplitPlan {
-  uint32_t lane, attended, chunk, splits;
-  bool live;
-};
-
-// Work decomposition shared by the attention and the reduce kernels.
-__device__ inline SplitPlan plan_token(const FastRagged &p, uint32_t token) {
-  SplitPlan plan{0, 0, 0, 0, false};
+// Work decomposition of one token.  attended == 0 with splits == 0 and lane == 0xffffffff marks a
+// token whose context exceeds its table (reported as a bad page).
+__device__ inline TokenPlan plan_token(const FastRagged &p, uint32_t token, uint32_t split_tokens) {
+  TokenPlan plan{0, 0, 0, 0};
   uint64_t attended;
   if (p.cu == nullptr) {
     if (p.activity && p.activity[0] == 0) return plan;
@@ -228,14 +236,12 @@ __device__ inline SplitPlan plan_token(const FastRagged &p, uint32_t token) {
     if (p.activity && p.activity[plan.lane] == 0) return plan;
     attended = (uint64_t)p.starts[plan.lane] + (token - p.cu[plan.lane]) + 1;
   }
-  uint64_t capacity = (uint64_t)p.table_pages * p.page_tokens;
-  plan.live = true;
-  if (attended > capacity) {
-    plan.attended = 0;  // reported as a bad page by the caller
+  if (attended > (uint64_t)p.table_pages * p.page_tokens) {
+    plan.lane = 0xffffffffu;
     return plan;
   }
   plan.attended = (uint32_t)attended;
-  uint32_t want = (plan.attended + kSplitTokens - 1) / kSplitTokens;
+  uint32_t want = (plan.attended + split_tokens - 1) / split_tokens;
   if (want > p.max_splits) want = p.max_splits;
   uint32_t chunk = (plan.attended + want - 1) / want;
   plan.chunk = (chunk + kTile - 1) / kTile * kTile;
@@ -243,43 +249,203 @@ __device__ inline SplitPlan plan_token(const FastRagged &p, uint32_t token) {
   return plan;
 }
 
+// One workgroup: plans every token, compacts the live (token, split) pairs and clears the
+// per-token failure flags.
+__global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlot *error) {
+  __shared__ uint32_t wave_totals[4];
+  __shared__ uint32_t running;
+  __shared__ unsigned long long total_attended;
+  if (threadIdx.x == 0) {
+    running = 0;
+    total_attended = 0;
+  }
+  __syncthreads();
+  // Split length: long enough that a wave's fixed start-up cost (plan, table, query) is small
+  // against its stream, short enough that the batch still yields ~kTargetItems work items.
+  uint32_t split_tokens = p.split_tokens;
+  if (split_tokens == 0) {
+    unsigned long long mine = 0;
+    for (uint32_t token = threadIdx.x; token < p.tokens; token += 256)
+      mine += plan_token(p, token, 1u << 30).attended;
+    for (int offset = 32; offset > 0; offset >>= 1) mine += __shfl_xor(mine, offset, 64);
+    if ((threadIdx.x & 63) == 0) atomicAdd(&total_attended, mine);
+    __syncthreads();
+    unsigned long long per_item = total_attended / kTargetItems;
+    split_tokens = (uint32_t)((per_item + kTile - 1) / kTile * kTile);
+    if (split_tokens < kMinSplitTokens) split_tokens = kMinSplitTokens;
+    if (split_tokens > kMaxSplitTokens) split_tokens = kMaxSplitTokens;
+  }
+  for (uint32_t base = 0; base < p.tokens; base += 256) {
+    uint32_t token = base + threadIdx.x;
+    TokenPlan plan{0, 0, 0, 0};
+    if (token < p.tokens) {
+      plan = plan_token(p, token, split_tokens);
+      uint32_t bad = 0;
+      if (plan.lane == 0xffffffffu) {
+        report_error(error, p.table_pages);
+        bad = 1;
+        plan.lane = 0;
+      }
+      p.bad[token] = bad;
+      p.plans[token] = plan;
+    }
+    uint32_t inclusive = plan.splits;
+    for (int offset = 1; offset < 64; offset <<= 1) {
+      uint32_t other = __shfl_up(inclusive, offset, 64);
+      if ((int)(threadIdx.x & 63) >= offset) inclusive += other;
+    }
+    if ((threadIdx.x & 63) == 63) wave_totals[threadIdx.x >> 6] = inclusive;
+    __syncthreads();
+    uint32_t before = running;
+    for (uint32_t w = 0; w < (threadIdx.x >> 6); ++w) before += wave_totals[w];
+    uint32_t first = before + inclusive - plan.splits;
+    for (uint32_t s = 0; s < plan.splits; ++s) p.items[first + s] = make_uint2(token, s);
+    __syncthreads();
+    if (threadIdx.x == 255) running = before + inclusive;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) p.item_count[0] = running;
+}
+
 __device__ inline uint32_t pack_bf16(float lo, float hi) {
   bf16x2 v = {(__bf16)lo, (__bf16)hi};
   return __builtin_bit_cast(uint32_t, v);
 }
 
-__global__ __launch_bounds__(64) void ragged_attention_mfma_kernel(FastRagged p, ErrorSlot *error) {
-  __shared__ __attribute__((aligned(16))) unsigned char v_tile[kTile * kVPitch];
-  const uint32_t lane = threadIdx.x, hl = lane & 15, g = lane >> 4;
-  const uint32_t split = blockIdx.x, token = blockIdx.y, kv_head = blockIdx.z;
-  const SplitPlan plan = plan_token(p, token);
-  if (!plan.live) return;
-  if (plan.attended == 0) {
-    if (split == 0 && kv_head == 0 && lane == 0) {
-      report_error(error, p.table_pages);
-      p.bad[token] = 1;
+__device__ inline uint32_t dword_of(const uint4 &v, int index) {
+  return index == 0 ? v.x : (index == 1 ? v.y : (index == 2 ? v.z : v.w));
+}
+
+struct TileRegs {
+  uint4 k[2][4];
+  uint4 v[8];
+};
+
+struct LaneConst {
+  uint32_t k_offset;  // elements from the first row of a 16-token half to this lane's K piece
+  uint32_t v_offset;  // likewise for slot 0 of this lane's V pieces
+  uint32_t row_elems; // elements per pool token row (Hkv * 128)
+};
+
+// Issues the 16 loads of one 32-token tile.  `physical` holds this lane's authenticated page of
+// the current 64-page group; a 16-token half never straddles a page, so each half is addressed
+// as a wave-uniform base plus a per-lane 32-bit offset.  kMasked tiles (the last, partial tile
+// of a split) load zeros past `end`: unused pool slots may hold anything and 0 * NaN would
+// poison the sum.
+template <bool kMasked>
+__device__ inline void load_tile(const FastRagged &p, TileRegs &r, uint32_t tile0, uint32_t end,
+                                 uint32_t page0, uint32_t physical, const LaneConst &lc,
+                                 uint32_t hl, uint32_t g) {
+  const uint32_t pt = p.page_tokens;
+  for (int sub = 0; sub < 2; ++sub) {
+    const uint32_t tok0 = tile0 + 16 * sub;
+    if (kMasked && tok0 >= end) {
+      for (int step = 0; step < 4; ++step) r.k[sub][step] = make_uint4(0, 0, 0, 0);
+      for (int i = 0; i < 4; ++i) r.v[4 * sub + i] = make_uint4(0, 0, 0, 0);
+      continue;
     }
-    return;
+    const uint32_t page =
+        __builtin_amdgcn_readfirstlane(__shfl(physical, (int)(tok0 / pt - page0), 64));
+    const uint64_t row0 = (uint64_t)page * pt + tok0 % pt;
+    const uint16_t *k_base = p.key_pool + row0 * lc.row_elems;
+    const uint16_t *v_base = p.value_pool + row0 * lc.row_elems;
+    for (int step = 0; step < 4; ++step) {
+      r.k[sub][step] = *(const uint4 *)(k_base + lc.k_offset + 32 * step);
+      if (kMasked && tok0 + hl >= end) r.k[sub][step] = make_uint4(0, 0, 0, 0);
+    }
+    for (int i = 0; i < 4; ++i) {
+      r.v[4 * sub + i] = *(const uint4 *)(v_base + lc.v_offset + i * lc.row_elems);
+      if (kMasked && tok0 + 4 * g + i >= end) r.v[4 * sub + i] = make_uint4(0, 0, 0, 0);
+    }
   }
-  if (split >= plan.splits) return;
+}
+
+struct Softmax {
+  float m, l;
+};
+
+// Scores, online softmax and the value product for one tile.
+template <bool kMasked>
+__device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[4], f32x4 (&o)[8],
+                                    Softmax &sm, uint32_t tile0, uint32_t end, float scale_log2,
+                                    uint32_t g) {
+  float s_val[8];
+  for (int sub = 0; sub < 2; ++sub) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int step = 0; step < 4; ++step)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, cur.k[sub][step]),
+                                                    __builtin_bit_cast(bf16x8, q_reg[step]), acc, 0,
+                                                    0, 0);
+    for (int j = 0; j < 4; ++j) {
+      s_val[4 * sub + j] = acc[j] * scale_log2;
+      if (kMasked && tile0 + 16 * sub + 4 * g + j >= end) s_val[4 * sub + j] = -__builtin_inff();
+    }
+  }
+  float tile_max = s_val[0];
+  for (int i = 1; i < 8; ++i) tile_max = fmaxf(tile_max, s_val[i]);
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+  const float m_new = fmaxf(sm.m, tile_max);
+  float p_val[8], p_sum = 0.0f;
+  for (int i = 0; i < 8; ++i) {
+    p_val[i] = __builtin_amdgcn_exp2f(s_val[i] - m_new);
+    p_sum += p_val[i];
+  }
+  // The running maximum settles after a few tiles; skip the rescale when no lane's moved.
+  if (__any(m_new != sm.m)) {
+    const float alpha = __builtin_amdgcn_exp2f(sm.m - m_new);
+    sm.l *= alpha;
+    for (int mt = 0; mt < 8; ++mt)
+      for (int j = 0; j < 4; ++j) o[mt][j] *= alpha;
+    sm.m = m_new;
+  }
+  sm.l += p_sum;
+  const uint4 p_reg = make_uint4(pack_bf16(p_val[0], p_val[1]), pack_bf16(p_val[2], p_val[3]),
+                                 pack_bf16(p_val[4], p_val[5]), pack_bf16(p_val[6], p_val[7]));
+  // O^T += V^T . P^T.  Tile mt takes element mt of each of the lane's 8 token pieces.
+  for (int mt = 0; mt < 8; ++mt) {
+    const uint32_t selector = (mt & 1) ? 0x07060302u : 0x05040100u;
+    uint32_t a_words[4];
+    for (int pair = 0; pair < 4; ++pair)
+      a_words[pair] = __builtin_amdgcn_perm(dword_of(cur.v[2 * pair + 1], mt >> 1),
+                                            dword_of(cur.v[2 * pair], mt >> 1), selector);
+    const uint4 a_reg = make_uint4(a_words[0], a_words[1], a_words[2], a_words[3]);
+    o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_reg),
+                                                   __builtin_bit_cast(bf16x8, p_reg), o[mt], 0, 0,
+                                                   0);
+  }
+}
+
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void ragged_attention_mfma_kernel(
+    FastRagged p, ErrorSlot *error) {
+  const uint32_t lane = threadIdx.x, hl = lane & 15, g = lane >> 4;
+  const uint32_t item = blockIdx.x / p.kv_heads, kv_head = blockIdx.x % p.kv_heads;
+  if (item >= p.item_count[0]) return;
+  const uint2 work = p.items[item];
+  const uint32_t token = work.x, split = work.y;
+  const TokenPlan plan = p.plans[token];
   const uint32_t begin = split * plan.chunk;
   const uint32_t end = min(plan.attended, begin + plan.chunk);
   const uint32_t pt = p.page_tokens;
   const uint32_t *table = p.tables + (uint64_t)plan.lane * p.table_pages * 2;
+  LaneConst lc;
+  lc.row_elems = p.kv_heads * 128;
+  lc.k_offset = (hl * p.kv_heads + kv_head) * 128 + 8 * g;
+  lc.v_offset = (4 * g * p.kv_heads + kv_head) * 128 + 8 * hl;
 
   // Query operand: head hl of this kv head's group (zero rows beyond the group).
   uint4 q_reg[4];
   {
     const uint32_t head = kv_head * p.group + hl;
     const uint16_t *q_row = p.q + (uint64_t)token * p.q_stride_t + (uint64_t)head * p.q_stride_h;
-    for (int step = 0; step < 4; ++step) {
+    for (int step = 0; step < 4; ++step) {  // same head-dim slice per (step, g) as the K operand
       q_reg[step] = make_uint4(0, 0, 0, 0);
-      if (hl < p.group) q_reg[step] = *(const uint4 *)(q_row + 32 * g + 8 * step);
+      if (hl < p.group) q_reg[step] = *(const uint4 *)(q_row + 32 * step + 8 * g);
     }
   }
   f32x4 o[8];
   for (int mt = 0; mt < 8; ++mt) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -__builtin_inff(), l_run = 0.0f;
+  Softmax sm{-__builtin_inff(), 0.0f};
 
   const uint32_t first_page = begin / pt, last_page = (end - 1) / pt;
   for (uint32_t page0 = first_page; page0 <= last_page; page0 += 64) {
@@ -300,160 +466,93 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_kernel(FastRagged p,
       return;
     }
     const uint32_t tok_lo = max(begin, page0 * pt);
-    const uint64_t tok_hi64 = min((uint64_t)end, ((uint64_t)page0 + 64) * pt);
-    const uint32_t tok_hi = (uint32_t)tok_hi64;
-    for (uint32_t tile0 = tok_lo; tile0 < tok_hi; tile0 += kTile) {
-      // Pool row of the first token of each 16-token half (a half never straddles a page).
-      uint64_t row0[2] = {0, 0};
-      for (int sub = 0; sub < 2; ++sub) {
-        uint32_t tok0 = tile0 + 16 * sub;
-        if (tok0 < end) {
-          uint32_t page = __shfl(physical, (int)(tok0 / pt - page0), 64);
-          row0[sub] = (uint64_t)page * pt + tok0 % pt;
-        }
-      }
-      // K: lane (token hl, group g) reads 64 contiguous bytes of its token row.
-      uint4 k_reg[2][4];
-      for (int sub = 0; sub < 2; ++sub) {
-        uint32_t tok = tile0 + 16 * sub + hl;
-        const uint16_t *k_row =
-            p.key_pool + ((row0[sub] + hl) * p.kv_heads + kv_head) * 128 + 32 * g;
-        for (int step = 0; step < 4; ++step) {
-          k_reg[sub][step] = make_uint4(0, 0, 0, 0);
-          if (tok < end) k_reg[sub][step] = *(const uint4 *)(k_row + 8 * step);
-        }
-      }
-      // V: coalesced 16-byte loads of the 32x128 tile (zeros past the end: unused pool slots may
-      // hold anything, and 0 * NaN would poison the product).
-      uint4 v_reg[8];
-      for (int j = 0; j < 8; ++j) {
-        uint32_t piece = lane + 64 * j, row = piece >> 4, col = piece & 15;
-        uint32_t tok = tile0 + row;
-        v_reg[j] = make_uint4(0, 0, 0, 0);
-        if (tok < end)
-          v_reg[j] = *(const uint4 *)(p.value_pool +
-                                      ((row0[row >> 4] + (row & 15)) * p.kv_heads + kv_head) * 128 +
-                                      8 * col);
-      }
-      __syncthreads();  // previous tile's transposed reads are done
-      for (int j = 0; j < 8; ++j) {
-        uint32_t piece = lane + 64 * j, row = piece >> 4, col = piece & 15;
-        uint2 *dst = (uint2 *)(v_tile + row * kVPitch + col * 16);
-        dst[0] = make_uint2(v_reg[j].x, v_reg[j].y);
-        dst[1] = make_uint2(v_reg[j].z, v_reg[j].w);
-      }
-      // Scores.
-      float s_val[8];
-      for (int sub = 0; sub < 2; ++sub) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int step = 0; step < 4; ++step)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              __builtin_bit_cast(bf16x8, k_reg[sub][step]), __builtin_bit_cast(bf16x8, q_reg[step]),
-              acc, 0, 0, 0);
-        for (int j = 0; j < 4; ++j) {
-          uint32_t tok = tile0 + 16 * sub + 4 * g + j;
-          s_val[4 * sub + j] = tok < end ? acc[j] * p.scale_log2 : -__builtin_inff();
-        }
-      }
-      float tile_max = s_val[0];
-      for (int i = 1; i < 8; ++i) tile_max = fmaxf(tile_max, s_val[i]);
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-      float m_new = fmaxf(m_run, tile_max);
-      float alpha = exp2f(m_run - m_new);
-      float p_val[8], p_sum = 0.0f;
-      for (int i = 0; i < 8; ++i) {
-        p_val[i] = exp2f(s_val[i] - m_new);
-        p_sum += p_val[i];
-      }
-      l_run = l_run * alpha + p_sum;
-      m_run = m_new;
-      uint4 p_reg = make_uint4(pack_bf16(p_val[0], p_val[1]), pack_bf16(p_val[2], p_val[3]),
-                               pack_bf16(p_val[4], p_val[5]), pack_bf16(p_val[6], p_val[7]));
-      for (int mt = 0; mt < 8; ++mt)
-        for (int j = 0; j < 4; ++j) o[mt][j] *= alpha;
-      __syncthreads();  // V tile visible
-      // O^T += V^T . P^T ; contraction slot i of lane group g is token (i<4 ? 4g+i : 16+4g+i-4).
-      const uint16_t *v_lds = (const uint16_t *)v_tile;
-      for (int mt = 0; mt < 8; ++mt) {
-        uint32_t a_words[4];
-        for (int pair = 0; pair < 4; ++pair) {
-          uint32_t i0 = 2 * pair, i1 = 2 * pair + 1;
-          uint32_t r0 = (i0 < 4 ? 4 * g + i0 : 16 + 4 * g + i0 - 4);
-          uint32_t r1 = (i1 < 4 ? 4 * g + i1 : 16 + 4 * g + i1 - 4);
-          uint32_t lo = v_lds[r0 * (kVPitch / 2) + 16 * mt + hl];
-          uint32_t hi = v_lds[r1 * (kVPitch / 2) + 16 * mt + hl];
-          a_words[pair] = lo | (hi << 16);
-        }
-        uint4 a_reg = make_uint4(a_words[0], a_words[1], a_words[2], a_words[3]);
-        o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_reg),
-                                                       __builtin_bit_cast(bf16x8, p_reg), o[mt], 0,
-                                                       0, 0);
-      }
+    const uint32_t tok_hi = (uint32_t)min((uint64_t)end, ((uint64_t)page0 + 64) * pt);
+    // Full tiles first (no bounds logic at all), then at most one partial tile.
+    const uint32_t full_hi = tok_lo + (tok_hi - tok_lo) / kTile * kTile;
+    TileRegs cur;
+    if (tok_lo < full_hi)
+      load_tile<false>(p, cur, tok_lo, end, page0, physical, lc, hl, g);
+    else
+      load_tile<true>(p, cur, tok_lo, end, page0, physical, lc, hl, g);
+    for (uint32_t tile0 = tok_lo; tile0 < full_hi; tile0 += kTile) {
+      // Software pipeline: the next tile's loads are in flight while this one is consumed.
+      TileRegs nxt;
+      const uint32_t next0 = tile0 + kTile;
+      if (next0 < full_hi)
+        load_tile<false>(p, nxt, next0, end, page0, physical, lc, hl, g);
+      else if (next0 < tok_hi)
+        load_tile<true>(p, nxt, next0, end, page0, physical, lc, hl, g);
+      consume_tile<false>(cur, q_reg, o, sm, tile0, end, p.scale_log2, g);
+      if (next0 < tok_hi) cur = nxt;
     }
+    if (full_hi < tok_hi) consume_tile<true>(cur, q_reg, o, sm, full_hi, end, p.scale_log2, g);
   }
+  float m_run = sm.m, l_run = sm.l;
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
   if (hl >= p.group) return;
+  // Lane (head hl, group g) holds value columns 32g + 8j + mt.
   const uint32_t head = kv_head * p.group + hl;
   if (plan.splits == 1) {
     float inv = 1.0f / l_run;
     uint16_t *out_row = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
-    for (int mt = 0; mt < 8; ++mt) {
-      uint2 packed = make_uint2(pack_bf16(o[mt][0] * inv, o[mt][1] * inv),
-                                pack_bf16(o[mt][2] * inv, o[mt][3] * inv));
-      *(uint2 *)(out_row + 16 * mt + 4 * g) = packed;
+    for (int j = 0; j < 4; ++j) {
+      uint2 lo = make_uint2(pack_bf16(o[0][j] * inv, o[1][j] * inv), pack_bf16(o[2][j] * inv, o[3][j] * inv));
+      uint2 hi = make_uint2(pack_bf16(o[4][j] * inv, o[5][j] * inv), pack_bf16(o[6][j] * inv, o[7][j] * inv));
+      *(uint2 *)(out_row + 32 * g + 8 * j) = lo;
+      *(uint2 *)(out_row + 32 * g + 8 * j + 4) = hi;
     }
     return;
   }
-  uint64_t item = ((uint64_t)token * p.max_splits + split) * p.query_heads + head;
-  float *po = p.partial_o + item * 128;
-  for (int mt = 0; mt < 8; ++mt)
-    *(float4 *)(po + 16 * mt + 4 * g) = make_float4(o[mt][0], o[mt][1], o[mt][2], o[mt][3]);
-  if (g == 0) p.partial_ml[item] = make_float2(m_run, l_run);
+  uint64_t slot = ((uint64_t)token * p.max_splits + split) * p.query_heads + head;
+  float *po = p.partial_o + slot * 128 + 32 * g;
+  for (int j = 0; j < 4; ++j) {
+    *(float4 *)(po + 8 * j) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
+    *(float4 *)(po + 8 * j + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
+  }
+  if (g == 0) p.partial_ml[slot] = make_float2(m_run, l_run);
 }
 
-// Merges the per-split partials of one token: out = sum_s O_s 2^(m_s-M) / sum_s l_s 2^(m_s-M).
-// Also writes the zero rows of inactive lanes, uncovered tokens and tokens whose page table was
-// refused.
-__global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
-  const uint32_t token = blockIdx.x;
-  const SplitPlan plan = plan_token(p, token);
-  const bool zero = !plan.live || plan.attended == 0 || p.bad[token] != 0;
+// Merges the per-split partials of one (token, head): out = sum_s O_s 2^(m_s-M) / sum_s l_s
+// 2^(m_s-M).  Also writes the zero rows of inactive lanes, uncovered tokens and tokens whose page
+// table was refused.
+__global__ __launch_bounds__(64) void ragged_reduce_kernel(FastRagged p) {
+  const uint32_t head = blockIdx.x, token = blockIdx.y;
+  const TokenPlan plan = p.plans[token];
+  const bool zero = plan.splits == 0 || p.bad[token] != 0;
   if (!zero && plan.splits == 1) return;
-  const uint32_t work = p.query_heads * 32;  // 4 value columns per thread
-  for (uint32_t item = threadIdx.x; item < work; item += blockDim.x) {
-    uint32_t head = item >> 5, column = (item & 31) * 4;
-    uint16_t *dst = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
-    if (zero) {
-      *(uint2 *)dst = make_uint2(0, 0);
-      continue;
-    }
-    uint64_t base = (uint64_t)token * p.max_splits * p.query_heads + head;
-    float m_all = -__builtin_inff();
-    for (uint32_t s = 0; s < plan.splits; ++s)
-      m_all = fmaxf(m_all, p.partial_ml[base + (uint64_t)s * p.query_heads].x);
-    float l_all = 0.0f;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t s = 0; s < plan.splits; ++s) {
-      uint64_t at = base + (uint64_t)s * p.query_heads;
-      float2 ml = p.partial_ml[at];
-      float w = exp2f(ml.x - m_all);
-      l_all += ml.y * w;
-      float4 part = *(const float4 *)(p.partial_o + at * 128 + column);
-      acc.x += part.x * w;
-      acc.y += part.y * w;
-      acc.z += part.z * w;
-      acc.w += part.w * w;
-    }
+  const uint32_t lane = threadIdx.x, column = (lane & 31) * 4, half = lane >> 5;
+  uint16_t *dst = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
+  if (zero) {
+    if (half == 0) *(uint2 *)dst = make_uint2(0, 0);
+    return;
+  }
+  const uint64_t base = (uint64_t)token * p.max_splits * p.query_heads + head;
+  float m_all = -__builtin_inff();
+  for (uint32_t s = 0; s < plan.splits; ++s)
+    m_all = fmaxf(m_all, p.partial_ml[base + (uint64_t)s * p.query_heads].x);
+  float l_all = 0.0f;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (uint32_t s = half; s < plan.splits; s += 2) {
+    uint64_t at = base + (uint64_t)s * p.query_heads;
+    float2 ml = p.partial_ml[at];
+    float w = exp2f(ml.x - m_all);
+    l_all += ml.y * w;
+    float4 part = *(const float4 *)(p.partial_o + at * 128 + column);
+    acc.x += part.x * w;
+    acc.y += part.y * w;
+    acc.z += part.z * w;
+    acc.w += part.w * w;
+  }
+  l_all += __shfl_xor(l_all, 32, 64);
+  acc.x += __shfl_xor(acc.x, 32, 64);
+  acc.y += __shfl_xor(acc.y, 32, 64);
+  acc.z += __shfl_xor(acc.z, 32, 64);
+  acc.w += __shfl_xor(acc.w, 32, 64);
+  if (half == 0) {
     float inv = 1.0f / l_all;
     *(uint2 *)dst = make_uint2(pack_bf16(acc.x * inv, acc.y * inv), pack_bf16(acc.z * inv, acc.w * inv));
   }
-}
-
-__global__ void clear_flags_kernel(uint32_t *flags, uint32_t count) {
-  uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < count) flags[i] = 0;
 }
 
 bool fast_ragged_eligible(const RaggedAttention &p) {
@@ -483,23 +582,47 @@ uint32_t splits_for(uint32_t tokens) {
   return max_splits;
 }
 
-// Carves flags / (m,l) / O partial storage for `tokens` out of the backend workspace.
+// Carves flags / plans / work items / (m,l) / O partial storage out of the backend workspace.
 bool carve_partials(fh_backend *backend, FastRagged *f) {
-  uint64_t items = (uint64_t)f->tokens * f->max_splits * f->query_heads;
-  uint64_t flags_bytes = ((uint64_t)f->tokens * 4 + 255) / 256 * 256;
-  uint64_t ml_bytes = (items * sizeof(float2) + 255) / 256 * 256;
-  uint64_t o_bytes = items * 128 * sizeof(float);
-  char *ws = backend_workspace(backend, flags_bytes + ml_bytes + o_bytes);
+  static const uint32_t split_tokens = [] {
+    const char *env = getenv("FORJA_HIP_SPLIT_TOKENS");
+    uint32_t value = env ? (uint32_t)atoi(env) : 0;
+    return value >= 32 ? value / 32 * 32 : 0;  // 0 = chosen per launch from the batch
+  }();
+  f->split_tokens = split_tokens;
+  auto round = [](uint64_t bytes) { return (bytes + 255) / 256 * 256; };
+  uint64_t slots = (uint64_t)f->tokens * f->max_splits;
+  uint64_t flags_bytes = round((uint64_t)f->tokens * 4);
+  uint64_t plan_bytes = round((uint64_t)f->tokens * sizeof(TokenPlan));
+  uint64_t item_bytes = round(slots * sizeof(uint2));
+  uint64_t count_bytes = 256;
+  uint64_t ml_bytes = round(slots * f->query_heads * sizeof(float2));
+  uint64_t o_bytes = slots * f->query_heads * 128 * sizeof(float);
+  char *ws = backend_workspace(
+      backend, flags_bytes + plan_bytes + item_bytes + count_bytes + ml_bytes + o_bytes);
   if (!ws) return false;
   f->bad = (uint32_t *)ws;
-  f->partial_ml = (float2 *)(ws + flags_bytes);
-  f->partial_o = (float *)(ws + flags_bytes + ml_bytes);
+  ws += flags_bytes;
+  f->plans = (TokenPlan *)ws;
+  ws += plan_bytes;
+  f->items = (uint2 *)ws;
+  ws += item_bytes;
+  f->item_count = (uint32_t *)ws;
+  ws += count_bytes;
+  f->partial_ml = (float2 *)ws;
+  ws += ml_bytes;
+  f->partial_o = (float *)ws;
   return true;
 }
 
+void launch_plan(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
+  ragged_plan_kernel<<<dim3(1), 256, 0, stream>>>(f, error);
+}
+
 void launch_fast(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
-  ragged_attention_mfma_kernel<<<dim3(f.max_splits, f.tokens, f.kv_heads), 64, 0, stream>>>(f, error);
-  ragged_reduce_kernel<<<dim3(f.tokens), 256, 0, stream>>>(f);
+  uint64_t blocks = (uint64_t)f.tokens * f.max_splits * f.kv_heads;
+  ragged_attention_mfma_kernel<<<dim3((unsigned)blocks), 64, 0, stream>>>(f, error);
+  ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens), 64, 0, stream>>>(f);
 }
 
 }  // namespace
@@ -545,7 +668,7 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   f.out_stride_t = lane.out.stride[1];
   f.out_stride_h = lane.out.stride[0];
   hipStream_t stream = backend_stream(backend);
-  clear_flags_kernel<<<dim3((f.tokens + 255) / 256), 256, 0, stream>>>(f.bad, f.tokens);
+  launch_plan(stream, f, error);
   launch_fast(stream, f, error);
   return true;
 }
@@ -581,7 +704,7 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     f.physical_pages = p.physical_pages;
     f.table_pages = p.table_pages;
     f.scale_log2 = p.scale * 1.4426950408889634f;
-    clear_flags_kernel<<<dim3((p.tokens + 255) / 256), 256, 0, stream>>>(f.bad, p.tokens);
+    launch_plan(stream, f, error);
   }
   uint64_t append_work =
       (uint64_t)p.tokens * (p.kv_heads * p.width + p.kv_heads * p.value_width);

@@ -1,4 +1,21 @@
-// Specialised MLX-4bit affine quantised matmul kernels (dense and routed) for gfx950.
+// MLX-4bit affine group-quantised matmul on the gfx950 matrix cores, dense and routed (MoE).
+//
+// y[m,n] = sum_k x[m,k] * (scale[n,k/64] * q[n,k] + bias[n,k/64])      (affine_quant_dot,
+// crates/forja-cpu/src/lib.rs:1277-1310), q = nibble k%8 of word k/8, low nibble first.
+//
+// The work is HBM-bound on the packed weights, so the kernel is built around reading each weight
+// byte once, with 16-byte loads, and spending as few vector instructions per nibble as possible:
+//   * a nibble becomes the bf16 value 16+q with two integer ops for two nibbles
+//     ((w >> s) & 0x00780078 | 0x41804180: q lands in mantissa bits 3..6 of exponent 2^4); the
+//     pairs come out in the order (0,4)(1,5)(2,6)(3,7), and the activation tile is staged in LDS
+//     with the same permutation inside every 8 elements;
+//   * v_mfma_f32_32x32x16_bf16 contracts one 64-element quantisation group in four steps (each
+//     lane holds the four packed words = 32 values of "its" half of the group for one output
+//     column), giving part[m,n] = sum x * (16+q) exactly in f32;
+//   * the affine parameters are applied once per group: acc += scale*part + (bias-16*scale)*xsum,
+//     with xsum[m,group] = sum of the group's activations computed while staging.
+// The dequantised weight is never rounded to bf16, so results track the f32 reference closely.
+// Activations: bf16; 32 rows per MFMA tile (padded); a workgroup is 4 waves x 32 columns.
 #include "fast_kernels.hpp"
 
 #include <algorithm>
@@ -6,14 +23,410 @@
 
 namespace fh {
 
-bool try_fast_quant_matmul(hipStream_t, const QmmProblem &) { return false; }
+namespace {
 
-bool try_fast_gather_projection(fh_backend *, const GatherProblem &, int, bool, ErrorSlot *) {
-  return false;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int kWaves = 4;           // waves per workgroup
+constexpr int kColsPerWave = 32;
+constexpr int kGroup = 64;          // quantisation group handled by this path
+constexpr uint32_t kNoBlock = 0xffffffffu;
+
+enum Epilogue { kStore = 0, kSwiglu = 1 };
+
+struct QmmArgs {
+  const uint16_t *x;        // bf16 activations, innermost axis contiguous
+  uint64_t x_row_stride;    // elements between input rows
+  const uint32_t *packed[2];
+  const uint16_t *scales[2], *biases[2];
+  uint64_t expert_words;    // u32 words per expert matrix (N*K/8); 0 for dense
+  uint64_t expert_groups;   // scale entries per expert matrix (N*K/64)
+  void *out;                // bf16 or f32
+  uint64_t out_row_stride;  // elements
+  uint32_t out_f32;
+  uint32_t rows, inner, columns;
+  // routed form
+  const uint32_t *sorted_routes, *blocks, *n_blocks;
+  uint32_t route_div;       // input row = route / route_div
+};
+
+__device__ inline uint32_t pack2(float lo, float hi) {
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
 }
 
-bool try_fast_gather_weighted(fh_backend *, const GatherProblem &, const View *, ErrorSlot *) {
-  return false;
+__device__ inline float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+// Eight nibbles of `w` as bf16 (16+q), in slot order (0,4)(1,5)(2,6)(3,7).
+__device__ inline bf16x8 unpack_word(uint32_t w) {
+  const uint32_t mask = 0x00780078u, magic = 0x41804180u;
+  uint4 r;
+  r.x = ((w << 3) & mask) | magic;
+  r.y = ((w >> 1) & mask) | magic;
+  r.z = ((w >> 5) & mask) | magic;
+  r.w = ((w >> 9) & mask) | magic;
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+// MT = 32-row tiles per workgroup, KC = activation columns staged per pass.
+template <int MT, bool kPair, bool kRouted>
+__global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
+  constexpr int KC = 512 / MT;  // 33 KB of LDS either way: two workgroups per CU overlap staging
+  constexpr int kRows = 32 * MT;
+  constexpr int kPitch = 2 * KC + 16;  // bytes; +16 spreads consecutive rows over the banks
+  __shared__ __attribute__((aligned(16))) unsigned char xs[kRows * kPitch];
+  __shared__ __attribute__((aligned(16))) float xsum[(KC / kGroup) * kRows];
+  __shared__ uint32_t row_ids[kRows];
+
+  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint32_t nl = lane & 31, h = lane >> 5;
+  const uint32_t column = (blockIdx.x * kWaves + wave) * kColsPerWave + nl;
+  const uint32_t column_c = min(column, a.columns - 1);  // clamped for loads
+
+  uint32_t expert = 0, count = 0, first = 0;
+  if (kRouted) {
+    if (blockIdx.y >= a.n_blocks[0]) return;
+    expert = a.blocks[3 * blockIdx.y];
+    if (expert == kNoBlock) return;
+    first = a.blocks[3 * blockIdx.y + 1];
+    count = a.blocks[3 * blockIdx.y + 2];
+    if (tid < kRows) row_ids[tid] = tid < count ? a.sorted_routes[first + tid] : 0;
+  } else {
+    first = blockIdx.y * kRows;
+    count = min((uint32_t)kRows, a.rows - first);
+  }
+  const uint32_t words_per_row = a.inner / 8, groups_per_row = a.inner / kGroup;
+  const uint32_t *w_row[2];
+  const uint16_t *s_row[2], *b_row[2];
+  for (int pj = 0; pj < (kPair ? 2 : 1); ++pj) {
+    w_row[pj] = a.packed[pj] + expert * a.expert_words + (uint64_t)column_c * words_per_row + 4 * h;
+    s_row[pj] = a.scales[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
+    b_row[pj] = a.biases[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
+  }
+
+  f32x16 acc[kPair ? 2 : 1][MT];
+  for (int pj = 0; pj < (kPair ? 2 : 1); ++pj)
+    for (int mt = 0; mt < MT; ++mt)
+      for (int j = 0; j < 16; ++j) acc[pj][mt][j] = 0.0f;
+
+  for (uint32_t kc0 = 0; kc0 < a.inner; kc0 += KC) {
+    const uint32_t kc = min((uint32_t)KC, a.inner - kc0);
+    __syncthreads();  // the previous pass is consumed (and row_ids are visible)
+    // ---- stage activations: 16-byte pieces, permuted inside each 8, plus per-group sums
+    const uint32_t pieces_per_row = kc / 8;
+    for (uint32_t piece = tid; piece < kRows * pieces_per_row; piece += 256) {
+      const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (row < count) {
+        const uint64_t in_row = kRouted ? row_ids[row] / a.route_div : first + row;
+        v = *(const uint4 *)(a.x + in_row * a.x_row_stride + kc0 + 8 * pc);
+      }
+      float sum = bf16_bits_to_f32(v.x & 0xffffu) + bf16_bits_to_f32(v.x >> 16) +
+                  bf16_bits_to_f32(v.y & 0xffffu) + bf16_bits_to_f32(v.y >> 16) +
+                  bf16_bits_to_f32(v.z & 0xffffu) + bf16_bits_to_f32(v.z >> 16) +
+                  bf16_bits_to_f32(v.w & 0xffffu) + bf16_bits_to_f32(v.w >> 16);
+      uint4 permuted;
+      permuted.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
+      permuted.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
+      permuted.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+      permuted.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+      *(uint4 *)(xs + row * kPitch + pc * 16) = permuted;
+      // eight consecutive pieces (= lanes) make one quantisation group
+      sum += __shfl_xor(sum, 1, 64);
+      sum += __shfl_xor(sum, 2, 64);
+      sum += __shfl_xor(sum, 4, 64);
+      if ((pc & 7) == 0) xsum[(pc >> 3) * kRows + row] = sum;
+    }
+    __syncthreads();
+    // ---- stream the weights of this pass: 4 groups (256 columns of K) per unrolled round
+    const uint32_t groups = kc / kGroup;
+    const uint32_t word0 = kc0 / 8, group0 = kc0 / kGroup;
+    for (uint32_t g0 = 0; g0 < groups; g0 += 4) {
+      uint4 wq[kPair ? 2 : 1][4];
+      uint32_t sb[kPair ? 2 : 1][4][2];
+      for (int pj = 0; pj < (kPair ? 2 : 1); ++pj)
+        for (int u = 0; u < 4; ++u) {
+          wq[pj][u] = *(const uint4 *)(w_row[pj] + word0 + (g0 + u) * 8);
+          sb[pj][u][0] = s_row[pj][group0 + g0 + u];
+          sb[pj][u][1] = b_row[pj][group0 + g0 + u];
+        }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t gi = g0 + u;
+        f32x16 part[kPair ? 2 : 1][MT];
+        for (int pj = 0; pj < (kPair ? 2 : 1); ++pj)
+          for (int mt = 0; mt < MT; ++mt)
+            for (int j = 0; j < 16; ++j) part[pj][mt][j] = 0.0f;
+#pragma unroll
+        for (int step = 0; step < 4; ++step) {
+          bf16x8 b_op[kPair ? 2 : 1];
+          for (int pj = 0; pj < (kPair ? 2 : 1); ++pj) {
+            const uint32_t word = step == 0 ? wq[pj][u].x
+                                            : (step == 1 ? wq[pj][u].y
+                                                         : (step == 2 ? wq[pj][u].z : wq[pj][u].w));
+            b_op[pj] = unpack_word(word);
+          }
+          for (int mt = 0; mt < MT; ++mt) {
+            const uint4 a_raw = *(const uint4 *)(xs + (mt * 32 + nl) * kPitch +
+                                                 (gi * kGroup + 32 * h + 8 * step) * 2);
+            const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
+            for (int pj = 0; pj < (kPair ? 2 : 1); ++pj)
+              part[pj][mt] =
+                  __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op[pj], part[pj][mt], 0, 0, 0);
+          }
+        }
+        // ---- affine fix-up for this group; row blocks beyond `count` are skipped
+        for (int pj = 0; pj < (kPair ? 2 : 1); ++pj) {
+          const float scale = bf16_bits_to_f32(sb[pj][u][0]);
+          const float shift = bf16_bits_to_f32(sb[pj][u][1]) - 16.0f * scale;
+          for (int mt = 0; mt < MT; ++mt)
+            for (int jq = 0; jq < 4; ++jq) {
+              if ((uint32_t)(mt * 32 + 8 * jq) >= count) continue;
+              const float4 sums = *(const float4 *)(xsum + gi * kRows + mt * 32 + 8 * jq + 4 * h);
+              acc[pj][mt][4 * jq + 0] += scale * part[pj][mt][4 * jq + 0] + shift * sums.x;
+              acc[pj][mt][4 * jq + 1] += scale * part[pj][mt][4 * jq + 1] + shift * sums.y;
+              acc[pj][mt][4 * jq + 2] += scale * part[pj][mt][4 * jq + 2] + shift * sums.z;
+              acc[pj][mt][4 * jq + 3] += scale * part[pj][mt][4 * jq + 3] + shift * sums.w;
+            }
+        }
+      }
+    }
+  }
+  // ---- epilogue and store; lane (column nl, half h) holds rows 8*(j/4) + 4h + j%4 of each tile
+  if (column >= a.columns) return;
+  for (int mt = 0; mt < MT; ++mt)
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t row = mt * 32 + 8 * (j / 4) + 4 * h + (j % 4);
+      if (row >= count) continue;
+      float value = acc[0][mt][j];
+      if (kPair) {
+        const float gate = value, up = acc[kPair ? 1 : 0][mt][j];
+        value = gate * (1.0f / (1.0f + __expf(-gate))) * up;
+      }
+      const uint64_t out_row = kRouted ? row_ids[row] : first + row;
+      const uint64_t at = out_row * a.out_row_stride + column;
+      if (a.out_f32)
+        ((float *)a.out)[at] = value;
+      else
+        ((uint16_t *)a.out)[at] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+    }
+}
+
+// out[r, :] = residual[r, :] + sum_s weights[r, s] * partial[r*k + s, :], slots in ascending
+// order (execute_gather_quant_weighted_sum, crates/forja-cpu/src/lib.rs:1153-1199); routes that
+// name no valid expert contribute nothing.
+__global__ void combine_routes_kernel(const float *partial, View indices, View weights,
+                                      View residual, int has_residual, View out, uint32_t rows,
+                                      uint32_t routes, uint32_t columns, uint32_t experts) {
+  uint64_t flat = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (flat >= (uint64_t)rows * columns) return;
+  uint32_t row = (uint32_t)(flat / columns), column = (uint32_t)(flat % columns);
+  float value = 0.0f;
+  for (uint32_t slot = 0; slot < routes; ++slot) {
+    uint32_t expert = load_u32_at(indices, indices.offset + row * indices.stride[0] +
+                                               slot * indices.stride[1]);
+    if (expert >= experts) continue;
+    float weight = load_float_at(weights, weights.offset + row * weights.stride[0] +
+                                              slot * weights.stride[1]);
+    value += weight * partial[((uint64_t)row * routes + slot) * columns + column];
+  }
+  if (has_residual)
+    value += load_float_at(residual, residual.offset + row * residual.stride[0] +
+                                         column * residual.stride[1]);
+  store_float_at(out, out.offset + row * out.stride[0] + column * out.stride[1], value);
+}
+
+bool rows_contiguous(const View &v, uint32_t rank) {
+  // innermost axis contiguous and every outer stride the dense product (weights, scales)
+  uint64_t expected = 1;
+  for (int axis = (int)rank - 1; axis >= 0; --axis) {
+    if (v.shape[axis] != 1 && v.stride[axis] != expected) return false;
+    expected *= v.shape[axis];
+  }
+  return true;
+}
+
+bool weights_eligible(const View &packed, const View &scales, const View &biases, uint32_t rank,
+                      uint32_t inner, uint32_t bits, uint32_t group) {
+  if (bits != 4 || group != kGroup || inner % 256 != 0) return false;
+  if (scales.dtype != FH_BF16 || biases.dtype != FH_BF16) return false;
+  if (!rows_contiguous(packed, rank) || !rows_contiguous(scales, rank) ||
+      !rows_contiguous(biases, rank))
+    return false;
+  if (packed.offset % 4 != 0) return false;  // 16-byte aligned rows (K/8 words is a multiple of 32)
+  return true;
+}
+
+template <bool kPair, bool kRouted>
+void launch_qmm(hipStream_t stream, const QmmArgs &a, uint32_t row_blocks, int mt) {
+  dim3 grid((a.columns + kWaves * kColsPerWave - 1) / (kWaves * kColsPerWave), row_blocks);
+  if (mt == 1)
+    qmm_mfma_kernel<1, kPair, kRouted><<<grid, 256, 0, stream>>>(a);
+  else
+    qmm_mfma_kernel<2, kPair, kRouted><<<grid, 256, 0, stream>>>(a);
+}
+
+const uint32_t *u32_ptr(const View &v) { return (const uint32_t *)v.base + v.offset; }
+const uint16_t *u16_ptr(const View &v) { return (const uint16_t *)v.base + v.offset; }
+
+}  // namespace
+
+bool try_fast_quant_matmul(hipStream_t stream, const QmmProblem &p) {
+  if (p.x.dtype != FH_BF16) return false;
+  if (p.out.dtype != FH_BF16 && p.out.dtype != FH_F32) return false;
+  if (!weights_eligible(p.packed, p.scales, p.biases, 2, p.inner, p.bits, p.group)) return false;
+  if (p.x.stride[1] != 1 || p.x.stride[0] % 8 != 0 || p.x.offset % 8 != 0) return false;
+  if (p.out.stride[1] != 1) return false;
+  QmmArgs a{};
+  a.x = u16_ptr(p.x);
+  a.x_row_stride = p.x.stride[0];
+  a.packed[0] = u32_ptr(p.packed);
+  a.scales[0] = u16_ptr(p.scales);
+  a.biases[0] = u16_ptr(p.biases);
+  a.out = p.out.dtype == FH_F32 ? (void *)((float *)p.out.base + p.out.offset)
+                                : (void *)((uint16_t *)p.out.base + p.out.offset);
+  a.out_row_stride = p.out.stride[0];
+  a.out_f32 = p.out.dtype == FH_F32;
+  a.rows = p.rows;
+  a.inner = p.inner;
+  a.columns = p.columns;
+  int mt = p.rows <= 32 ? 1 : 2;
+  uint32_t row_blocks = (p.rows + 32 * mt - 1) / (32 * mt);
+  launch_qmm<false, false>(stream, a, row_blocks, mt);
+  return true;
+}
+
+namespace {
+
+constexpr uint32_t kRouteTile = 32;
+
+struct RoutePlan {
+  uint32_t *counts, *offsets, *sorted_routes, *blocks, *n_blocks;
+  uint32_t max_blocks;
+  char *rest;  // workspace after the plan
+};
+
+// Packs the routes on the device into `extra` + plan bytes of workspace.
+bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, ErrorSlot *error,
+                 RoutePlan *plan) {
+  uint64_t routes = (uint64_t)p.rows * p.k;
+  plan->max_blocks = p.experts + (uint32_t)(routes / kRouteTile) + 1;
+  auto round = [](uint64_t bytes) { return (bytes + 255) / 256 * 256; };
+  uint64_t counts_b = round(p.experts * 4ull), offsets_b = round((p.experts + 1) * 4ull),
+           sorted_b = round(routes * 4), blocks_b = round(plan->max_blocks * 12ull), nb_b = 256;
+  char *ws = backend_workspace(backend, counts_b + offsets_b + sorted_b + blocks_b + nb_b + extra);
+  if (!ws) return false;
+  plan->counts = (uint32_t *)ws;
+  ws += counts_b;
+  plan->offsets = (uint32_t *)ws;
+  ws += offsets_b;
+  plan->sorted_routes = (uint32_t *)ws;
+  ws += sorted_b;
+  plan->blocks = (uint32_t *)ws;
+  ws += blocks_b;
+  plan->n_blocks = (uint32_t *)ws;
+  ws += nb_b;
+  plan->rest = ws;
+  launch_route_pack(backend_stream(backend), p.indices, p.rows, p.k, p.experts, kRouteTile,
+                    plan->counts, plan->offsets, plan->sorted_routes, plan->blocks,
+                    plan->max_blocks, plan->n_blocks, error);
+  return true;
+}
+
+bool gather_eligible(const GatherProblem &p, int projections) {
+  if (p.x.dtype != FH_BF16) return false;
+  for (int pj = 0; pj < projections; ++pj)
+    if (!weights_eligible(p.packed[pj], p.scales[pj], p.biases[pj], 3, p.inner, p.bits, p.group))
+      return false;
+  if ((uint64_t)p.rows * p.k > (1u << 24)) return false;
+  return true;
+}
+
+}  // namespace
+
+bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int projections,
+                                bool swiglu, ErrorSlot *error) {
+  if (!gather_eligible(p, projections)) return false;
+  if (projections == 2 && !swiglu) return false;
+  if (p.out.dtype != FH_BF16 || ((uint64_t)p.rows * p.k * p.columns) % 2 != 0) return false;
+  // x [R,K] rows; out [R,k,N] must be dense so that route r*k+s is row r*k+s of [R*k, N]
+  if (p.x.stride[1] != 1 || p.x.stride[0] % 8 != 0 || p.x.offset % 8 != 0) return false;
+  if (p.out.stride[2] != 1 || p.out.stride[1] != p.columns ||
+      p.out.stride[0] != (uint64_t)p.k * p.columns)
+    return false;
+  RoutePlan plan;
+  if (!plan_routes(backend, p, 0, error, &plan)) return false;
+  hipStream_t stream = backend_stream(backend);
+  // Rows of bad routes stay zero: clear the output first (bad routes are never packed).
+  launch_fill_u32(stream, (uint32_t *)((uint16_t *)p.out.base + p.out.offset),
+                  (uint64_t)p.rows * p.k * p.columns / 2, 0);
+  QmmArgs a{};
+  a.x = u16_ptr(p.x);
+  a.x_row_stride = p.x.stride[0];
+  for (int pj = 0; pj < projections; ++pj) {
+    a.packed[pj] = u32_ptr(p.packed[pj]);
+    a.scales[pj] = u16_ptr(p.scales[pj]);
+    a.biases[pj] = u16_ptr(p.biases[pj]);
+  }
+  a.expert_words = (uint64_t)p.columns * p.inner / 8;
+  a.expert_groups = (uint64_t)p.columns * p.inner / kGroup;
+  a.out = (uint16_t *)p.out.base + p.out.offset;
+  a.out_row_stride = p.columns;
+  a.out_f32 = 0;
+  a.rows = p.rows * p.k;
+  a.inner = p.inner;
+  a.columns = p.columns;
+  a.sorted_routes = plan.sorted_routes;
+  a.blocks = plan.blocks;
+  a.n_blocks = plan.n_blocks;
+  a.route_div = p.k;
+  if (projections == 2)
+    launch_qmm<true, true>(stream, a, plan.max_blocks, 1);
+  else
+    launch_qmm<false, true>(stream, a, plan.max_blocks, 1);
+  return true;
+}
+
+bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const View *residual,
+                              ErrorSlot *error) {
+  if (!gather_eligible(p, 1)) return false;
+  // x [R,k,K] dense rows so that route r*k+s is row r*k+s of [R*k, K]
+  if (p.x.stride[2] != 1 || p.x.stride[1] % 8 != 0 || p.x.offset % 8 != 0 ||
+      p.x.stride[0] != (uint64_t)p.k * p.x.stride[1])
+    return false;
+  uint64_t partial_bytes = (uint64_t)p.rows * p.k * p.columns * sizeof(float);
+  RoutePlan plan;
+  if (!plan_routes(backend, p, partial_bytes, error, &plan)) return false;
+  hipStream_t stream = backend_stream(backend);
+  float *partial = (float *)plan.rest;
+  QmmArgs a{};
+  a.x = u16_ptr(p.x);
+  a.x_row_stride = p.x.stride[1];
+  a.packed[0] = u32_ptr(p.packed[0]);
+  a.scales[0] = u16_ptr(p.scales[0]);
+  a.biases[0] = u16_ptr(p.biases[0]);
+  a.expert_words = (uint64_t)p.columns * p.inner / 8;
+  a.expert_groups = (uint64_t)p.columns * p.inner / kGroup;
+  a.out = partial;
+  a.out_row_stride = p.columns;
+  a.out_f32 = 1;
+  a.rows = p.rows * p.k;
+  a.inner = p.inner;
+  a.columns = p.columns;
+  a.sorted_routes = plan.sorted_routes;
+  a.blocks = plan.blocks;
+  a.n_blocks = plan.n_blocks;
+  a.route_div = 1;
+  launch_qmm<false, true>(stream, a, plan.max_blocks, 1);
+  uint64_t work = (uint64_t)p.rows * p.columns;
+  View none{};
+  none.base = nullptr;
+  combine_routes_kernel<<<dim3((unsigned)((work + 255) / 256)), 256, 0, stream>>>(
+      partial, p.indices, p.weights, residual ? *residual : none, residual ? 1 : 0, p.out, p.rows,
+      p.k, p.columns, p.experts);
+  return true;
 }
 
 bool try_fast_program(hipStream_t, bool, const ProgramArgs &, uint64_t) { return false; }

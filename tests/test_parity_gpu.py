@@ -123,6 +123,10 @@ QMM_CASES = [
     (5, 24, 256, 4, 32, DType.F16),
     (3, 24, 256, 8, 128, DType.F32),
     (40, 72, 192, 4, 64, DType.BF16),
+    (1, 2048, 2048, 4, 64, DType.BF16),
+    (64, 100, 512, 4, 64, DType.BF16),      # column tail inside a wave
+    (130, 96, 768, 4, 64, DType.BF16),      # row tail across row blocks
+    (8, 512, 4096, 4, 64, DType.BF16),
 ]
 
 
@@ -176,7 +180,9 @@ def routed_case(seed, rows, k, experts, n, inner, bad=()):
 
 
 @pytest.mark.parametrize("rows,k,experts,n,inner", [(24, 4, 16, 128, 128), (256, 8, 128, 64, 128),
-                                                   (5, 2, 3, 64, 64), (40, 8, 8, 192, 256)])
+                                                   (5, 2, 3, 64, 64), (40, 8, 8, 192, 256),
+                                                   (64, 8, 16, 256, 256), (33, 4, 7, 512, 256),
+                                                   (256, 8, 128, 768, 2048)])   # last: BASELINE config 2
 def test_gather_projection_pair_and_weighted_sum(cpu, hip, rows, k, experts, n, inner):
     gate = Quantised(31, 1, (n, inner), experts=experts)
     up = Quantised(31, 11, (n, inner), experts=experts)

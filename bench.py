@@ -1,0 +1,247 @@
+#!/usr/bin/env python3
+"""Headline benchmark: decode tokens/s of the 4-bit Qwen3-Coder-30B-A3B-shaped ragged continuous
+batch on one MI355X (BASELINE.json metric, config 3).
+
+A step = one forward step of the whole batch: 128 decode lanes (contexts log-uniform over
+256..32768, non-contiguous block tables, page size 16), 48 MoE layers, lm_head and greedy argmax,
+recorded once as a command list and replayed; every step 8 sequences retire and 8 are admitted.
+Weights and K/V pools are synthetic, generated on the device, resident in HBM before timing.
+
+Prints one JSON line with the throughput, the roofline of the dominant kernel (paged attention,
+HBM-bound) measured with HIP events on the backend's stream inside the timed region, and the CPU
+baseline (the single-threaded oracle on a bounded sample of the same workload).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from forja_amd.core import CommandList, DType, Op  # noqa: E402
+from forja_amd.hip_backend import HipBackend  # noqa: E402
+from forja_amd.model import (QWEN3_CODER_30B_A3B, QWEN3_0_6B, DecodeSession, Model,  # noqa: E402
+                             ModelConfig)
+
+HBM_PEAK_GBPS = 8000.0
+KC_ATTENTION, KC_MOE, KC_QMM = 3, 2, 1
+KC_ATTENTION_KERNEL, KC_MOE_KERNEL, KC_QMM_KERNEL = 4, 5, 6
+
+
+def log_uniform(rng, lo, hi, count):
+    return np.exp(rng.uniform(math.log(lo), math.log(hi), count)).astype(np.int64)
+
+
+class Workload:
+    """Config 3: 128 decode lanes, 8 retire + 8 admit per step."""
+
+    def __init__(self, backend, config: ModelConfig, lanes, ctx_lo, ctx_hi, churn, seed, layers=None,
+                 capacity_factor=1.45):
+        self.rng = np.random.default_rng(seed)
+        self.lanes, self.ctx_lo, self.ctx_hi, self.churn = lanes, ctx_lo, ctx_hi, churn
+        contexts = log_uniform(self.rng, ctx_lo, ctx_hi, lanes)
+        pt = config.page_tokens
+        expected_tokens = lanes * (ctx_hi - ctx_lo) / math.log(ctx_hi / ctx_lo)
+        capacity_tokens = max(int(expected_tokens * capacity_factor), int(contexts.sum() * 1.1))
+        self.capacity_pages = capacity_tokens // pt + 2 * lanes
+        table_pages = (ctx_hi + 4096 + pt) // pt
+        self.model = Model(backend, config, seed=seed, layers=layers)
+        self.session = DecodeSession(self.model, contexts, seed=seed, physical_pages=self.capacity_pages,
+                                     table_pages=table_pages)
+        self.next_lane = 0
+
+    def churn_lanes(self):
+        s = self.session
+        pt = self.model.config.page_tokens
+        for _ in range(self.churn):
+            lane = self.next_lane
+            self.next_lane = (self.next_lane + 1) % self.lanes
+            s.cache.retire(lane)
+            # admit a new sequence whose cache fits the free pages (redraw otherwise)
+            for _attempt in range(16):
+                context = int(log_uniform(self.rng, self.ctx_lo, self.ctx_hi, 1)[0])
+                if (context + 64) // pt + 2 < len(s.cache.free) - 4 * self.lanes:
+                    break
+            else:
+                context = self.ctx_lo
+            s.contexts[lane] = context
+            s.cache.ensure(lane, context + 1)
+            s.cache.upload_tables([lane])
+
+
+def algorithmic_bytes(workload, contexts):
+    """SURVEY/DESIGN accounting: K/V rows read once per kv head, weights incl. scales+biases."""
+    model = workload.model
+    c = model.config
+    kv = int((contexts + 1).sum()) * (model.n_layers * 2 * c.kv_heads * c.head_dim * 2)
+    weights = model.weight_bytes_per_step(len(contexts))
+    return kv, weights
+
+
+def cpu_baseline(config, seed, sample_lanes, ctx_lo, ctx_hi):
+    """Times the CPU oracle (single thread, as the reference backend is single-threaded) on one
+    decoder layer over `sample_lanes` lanes of the same workload plus the lm_head on 2 rows, and
+    extrapolates linearly in layers and rows to a full step."""
+    from oracle.cpu_backend import CpuBackend
+    rng = np.random.default_rng(seed)
+    contexts = log_uniform(rng, ctx_lo, ctx_hi, 128)[:sample_lanes]
+    cpu = CpuBackend(threads=1)
+    model = Model(cpu, config, seed=seed, layers=1)
+    session = DecodeSession(model, contexts, seed=seed)
+    # time the layer: everything except lm_head/argmax, obtained by timing the full single-layer
+    # step and a separate lm_head-only dispatch
+    started = time.perf_counter()
+    session.step()
+    step_seconds = time.perf_counter() - started
+    b = session.buffers
+    head = CommandList()
+    head.dispatch(Op.quant_matmul(4, 64), [b.normalized[0].narrow(0, 0, 2), *model.lm_head.triple],
+                  b.logits.narrow(0, 0, 2))
+    started = time.perf_counter()
+    cpu.submit(head).wait()
+    head_seconds = time.perf_counter() - started
+    head_full_sample = head_seconds * sample_lanes / 2.0
+    layer_seconds = max(step_seconds - head_full_sample, 1e-9)
+    scale_rows = 128.0 / sample_lanes
+    full_step = config.layers * layer_seconds * scale_rows + head_seconds * 64.0
+    return {
+        "value": 128.0 / full_step, "unit": "tok/s", "cores": 1, "kind": "port",
+        "sample": (f"1 of {config.layers} layers x {sample_lanes} of 128 lanes (contexts "
+                   f"{int(contexts.min())}..{int(contexts.max())}) + lm_head on 2 rows, timed "
+                   f"{step_seconds + head_seconds:.1f} s; step time extrapolated linearly in "
+                   f"layers and rows"),
+        "extrapolated_ms_per_step": full_step * 1e3,
+    }
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=4)
+    parser.add_argument("--seed", type=int, default=20261)
+    parser.add_argument("--layers", type=int, default=None, help="debug: fewer layers")
+    parser.add_argument("--lanes", type=int, default=128)
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--cpu-sample-lanes", type=int, default=8)
+    parser.add_argument("--no-profile", action="store_true",
+                        help="skip the HIP-event kernel timing inside the timed region")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the ragged forward step on ONE MI355X; collectives and "
+              "sharding are not part of it, so --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    config = QWEN3_CODER_30B_A3B
+    ctx_lo, ctx_hi, churn = 256, 32768, 8
+    backend = HipBackend(0)
+    info = backend.device_info()
+    workload = Workload(backend, config, args.lanes, ctx_lo, ctx_hi, churn, args.seed, layers=args.layers)
+    session = workload.session
+    backend.synchronize()
+
+    def run_step():
+        contexts = session.contexts.copy()
+        submission = session.submit_step()
+        workload.churn_lanes()
+        return submission, contexts
+
+    for _ in range(args.warmup):
+        submission, _ = run_step()
+        submission.wait()
+        submission.free()
+    backend.synchronize()
+    if not args.no_profile:
+        backend.profile_enable(1)
+        backend.profile_reset()
+
+    kv_bytes_total, submissions = 0, []
+    backend.synchronize()
+    started = time.perf_counter()
+    for _ in range(args.steps):
+        submission, contexts = run_step()
+        kv_bytes_total += algorithmic_bytes(workload, contexts)[0]
+        submissions.append(submission)
+    backend.synchronize()
+    elapsed = time.perf_counter() - started
+    for submission in submissions:
+        submission.wait()            # surfaces any device error flag
+        submission.free()
+
+    tokens = args.lanes * args.steps
+    result = {
+        "metric": "decode tok/s, 4-bit 30B-A3B ragged batch; % HBM roofline; prefill % MFMA",
+        "value": tokens / elapsed, "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": ("BASELINE config 3: Qwen3-Coder-30B-A3B-shaped full model, "
+                         f"{workload.model.n_layers} layers, MLX-4bit random weights, {args.lanes} decode "
+                         f"lanes, contexts log-uniform {ctx_lo}-{ctx_hi}, paged bf16 KV page 16, "
+                         f"non-contiguous block tables, {churn} retire+admit per step"),
+            "lanes": args.lanes, "layers": workload.model.n_layers, "page_tokens": config.page_tokens,
+            "dispatches_per_step": session.dispatches, "device": info["family"],
+        },
+    }
+    weights = workload.model.weight_bytes_per_step(args.lanes)
+    kv_per_step = kv_bytes_total / args.steps
+    step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"]
+    result["step_algorithmic_gb"] = step_bytes / 1e9
+    result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS
+    if not args.no_profile:
+        ns, launches = backend.profile_read(KC_ATTENTION_KERNEL)
+        kernel_bytes = kv_bytes_total / max(launches, 1)          # per launch = per layer per step
+        average = ns / max(launches, 1) * 1e-9
+        achieved = kernel_bytes / average / 1e9 if average > 0 else 0.0
+        result["roofline"] = {
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "kernel": "ragged_attention_mfma_kernel", "launches": launches,
+            "avg_launch_us": average * 1e6, "algorithmic_bytes_per_launch": kernel_bytes,
+        }
+        # Secondary kernels over the same region, then a per-op breakdown from a few extra steps
+        # (every dispatch timed; not part of `value`).
+        moe_ns, moe_launches = backend.profile_read(KC_MOE_KERNEL)
+        qmm_ns, qmm_launches = backend.profile_read(KC_QMM_KERNEL)
+        secondary = {}
+        if moe_launches:
+            moe_bytes = weights["routed_all_experts"] * args.steps / moe_launches
+            secondary["routed_qmm_mfma_kernel"] = {
+                "avg_launch_us": moe_ns / moe_launches / 1e3,
+                "achieved_gbps": moe_bytes / (moe_ns / moe_launches * 1e-9) / 1e9,
+                "frac": moe_bytes / (moe_ns / moe_launches * 1e-9) / 1e9 / HBM_PEAK_GBPS,
+                "note": "weights of all experts counted once per projection launch"}
+        if qmm_launches:
+            qmm_bytes = weights["dense"] * args.steps / qmm_launches
+            secondary["dense_qmm_mfma_kernel"] = {
+                "avg_launch_us": qmm_ns / qmm_launches / 1e3,
+                "achieved_gbps": qmm_bytes / (qmm_ns / qmm_launches * 1e-9) / 1e9,
+                "frac": qmm_bytes / (qmm_ns / qmm_launches * 1e-9) / 1e9 / HBM_PEAK_GBPS}
+        result["secondary_kernels"] = secondary
+        backend.profile_enable(2)
+        backend.profile_reset()
+        extra = 4
+        for _ in range(extra):
+            submission, _ = run_step()
+            submission.wait()
+            submission.free()
+        breakdown = {}
+        for name, kc in (("attention_ops", KC_ATTENTION), ("routed_matmul_ops", KC_MOE),
+                         ("dense_matmul_ops", KC_QMM), ("other_ops", 0)):
+            class_ns, _ = backend.profile_read(kc)
+            breakdown[name] = class_ns / 1e6 / extra
+        result["gpu_ms_per_step_by_op"] = breakdown
+        backend.profile_enable(0)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(config, args.seed, args.cpu_sample_lanes, ctx_lo, ctx_hi)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libforja_hip.so")
 
-SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip"]
+SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "programs_fast.hip"]
 
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

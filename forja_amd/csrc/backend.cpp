@@ -31,6 +31,7 @@ struct Program {
   uint32_t kind = 0;  // 0 map, 1 row
   std::vector<fh_inst> insts;
   std::vector<uint32_t> pairs;  // (slot, value)
+  ProgramClass fast{};          // recognised fused form, if any
   uint32_t n_inputs = 0;
   uint32_t n_outputs = 0;
   uint32_t n_reduce = 0;
@@ -76,6 +77,7 @@ struct fh_submission {
   fh_backend *backend = nullptr;
   uint64_t serial = 0;
   uint32_t count = 0;
+  uint32_t error_capacity = 0;
   std::vector<uint32_t> ops;
   ErrorSlot *device_errors = nullptr;
   ErrorSlot *host_errors = nullptr;  // pinned
@@ -99,7 +101,7 @@ struct fh_backend {
   char *workspace = nullptr;
   uint64_t workspace_bytes = 0;
   // profiling
-  bool profiling = false;
+  int profiling = 0;  // 0 off, 1 kernel-level timers, 2 also one timer per dispatch
   struct Timed {
     hipEvent_t start, end;
     uint32_t kernel_class;
@@ -107,8 +109,19 @@ struct fh_backend {
   std::vector<Timed> timed;
   std::vector<hipEvent_t> event_pool;
   std::set<fh_submission *> submissions;  // live submissions owning device resources
-  uint64_t class_ns[FH_KC_COUNT] = {0, 0, 0, 0};
-  uint64_t class_launches[FH_KC_COUNT] = {0, 0, 0, 0};
+  // Recycled per-submission error records (device + pinned host), keyed by capacity.
+  struct ErrorBuffers {
+    ErrorSlot *device;
+    ErrorSlot *host;
+    uint32_t capacity;
+  };
+  std::vector<ErrorBuffers> error_pool;
+  std::vector<hipEvent_t> open_timers[FH_KC_COUNT];
+  // Pinned staging ring for small host->device writes, so fh_write need not wait for the stream.
+  char *ring = nullptr;
+  uint64_t ring_bytes = 0, ring_head = 0;
+  uint64_t class_ns[FH_KC_COUNT] = {};
+  uint64_t class_launches[FH_KC_COUNT] = {};
 
   char *ensure_workspace(uint64_t bytes) {
     if (bytes <= workspace_bytes) return workspace;
@@ -484,7 +497,7 @@ fh_status plan_program(fh_backend *b, const Planned &pl, bool execute) {
   uint64_t elements = element_count(first);
   if (it->second.kind == 1) FH_REQUIRE(first.shape[first.rank - 1] != 0);
   if (execute) {
-    if (try_fast_program(b->stream, it->second.kind == 1, args, elements)) return FH_OK;
+    if (try_fast_program(b->stream, it->second.fast, args, elements)) return FH_OK;
     launch_program(b->stream, args, it->second.kind == 1, elements);
   }
   return FH_OK;
@@ -507,7 +520,7 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
   if (!d.epilogue) {
     QmmProblem problem{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows, inner, columns,
                        d.bits, d.group_size};
-    if (try_fast_quant_matmul(b->stream, problem)) return FH_OK;
+    if (try_fast_quant_matmul(b, problem)) return FH_OK;
     launch_quant_matmul_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows,
                                 inner, columns, d.bits, d.group_size);
     return FH_OK;
@@ -518,7 +531,7 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
   View acc_view = contiguous_view(acc, FH_F32, out);
   QmmProblem problem{pl.in[0], pl.in[1], pl.in[2], pl.in[3], acc_view, rows, inner, columns,
                      d.bits, d.group_size};
-  if (!try_fast_quant_matmul(b->stream, problem))
+  if (!try_fast_quant_matmul(b, problem))
     launch_quant_matmul_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], acc_view, rows,
                                 inner, columns, d.bits, d.group_size);
   return run_epilogue(b, pl, primitive, acc, 1);
@@ -1066,6 +1079,17 @@ hipEvent_t take_event(fh_backend *b) {
   return e;
 }
 
+// Returns a finished submission's error record and events to the backend's pools.
+void recycle_submission(fh_backend *b, fh_submission *s) {
+  if (s->device_errors)
+    b->error_pool.push_back({s->device_errors, s->host_errors, s->error_capacity});
+  if (s->start) b->event_pool.push_back(s->start);
+  if (s->end) b->event_pool.push_back(s->end);
+  s->device_errors = nullptr;
+  s->host_errors = nullptr;
+  s->start = s->end = nullptr;
+}
+
 void drain_profile(fh_backend *b) {
   for (auto &t : b->timed) {
     float ms = 0.0f;
@@ -1132,6 +1156,13 @@ void fh_destroy(fh_backend *b) {
     for (auto &entry : b->programs)
       for (auto &typed : entry.second.typed) (void)hipFree(typed.second);
     if (b->workspace) (void)hipFree(b->workspace);
+    for (auto &e : b->error_pool) {
+      (void)hipFree(e.device);
+      (void)hipHostFree(e.host);
+    }
+    if (b->ring) (void)hipHostFree(b->ring);
+    for (auto &open : b->open_timers)
+      for (auto e : open) (void)hipEventDestroy(e);
     for (auto &t : b->timed) {
       (void)hipEventDestroy(t.start);
       (void)hipEventDestroy(t.end);
@@ -1200,10 +1231,37 @@ fh_status fh_write(fh_backend *b, fh_buffer buffer, uint64_t byte_offset, const 
     return FH_INVALID_INPUT;
   if (len == 0) return FH_OK;
   (void)hipSetDevice(b->device);
+  // Small writes are staged through a pinned ring and ordered on the stream without waiting for
+  // it; the caller's bytes may be reused as soon as this returns either way.
+  constexpr uint64_t kRingBytes = 32ull << 20, kRingPiece = 4ull << 20;
+  if (len <= kRingPiece) {
+    if (!b->ring) {
+      void *ptr = nullptr;
+      if (hipHostMalloc(&ptr, kRingBytes, hipHostMallocDefault) == hipSuccess) {
+        b->ring = (char *)ptr;
+        b->ring_bytes = kRingBytes;
+        b->ring_head = 0;
+      }
+    }
+    if (b->ring) {
+      uint64_t need = (len + 255) / 256 * 256;
+      if (b->ring_head + need > b->ring_bytes) {
+        // Wrap: every earlier staged copy must have left the ring.
+        if (hipStreamSynchronize(b->stream) != hipSuccess) return FH_DEVICE_EXECUTION_FAILED;
+        b->ring_head = 0;
+      }
+      char *stage = b->ring + b->ring_head;
+      memcpy(stage, bytes, len);
+      b->ring_head += need;
+      if (hipMemcpyAsync(it->second.ptr + byte_offset, stage, len, hipMemcpyHostToDevice,
+                         b->stream) != hipSuccess)
+        return FH_DEVICE_EXECUTION_FAILED;
+      return FH_OK;
+    }
+  }
   if (hipMemcpyAsync(it->second.ptr + byte_offset, bytes, len, hipMemcpyHostToDevice, b->stream) !=
       hipSuccess)
     return FH_DEVICE_EXECUTION_FAILED;
-  // The caller's bytes may be reused as soon as this returns.
   if (hipStreamSynchronize(b->stream) != hipSuccess) return FH_DEVICE_EXECUTION_FAILED;
   return FH_OK;
 }
@@ -1303,6 +1361,7 @@ fh_status fh_prepare_program(fh_backend *b, uint32_t kind, const fh_inst *insts,
       if (inst.kind == 0) uses_index_math = true;
     if (!uses_index_math) return status;
   }
+  p.fast = classify_program(kind, p.insts.data(), n_insts, p.pairs.data(), n_pairs);
   std::lock_guard<std::mutex> lock(b->mutex);
   uint64_t id = b->next_id++;
   b->programs[id] = std::move(p);
@@ -1340,30 +1399,46 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   s->count = count;
   s->ops.resize(count);
   uint32_t slots = count == 0 ? 1 : count;
-  void *dev = nullptr, *host = nullptr;
-  if (hipMalloc(&dev, slots * sizeof(ErrorSlot)) != hipSuccess ||
-      hipHostMalloc(&host, slots * sizeof(ErrorSlot), hipHostMallocDefault) != hipSuccess ||
-      hipEventCreate(&s->start) != hipSuccess || hipEventCreate(&s->end) != hipSuccess) {
-    if (dev) (void)hipFree(dev);
-    if (host) (void)hipHostFree(host);
-    delete s;
-    return FH_ALLOCATION_FAILED;
+  bool pooled = false;
+  for (size_t i = 0; i < b->error_pool.size(); ++i) {
+    if (b->error_pool[i].capacity >= slots) {
+      s->device_errors = b->error_pool[i].device;
+      s->host_errors = b->error_pool[i].host;
+      s->error_capacity = b->error_pool[i].capacity;
+      b->error_pool.erase(b->error_pool.begin() + (long)i);
+      pooled = true;
+      break;
+    }
   }
-  s->device_errors = (ErrorSlot *)dev;
-  s->host_errors = (ErrorSlot *)host;
+  if (!pooled) {
+    void *dev = nullptr, *host = nullptr;
+    uint32_t capacity = std::max<uint32_t>(slots, 1024);
+    if (hipMalloc(&dev, capacity * sizeof(ErrorSlot)) != hipSuccess ||
+        hipHostMalloc(&host, capacity * sizeof(ErrorSlot), hipHostMallocDefault) != hipSuccess) {
+      if (dev) (void)hipFree(dev);
+      if (host) (void)hipHostFree(host);
+      delete s;
+      return FH_ALLOCATION_FAILED;
+    }
+    s->device_errors = (ErrorSlot *)dev;
+    s->host_errors = (ErrorSlot *)host;
+    s->error_capacity = capacity;
+  }
+  s->start = take_event(b);
+  s->end = take_event(b);
   launch_init_errors(b->stream, s->device_errors, slots);
   (void)hipEventRecord(s->start, b->stream);
   fh_status status = FH_OK;
   for (uint32_t i = 0; i < count && status == FH_OK; ++i) {
     s->ops[i] = dispatches[i].op;
     hipEvent_t t0 = nullptr, t1 = nullptr;
-    if (b->profiling) {
+    if (b->profiling >= 2) {
       t0 = take_event(b);
       t1 = take_event(b);
       (void)hipEventRecord(t0, b->stream);
     }
     status = process(b, dispatches[i], &s->device_errors[i], true);
-    if (b->profiling) {
+    if (b->profiling >= 2) {
       (void)hipEventRecord(t1, b->stream);
       b->timed.push_back({t0, t1, kernel_class_of(dispatches[i].op)});
     }
@@ -1373,10 +1448,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
                        hipMemcpyDeviceToHost, b->stream);
   if (status != FH_OK) {
     (void)hipStreamSynchronize(b->stream);
-    (void)hipFree(s->device_errors);
-    (void)hipHostFree(s->host_errors);
-    (void)hipEventDestroy(s->start);
-    (void)hipEventDestroy(s->end);
+    recycle_submission(b, s);
     delete s;
     return status;
   }
@@ -1482,10 +1554,7 @@ void fh_submission_free(fh_submission *s) {
     (void)hipSetDevice(b->device);
     if (!s->waited) (void)hipStreamSynchronize(b->stream);
     b->submissions.erase(s);
-    (void)hipFree(s->device_errors);
-    (void)hipHostFree(s->host_errors);
-    (void)hipEventDestroy(s->start);
-    (void)hipEventDestroy(s->end);
+    recycle_submission(b, s);
   }
   delete s;
 }
@@ -1523,7 +1592,7 @@ fh_status fh_profile_enable(fh_backend *b, int enabled) {
   (void)hipSetDevice(b->device);
   (void)hipStreamSynchronize(b->stream);
   drain_profile(b);
-  b->profiling = enabled != 0;
+  b->profiling = enabled < 0 ? 0 : (enabled > 2 ? 2 : enabled);
   return FH_OK;
 }
 
@@ -1559,5 +1628,33 @@ char *backend_workspace(fh_backend *backend, uint64_t bytes) { return backend->e
 hipStream_t backend_stream(fh_backend *backend) { return backend->stream; }
 uint32_t backend_compute_units(fh_backend *backend) {
   return (uint32_t)backend->props.multiProcessorCount;
+}
+void backend_profile_begin(fh_backend *backend, uint32_t kernel_class) {
+  if (!backend->profiling || kernel_class >= FH_KC_COUNT) return;
+  hipEvent_t event = nullptr;
+  if (!backend->event_pool.empty()) {
+    event = backend->event_pool.back();
+    backend->event_pool.pop_back();
+  } else if (hipEventCreate(&event) != hipSuccess) {
+    return;
+  }
+  (void)hipEventRecord(event, backend->stream);
+  backend->open_timers[kernel_class].push_back(event);
+}
+void backend_profile_end(fh_backend *backend, uint32_t kernel_class) {
+  if (!backend->profiling || kernel_class >= FH_KC_COUNT) return;
+  if (backend->open_timers[kernel_class].empty()) return;
+  hipEvent_t start = backend->open_timers[kernel_class].back();
+  backend->open_timers[kernel_class].pop_back();
+  hipEvent_t end = nullptr;
+  if (!backend->event_pool.empty()) {
+    end = backend->event_pool.back();
+    backend->event_pool.pop_back();
+  } else if (hipEventCreate(&end) != hipSuccess) {
+    backend->event_pool.push_back(start);
+    return;
+  }
+  (void)hipEventRecord(end, backend->stream);
+  backend->timed.push_back({start, end, kernel_class});
 }
 }  // namespace fh

@@ -15,12 +15,24 @@ namespace fh {
 char *backend_workspace(fh_backend *backend, uint64_t bytes);
 hipStream_t backend_stream(fh_backend *backend);
 uint32_t backend_compute_units(fh_backend *backend);
+void backend_profile_begin(fh_backend *backend, uint32_t kernel_class);
+void backend_profile_end(fh_backend *backend, uint32_t kernel_class);
+
+// Brackets one kernel launch with HIP events when profiling is enabled.
+struct KernelTimer {
+  fh_backend *backend;
+  uint32_t kernel_class;
+  KernelTimer(fh_backend *b, uint32_t c) : backend(b), kernel_class(c) {
+    backend_profile_begin(backend, kernel_class);
+  }
+  ~KernelTimer() { backend_profile_end(backend, kernel_class); }
+};
 
 struct QmmProblem {
   View x, packed, scales, biases, out;
   uint32_t rows, inner, columns, bits, group;
 };
-bool try_fast_quant_matmul(hipStream_t stream, const QmmProblem &problem);
+bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &problem);
 
 struct GatherProblem {
   View x;           // projection: [R,K]; weighted sum: [R,k,K]
@@ -57,7 +69,17 @@ struct RaggedAttention {
 // false only when workspace allocation fails.
 bool run_ragged_attention(fh_backend *backend, const RaggedAttention &problem, ErrorSlot *error);
 
-bool try_fast_program(hipStream_t stream, bool row, const ProgramArgs &args, uint64_t elements);
+// Recognised guest row programs (by canonical expression) and their constants.
+enum ProgramKindFast { kProgramGeneric = 0, kProgramRmsNorm, kProgramResidualNorm, kProgramQkNormRope };
+struct ProgramClass {
+  int kind;
+  uint32_t axis;  // the axis the program's extent/index instruction names (must be the last)
+  float c[4];
+};
+ProgramClass classify_program(uint32_t kind, const fh_inst *insts, uint32_t n_insts,
+                              const uint32_t *pairs, uint32_t n_pairs);
+bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const ProgramArgs &args,
+                      uint64_t elements);
 
 // Epilogue recognisers: `acc + extra` and `silu(acc0) * acc1` in the instruction orders the SDK
 // emits (crates/forja-sdk/src/nn/blocks.rs:406-416) and commuted variants.

@@ -452,6 +452,60 @@ __global__ void argmax_kernel(View in, View out, uint32_t rows, uint32_t width) 
   }
 }
 
+// bf16 rows with a contiguous innermost axis: 16-byte loads, 1024 threads per row.
+__global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t *in, uint64_t row_stride,
+                                                           View out, uint32_t width) {
+  __shared__ int32_t keys[16];
+  __shared__ uint32_t idxs[16];
+  const uint32_t row = blockIdx.x;
+  const uint16_t *x = in + (uint64_t)row * row_stride;
+  int32_t best_key = (int32_t)0x80000000;
+  uint32_t best_index = 0xffffffffu;
+  for (uint32_t c = threadIdx.x * 8; c < width; c += 1024 * 8) {
+    uint4 v = *(const uint4 *)(x + c);
+    uint32_t words[4] = {v.x, v.y, v.z, v.w};
+    for (int i = 0; i < 4; ++i) {
+      int32_t lo = total_key(__uint_as_float(words[i] << 16));
+      int32_t hi = total_key(__uint_as_float(words[i] & 0xffff0000u));
+      if (best_index == 0xffffffffu || lo >= best_key) {
+        best_key = lo;
+        best_index = c + 2 * i;
+      }
+      if (hi >= best_key) {
+        best_key = hi;
+        best_index = c + 2 * i + 1;
+      }
+    }
+  }
+  for (int offset = 32; offset > 0; offset >>= 1) {
+    int32_t other_key = __shfl_xor(best_key, offset, 64);
+    uint32_t other_index = __shfl_xor(best_index, offset, 64);
+    if (other_index != 0xffffffffu &&
+        (best_index == 0xffffffffu || other_key > best_key ||
+         (other_key == best_key && other_index > best_index))) {
+      best_key = other_key;
+      best_index = other_index;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    keys[threadIdx.x >> 6] = best_key;
+    idxs[threadIdx.x >> 6] = best_index;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t key = keys[0];
+    uint32_t index = idxs[0];
+    for (uint32_t w = 1; w < 16; ++w) {
+      if (idxs[w] == 0xffffffffu) continue;
+      if (index == 0xffffffffu || keys[w] > key || (keys[w] == key && idxs[w] > index)) {
+        key = keys[w];
+        index = idxs[w];
+      }
+    }
+    ((uint32_t *)out.base)[view_offset(out, row)] = index;
+  }
+}
+
 // ---------------------------------------------------------------- glue
 
 // execute_quant_embed (lib.rs:748-813).
@@ -798,6 +852,12 @@ void launch_top_k(hipStream_t s, const View &in, const View &values, const View 
 
 void launch_argmax(hipStream_t s, const View &in, const View &out, uint32_t rows, uint32_t width) {
   if (rows == 0) return;
+  if (in.dtype == FH_BF16 && in.stride[1] == 1 && width % 8 == 0 && in.offset % 8 == 0 &&
+      (rows == 1 || in.stride[0] % 8 == 0)) {
+    argmax_bf16_kernel<<<dim3(rows), 1024, 0, s>>>((const uint16_t *)in.base + in.offset,
+                                                   in.stride[0], out, width);
+    return;
+  }
   argmax_kernel<<<dim3(rows), kBlock, 0, s>>>(in, out, rows, width);
 }
 

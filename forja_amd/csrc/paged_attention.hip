@@ -619,9 +619,12 @@ void launch_plan(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
   ragged_plan_kernel<<<dim3(1), 256, 0, stream>>>(f, error);
 }
 
-void launch_fast(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
+void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
   uint64_t blocks = (uint64_t)f.tokens * f.max_splits * f.kv_heads;
-  ragged_attention_mfma_kernel<<<dim3((unsigned)blocks), 64, 0, stream>>>(f, error);
+  {
+    KernelTimer timer(backend, FH_KC_ATTENTION_KERNEL);
+    ragged_attention_mfma_kernel<<<dim3((unsigned)blocks), 64, 0, stream>>>(f, error);
+  }
   ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens), 64, 0, stream>>>(f);
 }
 
@@ -669,7 +672,7 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   f.out_stride_h = lane.out.stride[0];
   hipStream_t stream = backend_stream(backend);
   launch_plan(stream, f, error);
-  launch_fast(stream, f, error);
+  launch_fast(backend, stream, f, error);
   return true;
 }
 
@@ -710,7 +713,7 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
       (uint64_t)p.tokens * (p.kv_heads * p.width + p.kv_heads * p.value_width);
   ragged_append_kernel<<<dim3((unsigned)((append_work + 255) / 256)), 256, 0, stream>>>(p, error);
   if (fast) {
-    launch_fast(stream, f, error);
+    launch_fast(backend, stream, f, error);
     return true;
   }
   uint32_t blocks = p.tokens * p.query_heads;

@@ -1,0 +1,343 @@
+// Fused kernels for the guest row programs every engine dispatches around the matmuls
+// (crates/forja-sdk/src/nn/blocks.rs:380-443): rms_norm_rows, residual_norm_rows and
+// qk_norm_rope_rows.  A program is recognised by its canonical expression (commutative operands
+// sorted, constants captured), never by name, so any instruction order the SDK emits matches;
+// everything else runs on the generic interpreter.  bf16 rows, innermost axis contiguous.
+#include "fast_kernels.hpp"
+
+#include <regex>
+#include <string>
+
+namespace fh {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+__device__ inline uint32_t pack2(float lo, float hi) {
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ inline float lo_f32(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ inline float hi_f32(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+__device__ inline float block_sum(float v, float *scratch) {
+  for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float total = 0.0f;
+  for (uint32_t w = 0; w < blockDim.x / 64; ++w) total += scratch[w];
+  __syncthreads();
+  return total;
+}
+
+struct RowArgs {
+  const uint16_t *x, *update, *weight;
+  uint16_t *out0, *out1;
+  uint64_t x_stride, update_stride, weight_stride, out0_stride, out1_stride;
+  uint32_t width;
+  float eps;
+};
+
+// out = x * rsqrt(mean(x^2) + eps) * w            (kResidual = false)
+// value = x + update; out0 = value; out1 = value * rsqrt(mean(value^2) + eps) * w
+template <bool kResidual>
+__global__ __launch_bounds__(256) void norm_rows_kernel(RowArgs a) {
+  __shared__ float scratch[4];
+  const uint64_t row = blockIdx.x;
+  const uint16_t *x = a.x + row * a.x_stride;
+  const uint16_t *u = kResidual ? a.update + row * a.update_stride : nullptr;
+  const uint16_t *w = a.weight + row * a.weight_stride;
+  float acc = 0.0f;
+  for (uint32_t c = threadIdx.x * 8; c < a.width; c += 256 * 8) {
+    uint4 v = *(const uint4 *)(x + c);
+    uint32_t words[4] = {v.x, v.y, v.z, v.w};
+    uint4 uv = make_uint4(0, 0, 0, 0);
+    if (kResidual) uv = *(const uint4 *)(u + c);
+    uint32_t uwords[4] = {uv.x, uv.y, uv.z, uv.w};
+    for (int i = 0; i < 4; ++i) {
+      float lo = lo_f32(words[i]), hi = hi_f32(words[i]);
+      if (kResidual) {
+        lo += lo_f32(uwords[i]);
+        hi += hi_f32(uwords[i]);
+      }
+      acc += lo * lo;
+      acc += hi * hi;
+    }
+  }
+  const float total = block_sum(acc, scratch);
+  const float inverse = 1.0f / sqrtf(total / (float)a.width + a.eps);
+  uint16_t *out_norm = (kResidual ? a.out1 + row * a.out1_stride : a.out0 + row * a.out0_stride);
+  for (uint32_t c = threadIdx.x * 8; c < a.width; c += 256 * 8) {
+    uint4 v = *(const uint4 *)(x + c);
+    uint4 wv = *(const uint4 *)(w + c);
+    uint32_t words[4] = {v.x, v.y, v.z, v.w}, wwords[4] = {wv.x, wv.y, wv.z, wv.w};
+    uint4 uv = make_uint4(0, 0, 0, 0);
+    if (kResidual) uv = *(const uint4 *)(u + c);
+    uint32_t uwords[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t value_words[4], norm_words[4];
+    for (int i = 0; i < 4; ++i) {
+      float lo = lo_f32(words[i]), hi = hi_f32(words[i]);
+      if (kResidual) {
+        lo += lo_f32(uwords[i]);
+        hi += hi_f32(uwords[i]);
+      }
+      value_words[i] = pack2(lo, hi);
+      norm_words[i] = pack2(lo * inverse * lo_f32(wwords[i]), hi * inverse * hi_f32(wwords[i]));
+    }
+    if (kResidual)
+      *(uint4 *)(a.out0 + row * a.out0_stride + c) =
+          make_uint4(value_words[0], value_words[1], value_words[2], value_words[3]);
+    *(uint4 *)(out_norm + c) = make_uint4(norm_words[0], norm_words[1], norm_words[2], norm_words[3]);
+  }
+}
+
+struct QkArgs {
+  const uint16_t *lo, *hi, *w_lo, *w_hi;
+  const float *positions;
+  uint16_t *out_lo, *out_hi;
+  uint64_t lo_s[2], hi_s[2], wlo_s[2], whi_s[2], pos_s[3], olo_s[2], ohi_s[2];
+  uint32_t rows, heads, width;
+  float head_dim, eps, theta, exponent_scale;
+};
+
+// One wave per (row, head): RMS-normalise the head over both halves, scale, rotate the
+// (lo, hi) pair by angle = position * theta^(i * exponent_scale).
+__global__ __launch_bounds__(256) void qk_norm_rope_kernel(QkArgs a) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint64_t item = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= (uint64_t)a.rows * a.heads) return;
+  const uint32_t row = (uint32_t)(item / a.heads), head = (uint32_t)(item % a.heads);
+  const bool live = lane < a.width;
+  float lo = 0.0f, hi = 0.0f;
+  if (live) {
+    lo = __uint_as_float((uint32_t)a.lo[row * a.lo_s[0] + head * a.lo_s[1] + lane] << 16);
+    hi = __uint_as_float((uint32_t)a.hi[row * a.hi_s[0] + head * a.hi_s[1] + lane] << 16);
+  }
+  float square_sum = lo * lo + hi * hi;
+  for (int offset = 32; offset > 0; offset >>= 1) square_sum += __shfl_xor(square_sum, offset, 64);
+  if (!live) return;
+  const float inverse = 1.0f / sqrtf(square_sum / a.head_dim + a.eps);
+  const float w_lo = __uint_as_float((uint32_t)a.w_lo[row * a.wlo_s[0] + head * a.wlo_s[1] + lane] << 16);
+  const float w_hi = __uint_as_float((uint32_t)a.w_hi[row * a.whi_s[0] + head * a.whi_s[1] + lane] << 16);
+  const float n_lo = lo * inverse * w_lo, n_hi = hi * inverse * w_hi;
+  const float position = a.positions[row * a.pos_s[0] + head * a.pos_s[1] + lane * a.pos_s[2]];
+  const float angle = position * powf(a.theta, (float)lane * a.exponent_scale);
+  const float c = cosf(angle), s = sinf(angle);
+  const float r_lo = n_lo * c - n_hi * s, r_hi = n_hi * c + n_lo * s;
+  a.out_lo[row * a.olo_s[0] + head * a.olo_s[1] + lane] = (uint16_t)(pack2(r_lo, 0.0f) & 0xffffu);
+  a.out_hi[row * a.ohi_s[0] + head * a.ohi_s[1] + lane] = (uint16_t)(pack2(r_hi, 0.0f) & 0xffffu);
+}
+
+// Canonical expression of value v: commutative operands sorted; constants carry their bits.
+std::string canonical(const fh_inst *insts, uint32_t count, uint32_t v, int depth = 0) {
+  if (v >= count || depth > 24) return "?";
+  const fh_inst &inst = insts[v];
+  char buffer[32];
+  switch (inst.kind) {
+  case 0: return "in" + std::to_string(inst.a);
+  case 1: snprintf(buffer, sizeof(buffer), "c%08x", inst.a); return buffer;
+  case 2: return "i" + std::to_string(inst.op);
+  case 3: return "e" + std::to_string(inst.op);
+  case 4: return "u" + std::to_string(inst.op) + "(" + canonical(insts, count, inst.a, depth + 1) + ")";
+  case 5: {
+    std::string l = canonical(insts, count, inst.a, depth + 1),
+                r = canonical(insts, count, inst.b, depth + 1);
+    if ((inst.op == 0 || inst.op == 2) && r < l) std::swap(l, r);
+    return "b" + std::to_string(inst.op) + "(" + l + "," + r + ")";
+  }
+  case 7: return "k" + std::to_string(inst.op) + "(" + canonical(insts, count, inst.a, depth + 1) + ")";
+  case 8: return "r" + std::to_string(inst.op) + "(" + canonical(insts, count, inst.a, depth + 1) + ")";
+  default: return "?";
+  }
+}
+
+float const_of(const std::string &hex) {
+  uint32_t bits = (uint32_t)strtoul(hex.c_str(), nullptr, 16);
+  float value;
+  memcpy(&value, &bits, 4);
+  return value;
+}
+
+std::string escape(const std::string &s) {
+  std::string out;
+  for (char ch : s) {
+    if (ch == '(' || ch == ')') out += '\\';
+    out += ch;
+  }
+  return out;
+}
+
+const std::string kConst = "c([0-9a-f]{8})";
+
+bool bf16_rows(const View &v, uint32_t rank) {
+  return v.dtype == FH_BF16 && v.rank == rank && v.stride[rank - 1] == 1;
+}
+
+}  // namespace
+
+ProgramClass classify_program(uint32_t kind, const fh_inst *insts, uint32_t n_insts,
+                              const uint32_t *pairs, uint32_t n_pairs) {
+  ProgramClass result{};
+  result.kind = kProgramGeneric;
+  if (kind != 1) return result;
+  std::smatch m;
+  auto value_of = [&](uint32_t slot) -> std::string {
+    for (uint32_t p = 0; p < n_pairs; ++p)
+      if (pairs[2 * p] == slot) return canonical(insts, n_insts, pairs[2 * p + 1]);
+    return "";
+  };
+  // x * rsqrt(sum(x*x) / f32(extent) + eps) * w
+  auto norm_of = [&](const std::string &x, const std::string &w) {
+    std::string xe = escape(x);
+    return "b2\\(b2\\(" + xe + ",u5\\(b0\\(b3\\(r0\\(b2\\(" + xe + "," + xe + "\\)\\),k0\\(e(\\d)\\)\\)," +
+           kConst + "\\)\\)\\)," + w + "\\)";
+  };
+  if (n_pairs == 1) {
+    std::string e = value_of(0);
+    if (std::regex_match(e, m, std::regex("^" + norm_of("in0", "in1") + "$"))) {
+      result.kind = kProgramRmsNorm;
+      result.axis = (uint32_t)atoi(m[1].str().c_str());
+      result.c[0] = const_of(m[2].str());
+    }
+    return result;
+  }
+  if (n_pairs != 2) return result;
+  std::string first = value_of(0), second = value_of(1);
+  if (first == "b0(in0,in1)" &&
+      std::regex_match(second, m, std::regex("^" + norm_of("b0(in0,in1)", "in2") + "$"))) {
+    result.kind = kProgramResidualNorm;
+    result.axis = (uint32_t)atoi(m[1].str().c_str());
+    result.c[0] = const_of(m[2].str());
+    return result;
+  }
+  // qk_norm_rope_rows(lo, hi, w_lo, w_hi, positions)
+  const std::string ss = "r0\\(b0\\(b2\\(in0,in0\\),b2\\(in1,in1\\)\\)\\)";
+  const std::string inv = "u5\\(b0\\(b3\\(" + ss + "," + kConst + "\\)," + kConst + "\\)\\)";
+  // later occurrences of the same sub-expression must repeat the captured constants
+  const std::string inv_again = "u5\\(b0\\(b3\\(" + ss + ",c\\1\\),c\\2\\)\\)";
+  const std::string angle = "b2\\(b6\\(" + kConst + ",b2\\(" + kConst + ",k0\\(i(\\d)\\)\\)\\),in4\\)";
+  const std::string angle_again = "b2\\(b6\\(c\\3,b2\\(c\\4,k0\\(i\\5\\)\\)\\),in4\\)";
+  const std::string n_lo = "b2\\(b2\\(in0," + inv + "\\),in2\\)";
+  const std::string n_lo_again = "b2\\(b2\\(in0," + inv_again + "\\),in2\\)";
+  const std::string n_hi_again = "b2\\(b2\\(in1," + inv_again + "\\),in3\\)";
+  const std::string out0 = "^b1\\(b2\\(" + n_lo + ",u7\\(" + angle + "\\)\\),b2\\(" + n_hi_again +
+                           ",u6\\(" + angle_again + "\\)\\)\\)$";
+  if (std::regex_match(first, m, std::regex(out0))) {
+    float head_dim = const_of(m[1].str()), eps = const_of(m[2].str()), theta = const_of(m[3].str()),
+          exponent_scale = const_of(m[4].str());
+    uint32_t axis = (uint32_t)atoi(m[5].str().c_str());
+    // second output: n_hi*cos + n_lo*sin with the same constants (sorted: the n_lo product first)
+    auto hex = [](float f) {
+      uint32_t bits;
+      memcpy(&bits, &f, 4);
+      char b[16];
+      snprintf(b, sizeof(b), "c%08x", bits);
+      return std::string(b);
+    };
+    std::string inv_s = "u5(b0(b3(r0(b0(b2(in0,in0),b2(in1,in1)))," + hex(head_dim) + ")," + hex(eps) + "))";
+    std::string angle_s = "b2(b6(" + hex(theta) + ",b2(" + hex(exponent_scale) + ",k0(i" +
+                          std::to_string(axis) + "))),in4)";
+    std::string nlo_s = "b2(b2(in0," + inv_s + "),in2)", nhi_s = "b2(b2(in1," + inv_s + "),in3)";
+    std::string expect = "b0(b2(" + nlo_s + ",u6(" + angle_s + ")),b2(" + nhi_s + ",u7(" + angle_s + ")))";
+    if (second == expect) {
+      result.kind = kProgramQkNormRope;
+      result.axis = axis;
+      result.c[0] = head_dim;
+      result.c[1] = eps;
+      result.c[2] = theta;
+      result.c[3] = exponent_scale;
+    }
+  }
+  return result;
+}
+
+bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const ProgramArgs &p,
+                      uint64_t elements) {
+  if (cls.kind == kProgramGeneric || elements == 0) return false;
+  const uint32_t rank = p.rank;
+  if (cls.axis != rank - 1) return false;
+  auto ptr = [](const View &v) { return (uint16_t *)v.base + v.offset; };
+  auto aligned = [&](const View &v) {
+    if (v.offset % 8) return false;
+    for (uint32_t axis = 0; axis + 1 < rank; ++axis)
+      if (v.stride[axis] % 8) return false;
+    return true;
+  };
+  if (cls.kind == kProgramRmsNorm || cls.kind == kProgramResidualNorm) {
+    const bool residual = cls.kind == kProgramResidualNorm;
+    if (rank != 2 || p.n_inputs != (residual ? 3u : 2u)) return false;
+    const uint32_t n_out = residual ? 2 : 1;
+    for (uint32_t i = 0; i < p.n_inputs; ++i)
+      if (!bf16_rows(p.inputs[i], 2) || !aligned(p.inputs[i])) return false;
+    for (uint32_t i = 0; i < n_out; ++i)
+      if (!bf16_rows(p.outputs[i], 2) || !aligned(p.outputs[i])) return false;
+    const uint32_t width = p.shape[1];
+    if (width % 8 != 0) return false;
+    RowArgs a{};
+    a.x = ptr(p.inputs[0]);
+    a.x_stride = p.inputs[0].stride[0];
+    const View &w = p.inputs[residual ? 2 : 1];
+    a.weight = ptr(w);
+    a.weight_stride = w.stride[0];
+    if (residual) {
+      a.update = ptr(p.inputs[1]);
+      a.update_stride = p.inputs[1].stride[0];
+    }
+    // out_slot maps pairs to output tensors; pairs are (slot, value) with slot = output index
+    a.out0 = ptr(p.outputs[0]);
+    a.out0_stride = p.outputs[0].stride[0];
+    if (residual) {
+      a.out1 = ptr(p.outputs[1]);
+      a.out1_stride = p.outputs[1].stride[0];
+    }
+    a.width = width;
+    a.eps = cls.c[0];
+    if (residual)
+      norm_rows_kernel<true><<<dim3(p.shape[0]), 256, 0, stream>>>(a);
+    else
+      norm_rows_kernel<false><<<dim3(p.shape[0]), 256, 0, stream>>>(a);
+    return true;
+  }
+  if (cls.kind == kProgramQkNormRope) {
+    if (rank != 3 || p.n_inputs != 5 || p.shape[2] > 64) return false;
+    for (uint32_t i = 0; i < 4; ++i)
+      if (!bf16_rows(p.inputs[i], 3)) return false;
+    if (p.inputs[4].dtype != FH_F32 || p.inputs[4].rank != 3) return false;
+    for (uint32_t i = 0; i < 2; ++i)
+      if (!bf16_rows(p.outputs[i], 3)) return false;
+    QkArgs a{};
+    auto set = [](uint64_t (&dst)[2], const View &v) {
+      dst[0] = v.stride[0];
+      dst[1] = v.stride[1];
+    };
+    a.lo = ptr(p.inputs[0]);
+    a.hi = ptr(p.inputs[1]);
+    a.w_lo = ptr(p.inputs[2]);
+    a.w_hi = ptr(p.inputs[3]);
+    a.positions = (const float *)p.inputs[4].base + p.inputs[4].offset;
+    a.out_lo = ptr(p.outputs[0]);
+    a.out_hi = ptr(p.outputs[1]);
+    set(a.lo_s, p.inputs[0]);
+    set(a.hi_s, p.inputs[1]);
+    set(a.wlo_s, p.inputs[2]);
+    set(a.whi_s, p.inputs[3]);
+    for (int axis = 0; axis < 3; ++axis) a.pos_s[axis] = p.inputs[4].stride[axis];
+    set(a.olo_s, p.outputs[0]);
+    set(a.ohi_s, p.outputs[1]);
+    a.rows = p.shape[0];
+    a.heads = p.shape[1];
+    a.width = p.shape[2];
+    a.head_dim = cls.c[0];
+    a.eps = cls.c[1];
+    a.theta = cls.c[2];
+    a.exponent_scale = cls.c[3];
+    uint64_t items = (uint64_t)a.rows * a.heads;
+    qk_norm_rope_kernel<<<dim3((unsigned)((items + 3) / 4)), 256, 0, stream>>>(a);
+    return true;
+  }
+  return false;
+}
+
+}  // namespace fh

@@ -70,9 +70,15 @@ __device__ inline bf16x8 unpack_word(uint32_t w) {
   return __builtin_bit_cast(bf16x8, r);
 }
 
-// MT = 32-row tiles per workgroup, KC = activation columns staged per pass.
-template <int MT, bool kPair, bool kRouted>
+// MT = 32-row tiles per workgroup, KC = activation columns staged per pass.  The four waves of a
+// workgroup share the staged activations and either own 32 output columns each (kSplitK false)
+// or all work on the same 32 columns, each on a quarter of every staged pass, and add their
+// accumulators through LDS at the end (kSplitK true: narrow outputs, where column blocks alone
+// would leave most CUs idle and each block would crawl through all of K).
+template <int MT, bool kPair, bool kRouted, bool kSplitK>
 __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
+  constexpr int NW = kWaves;
+  constexpr int kThreads = 64 * NW;
   constexpr int KC = 512 / MT;  // 33 KB of LDS either way: two workgroups per CU overlap staging
   constexpr int kRows = 32 * MT;
   constexpr int kPitch = 2 * KC + 16;  // bytes; +16 spreads consecutive rows over the banks
@@ -82,7 +88,8 @@ __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
 
   const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const uint32_t nl = lane & 31, h = lane >> 5;
-  const uint32_t column = (blockIdx.x * kWaves + wave) * kColsPerWave + nl;
+  const uint32_t column =
+      (kSplitK ? blockIdx.x : blockIdx.x * NW + wave) * kColsPerWave + nl;
   const uint32_t column_c = min(column, a.columns - 1);  // clamped for loads
 
   uint32_t expert = 0, count = 0, first = 0;
@@ -92,7 +99,8 @@ __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
     if (expert == kNoBlock) return;
     first = a.blocks[3 * blockIdx.y + 1];
     count = a.blocks[3 * blockIdx.y + 2];
-    if (tid < kRows) row_ids[tid] = tid < count ? a.sorted_routes[first + tid] : 0;
+    for (uint32_t r = tid; r < kRows; r += kThreads)
+      row_ids[r] = r < count ? a.sorted_routes[first + r] : 0;
   } else {
     first = blockIdx.y * kRows;
     count = min((uint32_t)kRows, a.rows - first);
@@ -106,93 +114,170 @@ __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
     b_row[pj] = a.biases[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
   }
 
-  f32x16 acc[kPair ? 2 : 1][MT];
-  for (int pj = 0; pj < (kPair ? 2 : 1); ++pj)
+  constexpr int kP = kPair ? 2 : 1;
+  constexpr int kPieces = kRows * KC / 8 / kThreads;  // 16-byte activation pieces per thread per pass
+  constexpr int kGroupsPerPass = KC / kGroup;
+  f32x16 acc[kP][MT];
+  for (int pj = 0; pj < kP; ++pj)
     for (int mt = 0; mt < MT; ++mt)
       for (int j = 0; j < 16; ++j) acc[pj][mt][j] = 0.0f;
 
-  for (uint32_t kc0 = 0; kc0 < a.inner; kc0 += KC) {
+  // Two independent software pipelines hide memory latency:
+  //  * weights: a ring of four groups' packed words and affine parameters; a slot is reloaded
+  //    (four groups ahead) as soon as its group has been consumed - the weight stream does not
+  //    care about staging passes;
+  //  * activations: the next pass's pieces are fetched into registers while the current pass is
+  //    consumed from LDS.
+  // A wave consumes kGw groups of every staged pass.
+  constexpr int kGw = kSplitK ? kGroupsPerPass / NW : kGroupsPerPass;
+  const uint32_t total_groups = a.inner / kGroup;
+  const uint32_t passes = (a.inner + KC - 1) / KC;
+  uint4 wq[kP][4];
+  uint32_t sb[kP][4][2];
+  auto load_group = [&](int slot, uint32_t group) {
+    if (group >= total_groups) return;
+    for (int pj = 0; pj < kP; ++pj) {
+      wq[pj][slot] = *(const uint4 *)(w_row[pj] + (uint64_t)group * 8);
+      sb[pj][slot][0] = s_row[pj][group];
+      sb[pj][slot][1] = b_row[pj][group];
+    }
+  };
+  uint4 x_regs[kPieces];
+  auto fetch_pass = [&](uint32_t kc0) {
     const uint32_t kc = min((uint32_t)KC, a.inner - kc0);
-    __syncthreads();  // the previous pass is consumed (and row_ids are visible)
-    // ---- stage activations: 16-byte pieces, permuted inside each 8, plus per-group sums
     const uint32_t pieces_per_row = kc / 8;
-    for (uint32_t piece = tid; piece < kRows * pieces_per_row; piece += 256) {
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const uint32_t piece = tid + i * kThreads;
       const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (row < count) {
+      x_regs[i] = make_uint4(0, 0, 0, 0);
+      if (row < count) {  // rows beyond kRows only arise in a short last pass and are >= count
         const uint64_t in_row = kRouted ? row_ids[row] / a.route_div : first + row;
-        v = *(const uint4 *)(a.x + in_row * a.x_row_stride + kc0 + 8 * pc);
+        x_regs[i] = *(const uint4 *)(a.x + in_row * a.x_row_stride + kc0 + 8 * pc);
       }
+    }
+  };
+  // Pass switch: publish the fetched activations (permuted inside each 8, plus per-group sums),
+  // then start fetching the pass after.
+  auto pass_switch = [&](uint32_t pass) {
+    const uint32_t kc0 = pass * KC;
+    const uint32_t kc = min((uint32_t)KC, a.inner - kc0);
+    const uint32_t pieces_per_row = kc / 8;
+    __syncthreads();  // the previous pass is consumed
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const uint32_t piece = tid + i * kThreads;
+      const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
+      const uint4 v = x_regs[i];
       float sum = bf16_bits_to_f32(v.x & 0xffffu) + bf16_bits_to_f32(v.x >> 16) +
                   bf16_bits_to_f32(v.y & 0xffffu) + bf16_bits_to_f32(v.y >> 16) +
                   bf16_bits_to_f32(v.z & 0xffffu) + bf16_bits_to_f32(v.z >> 16) +
                   bf16_bits_to_f32(v.w & 0xffffu) + bf16_bits_to_f32(v.w >> 16);
-      uint4 permuted;
-      permuted.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
-      permuted.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
-      permuted.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
-      permuted.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
-      *(uint4 *)(xs + row * kPitch + pc * 16) = permuted;
       // eight consecutive pieces (= lanes) make one quantisation group
       sum += __shfl_xor(sum, 1, 64);
       sum += __shfl_xor(sum, 2, 64);
       sum += __shfl_xor(sum, 4, 64);
-      if ((pc & 7) == 0) xsum[(pc >> 3) * kRows + row] = sum;
-    }
-    __syncthreads();
-    // ---- stream the weights of this pass: 4 groups (256 columns of K) per unrolled round
-    const uint32_t groups = kc / kGroup;
-    const uint32_t word0 = kc0 / 8, group0 = kc0 / kGroup;
-    for (uint32_t g0 = 0; g0 < groups; g0 += 4) {
-      uint4 wq[kPair ? 2 : 1][4];
-      uint32_t sb[kPair ? 2 : 1][4][2];
-      for (int pj = 0; pj < (kPair ? 2 : 1); ++pj)
-        for (int u = 0; u < 4; ++u) {
-          wq[pj][u] = *(const uint4 *)(w_row[pj] + word0 + (g0 + u) * 8);
-          sb[pj][u][0] = s_row[pj][group0 + g0 + u];
-          sb[pj][u][1] = b_row[pj][group0 + g0 + u];
-        }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const uint32_t gi = g0 + u;
-        f32x16 part[kPair ? 2 : 1][MT];
-        for (int pj = 0; pj < (kPair ? 2 : 1); ++pj)
-          for (int mt = 0; mt < MT; ++mt)
-            for (int j = 0; j < 16; ++j) part[pj][mt][j] = 0.0f;
-#pragma unroll
-        for (int step = 0; step < 4; ++step) {
-          bf16x8 b_op[kPair ? 2 : 1];
-          for (int pj = 0; pj < (kPair ? 2 : 1); ++pj) {
-            const uint32_t word = step == 0 ? wq[pj][u].x
-                                            : (step == 1 ? wq[pj][u].y
-                                                         : (step == 2 ? wq[pj][u].z : wq[pj][u].w));
-            b_op[pj] = unpack_word(word);
-          }
-          for (int mt = 0; mt < MT; ++mt) {
-            const uint4 a_raw = *(const uint4 *)(xs + (mt * 32 + nl) * kPitch +
-                                                 (gi * kGroup + 32 * h + 8 * step) * 2);
-            const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
-            for (int pj = 0; pj < (kPair ? 2 : 1); ++pj)
-              part[pj][mt] =
-                  __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op[pj], part[pj][mt], 0, 0, 0);
-          }
-        }
-        // ---- affine fix-up for this group; row blocks beyond `count` are skipped
-        for (int pj = 0; pj < (kPair ? 2 : 1); ++pj) {
-          const float scale = bf16_bits_to_f32(sb[pj][u][0]);
-          const float shift = bf16_bits_to_f32(sb[pj][u][1]) - 16.0f * scale;
-          for (int mt = 0; mt < MT; ++mt)
-            for (int jq = 0; jq < 4; ++jq) {
-              if ((uint32_t)(mt * 32 + 8 * jq) >= count) continue;
-              const float4 sums = *(const float4 *)(xsum + gi * kRows + mt * 32 + 8 * jq + 4 * h);
-              acc[pj][mt][4 * jq + 0] += scale * part[pj][mt][4 * jq + 0] + shift * sums.x;
-              acc[pj][mt][4 * jq + 1] += scale * part[pj][mt][4 * jq + 1] + shift * sums.y;
-              acc[pj][mt][4 * jq + 2] += scale * part[pj][mt][4 * jq + 2] + shift * sums.z;
-              acc[pj][mt][4 * jq + 3] += scale * part[pj][mt][4 * jq + 3] + shift * sums.w;
-            }
-        }
+      if (row < (uint32_t)kRows) {
+        uint4 permuted;
+        permuted.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
+        permuted.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
+        permuted.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+        permuted.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+        *(uint4 *)(xs + row * kPitch + pc * 16) = permuted;
+        if ((pc & 7) == 0) xsum[(pc >> 3) * kRows + row] = sum;
       }
     }
+    __syncthreads();
+    if (kc0 + KC < a.inner) fetch_pass(kc0 + KC);
+  };
+  // One quantisation group: four MFMA steps per row tile, then the affine fix-up.
+  auto consume = [&](int slot, uint32_t group) {
+    const uint32_t gi = group % kGroupsPerPass;  // group index inside the staged pass
+    f32x16 part[kP][MT];
+    for (int pj = 0; pj < kP; ++pj)
+      for (int mt = 0; mt < MT; ++mt)
+        for (int j = 0; j < 16; ++j) part[pj][mt][j] = 0.0f;
+#pragma unroll
+    for (int step = 0; step < 4; ++step) {
+      bf16x8 b_op[kP];
+      for (int pj = 0; pj < kP; ++pj) {
+        const uint32_t word = step == 0 ? wq[pj][slot].x
+                                        : (step == 1 ? wq[pj][slot].y
+                                                     : (step == 2 ? wq[pj][slot].z : wq[pj][slot].w));
+        b_op[pj] = unpack_word(word);
+      }
+      for (int mt = 0; mt < MT; ++mt) {
+        const uint4 a_raw = *(const uint4 *)(xs + (mt * 32 + nl) * kPitch +
+                                             (gi * kGroup + 32 * h + 8 * step) * 2);
+        const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
+        for (int pj = 0; pj < kP; ++pj)
+          part[pj][mt] =
+              __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op[pj], part[pj][mt], 0, 0, 0);
+      }
+    }
+    // affine fix-up for this group; row blocks beyond `count` are skipped
+    for (int pj = 0; pj < kP; ++pj) {
+      const float scale = bf16_bits_to_f32(sb[pj][slot][0]);
+      const float shift = bf16_bits_to_f32(sb[pj][slot][1]) - 16.0f * scale;
+      for (int mt = 0; mt < MT; ++mt)
+        for (int jq = 0; jq < 4; ++jq) {
+          if ((uint32_t)(mt * 32 + 8 * jq) >= count) continue;
+          const float4 sums = *(const float4 *)(xsum + gi * kRows + mt * 32 + 8 * jq + 4 * h);
+          acc[pj][mt][4 * jq + 0] += scale * part[pj][mt][4 * jq + 0] + shift * sums.x;
+          acc[pj][mt][4 * jq + 1] += scale * part[pj][mt][4 * jq + 1] + shift * sums.y;
+          acc[pj][mt][4 * jq + 2] += scale * part[pj][mt][4 * jq + 2] + shift * sums.z;
+          acc[pj][mt][4 * jq + 3] += scale * part[pj][mt][4 * jq + 3] + shift * sums.w;
+        }
+    }
+  };
+  if (kRouted) __syncthreads();  // row_ids visible
+  fetch_pass(0);
+  if (!kSplitK) {
+    // Weight ring of four groups, refilled four groups ahead, independent of the passes.
+#pragma unroll
+    for (int u = 0; u < 4; ++u) load_group(u, u);
+    for (uint32_t g0 = 0; g0 < total_groups; g0 += 4) {
+      if (g0 % kGroupsPerPass == 0) pass_switch(g0 / kGroupsPerPass);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        consume(u, g0 + u);
+        load_group(u, g0 + u + 4);
+      }
+    }
+  } else {
+    // This wave's kGw groups of each pass; the next pass's are loaded while these are consumed.
+    const uint32_t mine = wave * kGw;
+#pragma unroll
+    for (int j = 0; j < kGw; ++j) load_group(j, mine + j);
+    for (uint32_t pass = 0; pass < passes; ++pass) {
+      pass_switch(pass);
+#pragma unroll
+      for (int j = 0; j < kGw; ++j) {
+        const uint32_t group = pass * kGroupsPerPass + mine + j;
+        if (group < total_groups) consume(j, group);
+        load_group(j, group + kGroupsPerPass);
+      }
+    }
+  }
+  if (kSplitK) {
+    // ---- add the four waves' partial accumulators through LDS (reusing the staging area)
+    static_assert(!kSplitK || !kPair, "split-K is for single projections");
+    float *red = (float *)xs;
+    __syncthreads();
+    for (int mt = 0; mt < MT; ++mt)
+      for (int j = 0; j < 16; ++j) {
+        const uint32_t row = mt * 32 + 8 * (j / 4) + 4 * h + (j % 4);
+        red[(wave * kRows + row) * 32 + nl] = acc[0][mt][j];
+      }
+    __syncthreads();
+    if (wave != 0) return;
+    for (int mt = 0; mt < MT; ++mt)
+      for (int j = 0; j < 16; ++j) {
+        const uint32_t row = mt * 32 + 8 * (j / 4) + 4 * h + (j % 4);
+        float total = 0.0f;
+        for (int w = 0; w < NW; ++w) total += red[(w * kRows + row) * 32 + nl];
+        acc[0][mt][j] = total;
+      }
   }
   // ---- epilogue and store; lane (column nl, half h) holds rows 8*(j/4) + 4h + j%4 of each tile
   if (column >= a.columns) return;
@@ -261,11 +346,20 @@ bool weights_eligible(const View &packed, const View &scales, const View &biases
 
 template <bool kPair, bool kRouted>
 void launch_qmm(hipStream_t stream, const QmmArgs &a, uint32_t row_blocks, int mt) {
-  dim3 grid((a.columns + kWaves * kColsPerWave - 1) / (kWaves * kColsPerWave), row_blocks);
+  uint32_t wide_blocks = (a.columns + kWaves * kColsPerWave - 1) / (kWaves * kColsPerWave);
+  if (!kPair && !kRouted && (uint64_t)wide_blocks * row_blocks < 256) {
+    dim3 grid((a.columns + kColsPerWave - 1) / kColsPerWave, row_blocks);
+    if (mt == 1)
+      qmm_mfma_kernel<1, false, false, true><<<grid, 256, 0, stream>>>(a);
+    else
+      qmm_mfma_kernel<2, false, false, true><<<grid, 256, 0, stream>>>(a);
+    return;
+  }
+  dim3 grid(wide_blocks, row_blocks);
   if (mt == 1)
-    qmm_mfma_kernel<1, kPair, kRouted><<<grid, 256, 0, stream>>>(a);
+    qmm_mfma_kernel<1, kPair, kRouted, false><<<grid, 256, 0, stream>>>(a);
   else
-    qmm_mfma_kernel<2, kPair, kRouted><<<grid, 256, 0, stream>>>(a);
+    qmm_mfma_kernel<2, kPair, kRouted, false><<<grid, 256, 0, stream>>>(a);
 }
 
 const uint32_t *u32_ptr(const View &v) { return (const uint32_t *)v.base + v.offset; }
@@ -273,7 +367,8 @@ const uint16_t *u16_ptr(const View &v) { return (const uint16_t *)v.base + v.off
 
 }  // namespace
 
-bool try_fast_quant_matmul(hipStream_t stream, const QmmProblem &p) {
+bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
+  hipStream_t stream = backend_stream(backend);
   if (p.x.dtype != FH_BF16) return false;
   if (p.out.dtype != FH_BF16 && p.out.dtype != FH_F32) return false;
   if (!weights_eligible(p.packed, p.scales, p.biases, 2, p.inner, p.bits, p.group)) return false;
@@ -294,6 +389,7 @@ bool try_fast_quant_matmul(hipStream_t stream, const QmmProblem &p) {
   a.columns = p.columns;
   int mt = p.rows <= 32 ? 1 : 2;
   uint32_t row_blocks = (p.rows + 32 * mt - 1) / (32 * mt);
+  KernelTimer timer(backend, FH_KC_QMM_KERNEL);
   launch_qmm<false, false>(stream, a, row_blocks, mt);
   return true;
 }
@@ -382,6 +478,7 @@ bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int
   a.blocks = plan.blocks;
   a.n_blocks = plan.n_blocks;
   a.route_div = p.k;
+  KernelTimer timer(backend, FH_KC_MOE_KERNEL);
   if (projections == 2)
     launch_qmm<true, true>(stream, a, plan.max_blocks, 1);
   else
@@ -419,7 +516,10 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
   a.blocks = plan.blocks;
   a.n_blocks = plan.n_blocks;
   a.route_div = 1;
-  launch_qmm<false, true>(stream, a, plan.max_blocks, 1);
+  {
+    KernelTimer timer(backend, FH_KC_MOE_KERNEL);
+    launch_qmm<false, true>(stream, a, plan.max_blocks, 1);
+  }
   uint64_t work = (uint64_t)p.rows * p.columns;
   View none{};
   none.base = nullptr;
@@ -428,8 +528,6 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
       p.k, p.columns, p.experts);
   return true;
 }
-
-bool try_fast_program(hipStream_t, bool, const ProgramArgs &, uint64_t) { return false; }
 
 namespace {
 

@@ -310,8 +310,9 @@ class HipBackend:
         return value.value
 
     # ---- profiling aid
-    def profile_enable(self, enabled: bool):
-        _check(self._lib.fh_profile_enable(self._handle, int(enabled)))
+    def profile_enable(self, level: int):
+        """0 off, 1 single-kernel timers, 2 also one timer per dispatch."""
+        _check(self._lib.fh_profile_enable(self._handle, int(level)))
 
     def profile_reset(self):
         _check(self._lib.fh_profile_reset(self._handle))

@@ -197,15 +197,21 @@ FH_API fh_status fh_memory_usage(fh_backend *backend, uint64_t *bytes);
 /* Blocks until all submitted work has finished. */
 FH_API fh_status fh_synchronize(fh_backend *backend);
 
-/* Profiling aid: device time in ns spent by kernels whose name class matches `kernel_class`
- * (see fh_kernel_class) since the last fh_profile_reset, measured with HIP events on the
- * backend's stream; `launches` receives the launch count.  Enabled by fh_profile_enable(1). */
+/* Profiling aid: device time in ns spent in `kernel_class` (see fh_kernel_class) since the last
+ * fh_profile_reset, measured with HIP events recorded on the backend's stream around each
+ * dispatch / kernel launch; `launches` receives the count.  fh_profile_enable level: 0 off,
+ * 1 times only the single-kernel classes, 2 also times every dispatch. */
 typedef enum fh_kernel_class {
+  /* whole dispatches, by op */
   FH_KC_OTHER = 0,
-  FH_KC_QMM = 1,
-  FH_KC_MOE = 2,
-  FH_KC_ATTENTION = 3,
-  FH_KC_COUNT = 4
+  FH_KC_QMM = 1,       /* FH_OP_QUANT_MATMUL */
+  FH_KC_MOE = 2,       /* FH_OP_GATHER_QUANT_MATMUL (packing + grouped matmul + combine) */
+  FH_KC_ATTENTION = 3, /* paged attention ops (plan + append + attention + merge) */
+  /* single kernels: the launch that dominates each class */
+  FH_KC_ATTENTION_KERNEL = 4, /* ragged_attention_mfma_kernel */
+  FH_KC_MOE_KERNEL = 5,       /* routed qmm_mfma_kernel */
+  FH_KC_QMM_KERNEL = 6,       /* dense qmm_mfma_kernel */
+  FH_KC_COUNT = 7
 } fh_kernel_class;
 FH_API fh_status fh_profile_enable(fh_backend *backend, int enabled);
 FH_API fh_status fh_profile_reset(fh_backend *backend);

@@ -75,7 +75,8 @@ class Workload:
 
 
 def algorithmic_bytes(workload, contexts):
-    """SURVEY/DESIGN accounting: K/V rows read once per kv head, weights incl. scales+biases."""
+    """Logical bytes of a step: every K/V row read once per kv head, weights with their scales and
+    biases (the accounting of crates/forja-core/src/cost/attention.rs:5-90 and cost.rs:111-153)."""
     model = workload.model
     c = model.config
     kv = int((contexts + 1).sum()) * (model.n_layers * 2 * c.kv_heads * c.head_dim * 2)
@@ -131,7 +132,22 @@ def main():
     parser.add_argument("--cpu-sample-lanes", type=int, default=8)
     parser.add_argument("--no-profile", action="store_true",
                         help="skip the HIP-event kernel timing inside the timed region")
+    parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                        help="only run 8 plain copies of MIB mebibytes (a known-size kernel to "
+                             "scale hardware traffic counters by) and exit")
     args = parser.parse_args()
+    if args.calibrate_copy:
+        backend = HipBackend(0)
+        elements = args.calibrate_copy * (1 << 20) // 4
+        source = backend.alloc(DType.U32, [elements])
+        target = backend.alloc(DType.U32, [elements])
+        for _ in range(8):
+            commands = CommandList()
+            commands.dispatch(Op.copy(), [source], target)
+            backend.submit(commands).wait()
+        print(json.dumps({"copy_bytes_read": elements * 4, "copy_bytes_written": elements * 4,
+                          "kernel": "copy_kernel", "launches": 8}))
+        return
     if args.gpus != 1:
         print("bench.py: this build runs the ragged forward step on ONE MI355X; collectives and "
               "sharding are not part of it, so --gpus must be 1", file=sys.stderr)

@@ -299,6 +299,229 @@ __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
     }
 }
 
+// ---- decode-sized dense products: at most 128 activation rows -------------------------------
+//
+// With so few rows the weights are a few megabytes, and what a compute unit can pull from L2
+// (about 50 GB/s) bounds the launch long before HBM does.  So the product is cut into slabs that
+// make every byte a CU fetches count: a workgroup of eight waves takes 256 output columns (32
+// per wave) and 256 values of K for all rows, stages that activation slab in LDS once (64 KB for
+// 128 rows), and every wave contracts it with its own four groups of packed weights, which were
+// requested before anything else.  There is a single pass and a single barrier.  The K slabs of
+// a column block leave f32 partial tiles in workspace and sum_slabs_kernel adds them in slab
+// order (a fixed order: results do not depend on scheduling).
+struct SlabArgs {
+  const uint16_t *x;
+  uint64_t x_row_stride;
+  const uint32_t *packed;
+  const uint16_t *scales, *biases;
+  float *partials;      // [K/256][rows][columns]
+  void *out;            // used directly when there is a single slab
+  uint64_t out_row_stride;
+  uint32_t out_f32;
+  uint32_t rows, inner, columns;
+};
+
+constexpr int kSlabK = 256, kSlabWaves = 8, kSlabThreads = 64 * kSlabWaves;
+constexpr int kSlabP = 1;                     // 32-column operands per wave
+constexpr int kSlabColsPerWave = 32 * kSlabP;
+constexpr int kSlabPitch = 2 * kSlabK + 16;   // bytes per staged row
+
+template <int MT>
+constexpr uint32_t slab_lds_bytes() {
+  return 32 * MT * kSlabPitch + (kSlabK / kGroup) * 32 * MT * 4;
+}
+
+template <int MT>
+__global__ __launch_bounds__(kSlabThreads) void qmm_slab_kernel(SlabArgs a) {
+  constexpr int kP = kSlabP;
+  constexpr int kRows = 32 * MT;
+  constexpr int kGroups = kSlabK / kGroup;   // 4
+  extern __shared__ __attribute__((aligned(16))) unsigned char slab_lds[];
+  unsigned char *xs = slab_lds;
+  float *xsum = (float *)(slab_lds + kRows * kSlabPitch);
+  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint32_t nl = lane & 31, h = lane >> 5;
+  const uint32_t slab = blockIdx.y, k0 = slab * kSlabK;
+  const uint32_t groups_per_row = a.inner / kGroup;
+  uint32_t column[kP];
+  for (int pj = 0; pj < kP; ++pj)
+    column[pj] = (blockIdx.x * kSlabWaves + wave) * kSlabColsPerWave + 32 * pj + nl;
+
+  // weights first: they come from cold memory
+  uint4 wq[kP][kGroups];
+  uint32_t scale_bits[kP][kGroups], bias_bits[kP][kGroups];
+#pragma unroll
+  for (int pj = 0; pj < kP; ++pj) {
+    const uint32_t column_c = min(column[pj], a.columns - 1);
+    const uint32_t *w_row = a.packed + (uint64_t)column_c * (a.inner / 8) + k0 / 8 + 4 * h;
+    const uint16_t *s_row = a.scales + (uint64_t)column_c * groups_per_row + k0 / kGroup;
+    const uint16_t *b_row = a.biases + (uint64_t)column_c * groups_per_row + k0 / kGroup;
+#pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+      wq[pj][g] = *(const uint4 *)(w_row + 8 * g);
+      scale_bits[pj][g] = s_row[g];
+      bias_bits[pj][g] = b_row[g];
+    }
+  }
+  // stage the activation slab: permuted inside each 8, with per-group row sums
+  constexpr int kPieces = kRows * (kSlabK / 8) / kSlabThreads;
+#pragma unroll
+  for (int i0 = 0; i0 < kPieces; i0 += 8) {
+    uint4 x_regs[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i0 + i >= kPieces) break;
+      const uint32_t piece = tid + (i0 + i) * kSlabThreads;
+      const uint32_t row = piece / (kSlabK / 8), pc = piece % (kSlabK / 8);
+      x_regs[i] = make_uint4(0, 0, 0, 0);
+      if (row < a.rows)
+        x_regs[i] = *(const uint4 *)(a.x + (uint64_t)row * a.x_row_stride + k0 + 8 * pc);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i0 + i >= kPieces) break;
+      const uint32_t piece = tid + (i0 + i) * kSlabThreads;
+      const uint32_t row = piece / (kSlabK / 8), pc = piece % (kSlabK / 8);
+      const uint4 v = x_regs[i];
+      float sum = bf16_bits_to_f32(v.x & 0xffffu) + bf16_bits_to_f32(v.x >> 16) +
+                  bf16_bits_to_f32(v.y & 0xffffu) + bf16_bits_to_f32(v.y >> 16) +
+                  bf16_bits_to_f32(v.z & 0xffffu) + bf16_bits_to_f32(v.z >> 16) +
+                  bf16_bits_to_f32(v.w & 0xffffu) + bf16_bits_to_f32(v.w >> 16);
+      sum += __shfl_xor(sum, 1, 64);   // eight consecutive pieces (= lanes) make one group
+      sum += __shfl_xor(sum, 2, 64);
+      sum += __shfl_xor(sum, 4, 64);
+      uint4 permuted;
+      permuted.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
+      permuted.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
+      permuted.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+      permuted.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+      *(uint4 *)(xs + row * kSlabPitch + pc * 16) = permuted;
+      if ((pc & 7) == 0) xsum[(pc >> 3) * kRows + row] = sum;
+    }
+  }
+  __syncthreads();
+
+  f32x16 acc[kP][MT];
+  for (int pj = 0; pj < kP; ++pj)
+    for (int mt = 0; mt < MT; ++mt)
+      for (int j = 0; j < 16; ++j) acc[pj][mt][j] = 0.0f;
+  // The bias term sum_g (bias_g - 16 scale_g) * xsum_g[row] is itself a small product over the
+  // groups: an f32 MFMA (K = 2 groups per instruction; lane half h supplies group 2p + h of
+  // both operands) adds it straight into the accumulators.
+#pragma unroll
+  for (int pair = 0; pair < kGroups / 2; ++pair)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const float sums = xsum[(2 * pair + h) * kRows + mt * 32 + nl];
+#pragma unroll
+      for (int pj = 0; pj < kP; ++pj) {
+        const float shift_even = bf16_bits_to_f32(bias_bits[pj][2 * pair]) -
+                                 16.0f * bf16_bits_to_f32(scale_bits[pj][2 * pair]);
+        const float shift_odd = bf16_bits_to_f32(bias_bits[pj][2 * pair + 1]) -
+                                16.0f * bf16_bits_to_f32(scale_bits[pj][2 * pair + 1]);
+        acc[pj][mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(sums, h ? shift_odd : shift_even,
+                                                           acc[pj][mt], 0, 0, 0);
+      }
+    }
+  // The group loop is kept rolled (a compact body keeps the register count down); the weight
+  // registers rotate so that slot 0 is always the current group.
+#pragma unroll 1
+  for (int g = 0; g < kGroups; ++g) {
+    bf16x8 b_op[kP][4];
+    float scale[kP];
+#pragma unroll
+    for (int pj = 0; pj < kP; ++pj) {
+      scale[pj] = bf16_bits_to_f32(scale_bits[pj][0]);
+      b_op[pj][0] = unpack_word(wq[pj][0].x);
+      b_op[pj][1] = unpack_word(wq[pj][0].y);
+      b_op[pj][2] = unpack_word(wq[pj][0].z);
+      b_op[pj][3] = unpack_word(wq[pj][0].w);
+    }
+    // up to four independent accumulation chains at a time keep the matrix pipe busy
+    constexpr int kChunk = (MT * kP >= 4) ? 4 / kP : MT;
+#pragma unroll
+    for (int mt0 = 0; mt0 < MT; mt0 += kChunk) {
+      f32x16 part[kP][kChunk];
+#pragma unroll
+      for (int pj = 0; pj < kP; ++pj)
+        for (int c = 0; c < kChunk; ++c)
+          for (int j = 0; j < 16; ++j) part[pj][c][j] = 0.0f;
+#pragma unroll
+      for (int step = 0; step < 4; ++step)
+#pragma unroll
+        for (int c = 0; c < kChunk; ++c) {
+          const uint4 a_raw = *(const uint4 *)(xs + ((mt0 + c) * 32 + nl) * kSlabPitch +
+                                               (g * kGroup + 32 * h + 8 * step) * 2);
+          const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
+#pragma unroll
+          for (int pj = 0; pj < kP; ++pj)
+            part[pj][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op[pj][step],
+                                                                  part[pj][c], 0, 0, 0);
+        }
+#pragma unroll
+      for (int pj = 0; pj < kP; ++pj)
+#pragma unroll
+        for (int c = 0; c < kChunk; ++c)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) acc[pj][mt0 + c][j] += scale[pj] * part[pj][c][j];
+    }
+#pragma unroll
+    for (int pj = 0; pj < kP; ++pj)
+#pragma unroll
+      for (int r = 0; r + 1 < kGroups; ++r) {
+        wq[pj][r] = wq[pj][r + 1];
+        scale_bits[pj][r] = scale_bits[pj][r + 1];
+      }
+  }
+  const bool direct = gridDim.y == 1;
+  float *mine = a.partials + (uint64_t)slab * a.rows * a.columns;
+#pragma unroll
+  for (int pj = 0; pj < kP; ++pj) {
+    if (column[pj] >= a.columns) continue;
+    for (int mt = 0; mt < MT; ++mt)
+      for (int j = 0; j < 16; ++j) {
+        const uint32_t row = mt * 32 + 8 * (j / 4) + 4 * h + (j % 4);
+        if (row >= a.rows) continue;
+        if (!direct) {
+          mine[(uint64_t)row * a.columns + column[pj]] = acc[pj][mt][j];
+        } else {
+          const uint64_t at = (uint64_t)row * a.out_row_stride + column[pj];
+          if (a.out_f32)
+            ((float *)a.out)[at] = acc[pj][mt][j];
+          else
+            ((uint16_t *)a.out)[at] = (uint16_t)(pack2(acc[pj][mt][j], 0.0f) & 0xffffu);
+        }
+      }
+  }
+}
+
+// out[row, column] = sum over slabs (ascending) of partials[slab][row][column]; a thread takes
+// four consecutive columns (the host guarantees columns % 4 == 0 and aligned output rows).
+__global__ void sum_slabs_kernel(const float *partials, uint32_t slabs, uint32_t rows,
+                                 uint32_t columns, void *out, uint64_t out_row_stride,
+                                 uint32_t out_f32) {
+  const uint64_t flat = 4 * ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x);
+  const uint64_t plane = (uint64_t)rows * columns;
+  if (flat >= plane) return;
+  float4 total = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  for (uint32_t s = 0; s < slabs; ++s) {
+    const float4 v = *(const float4 *)(partials + s * plane + flat);
+    total.x += v.x;
+    total.y += v.y;
+    total.z += v.z;
+    total.w += v.w;
+  }
+  const uint64_t at = (flat / columns) * out_row_stride + flat % columns;
+  if (out_f32) {
+    *(float4 *)((float *)out + at) = total;
+  } else {
+    uint2 packed;
+    packed.x = pack2(total.x, total.y);
+    packed.y = pack2(total.z, total.w);
+    *(uint2 *)((uint16_t *)out + at) = packed;
+  }
+}
+
 // out[r, :] = residual[r, :] + sum_s weights[r, s] * partial[r*k + s, :], slots in ascending
 // order (execute_gather_quant_weighted_sum, crates/forja-cpu/src/lib.rs:1153-1199); routes that
 // name no valid expert contribute nothing.
@@ -362,6 +585,53 @@ void launch_qmm(hipStream_t stream, const QmmArgs &a, uint32_t row_blocks, int m
     qmm_mfma_kernel<2, kPair, kRouted, false><<<grid, 256, 0, stream>>>(a);
 }
 
+// Decode-sized dense product through the slab kernels; false when workspace is short.
+template <int MT>
+void launch_slab(hipStream_t stream, const SlabArgs &s, dim3 grid) {
+  static bool configured = false;   // raise the dynamic LDS limit once per process
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_slab_kernel<MT>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)slab_lds_bytes<MT>());
+    configured = true;
+  }
+  qmm_slab_kernel<MT><<<grid, kSlabThreads, slab_lds_bytes<MT>(), stream>>>(s);
+}
+
+bool launch_skinny(fh_backend *backend, const QmmArgs &q) {
+  hipStream_t stream = backend_stream(backend);
+  const uint32_t slabs = q.inner / kSlabK;
+  const uint64_t plane = (uint64_t)q.rows * q.columns;
+  SlabArgs s{};
+  if (slabs > 1) {
+    s.partials = (float *)backend_workspace(backend, slabs * plane * sizeof(float));
+    if (!s.partials) return false;
+  }
+  s.x = q.x;
+  s.x_row_stride = q.x_row_stride;
+  s.packed = q.packed[0];
+  s.scales = q.scales[0];
+  s.biases = q.biases[0];
+  s.out = q.out;
+  s.out_row_stride = q.out_row_stride;
+  s.out_f32 = q.out_f32;
+  s.rows = q.rows;
+  s.inner = q.inner;
+  s.columns = q.columns;
+  KernelTimer timer(backend, FH_KC_QMM_KERNEL);
+  dim3 grid((q.columns + kSlabWaves * kSlabColsPerWave - 1) / (kSlabWaves * kSlabColsPerWave), slabs);
+  if (q.rows <= 32)
+    launch_slab<1>(stream, s, grid);
+  else if (q.rows <= 64)
+    launch_slab<2>(stream, s, grid);
+  else
+    launch_slab<4>(stream, s, grid);
+  if (slabs > 1)
+    sum_slabs_kernel<<<(uint32_t)((plane / 4 + 255) / 256), 256, 0, stream>>>(
+        s.partials, slabs, q.rows, q.columns, q.out, q.out_row_stride, q.out_f32);
+  return true;
+}
+
 const uint32_t *u32_ptr(const View &v) { return (const uint32_t *)v.base + v.offset; }
 const uint16_t *u16_ptr(const View &v) { return (const uint16_t *)v.base + v.offset; }
 
@@ -387,6 +657,11 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
   a.rows = p.rows;
   a.inner = p.inner;
   a.columns = p.columns;
+  if (p.rows <= 128 && p.columns <= 16384 && p.columns % 4 == 0 && p.out.stride[0] % 4 == 0 &&
+      p.out.offset % 4 == 0) {
+    if (!launch_skinny(backend, a)) return false;
+    return true;
+  }
   int mt = p.rows <= 32 ? 1 : 2;
   uint32_t row_blocks = (p.rows + 32 * mt - 1) / (32 * mt);
   KernelTimer timer(backend, FH_KC_QMM_KERNEL);

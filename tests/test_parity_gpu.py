@@ -127,6 +127,12 @@ QMM_CASES = [
     (64, 100, 512, 4, 64, DType.BF16),      # column tail inside a wave
     (130, 96, 768, 4, 64, DType.BF16),      # row tail across row blocks
     (8, 512, 4096, 4, 64, DType.BF16),
+    (128, 5120, 2048, 4, 64, DType.BF16),   # C3 stacked qkv: packed-activation path, 2 splits
+    (128, 2048, 4096, 4, 64, DType.BF16),   # C3 o_proj: 4 splits
+    (100, 130, 2048, 4, 64, DType.BF16),    # row and column tails, 8 splits
+    (64, 96, 256, 4, 64, DType.BF16),       # a single group per wave, no split
+    (65, 32, 3072, 4, 64, DType.BF16),      # 12 splits
+    (192, 4096, 2048, 4, 64, DType.BF16),   # more rows than the decode path takes
 ]
 
 

@@ -29,6 +29,11 @@ from forja_amd.model import (QWEN3_CODER_30B_A3B, QWEN3_0_6B, DecodeSession, Mod
                              ModelConfig)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes moved by ragged_attention_mfma_kernel per algorithmic byte on this workload, from the
+# hardware counters: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over the same launches, each
+# scaled by what the counter reads for a 1 GiB copy (FETCH_SIZE counts half of it, WRITE_SIZE all
+# of it); figures and commands in profiles/c3_decode_step_hbm_traffic.txt.
+ATTENTION_TRAFFIC_RATIO = 1.022
 KC_ATTENTION, KC_MOE, KC_QMM = 3, 2, 1
 KC_ATTENTION_KERNEL, KC_MOE_KERNEL, KC_QMM_KERNEL = 4, 5, 6
 
@@ -155,6 +160,7 @@ def main():
 
     config = QWEN3_CODER_30B_A3B
     ctx_lo, ctx_hi, churn = 256, 32768, 8
+    default_workload = args.layers is None and args.lanes == 128 and args.seed == 20261
     backend = HipBackend(0)
     info = backend.device_info()
     workload = Workload(backend, config, args.lanes, ctx_lo, ctx_hi, churn, args.seed, layers=args.layers)
@@ -207,9 +213,7 @@ def main():
     }
     weights = workload.model.weight_bytes_per_step(args.lanes)
     kv_per_step = kv_bytes_total / args.steps
-    step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"]
-    result["step_algorithmic_gb"] = step_bytes / 1e9
-    result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS
+    routed_fraction = 1.0
     if not args.no_profile:
         ns, launches = backend.profile_read(KC_ATTENTION_KERNEL)
         kernel_bytes = kv_bytes_total / max(launches, 1)          # per launch = per layer per step
@@ -217,7 +221,8 @@ def main():
         achieved = kernel_bytes / average / 1e9 if average > 0 else 0.0
         result["roofline"] = {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": kernel_bytes * ATTENTION_TRAFFIC_RATIO if default_workload else None,
             "kernel": "ragged_attention_mfma_kernel", "launches": launches,
             "avg_launch_us": average * 1e6, "algorithmic_bytes_per_launch": kernel_bytes,
         }
@@ -227,12 +232,31 @@ def main():
         qmm_ns, qmm_launches = backend.profile_read(KC_QMM_KERNEL)
         secondary = {}
         if moe_launches:
-            moe_bytes = weights["routed_all_experts"] * args.steps / moe_launches
+            # one more (untimed) step that also copies out every layer's expert choices: the
+            # routed kernels read the weights of the DISTINCT experts chosen, nothing else
+            from forja_amd.model import record_step
+            trace = backend.alloc(DType.U32, (workload.model.n_layers, args.lanes, config.top_k))
+            traced = CommandList()
+            record_step(workload.model, session.cache, session.buffers, traced, feed_back=True,
+                        route_trace=trace)
+            session.upload_positions()
+            backend.submit(traced).wait()
+            session.contexts += 1
+            chosen = np.frombuffer(backend.read(trace), np.uint32).reshape(
+                workload.model.n_layers, args.lanes * config.top_k)
+            distinct = np.array([len(np.unique(layer)) for layer in chosen])
+            fraction = float(distinct.mean()) / config.experts
+            moe_bytes = weights["routed_all_experts"] * fraction * args.steps / moe_launches
             secondary["routed_qmm_mfma_kernel"] = {
                 "avg_launch_us": moe_ns / moe_launches / 1e3,
                 "achieved_gbps": moe_bytes / (moe_ns / moe_launches * 1e-9) / 1e9,
                 "frac": moe_bytes / (moe_ns / moe_launches * 1e-9) / 1e9 / HBM_PEAK_GBPS,
-                "note": "weights of all experts counted once per projection launch"}
+                "distinct_experts_per_layer": {"mean": float(distinct.mean()),
+                                               "min": int(distinct.min()), "max": int(distinct.max()),
+                                               "of": config.experts},
+                "note": ("bytes = weights of the distinct experts the router chose (measured on "
+                         "one traced step), per projection launch")}
+            routed_fraction = fraction
         if qmm_launches:
             qmm_bytes = weights["dense"] * args.steps / qmm_launches
             secondary["dense_qmm_mfma_kernel"] = {
@@ -254,6 +278,9 @@ def main():
             breakdown[name] = class_ns / 1e6 / extra
         result["gpu_ms_per_step_by_op"] = breakdown
         backend.profile_enable(0)
+    step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction
+    result["step_algorithmic_gb"] = step_bytes / 1e9
+    result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(config, args.seed, args.cpu_sample_lanes, ctx_lo, ctx_hi)
     print(json.dumps(result))

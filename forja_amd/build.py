@@ -6,6 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libforja_hip.so")
+CONFORMANCE = os.path.join(HERE, "host", "conformance")
 
 SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "programs_fast.hip"]
 
@@ -44,7 +45,19 @@ def build(verbose=False, jobs=8):
         raise RuntimeError("hipcc failed")
     link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objects
     subprocess.run(link, check=True)
+    build_host()
     return LIB
+
+
+def build_host():
+    """Compiles the C++ host interface's known-answer program against the built library."""
+    host = os.path.join(HERE, "host")
+    include = os.path.join(os.path.dirname(HERE), "include")
+    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-I" + include, "-I" + host,
+           os.path.join(host, "conformance.cpp"), "-o", CONFORMANCE, "-L" + HERE, "-lforja_hip",
+           "-Wl,-rpath,$ORIGIN/.."]
+    subprocess.run(cmd, check=True)
+    return CONFORMANCE
 
 
 if __name__ == "__main__":

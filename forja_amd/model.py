@@ -259,9 +259,11 @@ class StepBuffers:
 
 
 def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: CommandList,
-                feed_back: bool = False) -> None:
+                feed_back: bool = False, route_trace: Optional[Tensor] = None) -> None:
     """Appends one forward step over the packed batch to `commands`.  With `feed_back` the greedy
-    tokens are copied into the id buffer for the next step (device to device)."""
+    tokens are copied into the id buffer for the next step (device to device).  `route_trace`
+    (u32 [layers, tokens, top_k]) receives a copy of every layer's expert choices, for
+    diagnostics."""
     c, b = model.config, buffers
     tokens = b.tokens
     heads = c.q_heads + c.kv_heads
@@ -309,6 +311,9 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
             commands.dispatch(q4, [normalized, *layer.router.triple], b.router_logits)
             commands.dispatch_many(Op.top_k(c.top_k, True), [b.router_logits],
                                    [b.route_weights, b.route_indices])
+            if route_trace is not None:
+                commands.dispatch(Op.copy(), [b.route_indices],
+                                  route_trace.narrow(0, index, 1).reshape((tokens, c.top_k)))
             commands.dispatch_epilogue(gq4, [normalized, *layer.gate.triple, *layer.up.triple,
                                              b.route_indices], b.activated, model.swiglu_epilogue, [])
             commands.dispatch_epilogue(gq4, [b.activated, *layer.down.triple, b.route_indices,

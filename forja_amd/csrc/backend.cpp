@@ -100,6 +100,11 @@ struct fh_backend {
   uint64_t used_bytes = 0;
   char *workspace = nullptr;
   uint64_t workspace_bytes = 0;
+  // route plan kept between the routed projections of a layer
+  char *route_plan = nullptr;
+  uint64_t route_plan_bytes = 0;
+  bool route_plan_valid = false;
+  RoutePlanKey route_plan_key{};
   // profiling
   int profiling = 0;  // 0 off, 1 kernel-level timers, 2 also one timer per dispatch
   struct Timed {
@@ -567,6 +572,7 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
     problem.scales[0] = pl.in[2];
     problem.biases[0] = pl.in[3];
     problem.indices = pl.in[4];
+    problem.indices_buffer = d.inputs[4].buffer;
     problem.weights = pl.in[5];
     problem.rows = rows;
     problem.k = routes;
@@ -633,6 +639,7 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
     problem.biases[1] = pl.in[6];
   }
   problem.indices = pl.in[primitive - 1];
+  problem.indices_buffer = d.inputs[primitive - 1].buffer;
   problem.out = pl.out[0];
   problem.rows = rows;
   problem.k = k;
@@ -983,7 +990,8 @@ fh_status plan_route_pack(fh_backend *b, const Planned &pl, ErrorSlot *error, bo
   for (uint32_t o = 0; o < 4; ++o)
     FH_REQUIRE(d.outputs[o].dtype == FH_U32 && is_contiguous(d.outputs[o]));
   uint32_t experts = d.outputs[0].shape[0];
-  FH_REQUIRE(d.outputs[0].rank == 1 && experts != 0 && experts <= 4096);
+  FH_REQUIRE(d.outputs[0].rank == 1 && experts != 0);
+  if (experts > 512) return FH_UNSUPPORTED_OPERATION;  // per-wave counts of all experts live in LDS
   FH_REQUIRE(shape_is(d.outputs[1], {experts + 1}));
   uint64_t routes = (uint64_t)idx.shape[0] * idx.shape[1];
   FH_REQUIRE(routes <= (1u << 24) && shape_is(d.outputs[2], {(uint32_t)routes}));
@@ -1156,6 +1164,7 @@ void fh_destroy(fh_backend *b) {
     for (auto &entry : b->programs)
       for (auto &typed : entry.second.typed) (void)hipFree(typed.second);
     if (b->workspace) (void)hipFree(b->workspace);
+    if (b->route_plan) (void)hipFree(b->route_plan);
     for (auto &e : b->error_pool) {
       (void)hipFree(e.device);
       (void)hipHostFree(e.host);
@@ -1426,6 +1435,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   }
   s->start = take_event(b);
   s->end = take_event(b);
+  b->route_plan_valid = false;  // host writes between submissions are not tracked
   launch_init_errors(b->stream, s->device_errors, slots);
   (void)hipEventRecord(s->start, b->stream);
   fh_status status = FH_OK;
@@ -1438,6 +1448,9 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
       (void)hipEventRecord(t0, b->stream);
     }
     status = process(b, dispatches[i], &s->device_errors[i], true);
+    if (b->route_plan_valid)
+      for (uint32_t o = 0; o < dispatches[i].n_outputs && o < FH_MAX_OUTPUTS; ++o)
+        if (dispatches[i].outputs[o].buffer == b->route_plan_key.buffer) b->route_plan_valid = false;
     if (b->profiling >= 2) {
       (void)hipEventRecord(t1, b->stream);
       b->timed.push_back({t0, t1, kernel_class_of(dispatches[i].op)});
@@ -1625,6 +1638,29 @@ fh_status fh_profile_read(fh_backend *b, uint32_t kernel_class, uint64_t *nanose
 
 namespace fh {
 char *backend_workspace(fh_backend *backend, uint64_t bytes) { return backend->ensure_workspace(bytes); }
+char *backend_route_plan(fh_backend *b, const RoutePlanKey &key, uint64_t bytes, bool *reuse) {
+  const RoutePlanKey &have = b->route_plan_key;
+  *reuse = b->route_plan_valid && bytes <= b->route_plan_bytes && have.buffer == key.buffer &&
+           have.offset == key.offset && have.stride0 == key.stride0 && have.stride1 == key.stride1 &&
+           have.rows == key.rows && have.k == key.k && have.experts == key.experts &&
+           have.tile == key.tile;
+  if (*reuse) return b->route_plan;
+  b->route_plan_valid = false;
+  if (bytes > b->route_plan_bytes) {
+    (void)hipStreamSynchronize(b->stream);
+    if (b->route_plan) (void)hipFree(b->route_plan);
+    b->route_plan = nullptr;
+    b->route_plan_bytes = 0;
+    uint64_t want = std::max<uint64_t>(bytes, 1ull << 20);
+    void *ptr = nullptr;
+    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
+    b->route_plan = (char *)ptr;
+    b->route_plan_bytes = want;
+  }
+  b->route_plan_key = key;
+  b->route_plan_valid = true;
+  return b->route_plan;
+}
 hipStream_t backend_stream(fh_backend *backend) { return backend->stream; }
 uint32_t backend_compute_units(fh_backend *backend) {
   return (uint32_t)backend->props.multiProcessorCount;

@@ -18,6 +18,17 @@ uint32_t backend_compute_units(fh_backend *backend);
 void backend_profile_begin(fh_backend *backend, uint32_t kernel_class);
 void backend_profile_end(fh_backend *backend, uint32_t kernel_class);
 
+// Identity of a route plan: the indices view it was packed from and the tiling.
+struct RoutePlanKey {
+  uint64_t buffer, offset, stride0, stride1;
+  uint32_t rows, k, experts, tile;
+};
+// Device storage (at least `bytes`) for a route plan that outlives its dispatch, so that the two
+// routed projections of a layer pack their shared indices once.  `*reuse` is set when the storage
+// already holds the plan for `key`: the same indices view, not written since it was packed, in
+// the same submission.  Null when allocation fails.
+char *backend_route_plan(fh_backend *backend, const RoutePlanKey &key, uint64_t bytes, bool *reuse);
+
 // Brackets one kernel launch with HIP events when profiling is enabled.
 struct KernelTimer {
   fh_backend *backend;
@@ -38,6 +49,7 @@ struct GatherProblem {
   View x;           // projection: [R,K]; weighted sum: [R,k,K]
   View packed[2], scales[2], biases[2];
   View indices;     // [R,k]
+  uint64_t indices_buffer;  // allocation identity of `indices`
   View weights;     // weighted sum only: [R,k]
   View out;         // projection: [R,k,N]; weighted sum: [R,N]
   uint32_t rows, k, inner, experts, columns, bits, group;

@@ -11,103 +11,127 @@ namespace fh {
 
 namespace {
 
-// One wave does the whole plan: at decode sizes (<= a few thousand routes) the work is a handful
-// of 64-route rounds and a single launch beats three.
-__global__ void route_pack_kernel(View indices, uint32_t rows, uint32_t k, uint32_t experts,
-                                  uint32_t tile_rows, uint32_t *counts, uint32_t *offsets,
-                                  uint32_t *sorted_routes, uint32_t *blocks, uint32_t max_blocks,
-                                  uint32_t *n_blocks, ErrorSlot *error) {
+// One workgroup of 16 waves does the whole plan in a single launch: at decode sizes (a few
+// thousand routes) everything fits one or two 1024-route rounds, and what matters is the number
+// of dependent memory round trips, not throughput.
+constexpr uint32_t kPackThreads = 1024, kPackWaves = kPackThreads / 64;
+
+__global__ __launch_bounds__(1024) void route_pack_kernel(
+    View indices, uint32_t rows, uint32_t k, uint32_t experts, uint32_t tile_rows, uint32_t *counts,
+    uint32_t *offsets, uint32_t *sorted_routes, uint32_t *blocks, uint32_t max_blocks,
+    uint32_t *n_blocks, ErrorSlot *error) {
   extern __shared__ uint32_t lds[];
-  uint32_t *lds_counts = lds;            // [experts]
-  uint32_t *lds_cursor = lds + experts;  // [experts]
-  const uint32_t lane = threadIdx.x;
+  uint32_t *lds_counts = lds;                    // [experts]
+  uint32_t *lds_cursor = lds + experts;          // [experts] next free position per expert
+  uint32_t *wave_counts = lds + 2 * experts;     // [kPackWaves][experts] per round
+  uint32_t *scan = lds + (2 + kPackWaves) * experts;  // [kPackWaves + 1]
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t routes = rows * k;
-  for (uint32_t e = lane; e < experts; e += 64) lds_counts[e] = 0;
+  auto expert_of = [&](uint32_t route) {
+    return load_u32_at(indices, indices.offset + (uint64_t)(route / k) * indices.stride[0] +
+                                    (uint64_t)(route % k) * indices.stride[1]);
+  };
+  for (uint32_t e = tid; e < experts; e += kPackThreads) lds_counts[e] = 0;
   __syncthreads();
-  for (uint32_t route = lane; route < routes; route += 64) {
-    uint32_t expert = load_u32_at(indices, indices.offset + (uint64_t)(route / k) * indices.stride[0] +
-                                               (uint64_t)(route % k) * indices.stride[1]);
+  // the first round's expert ids stay in a register for the arrange pass
+  const uint32_t first_expert = tid < routes ? expert_of(tid) : 0xffffffffu;
+  for (uint32_t route = tid; route < routes; route += kPackThreads) {
+    const uint32_t expert = route == tid ? first_expert : expert_of(route);
     if (expert >= experts)
       report_error(error, expert);
     else
       atomicAdd(&lds_counts[expert], 1u);
   }
   __syncthreads();
-  // Exclusive scan of counts, 64 experts per round.
-  uint32_t running = 0;
-  for (uint32_t base = 0; base < experts; base += 64) {
-    uint32_t e = base + lane;
-    uint32_t c = e < experts ? lds_counts[e] : 0;
-    uint32_t inclusive = c;
+  // Exclusive scans over the experts of the route counts (-> offsets) and of the tile counts
+  // (-> first row block of each expert): one expert per thread per round, wave scans stitched
+  // through LDS.
+  uint32_t running = 0, block_running = 0;
+  for (uint32_t base = 0; base < experts; base += kPackThreads) {
+    const uint32_t e = base + tid;
+    const uint32_t c = e < experts ? lds_counts[e] : 0;
+    const uint32_t tiles = (c + tile_rows - 1) / tile_rows;
+    uint32_t inclusive = c, inclusive_tiles = tiles;
     for (int offset = 1; offset < 64; offset <<= 1) {
-      uint32_t other = __shfl_up(inclusive, offset, 64);
-      if ((int)lane >= offset) inclusive += other;
+      const uint32_t other = __shfl_up(inclusive, offset, 64);
+      const uint32_t other_tiles = __shfl_up(inclusive_tiles, offset, 64);
+      if ((int)lane >= offset) {
+        inclusive += other;
+        inclusive_tiles += other_tiles;
+      }
     }
-    uint32_t exclusive = running + inclusive - c;
+    if (lane == 63) {
+      scan[wave] = inclusive;
+      scan[kPackWaves + 1 + wave] = inclusive_tiles;
+    }
+    __syncthreads();
+    uint32_t before = running, before_tiles = block_running, total = 0, total_tiles = 0;
+    for (uint32_t w = 0; w < kPackWaves; ++w) {
+      if (w < wave) {
+        before += scan[w];
+        before_tiles += scan[kPackWaves + 1 + w];
+      }
+      total += scan[w];
+      total_tiles += scan[kPackWaves + 1 + w];
+    }
     if (e < experts) {
+      const uint32_t start = before + inclusive - c;
       counts[e] = c;
-      offsets[e] = exclusive;
-      lds_cursor[e] = exclusive;
-    }
-    running += __shfl(inclusive, 63, 64);
-  }
-  if (lane == 0) offsets[experts] = running;
-  __syncthreads();
-  // Stable arrange: within a round, a route's rank is the number of lower lanes naming the same
-  // expert; rounds run in ascending route order.
-  for (uint32_t base = 0; base < routes; base += 64) {
-    uint32_t route = base + lane;
-    uint32_t expert = 0xffffffffu;
-    if (route < routes)
-      expert = load_u32_at(indices, indices.offset + (uint64_t)(route / k) * indices.stride[0] +
-                                        (uint64_t)(route % k) * indices.stride[1]);
-    bool valid = route < routes && expert < experts;
-    unsigned long long same = __ballot(valid);
-    for (uint32_t bit = 0; (experts - 1) >> bit; ++bit) {
-      unsigned long long set = __ballot(valid && ((expert >> bit) & 1u));
-      same &= ((expert >> bit) & 1u) ? set : ~set;
-    }
-    uint32_t rank = __popcll(same & ((1ull << lane) - 1ull));
-    uint32_t group = __popcll(same);
-    uint32_t position = 0;
-    if (valid) position = lds_cursor[expert] + rank;
-    __syncthreads();
-    if (valid) {
-      sorted_routes[position] = route;
-      if (rank + 1 == group) lds_cursor[expert] = position + 1;
-    }
-    __syncthreads();
-  }
-  // Row blocks in ascending (expert, start) order.
-  uint32_t block_running = 0;
-  for (uint32_t base = 0; base < experts; base += 64) {
-    uint32_t e = base + lane;
-    uint32_t c = e < experts ? lds_counts[e] : 0;
-    uint32_t tiles = (c + tile_rows - 1) / tile_rows;
-    uint32_t inclusive = tiles;
-    for (int offset = 1; offset < 64; offset <<= 1) {
-      uint32_t other = __shfl_up(inclusive, offset, 64);
-      if ((int)lane >= offset) inclusive += other;
-    }
-    uint32_t first = block_running + inclusive - tiles;
-    if (e < experts) {
-      uint32_t start = lds_cursor[e] - c;  // cursor now sits at the end of the expert's span
+      offsets[e] = start;
+      lds_cursor[e] = start;
+      const uint32_t first = before_tiles + inclusive_tiles - tiles;
       for (uint32_t t = 0; t < tiles; ++t) {
-        uint32_t b = first + t;
+        const uint32_t b = first + t;
         if (b >= max_blocks) break;
-        uint32_t remaining = c - t * tile_rows;
+        const uint32_t remaining = c - t * tile_rows;
         blocks[3 * b + 0] = e;
         blocks[3 * b + 1] = start + t * tile_rows;
         blocks[3 * b + 2] = remaining < tile_rows ? remaining : tile_rows;
       }
     }
-    block_running += __shfl(inclusive, 63, 64);
+    running += total;
+    block_running += total_tiles;
+    __syncthreads();
   }
-  if (lane == 0) n_blocks[0] = block_running < max_blocks ? block_running : max_blocks;
-  for (uint32_t b = block_running + lane; b < max_blocks; b += 64) {
+  if (tid == 0) {
+    offsets[experts] = running;
+    n_blocks[0] = block_running < max_blocks ? block_running : max_blocks;
+  }
+  for (uint32_t b = block_running + tid; b < max_blocks; b += kPackThreads) {
     blocks[3 * b + 0] = 0xffffffffu;
     blocks[3 * b + 1] = 0;
     blocks[3 * b + 2] = 0;
+  }
+  // Stable arrange, 1024 routes per round in ascending route order: a route's position is its
+  // expert's cursor + the routes of the same expert in lower waves of the round + its rank among
+  // the lower lanes of its own wave.
+  for (uint32_t base = 0; base < routes; base += kPackThreads) {
+    const uint32_t route = base + tid;
+    for (uint32_t i = tid; i < kPackWaves * experts; i += kPackThreads) wave_counts[i] = 0;
+    uint32_t expert = 0xffffffffu;
+    if (route < routes) expert = base == 0 ? first_expert : expert_of(route);
+    const bool valid = route < routes && expert < experts;
+    unsigned long long same = __ballot(valid);
+    for (uint32_t bit = 0; (experts - 1) >> bit; ++bit) {
+      const unsigned long long set = __ballot(valid && ((expert >> bit) & 1u));
+      same &= ((expert >> bit) & 1u) ? set : ~set;
+    }
+    const uint32_t rank = __popcll(same & ((1ull << lane) - 1ull));
+    __syncthreads();  // wave_counts cleared
+    if (valid && rank == 0) wave_counts[wave * experts + expert] = __popcll(same);
+    __syncthreads();
+    if (valid) {
+      uint32_t position = lds_cursor[expert] + rank;
+      for (uint32_t w = 0; w < wave; ++w) position += wave_counts[w * experts + expert];
+      sorted_routes[position] = route;
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < experts; e += kPackThreads) {
+      uint32_t added = 0;
+      for (uint32_t w = 0; w < kPackWaves; ++w) added += wave_counts[w * experts + e];
+      lds_cursor[e] += added;
+    }
+    __syncthreads();
   }
 }
 
@@ -117,8 +141,8 @@ void launch_route_pack(hipStream_t s, const View &indices, uint32_t rows, uint32
                        uint32_t experts, uint32_t tile_rows, uint32_t *counts, uint32_t *offsets,
                        uint32_t *sorted_routes, uint32_t *blocks, uint32_t max_blocks,
                        uint32_t *n_blocks, ErrorSlot *error) {
-  size_t lds = (size_t)experts * 2 * sizeof(uint32_t);
-  route_pack_kernel<<<dim3(1), 64, lds, s>>>(indices, rows, k, experts, tile_rows, counts, offsets,
+  size_t lds = ((size_t)experts * (2 + kPackWaves) + 2 * (kPackWaves + 1)) * sizeof(uint32_t);
+  route_pack_kernel<<<dim3(1), kPackThreads, lds, s>>>(indices, rows, k, experts, tile_rows, counts, offsets,
                                              sorted_routes, blocks, max_blocks, n_blocks, error);
 }
 

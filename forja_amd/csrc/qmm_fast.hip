@@ -679,7 +679,8 @@ struct RoutePlan {
   char *rest;  // workspace after the plan
 };
 
-// Packs the routes on the device into `extra` + plan bytes of workspace.
+// Packs the routes on the device (or reuses the plan the previous routed projection packed from
+// the same indices); `extra` bytes of ordinary workspace are returned in plan->rest.
 bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, ErrorSlot *error,
                  RoutePlan *plan) {
   uint64_t routes = (uint64_t)p.rows * p.k;
@@ -687,8 +688,16 @@ bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, Er
   auto round = [](uint64_t bytes) { return (bytes + 255) / 256 * 256; };
   uint64_t counts_b = round(p.experts * 4ull), offsets_b = round((p.experts + 1) * 4ull),
            sorted_b = round(routes * 4), blocks_b = round(plan->max_blocks * 12ull), nb_b = 256;
-  char *ws = backend_workspace(backend, counts_b + offsets_b + sorted_b + blocks_b + nb_b + extra);
+  RoutePlanKey key{p.indices_buffer, p.indices.offset, p.indices.stride[0], p.indices.stride[1],
+                   p.rows, p.k, p.experts, kRouteTile};
+  bool reuse = false;
+  char *ws = backend_route_plan(backend, key, counts_b + offsets_b + sorted_b + blocks_b + nb_b, &reuse);
   if (!ws) return false;
+  plan->rest = nullptr;
+  if (extra) {
+    plan->rest = backend_workspace(backend, extra);
+    if (!plan->rest) return false;
+  }
   plan->counts = (uint32_t *)ws;
   ws += counts_b;
   plan->offsets = (uint32_t *)ws;
@@ -698,11 +707,10 @@ bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, Er
   plan->blocks = (uint32_t *)ws;
   ws += blocks_b;
   plan->n_blocks = (uint32_t *)ws;
-  ws += nb_b;
-  plan->rest = ws;
-  launch_route_pack(backend_stream(backend), p.indices, p.rows, p.k, p.experts, kRouteTile,
-                    plan->counts, plan->offsets, plan->sorted_routes, plan->blocks,
-                    plan->max_blocks, plan->n_blocks, error);
+  if (!reuse)
+    launch_route_pack(backend_stream(backend), p.indices, p.rows, p.k, p.experts, kRouteTile,
+                      plan->counts, plan->offsets, plan->sorted_routes, plan->blocks,
+                      plan->max_blocks, plan->n_blocks, error);
   return true;
 }
 
@@ -711,7 +719,7 @@ bool gather_eligible(const GatherProblem &p, int projections) {
   for (int pj = 0; pj < projections; ++pj)
     if (!weights_eligible(p.packed[pj], p.scales[pj], p.biases[pj], 3, p.inner, p.bits, p.group))
       return false;
-  if ((uint64_t)p.rows * p.k > (1u << 24)) return false;
+  if ((uint64_t)p.rows * p.k > (1u << 24) || p.experts > 512) return false;
   return true;
 }
 

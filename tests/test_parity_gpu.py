@@ -264,10 +264,14 @@ def test_gather_with_an_unrecognised_epilogue_uses_the_interpreter(cpu, hip):
 
 
 @pytest.mark.parametrize("rows,k,experts,tile", [(256, 8, 128, 16), (128, 8, 128, 32), (7, 3, 5, 2),
-                                                (1, 1, 1, 1), (300, 8, 128, 32), (64, 2, 200, 8)])
+                                                (1, 1, 1, 1), (300, 8, 128, 32), (64, 2, 200, 8),
+                                                (100, 8, 512, 32), (333, 8, 3, 32)])
 def test_route_pack_is_bit_exact(cpu, hip, rows, k, experts, tile):
     rng = np.random.default_rng(rows * 31 + k)
     indices = rng.integers(0, experts, (rows, k)).astype(np.uint32)
+    if experts == 3:
+        indices[:] = 1      # every route names the same expert: one long run across rounds
+        indices[5, 2] = 0
 
     def build(backend):
         idx = upload(backend, indices, DType.U32)

@@ -404,6 +404,76 @@ __global__ void top_k_kernel(View in, View values, View indices, uint32_t rows, 
   }
 }
 
+// Rows of at most 64 * kPer values (router logits): the whole row is loaded once into registers
+// and the k selections run on registers only.  Same order and results as top_k_kernel.
+template <int kPer>
+__global__ void top_k_registers_kernel(View in, View values, View indices, uint32_t rows,
+                                       uint32_t width, uint32_t k, int normalize) {
+  __shared__ float selected[64 * kPer];
+  const uint32_t row = blockIdx.x, lane = threadIdx.x;
+  const uint64_t in_row = in.offset + (uint64_t)row * in.stride[0];
+  int32_t keys[kPer];
+  bool live[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const uint32_t index = lane + 64 * i;
+    live[i] = index < width;
+    keys[i] = live[i] ? total_key(load_float_at(in, in_row + (uint64_t)index * in.stride[1]))
+                      : (int32_t)0x80000000;
+  }
+  for (uint32_t slot = 0; slot < k; ++slot) {
+    Candidate best = {(int32_t)0x80000000, 0xffffffffu};
+    bool have = false;
+    int mine = -1;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      Candidate c = {keys[i], lane + 64 * i};
+      if (live[i] && (!have || before(c, best))) {
+        best = c;
+        have = true;
+        mine = i;
+      }
+    }
+    const uint32_t my_index = best.index;
+    for (int offset = 32; offset > 0; offset >>= 1) {
+      Candidate other;
+      other.key = __shfl_xor(best.key, offset, 64);
+      other.index = __shfl_xor(best.index, offset, 64);
+      int other_have = __shfl_xor((int)have, offset, 64);
+      if (other_have && (!have || before(other, best))) {
+        best = other;
+        have = true;
+      }
+    }
+    // the owner retires the selected element
+#pragma unroll
+    for (int i = 0; i < kPer; ++i)
+      if (mine == i && my_index == best.index) live[i] = false;
+    if (lane == 0) {
+      const int32_t bits = best.key ^ (int32_t)(((uint32_t)(best.key >> 31)) >> 1);
+      selected[slot] = __uint_as_float((uint32_t)bits);
+      ((uint32_t *)indices.base)[indices.offset + (uint64_t)row * indices.stride[0] +
+                                 (uint64_t)slot * indices.stride[1]] = best.index;
+    }
+  }
+  if (lane == 0) {
+    if (normalize) {
+      float maximum = selected[0];
+      float sum = 0.0f;
+      for (uint32_t slot = 0; slot < k; ++slot) {
+        selected[slot] = expf(selected[slot] - maximum);
+        sum += selected[slot];
+      }
+      for (uint32_t slot = 0; slot < k; ++slot) selected[slot] /= sum;
+    }
+    for (uint32_t slot = 0; slot < k; ++slot)
+      store_float_at(values,
+                     values.offset + (uint64_t)row * values.stride[0] +
+                         (uint64_t)slot * values.stride[1],
+                     selected[slot]);
+  }
+}
+
 // Highest index among equal maxima under total order (lib.rs:530-539).
 __global__ void argmax_kernel(View in, View out, uint32_t rows, uint32_t width) {
   __shared__ int32_t keys[kBlock / 64];
@@ -847,6 +917,16 @@ void launch_gather_weighted_generic(hipStream_t s, const View &x, const View &pa
 void launch_top_k(hipStream_t s, const View &in, const View &values, const View &indices,
                   uint32_t rows, uint32_t width, uint32_t k, bool normalize) {
   if (rows == 0) return;
+  if (width <= 128) {
+    top_k_registers_kernel<2><<<dim3(rows), 64, 0, s>>>(in, values, indices, rows, width, k,
+                                                        normalize ? 1 : 0);
+    return;
+  }
+  if (width <= 512) {
+    top_k_registers_kernel<8><<<dim3(rows), 64, 0, s>>>(in, values, indices, rows, width, k,
+                                                        normalize ? 1 : 0);
+    return;
+  }
   top_k_kernel<<<dim3(rows), 64, 0, s>>>(in, values, indices, rows, width, k, normalize ? 1 : 0);
 }
 

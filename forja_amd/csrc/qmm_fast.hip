@@ -71,12 +71,9 @@ __device__ inline bf16x8 unpack_word(uint32_t w) {
 }
 
 // MT = 32-row tiles per workgroup, KC = activation columns staged per pass.  The four waves of a
-// workgroup share the staged activations and either own 32 output columns each (kSplitK false)
-// or all work on the same 32 columns, each on a quarter of every staged pass, and add their
-// accumulators through LDS at the end (kSplitK true: narrow outputs, where column blocks alone
-// would leave most CUs idle and each block would crawl through all of K).
-template <int MT, bool kPair, bool kRouted, bool kSplitK>
-__global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
+// workgroup share the staged activations and own 32 output columns each.
+template <int MT, bool kPair, bool kRouted>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qmm_mfma_kernel(QmmArgs a) {
   constexpr int NW = kWaves;
   constexpr int kThreads = 64 * NW;
   constexpr int KC = 512 / MT;  // 33 KB of LDS either way: two workgroups per CU overlap staging
@@ -88,8 +85,7 @@ __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
 
   const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const uint32_t nl = lane & 31, h = lane >> 5;
-  const uint32_t column =
-      (kSplitK ? blockIdx.x : blockIdx.x * NW + wave) * kColsPerWave + nl;
+  const uint32_t column = (blockIdx.x * NW + wave) * kColsPerWave + nl;
   const uint32_t column_c = min(column, a.columns - 1);  // clamped for loads
 
   uint32_t expert = 0, count = 0, first = 0;
@@ -123,23 +119,24 @@ __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
       for (int j = 0; j < 16; ++j) acc[pj][mt][j] = 0.0f;
 
   // Two independent software pipelines hide memory latency:
-  //  * weights: a ring of four groups' packed words and affine parameters; a slot is reloaded
-  //    (four groups ahead) as soon as its group has been consumed - the weight stream does not
-  //    care about staging passes;
+  //  * weights: a ring of two quads of groups.  A quad is four consecutive groups = one whole
+  //    128-byte line of every weight row, requested with four back-to-back loads so that the
+  //    line is fetched from L2 exactly once whatever the L1 does; a slot is reloaded two quads
+  //    ahead as soon as it has been consumed - the weight stream does not care about staging
+  //    passes;
   //  * activations: the next pass's pieces are fetched into registers while the current pass is
   //    consumed from LDS.
-  // A wave consumes kGw groups of every staged pass.
-  constexpr int kGw = kSplitK ? kGroupsPerPass / NW : kGroupsPerPass;
-  const uint32_t total_groups = a.inner / kGroup;
-  const uint32_t passes = (a.inner + KC - 1) / KC;
-  uint4 wq[kP][4];
-  uint32_t sb[kP][4][2];
-  auto load_group = [&](int slot, uint32_t group) {
-    if (group >= total_groups) return;
+  const uint32_t total_quads = a.inner / (4 * kGroup);
+  uint4 wq[kP][2][4];
+  uint2 scale_q[kP][2], bias_q[kP][2];   // four bf16 each
+  auto load_quad = [&](int slot, uint32_t quad) {
+    const uint32_t qd = min(quad, total_quads - 1);  // unconditional: the tail reloads the last quad
     for (int pj = 0; pj < kP; ++pj) {
-      wq[pj][slot] = *(const uint4 *)(w_row[pj] + (uint64_t)group * 8);
-      sb[pj][slot][0] = s_row[pj][group];
-      sb[pj][slot][1] = b_row[pj][group];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        wq[pj][slot][i] = *(const uint4 *)(w_row[pj] + (uint64_t)(4 * qd + i) * 8);
+      scale_q[pj][slot] = *(const uint2 *)(s_row[pj] + 4 * qd);
+      bias_q[pj][slot] = *(const uint2 *)(b_row[pj] + 4 * qd);
     }
   };
   uint4 x_regs[kPieces];
@@ -190,94 +187,72 @@ __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
     __syncthreads();
     if (kc0 + KC < a.inner) fetch_pass(kc0 + KC);
   };
-  // One quantisation group: four MFMA steps per row tile, then the affine fix-up.
-  auto consume = [&](int slot, uint32_t group) {
-    const uint32_t gi = group % kGroupsPerPass;  // group index inside the staged pass
-    f32x16 part[kP][MT];
-    for (int pj = 0; pj < kP; ++pj)
-      for (int mt = 0; mt < MT; ++mt)
-        for (int j = 0; j < 16; ++j) part[pj][mt][j] = 0.0f;
+  // Two consecutive quantisation groups (members i0, i0+1 of ring slot `slot`; `group` is the
+  // first one's number): four MFMA steps per group and row tile on independent accumulation
+  // chains, the scales applied per group, and the bias term
+  // sum_g (bias_g - 16 scale_g) * xsum_g[row] as one f32 MFMA over the two groups (lane half h
+  // supplies group + h of both operands).
+  auto consume_pair = [&](int slot, int i0, uint32_t group) {
+    const uint32_t gi = group % kGroupsPerPass;  // index of the first group inside the staged pass
+    f32x16 part[2][kP][MT];
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      for (int pj = 0; pj < kP; ++pj)
+        for (int mt = 0; mt < MT; ++mt)
+          for (int j = 0; j < 16; ++j) part[q][pj][mt][j] = 0.0f;
 #pragma unroll
     for (int step = 0; step < 4; ++step) {
-      bf16x8 b_op[kP];
-      for (int pj = 0; pj < kP; ++pj) {
-        const uint32_t word = step == 0 ? wq[pj][slot].x
-                                        : (step == 1 ? wq[pj][slot].y
-                                                     : (step == 2 ? wq[pj][slot].z : wq[pj][slot].w));
-        b_op[pj] = unpack_word(word);
-      }
-      for (int mt = 0; mt < MT; ++mt) {
-        const uint4 a_raw = *(const uint4 *)(xs + (mt * 32 + nl) * kPitch +
-                                             (gi * kGroup + 32 * h + 8 * step) * 2);
-        const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
-        for (int pj = 0; pj < kP; ++pj)
-          part[pj][mt] =
-              __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op[pj], part[pj][mt], 0, 0, 0);
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        bf16x8 b_op[kP];
+        for (int pj = 0; pj < kP; ++pj) {
+          const uint4 w = wq[pj][slot][i0 + q];
+          b_op[pj] = unpack_word(step == 0 ? w.x : (step == 1 ? w.y : (step == 2 ? w.z : w.w)));
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const uint4 a_raw = *(const uint4 *)(xs + (mt * 32 + nl) * kPitch +
+                                               ((gi + q) * kGroup + 32 * h + 8 * step) * 2);
+          const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
+          for (int pj = 0; pj < kP; ++pj)
+            part[q][pj][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op[pj],
+                                                                      part[q][pj][mt], 0, 0, 0);
+        }
       }
     }
-    // affine fix-up for this group; row blocks beyond `count` are skipped
+#pragma unroll
     for (int pj = 0; pj < kP; ++pj) {
-      const float scale = bf16_bits_to_f32(sb[pj][slot][0]);
-      const float shift = bf16_bits_to_f32(sb[pj][slot][1]) - 16.0f * scale;
-      for (int mt = 0; mt < MT; ++mt)
-        for (int jq = 0; jq < 4; ++jq) {
-          if ((uint32_t)(mt * 32 + 8 * jq) >= count) continue;
-          const float4 sums = *(const float4 *)(xsum + gi * kRows + mt * 32 + 8 * jq + 4 * h);
-          acc[pj][mt][4 * jq + 0] += scale * part[pj][mt][4 * jq + 0] + shift * sums.x;
-          acc[pj][mt][4 * jq + 1] += scale * part[pj][mt][4 * jq + 1] + shift * sums.y;
-          acc[pj][mt][4 * jq + 2] += scale * part[pj][mt][4 * jq + 2] + shift * sums.z;
-          acc[pj][mt][4 * jq + 3] += scale * part[pj][mt][4 * jq + 3] + shift * sums.w;
-        }
+      const uint32_t scale_bits = i0 == 0 ? scale_q[pj][slot].x : scale_q[pj][slot].y;
+      const uint32_t bias_bits = i0 == 0 ? bias_q[pj][slot].x : bias_q[pj][slot].y;
+      const float scale0 = bf16_bits_to_f32(scale_bits & 0xffffu);
+      const float scale1 = bf16_bits_to_f32(scale_bits >> 16);
+      const float shift0 = bf16_bits_to_f32(bias_bits & 0xffffu) - 16.0f * scale0;
+      const float shift1 = bf16_bits_to_f32(bias_bits >> 16) - 16.0f * scale1;
+      const float shift = h ? shift1 : shift0;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          acc[pj][mt][j] += scale0 * part[0][pj][mt][j] + scale1 * part[1][pj][mt][j];
+        acc[pj][mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+            xsum[(gi + h) * kRows + mt * 32 + nl], shift, acc[pj][mt], 0, 0, 0);
+      }
     }
   };
   if (kRouted) __syncthreads();  // row_ids visible
   fetch_pass(0);
-  if (!kSplitK) {
-    // Weight ring of four groups, refilled four groups ahead, independent of the passes.
+  load_quad(0, 0);
+  load_quad(1, 1);
+  for (uint32_t q0 = 0; q0 < total_quads; q0 += 2) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) load_group(u, u);
-    for (uint32_t g0 = 0; g0 < total_groups; g0 += 4) {
-      if (g0 % kGroupsPerPass == 0) pass_switch(g0 / kGroupsPerPass);
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        consume(u, g0 + u);
-        load_group(u, g0 + u + 4);
-      }
+    for (int uq = 0; uq < 2; ++uq) {
+      const uint32_t quad = q0 + uq;
+      if (quad >= total_quads) break;
+      if ((uq * 4) % kGroupsPerPass == 0) pass_switch(quad * 4 / kGroupsPerPass);
+      consume_pair(uq, 0, 4 * quad);
+      consume_pair(uq, 2, 4 * quad + 2);
+      load_quad(uq, quad + 2);
     }
-  } else {
-    // This wave's kGw groups of each pass; the next pass's are loaded while these are consumed.
-    const uint32_t mine = wave * kGw;
-#pragma unroll
-    for (int j = 0; j < kGw; ++j) load_group(j, mine + j);
-    for (uint32_t pass = 0; pass < passes; ++pass) {
-      pass_switch(pass);
-#pragma unroll
-      for (int j = 0; j < kGw; ++j) {
-        const uint32_t group = pass * kGroupsPerPass + mine + j;
-        if (group < total_groups) consume(j, group);
-        load_group(j, group + kGroupsPerPass);
-      }
-    }
-  }
-  if (kSplitK) {
-    // ---- add the four waves' partial accumulators through LDS (reusing the staging area)
-    static_assert(!kSplitK || !kPair, "split-K is for single projections");
-    float *red = (float *)xs;
-    __syncthreads();
-    for (int mt = 0; mt < MT; ++mt)
-      for (int j = 0; j < 16; ++j) {
-        const uint32_t row = mt * 32 + 8 * (j / 4) + 4 * h + (j % 4);
-        red[(wave * kRows + row) * 32 + nl] = acc[0][mt][j];
-      }
-    __syncthreads();
-    if (wave != 0) return;
-    for (int mt = 0; mt < MT; ++mt)
-      for (int j = 0; j < 16; ++j) {
-        const uint32_t row = mt * 32 + 8 * (j / 4) + 4 * h + (j % 4);
-        float total = 0.0f;
-        for (int w = 0; w < NW; ++w) total += red[(w * kRows + row) * 32 + nl];
-        acc[0][mt][j] = total;
-      }
   }
   // ---- epilogue and store; lane (column nl, half h) holds rows 8*(j/4) + 4h + j%4 of each tile
   if (column >= a.columns) return;
@@ -297,6 +272,170 @@ __global__ __launch_bounds__(256) void qmm_mfma_kernel(QmmArgs a) {
       else
         ((uint16_t *)a.out)[at] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
     }
+}
+
+// ---- routed tiles with the whole K resident in LDS ------------------------------------------
+//
+// A route tile is at most 32 rows, so for K up to 2048 its activations (32 x K bf16, at most
+// 128 KB) fit the 160 KB of LDS whole.  A workgroup of eight waves stages the tile once (one
+// memory round trip, one barrier) and then every wave streams the packed weights of its own 32
+// output columns (both projections for the gate/up pair) with no further synchronisation, a quad
+// of groups (one 128-byte line per weight row) at a time, two quads ahead.
+template <bool kPair>
+__global__ __launch_bounds__(512) void qmm_routed_tile_kernel(QmmArgs a) {
+  constexpr int kTileWaves = 8, kTileThreads = 64 * kTileWaves, kRows = 32;
+  constexpr int kP = kPair ? 2 : 1;
+  extern __shared__ __attribute__((aligned(16))) unsigned char tile_lds[];
+  const uint32_t pitch = 2 * a.inner + 16;  // bytes per staged row
+  unsigned char *xs = tile_lds;
+  float *xsum = (float *)(tile_lds + kRows * pitch);      // [K/64][32]
+  uint32_t *row_ids = (uint32_t *)(xsum + (a.inner / kGroup) * kRows);
+
+  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint32_t nl = lane & 31, h = lane >> 5;
+  const uint32_t column = (blockIdx.x * kTileWaves + wave) * kColsPerWave + nl;
+  const uint32_t column_c = min(column, a.columns - 1);
+  if (blockIdx.y >= a.n_blocks[0]) return;
+  const uint32_t expert = a.blocks[3 * blockIdx.y];
+  if (expert == kNoBlock) return;
+  const uint32_t first = a.blocks[3 * blockIdx.y + 1], count = a.blocks[3 * blockIdx.y + 2];
+  if (tid < kRows) row_ids[tid] = tid < count ? a.sorted_routes[first + tid] : 0;
+
+  const uint32_t words_per_row = a.inner / 8, groups_per_row = a.inner / kGroup;
+  const uint32_t total_quads = a.inner / (4 * kGroup);
+  const uint32_t *w_row[kP];
+  const uint16_t *s_row[kP], *b_row[kP];
+  for (int pj = 0; pj < kP; ++pj) {
+    w_row[pj] = a.packed[pj] + expert * a.expert_words + (uint64_t)column_c * words_per_row + 4 * h;
+    s_row[pj] = a.scales[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
+    b_row[pj] = a.biases[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
+  }
+  uint4 wq[kP][2][4];
+  uint2 scale_q[kP][2], bias_q[kP][2];
+  auto load_quad = [&](int slot, uint32_t quad) {
+    const uint32_t qd = min(quad, total_quads - 1);  // unconditional: the tail reloads the last quad
+    for (int pj = 0; pj < kP; ++pj) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        wq[pj][slot][i] = *(const uint4 *)(w_row[pj] + (uint64_t)(4 * qd + i) * 8);
+      scale_q[pj][slot] = *(const uint2 *)(s_row[pj] + 4 * qd);
+      bias_q[pj][slot] = *(const uint2 *)(b_row[pj] + 4 * qd);
+    }
+  };
+  load_quad(0, 0);   // cold memory: request before anything else
+  load_quad(1, 1);
+  __syncthreads();   // row_ids visible
+  // ---- stage the tile: permuted inside each 8, with per-group row sums
+  const uint32_t pieces_per_row = a.inner / 8, pieces = kRows * pieces_per_row;
+  for (uint32_t base = 0; base < pieces; base += 8 * kTileThreads) {
+    uint4 x_regs[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t piece = base + tid + i * kTileThreads;
+      const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
+      x_regs[i] = make_uint4(0, 0, 0, 0);
+      if (piece < pieces && row < count)
+        x_regs[i] = *(const uint4 *)(a.x + (uint64_t)(row_ids[row] / a.route_div) * a.x_row_stride + 8 * pc);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t piece = base + tid + i * kTileThreads;
+      const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
+      const uint4 v = x_regs[i];
+      float sum = bf16_bits_to_f32(v.x & 0xffffu) + bf16_bits_to_f32(v.x >> 16) +
+                  bf16_bits_to_f32(v.y & 0xffffu) + bf16_bits_to_f32(v.y >> 16) +
+                  bf16_bits_to_f32(v.z & 0xffffu) + bf16_bits_to_f32(v.z >> 16) +
+                  bf16_bits_to_f32(v.w & 0xffffu) + bf16_bits_to_f32(v.w >> 16);
+      sum += __shfl_xor(sum, 1, 64);   // eight consecutive pieces (= lanes) make one group
+      sum += __shfl_xor(sum, 2, 64);
+      sum += __shfl_xor(sum, 4, 64);
+      if (piece < pieces) {
+        uint4 permuted;
+        permuted.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
+        permuted.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
+        permuted.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+        permuted.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+        *(uint4 *)(xs + row * pitch + pc * 16) = permuted;
+        if ((pc & 7) == 0) xsum[(pc >> 3) * kRows + row] = sum;
+      }
+    }
+  }
+  __syncthreads();
+
+  f32x16 acc[kP];
+  for (int pj = 0; pj < kP; ++pj)
+    for (int j = 0; j < 16; ++j) acc[pj][j] = 0.0f;
+  const unsigned char *my_row = xs + nl * pitch + 64 * h;
+  // Two consecutive groups (members i0, i0+1 of ring slot `slot`): independent accumulation
+  // chains per group and projection, scales applied per group, bias term as one f32 MFMA over
+  // the two groups (lane half h supplies group + h of both operands).
+  auto consume_pair = [&](int slot, int i0, uint32_t group) {
+    f32x16 part[2][kP];
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      for (int pj = 0; pj < kP; ++pj)
+        for (int j = 0; j < 16; ++j) part[q][pj][j] = 0.0f;
+#pragma unroll
+    for (int step = 0; step < 4; ++step)
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const uint4 a_raw = *(const uint4 *)(my_row + (group + q) * (2 * kGroup) + 16 * step);
+        const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
+#pragma unroll
+        for (int pj = 0; pj < kP; ++pj) {
+          const uint4 w = wq[pj][slot][i0 + q];
+          const bf16x8 b_op =
+              unpack_word(step == 0 ? w.x : (step == 1 ? w.y : (step == 2 ? w.z : w.w)));
+          part[q][pj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op, part[q][pj], 0, 0, 0);
+        }
+      }
+#pragma unroll
+    for (int pj = 0; pj < kP; ++pj) {
+      const uint32_t scale_bits = i0 == 0 ? scale_q[pj][slot].x : scale_q[pj][slot].y;
+      const uint32_t bias_bits = i0 == 0 ? bias_q[pj][slot].x : bias_q[pj][slot].y;
+      const float scale0 = bf16_bits_to_f32(scale_bits & 0xffffu);
+      const float scale1 = bf16_bits_to_f32(scale_bits >> 16);
+      const float shift0 = bf16_bits_to_f32(bias_bits & 0xffffu) - 16.0f * scale0;
+      const float shift1 = bf16_bits_to_f32(bias_bits >> 16) - 16.0f * scale1;
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        acc[pj][j] += scale0 * part[0][pj][j] + scale1 * part[1][pj][j];
+      acc[pj] = __builtin_amdgcn_mfma_f32_32x32x2f32(xsum[(group + h) * kRows + nl],
+                                                     h ? shift1 : shift0, acc[pj], 0, 0, 0);
+    }
+  };
+  for (uint32_t q0 = 0; q0 < total_quads; q0 += 2) {
+#pragma unroll
+    for (int uq = 0; uq < 2; ++uq) {
+      const uint32_t quad = q0 + uq;
+      if (quad >= total_quads) break;
+      consume_pair(uq, 0, 4 * quad);
+      consume_pair(uq, 2, 4 * quad + 2);
+      load_quad(uq, quad + 2);
+    }
+  }
+  // ---- epilogue and store; lane (column nl, half h) holds rows 8*(j/4) + 4h + j%4
+  if (column >= a.columns) return;
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t row = 8 * (j / 4) + 4 * h + (j % 4);
+    if (row >= count) continue;
+    float value = acc[0][j];
+    if (kPair) {
+      const float gate = value, up = acc[kP - 1][j];
+      value = gate * (1.0f / (1.0f + __expf(-gate))) * up;
+    }
+    const uint64_t at = (uint64_t)row_ids[row] * a.out_row_stride + column;
+    if (a.out_f32)
+      ((float *)a.out)[at] = value;
+    else
+      ((uint16_t *)a.out)[at] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+  }
+}
+
+constexpr uint32_t kTileMaxInner = 2048;   // 32 x 2048 bf16 + sums = 133 KB of the 160 KB of LDS
+
+inline uint32_t routed_tile_lds_bytes(uint32_t inner) {
+  return 32 * (2 * inner + 16) + (inner / kGroup) * 32 * 4 + 32 * 4;
 }
 
 // ---- decode-sized dense products: at most 128 activation rows -------------------------------
@@ -564,25 +703,18 @@ bool weights_eligible(const View &packed, const View &scales, const View &biases
       !rows_contiguous(biases, rank))
     return false;
   if (packed.offset % 4 != 0) return false;  // 16-byte aligned rows (K/8 words is a multiple of 32)
+  if (scales.offset % 4 != 0 || biases.offset % 4 != 0) return false;  // 8-byte aligned quads
   return true;
 }
 
 template <bool kPair, bool kRouted>
 void launch_qmm(hipStream_t stream, const QmmArgs &a, uint32_t row_blocks, int mt) {
   uint32_t wide_blocks = (a.columns + kWaves * kColsPerWave - 1) / (kWaves * kColsPerWave);
-  if (!kPair && !kRouted && (uint64_t)wide_blocks * row_blocks < 256) {
-    dim3 grid((a.columns + kColsPerWave - 1) / kColsPerWave, row_blocks);
-    if (mt == 1)
-      qmm_mfma_kernel<1, false, false, true><<<grid, 256, 0, stream>>>(a);
-    else
-      qmm_mfma_kernel<2, false, false, true><<<grid, 256, 0, stream>>>(a);
-    return;
-  }
   dim3 grid(wide_blocks, row_blocks);
   if (mt == 1)
-    qmm_mfma_kernel<1, kPair, kRouted, false><<<grid, 256, 0, stream>>>(a);
+    qmm_mfma_kernel<1, kPair, kRouted><<<grid, 256, 0, stream>>>(a);
   else
-    qmm_mfma_kernel<2, kPair, kRouted, false><<<grid, 256, 0, stream>>>(a);
+    qmm_mfma_kernel<2, kPair, kRouted><<<grid, 256, 0, stream>>>(a);
 }
 
 // Decode-sized dense product through the slab kernels; false when workspace is short.
@@ -714,6 +846,25 @@ bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, Er
   return true;
 }
 
+// Routed product over the packed tiles: whole-K tile kernel when the tile fits LDS, else the
+// multi-pass kernel.
+template <bool kPair>
+void launch_routed(hipStream_t stream, const QmmArgs &a, uint32_t max_blocks) {
+  if (a.inner <= kTileMaxInner) {
+    static bool configured = false;   // raise the dynamic LDS limit once per process
+    if (!configured) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_routed_tile_kernel<kPair>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)routed_tile_lds_bytes(kTileMaxInner));
+      configured = true;
+    }
+    dim3 grid((a.columns + 8 * kColsPerWave - 1) / (8 * kColsPerWave), max_blocks);
+    qmm_routed_tile_kernel<kPair><<<grid, 512, routed_tile_lds_bytes(a.inner), stream>>>(a);
+    return;
+  }
+  launch_qmm<kPair, true>(stream, a, max_blocks, 1);
+}
+
 bool gather_eligible(const GatherProblem &p, int projections) {
   if (p.x.dtype != FH_BF16) return false;
   for (int pj = 0; pj < projections; ++pj)
@@ -763,9 +914,9 @@ bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int
   a.route_div = p.k;
   KernelTimer timer(backend, FH_KC_MOE_KERNEL);
   if (projections == 2)
-    launch_qmm<true, true>(stream, a, plan.max_blocks, 1);
+    launch_routed<true>(stream, a, plan.max_blocks);
   else
-    launch_qmm<false, true>(stream, a, plan.max_blocks, 1);
+    launch_routed<false>(stream, a, plan.max_blocks);
   return true;
 }
 
@@ -801,7 +952,7 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
   a.route_div = 1;
   {
     KernelTimer timer(backend, FH_KC_MOE_KERNEL);
-    launch_qmm<false, true>(stream, a, plan.max_blocks, 1);
+    launch_routed<false>(stream, a, plan.max_blocks);
   }
   uint64_t work = (uint64_t)p.rows * p.columns;
   View none{};

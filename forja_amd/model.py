@@ -380,8 +380,8 @@ class DecodeSession:
         backend.write(b.q_starts, self.contexts.astype(np.uint32).tobytes())
         backend.write(b.positions, self.contexts.astype(np.float32).tobytes())
 
-    def submit_step(self):
-        """Uploads this step's metadata and enqueues the step; returns the submission."""
+    def prepare_step(self):
+        """Makes room for this step's token in every lane and uploads the step's metadata."""
         grown = []
         for lane in range(len(self.contexts)):
             before = len(self.cache.lane_pages[lane])
@@ -391,6 +391,10 @@ class DecodeSession:
         if grown:
             self.cache.upload_tables(grown)
         self.upload_positions()
+
+    def submit_step(self):
+        """Uploads this step's metadata and enqueues the step; returns the submission."""
+        self.prepare_step()
         submission = self.model.backend.submit(self.encoded)
         self.contexts += 1
         return submission

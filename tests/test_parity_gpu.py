@@ -303,7 +303,8 @@ def test_route_pack_skips_bad_routes_and_reports_the_lowest(cpu, hip):
 
 # ------------------------------------------------------------------ selection
 
-@pytest.mark.parametrize("width,k", [(1, 1), (64, 8), (128, 8), (2050, 64)])
+@pytest.mark.parametrize("width,k", [(1, 1), (64, 8), (100, 8), (128, 8), (300, 16), (512, 64),
+                                     (2050, 64)])
 def test_top_k_edge_widths_ties_and_nans(cpu, hip, width, k):
     values = top_k_case(width)
 

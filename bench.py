@@ -178,6 +178,57 @@ def moe_block_c2(backend, model, tokens=256, seed=77):
     }
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def prefill_gemm_c4(backend, rows=8256, seed=91, repeats=3):
+    """The quantised projections of one BASELINE config 4 layer (dense 27B-class shape) over the
+    8192-token prefill chunk plus its 64 decode rows: stacked qkv, o, stacked gate/up, down.
+    Each product runs `repeats` times after one warm-up; device time from HIP events around the
+    kernels."""
+    from forja_amd.model import DENSE_27B, QuantLinear
+    c = DENSE_27B
+    qkv_width = (c.q_heads + 2 * c.kv_heads) * c.head_dim
+    shapes = [("qkv", qkv_width, c.hidden), ("o_proj", c.hidden, c.q_heads * c.head_dim),
+              ("gate_up", 2 * c.intermediate, c.hidden), ("down", c.hidden, c.intermediate)]
+    products, total_flops, total_ns = {}, 0.0, 0.0
+    for index, (name, n, k) in enumerate(shapes):
+        linear = QuantLinear(backend, n, k)
+        x = backend.alloc(DType.BF16, (rows, k))
+        out = backend.alloc(DType.BF16, (rows, n))
+        fill = CommandList()
+        linear.fill(fill, seed, 10 * index)
+        fill.dispatch(Op.fill_seeded(2, seed, 10 * index + 5), [], x)
+        backend.submit(fill).wait()
+        commands = CommandList()
+        commands.dispatch(Op.quant_matmul(4, 64), [x, *linear.triple], out)
+        encoded = backend.encode(commands)
+        backend.submit(encoded).wait()
+        backend.profile_enable(1)
+        backend.profile_reset()
+        for _ in range(repeats):
+            backend.submit(encoded).wait()
+        ns, launches = backend.profile_read(KC_QMM_KERNEL)
+        backend.profile_enable(0)
+        flops = 2.0 * rows * n * k
+        per_launch = ns / max(launches, 1)
+        products[name] = {"n": n, "k": k, "us": per_launch / 1e3,
+                          "tflops": flops / (per_launch * 1e-9) / 1e12 if per_launch else 0.0}
+        total_flops += flops
+        total_ns += per_launch
+        for tensor in (x, out, *linear.triple):
+            backend.release(tensor)
+    achieved = total_flops / (total_ns * 1e-9) / 1e12 if total_ns else 0.0
+    return {
+        "workload": (f"BASELINE config 4 layer projections: {rows} rows (8192-token prefill chunk + "
+                     f"64 decode rows), hidden {c.hidden}, intermediate {c.intermediate}, MLX-4bit"),
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "kernel": "qmm_gemm_kernel"},
+        "ms_per_layer_projections": total_ns / 1e6, "products": products,
+    }
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -190,6 +241,8 @@ def main():
     parser.add_argument("--cpu-sample-lanes", type=int, default=8)
     parser.add_argument("--no-profile", action="store_true",
                         help="skip the HIP-event kernel timing inside the timed region")
+    parser.add_argument("--prefill-only", action="store_true",
+                        help="only run the config 4 prefill projection measurement and exit")
     parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                         help="only run 8 plain copies of MIB mebibytes (a known-size kernel to "
                              "scale hardware traffic counters by) and exit")
@@ -205,6 +258,9 @@ def main():
             backend.submit(commands).wait()
         print(json.dumps({"copy_bytes_read": elements * 4, "copy_bytes_written": elements * 4,
                           "kernel": "copy_kernel", "launches": 8}))
+        return
+    if args.prefill_only:
+        print(json.dumps(prefill_gemm_c4(HipBackend(0))))
         return
     if args.gpus != 1:
         print("bench.py: this build runs the ragged forward step on ONE MI355X; collectives and "
@@ -331,8 +387,9 @@ def main():
             breakdown[name] = class_ns / 1e6 / extra
         result["gpu_ms_per_step_by_op"] = breakdown
         backend.profile_enable(0)
+        result["secondary_workloads"] = {"prefill_gemm_c4": prefill_gemm_c4(backend)}
         if config.moe:
-            result["secondary_workloads"] = {"moe_block_c2": moe_block_c2(backend, workload.model)}
+            result["secondary_workloads"]["moe_block_c2"] = moe_block_c2(backend, workload.model)
     step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction
     result["step_algorithmic_gb"] = step_bytes / 1e9
     result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS

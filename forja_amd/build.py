@@ -8,7 +8,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libforja_hip.so")
 CONFORMANCE = os.path.join(HERE, "host", "conformance")
 
-SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "programs_fast.hip"]
+SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "qmm_gemm.hip", "programs_fast.hip"]
 
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

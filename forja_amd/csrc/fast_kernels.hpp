@@ -44,6 +44,9 @@ struct QmmProblem {
   uint32_t rows, inner, columns, bits, group;
 };
 bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &problem);
+// Tiled GEMM with weights dequantised into LDS, for many rows; operands as checked by
+// try_fast_quant_matmul.  False when the launch could not be configured.
+bool launch_quant_gemm(fh_backend *backend, const QmmProblem &problem);
 
 struct GatherProblem {
   View x;           // projection: [R,K]; weighted sum: [R,k,K]

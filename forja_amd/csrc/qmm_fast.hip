@@ -794,6 +794,7 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
     if (!launch_skinny(backend, a)) return false;
     return true;
   }
+  if (p.rows > 128 && launch_quant_gemm(backend, p)) return true;
   int mt = p.rows <= 32 ? 1 : 2;
   uint32_t row_blocks = (p.rows + 32 * mt - 1) / (32 * mt);
   KernelTimer timer(backend, FH_KC_QMM_KERNEL);

@@ -1,0 +1,292 @@
+// MLX-4bit quantised matmul for many activation rows (prefill chunks): a tiled f16 MFMA GEMM
+// whose weight tiles are dequantised on their way into LDS.
+//
+// y[m,n] = sum_k x[m,k] * (scale[n,k/64] * q[n,k] + bias[n,k/64])   (affine_quant_dot,
+// crates/forja-cpu/src/lib.rs:1277-1310).  With hundreds of rows per weight the work is bound by
+// the matrix cores, not by HBM, so the kernel is a classic GEMM:
+//   * operands are fp16, not bf16: a dequantised weight scale*q+bias rounded to bf16 (8
+//     significant bits) is too coarse for the stated tolerance on outputs that cancel, fp16 (11
+//     bits) is not, and the matrix cores run both at the same rate.  bf16 activations convert to
+//     fp16 exactly; prepare_rows_kernel does that once per product (scaling a row by a power of
+//     two first if it holds values beyond the fp16 range, undone exactly in the epilogue) and
+//     stores every 8 values in the order (0,4,1,5,2,6,3,7) in which nibbles unpack pairwise;
+//   * workgroup tile 256 rows x 256 columns, K step 64 (one quantisation group); four waves in
+//     a 2 x 2 arrangement, each owning 128 x 128 outputs = 16 accumulator tiles of
+//     v_mfma_f32_32x32x16_f16 (256 accumulator registers);
+//   * both operand tiles live in LDS, double buffered (2 x 2 x 36 KB of the 160 KB), rows padded
+//     to 144 bytes so that the 16-byte operand reads are bank-conflict free; the next K step is
+//     fetched into registers while the current one is multiplied, then stored, one barrier per
+//     step;
+//   * a thread dequantises one weight row of the tile per step (64 nibbles): two nibbles become
+//     the fp16 pair (1024+q) with one and-or, minus 1024 exactly, then one packed fused
+//     multiply-add gives scale*q+bias rounded once; scales outside the fp16 normal range take an
+//     f32 path.  Every weight byte is read from HBM once per 256 rows and unpacked once per
+//     workgroup;
+//   * the workgroup -> tile map walks all row tiles of a column tile before moving on and keeps
+//     the walk of one XCD contiguous, so a weight tile is fetched into that XCD's L2 once.
+// Accumulation is f32.
+#include "fast_kernels.hpp"
+
+namespace fh {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int kBM = 256, kBN = 256, kBK = 64;
+constexpr int kPitch = 2 * kBK + 16;              // bytes per staged row
+constexpr int kTileBytes = kBM * kPitch;          // one operand tile
+constexpr int kGemmLds = 4 * kTileBytes;          // A and B, double buffered
+
+struct GemmArgs {
+  const uint16_t *x;        // fp16 rows prepared by prepare_rows_kernel, stride = inner
+  const float *row_unscale; // per row: multiply the result by this
+  uint64_t x_row_stride;
+  const uint32_t *packed;
+  const uint16_t *scales, *biases;
+  void *out;
+  uint64_t out_row_stride;
+  uint32_t out_f32;
+  uint32_t rows, inner, columns;
+  uint32_t row_tiles, column_tiles;
+};
+
+__device__ inline uint32_t pack2(float lo, float hi) {
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ inline float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+__device__ inline uint32_t pack_f16(float lo, float hi) {
+  f16x2 v = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Eight nibbles of `w`, dequantised to fp16, as the four pairs (0,4)(1,5)(2,6)(3,7).
+// Fast form: (1024+q) pairs by and-or, minus 1024 (exact), then fused scale*q+bias per pair.
+__device__ inline uint4 dequantise_word(uint32_t w, f16x2 scale2, f16x2 bias2) {
+  const uint32_t mask = 0x000f000fu, magic = 0x64006400u;
+  const f16x2 offset = {(_Float16)1024.0f, (_Float16)1024.0f};
+  uint32_t raw[4] = {(w & mask) | magic, ((w >> 4) & mask) | magic, ((w >> 8) & mask) | magic,
+                     ((w >> 12) & mask) | magic};
+  uint32_t out[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const f16x2 q = __builtin_bit_cast(f16x2, raw[i]) - offset;
+    out[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(q, scale2, bias2));
+  }
+  return make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+// The same in f32 with one rounding to fp16, for scales or biases outside the fp16 normal range.
+__device__ inline uint4 dequantise_word_wide(uint32_t w, float scale, float bias) {
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(scale, (float)((w >> (4 * i)) & 15u), bias);
+  return make_uint4(pack_f16(v[0], v[4]), pack_f16(v[1], v[5]), pack_f16(v[2], v[6]),
+                    pack_f16(v[3], v[7]));
+}
+
+__device__ inline bool f16_exact(float value) {
+  const float magnitude = fabsf(value);
+  return magnitude == 0.0f || (magnitude >= 6.103515625e-05f && magnitude <= 4096.0f);
+}
+
+// x bf16 [rows, inner] -> fp16 [rows, inner] (every 8 values stored as 0,4,1,5,2,6,3,7), each row
+// multiplied by a power of two that brings its largest magnitude under 2^15; unscale[row] is the
+// inverse.  One wave per row.
+__global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, uint64_t x_row_stride,
+                                                           uint32_t rows, uint32_t inner,
+                                                           uint16_t *out, float *unscale) {
+  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const uint16_t *in_row = x + (uint64_t)row * x_row_stride;
+  uint32_t top = 0;   // largest magnitude bits (bf16 without sign) in the row
+  for (uint32_t piece = lane; piece < inner / 8; piece += 64) {
+    const uint4 v = *(const uint4 *)(in_row + 8 * piece);
+    const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t lo = words[i] & 0x7fffu, hi = (words[i] >> 16) & 0x7fffu;
+      // NaN and infinity (exponent 255) pass through the conversion unchanged; leave them out
+      if (lo < 0x7f80u) top = max(top, lo);
+      if (hi < 0x7f80u) top = max(top, hi);
+    }
+  }
+  for (int offset = 32; offset > 0; offset >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, offset, 64));
+  const int exponent = (int)(top >> 7) - 127;                    // floor(log2(max |x|))
+  const int down = exponent > 14 ? exponent - 14 : 0;            // scale by 2^-down
+  const float scale = __uint_as_float((uint32_t)(127 - down) << 23);
+  if (lane == 0) unscale[row] = __uint_as_float((uint32_t)(127 + down) << 23);
+  uint16_t *out_row = out + (uint64_t)row * inner;
+  for (uint32_t piece = lane; piece < inner / 8; piece += 64) {
+    const uint4 v = *(const uint4 *)(in_row + 8 * piece);
+    const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(words[i] << 16) * scale;
+      f[2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u) * scale;
+    }
+    *(uint4 *)(out_row + 8 * piece) = make_uint4(pack_f16(f[0], f[4]), pack_f16(f[1], f[5]),
+                                                 pack_f16(f[2], f[6]), pack_f16(f[3], f[7]));
+  }
+}
+
+__global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
+  unsigned char *a_tiles = gemm_lds;                    // [2][kBM][kPitch]
+  unsigned char *b_tiles = gemm_lds + 2 * kTileBytes;   // [2][kBN][kPitch]
+  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint32_t wm = wave >> 1, wn = wave & 1;
+  const uint32_t l32 = lane & 31, kh = lane >> 5;
+
+  // workgroup -> tile: workgroups are dealt round-robin to the 8 XCDs; give each XCD a
+  // contiguous run of tiles, column tile major
+  const uint32_t tiles = a.row_tiles * a.column_tiles;
+  const uint32_t per_xcd = (tiles + 7) / 8;
+  const uint32_t tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (tile >= tiles) return;
+  const uint32_t bn = tile / a.row_tiles, bm = tile % a.row_tiles;
+  const uint32_t row0 = bm * kBM, col0 = bn * kBN;
+
+  // staging assignments
+  const uint32_t a_piece = tid & 7, a_row = tid >> 3;   // rows a_row + 32 i, 16-byte piece
+  const uint32_t b_col = min(col0 + tid, a.columns - 1);
+  const uint32_t groups_per_row = a.inner / kBK;
+  const uint32_t *w_row = a.packed + (uint64_t)b_col * (a.inner / 8);
+  const uint16_t *s_row = a.scales + (uint64_t)b_col * groups_per_row;
+  const uint16_t *b_row = a.biases + (uint64_t)b_col * groups_per_row;
+
+  uint4 a_regs[8], w_regs[2];
+  uint32_t scale_bits, bias_bits;
+  auto fetch = [&](uint32_t step) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t row = row0 + a_row + 32 * i;
+      a_regs[i] = make_uint4(0, 0, 0, 0);
+      if (row < a.rows)
+        a_regs[i] = *(const uint4 *)(a.x + (uint64_t)row * a.x_row_stride + step * kBK + 8 * a_piece);
+    }
+    w_regs[0] = *(const uint4 *)(w_row + step * 8);
+    w_regs[1] = *(const uint4 *)(w_row + step * 8 + 4);
+    scale_bits = s_row[step];
+    bias_bits = b_row[step];
+  };
+  auto stage = [&](uint32_t buffer) {
+    unsigned char *at = a_tiles + buffer * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      *(uint4 *)(at + (a_row + 32 * i) * kPitch + 16 * a_piece) = a_regs[i];
+    unsigned char *bt = b_tiles + buffer * kTileBytes + tid * kPitch;
+    const float scale = bf16_bits_to_f32(scale_bits), bias = bf16_bits_to_f32(bias_bits);
+    const uint32_t words[8] = {w_regs[0].x, w_regs[0].y, w_regs[0].z, w_regs[0].w,
+                               w_regs[1].x, w_regs[1].y, w_regs[1].z, w_regs[1].w};
+    if (f16_exact(scale) && f16_exact(bias)) {
+      const f16x2 scale2 = {(_Float16)scale, (_Float16)scale}, bias2 = {(_Float16)bias, (_Float16)bias};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) *(uint4 *)(bt + 16 * i) = dequantise_word(words[i], scale2, bias2);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) *(uint4 *)(bt + 16 * i) = dequantise_word_wide(words[i], scale, bias);
+    }
+  };
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const uint32_t steps = a.inner / kBK;
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  for (uint32_t step = 0; step < steps; ++step) {
+    const uint32_t buffer = step & 1;
+    if (step + 1 < steps) fetch(step + 1);
+    const unsigned char *at = a_tiles + buffer * kTileBytes + (128 * wm + l32) * kPitch + 16 * kh;
+    const unsigned char *bt = b_tiles + buffer * kTileBytes + (128 * wn + l32) * kPitch + 16 * kh;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      f16x8 a_op[4], b_op[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * kPitch + 32 * s));
+        b_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kPitch + 32 * s));
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
+    }
+    if (step + 1 < steps) stage(buffer ^ 1);
+    __syncthreads();
+  }
+  // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t column = col0 + 128 * wn + 32 * j + l32;
+      if (column >= a.columns) continue;
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = row0 + 128 * wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+        if (row >= a.rows) continue;
+        const uint64_t at_out = (uint64_t)row * a.out_row_stride + column;
+        const float value = acc[i][j][r] * a.row_unscale[row];
+        if (a.out_f32)
+          ((float *)a.out)[at_out] = value;
+        else
+          ((uint16_t *)a.out)[at_out] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+      }
+    }
+}
+
+}  // namespace
+
+bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
+  const uint64_t rows_bytes = ((uint64_t)p.rows * p.inner * 2 + 255) / 256 * 256;
+  char *ws = backend_workspace(backend, rows_bytes + (uint64_t)p.rows * sizeof(float));
+  if (!ws) return false;
+  hipStream_t stream = backend_stream(backend);
+  GemmArgs a{};
+  a.x = (const uint16_t *)ws;
+  a.row_unscale = (const float *)(ws + rows_bytes);
+  a.x_row_stride = p.inner;
+  a.packed = (const uint32_t *)p.packed.base + p.packed.offset;
+  a.scales = (const uint16_t *)p.scales.base + p.scales.offset;
+  a.biases = (const uint16_t *)p.biases.base + p.biases.offset;
+  a.out = p.out.dtype == FH_F32 ? (void *)((float *)p.out.base + p.out.offset)
+                                : (void *)((uint16_t *)p.out.base + p.out.offset);
+  a.out_row_stride = p.out.stride[0];
+  a.out_f32 = p.out.dtype == FH_F32;
+  a.rows = p.rows;
+  a.inner = p.inner;
+  a.columns = p.columns;
+  a.row_tiles = (p.rows + kBM - 1) / kBM;
+  a.column_tiles = (p.columns + kBN - 1) / kBN;
+  static bool configured = false;   // raise the dynamic LDS limit once per process
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_gemm_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds) != hipSuccess)
+      return false;
+    configured = true;
+  }
+  const uint32_t tiles = a.row_tiles * a.column_tiles;
+  const uint32_t grid = ((tiles + 7) / 8) * 8;
+  KernelTimer timer(backend, FH_KC_QMM_KERNEL);
+  prepare_rows_kernel<<<(p.rows + 3) / 4, 256, 0, stream>>>(
+      (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, (uint16_t *)ws,
+      (float *)(ws + rows_bytes));
+  qmm_gemm_kernel<<<grid, 256, kGemmLds, stream>>>(a);
+  return true;
+}
+
+}  // namespace fh

@@ -132,7 +132,10 @@ QMM_CASES = [
     (100, 130, 2048, 4, 64, DType.BF16),    # row and column tails, 8 splits
     (64, 96, 256, 4, 64, DType.BF16),       # a single group per wave, no split
     (65, 32, 3072, 4, 64, DType.BF16),      # 12 splits
-    (192, 4096, 2048, 4, 64, DType.BF16),   # more rows than the decode path takes
+    (192, 4096, 2048, 4, 64, DType.BF16),   # more rows than the decode path takes: tiled GEMM
+    (257, 300, 512, 4, 64, DType.BF16),     # GEMM with row and column tails
+    (1000, 96, 256, 4, 64, DType.BF16),     # GEMM, a single column tile, four row tiles
+    (512, 1024, 2048, 4, 64, DType.BF16),   # GEMM, whole tiles
 ]
 
 

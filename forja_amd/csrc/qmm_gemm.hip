@@ -13,10 +13,12 @@
 //   * workgroup tile 256 rows x 256 columns, K step 64 (one quantisation group); four waves in
 //     a 2 x 2 arrangement, each owning 128 x 128 outputs = 16 accumulator tiles of
 //     v_mfma_f32_32x32x16_f16 (256 accumulator registers);
-//   * both operand tiles live in LDS, double buffered (2 x 2 x 36 KB of the 160 KB), rows padded
-//     to 144 bytes so that the 16-byte operand reads are bank-conflict free; the next K step is
-//     fetched into registers while the current one is multiplied, then stored, one barrier per
-//     step;
+//   * both operand tiles live in LDS, double buffered.  The activation tile goes from memory
+//     straight into LDS (global_load_lds, no registers), its 16-byte pieces XOR-swizzled inside
+//     each 128-byte row so that operand reads are bank-conflict free without padding; the weight
+//     tile passes through registers to be dequantised and is stored in rows padded to 144 bytes.
+//     The next K step is staged while the current one is multiplied, one barrier per step;
+//     packed weights are requested two steps ahead (they are cold in HBM);
 //   * a thread dequantises one weight row of the tile per step (64 nibbles): two nibbles become
 //     the fp16 pair (1024+q) with one and-or, minus 1024 exactly, then one packed fused
 //     multiply-add gives scale*q+bias rounded once; scales outside the fp16 normal range take an
@@ -37,9 +39,10 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int kBM = 256, kBN = 256, kBK = 64;
-constexpr int kPitch = 2 * kBK + 16;              // bytes per staged row
-constexpr int kTileBytes = kBM * kPitch;          // one operand tile
-constexpr int kGemmLds = 4 * kTileBytes;          // A and B, double buffered
+constexpr int kPitch = 2 * kBK + 16;              // bytes per staged weight row
+constexpr int kATileBytes = kBM * 2 * kBK;        // activation tile, swizzled, no padding
+constexpr int kBTileBytes = kBN * kPitch;         // weight tile
+constexpr int kGemmLds = 2 * (kATileBytes + kBTileBytes);
 
 struct GemmArgs {
   const uint16_t *x;        // fp16 rows prepared by prepare_rows_kernel, stride = inner
@@ -139,8 +142,8 @@ __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, ui
 
 __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
-  unsigned char *a_tiles = gemm_lds;                    // [2][kBM][kPitch]
-  unsigned char *b_tiles = gemm_lds + 2 * kTileBytes;   // [2][kBN][kPitch]
+  unsigned char *a_tiles = gemm_lds;                      // [2][kBM][128], pieces swizzled
+  unsigned char *b_tiles = gemm_lds + 2 * kATileBytes;    // [2][kBN][kPitch]
   const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const uint32_t wm = wave >> 1, wn = wave & 1;
   const uint32_t l32 = lane & 31, kh = lane >> 5;
@@ -154,38 +157,43 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   const uint32_t bn = tile / a.row_tiles, bm = tile % a.row_tiles;
   const uint32_t row0 = bm * kBM, col0 = bn * kBN;
 
-  // staging assignments
-  const uint32_t a_piece = tid & 7, a_row = tid >> 3;   // rows a_row + 32 i, 16-byte piece
-  const uint32_t b_col = min(col0 + tid, a.columns - 1);
-  const uint32_t groups_per_row = a.inner / kBK;
-  const uint32_t *w_row = a.packed + (uint64_t)b_col * (a.inner / 8);
-  const uint16_t *s_row = a.scales + (uint64_t)b_col * groups_per_row;
-  const uint16_t *b_row = a.biases + (uint64_t)b_col * groups_per_row;
-
-  uint4 a_regs[8], w_regs[2];
-  uint32_t scale_bits, bias_bits;
-  auto fetch = [&](uint32_t step) {
+  // Activation staging: a wave owns 64 rows of the tile; one instruction moves 8 rows (lane ->
+  // row lane/8, LDS slot lane%8), and the piece a lane fetches is its slot XOR ((row >> 1) & 7).
+  const uint16_t *a_src[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t row = row0 + a_row + 32 * i;
-      a_regs[i] = make_uint4(0, 0, 0, 0);
-      if (row < a.rows)
-        a_regs[i] = *(const uint4 *)(a.x + (uint64_t)row * a.x_row_stride + step * kBK + 8 * a_piece);
-    }
-    w_regs[0] = *(const uint4 *)(w_row + step * 8);
-    w_regs[1] = *(const uint4 *)(w_row + step * 8 + 4);
-    scale_bits = s_row[step];
-    bias_bits = b_row[step];
-  };
-  auto stage = [&](uint32_t buffer) {
-    unsigned char *at = a_tiles + buffer * kTileBytes;
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t in_tile = 64 * wave + 8 * i + lane / 8;
+    const uint32_t row = min(row0 + in_tile, a.rows - 1);   // tail rows reload the last row; never stored
+    const uint32_t piece = (lane % 8) ^ ((in_tile >> 1) & 7);
+    a_src[i] = a.x + (uint64_t)row * a.x_row_stride + 8 * piece;
+  }
+  auto stage_a = [&](uint32_t buffer, uint32_t step) {
+    unsigned char *to = a_tiles + buffer * kATileBytes + 64 * wave * 128;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      *(uint4 *)(at + (a_row + 32 * i) * kPitch + 16 * a_piece) = a_regs[i];
-    unsigned char *bt = b_tiles + buffer * kTileBytes + tid * kPitch;
-    const float scale = bf16_bits_to_f32(scale_bits), bias = bf16_bits_to_f32(bias_bits);
-    const uint32_t words[8] = {w_regs[0].x, w_regs[0].y, w_regs[0].z, w_regs[0].w,
-                               w_regs[1].x, w_regs[1].y, w_regs[1].z, w_regs[1].w};
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void *)(a_src[i] + step * kBK),
+          (__attribute__((address_space(3))) void *)(to + 8 * i * 128), 16, 0, 0);
+  };
+  // Weight staging: thread t dequantises row t of the tile.
+  const uint32_t b_col = min(col0 + tid, a.columns - 1);
+  const uint32_t steps = a.inner / kBK;
+  const uint32_t *w_row = a.packed + (uint64_t)b_col * (a.inner / 8);
+  const uint16_t *s_row = a.scales + (uint64_t)b_col * steps;
+  const uint16_t *b_row = a.biases + (uint64_t)b_col * steps;
+  uint4 w_now[2], w_next[2];
+  uint32_t affine_now, affine_next;   // scale | bias << 16
+  auto fetch_w = [&](uint32_t step) {
+    const uint32_t st = min(step, steps - 1);
+    w_next[0] = *(const uint4 *)(w_row + st * 8);
+    w_next[1] = *(const uint4 *)(w_row + st * 8 + 4);
+    affine_next = (uint32_t)s_row[st] | ((uint32_t)b_row[st] << 16);
+  };
+  auto stage_b = [&](uint32_t buffer) {
+    unsigned char *bt = b_tiles + buffer * kBTileBytes + tid * kPitch;
+    const float scale = bf16_bits_to_f32(affine_now & 0xffffu), bias = bf16_bits_to_f32(affine_now >> 16);
+    const uint32_t words[8] = {w_now[0].x, w_now[0].y, w_now[0].z, w_now[0].w,
+                               w_now[1].x, w_now[1].y, w_now[1].z, w_now[1].w};
     if (f16_exact(scale) && f16_exact(bias)) {
       const f16x2 scale2 = {(_Float16)scale, (_Float16)scale}, bias2 = {(_Float16)bias, (_Float16)bias};
 #pragma unroll
@@ -203,21 +211,32 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
     for (int j = 0; j < 4; ++j)
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  const uint32_t steps = a.inner / kBK;
-  fetch(0);
-  stage(0);
+  // prologue: step 0 staged, weights of step 1 in flight
+  stage_a(0, 0);
+  fetch_w(0);
+  w_now[0] = w_next[0];
+  w_now[1] = w_next[1];
+  affine_now = affine_next;
+  fetch_w(1);
+  stage_b(0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's rows have landed in LDS
   __syncthreads();
+  const uint32_t swizzle = (l32 >> 1) & 7;
   for (uint32_t step = 0; step < steps; ++step) {
     const uint32_t buffer = step & 1;
-    if (step + 1 < steps) fetch(step + 1);
-    const unsigned char *at = a_tiles + buffer * kTileBytes + (128 * wm + l32) * kPitch + 16 * kh;
-    const unsigned char *bt = b_tiles + buffer * kTileBytes + (128 * wn + l32) * kPitch + 16 * kh;
+    stage_a(buffer ^ 1, min(step + 1, steps - 1));
+    w_now[0] = w_next[0];   // weights of step+1: requested a whole step ago
+    w_now[1] = w_next[1];
+    affine_now = affine_next;
+    fetch_w(step + 2);
+    const unsigned char *at = a_tiles + buffer * kATileBytes + (128 * wm + l32) * 128;
+    const unsigned char *bt = b_tiles + buffer * kBTileBytes + (128 * wn + l32) * kPitch + 16 * kh;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       f16x8 a_op[4], b_op[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        a_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * kPitch + 32 * s));
+        a_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * 128 + 16 * ((2 * s + kh) ^ swizzle)));
         b_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kPitch + 32 * s));
       }
 #pragma unroll
@@ -226,7 +245,8 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
     }
-    if (step + 1 < steps) stage(buffer ^ 1);
+    stage_b(buffer ^ 1);
+    __builtin_amdgcn_s_waitcnt(0x0f74);   // vmcnt(4): all but the four weight loads just issued
     __syncthreads();
   }
   // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile

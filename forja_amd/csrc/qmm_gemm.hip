@@ -21,8 +21,10 @@
 //     packed weights are requested two steps ahead (they are cold in HBM);
 //   * a thread dequantises one weight row of the tile per step (64 nibbles): two nibbles become
 //     the fp16 pair (1024+q) with one and-or, minus 1024 exactly, then one packed fused
-//     multiply-add gives scale*q+bias rounded once; scales outside the fp16 normal range take an
-//     f32 path.  Every weight byte is read from HBM once per 256 rows and unpacked once per
+//     multiply-add gives scale*q+bias rounded once.  That needs every scale and bias to be an
+//     fp16 normal number (or zero); check_affine_kernel scans them first and raises a flag
+//     otherwise, and then a second instantiation of the kernel, which dequantises in f32, does
+//     the work instead (both are launched; the one whose turn it is not returns at once).  Every weight byte is read from HBM once per 256 rows and unpacked once per
 //     workgroup;
 //   * the workgroup -> tile map walks all row tiles of a column tile before moving on and keeps
 //     the walk of one XCD contiguous, so a weight tile is fetched into that XCD's L2 once.
@@ -55,6 +57,7 @@ struct GemmArgs {
   uint32_t out_f32;
   uint32_t rows, inner, columns;
   uint32_t row_tiles, column_tiles;
+  const uint32_t *wide_flag;   // non-zero: some scale or bias is not an fp16 normal number
 };
 
 __device__ inline uint32_t pack2(float lo, float hi) {
@@ -140,7 +143,17 @@ __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, ui
   }
 }
 
+// flag[0] = 1 if any scale or bias of the matrix is not exactly an fp16 normal number or zero.
+__global__ void check_affine_kernel(const uint16_t *scales, const uint16_t *biases, uint64_t count,
+                                    uint32_t *flag) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  if (!f16_exact(bf16_bits_to_f32(scales[i])) || !f16_exact(bf16_bits_to_f32(biases[i]))) flag[0] = 1;
+}
+
+template <bool kWide>
 __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
+  if ((a.wide_flag[0] != 0) != kWide) return;
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
   unsigned char *a_tiles = gemm_lds;                      // [2][kBM][128], pieces swizzled
   unsigned char *b_tiles = gemm_lds + 2 * kATileBytes;    // [2][kBN][kPitch]
@@ -189,18 +202,19 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
     w_next[1] = *(const uint4 *)(w_row + st * 8 + 4);
     affine_next = (uint32_t)s_row[st] | ((uint32_t)b_row[st] << 16);
   };
-  auto stage_b = [&](uint32_t buffer) {
-    unsigned char *bt = b_tiles + buffer * kBTileBytes + tid * kPitch;
+  // quarter `part` of the weight row: two packed words = 16 values
+  auto stage_b = [&](uint32_t buffer, int part) {
+    unsigned char *bt = b_tiles + buffer * kBTileBytes + tid * kPitch + 32 * part;
     const float scale = bf16_bits_to_f32(affine_now & 0xffffu), bias = bf16_bits_to_f32(affine_now >> 16);
-    const uint32_t words[8] = {w_now[0].x, w_now[0].y, w_now[0].z, w_now[0].w,
-                               w_now[1].x, w_now[1].y, w_now[1].z, w_now[1].w};
-    if (f16_exact(scale) && f16_exact(bias)) {
-      const f16x2 scale2 = {(_Float16)scale, (_Float16)scale}, bias2 = {(_Float16)bias, (_Float16)bias};
-#pragma unroll
-      for (int i = 0; i < 8; ++i) *(uint4 *)(bt + 16 * i) = dequantise_word(words[i], scale2, bias2);
+    const uint4 w = w_now[part / 2];
+    const uint32_t first = (part & 1) ? w.z : w.x, second = (part & 1) ? w.w : w.y;
+    if (kWide) {
+      *(uint4 *)(bt) = dequantise_word_wide(first, scale, bias);
+      *(uint4 *)(bt + 16) = dequantise_word_wide(second, scale, bias);
     } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) *(uint4 *)(bt + 16 * i) = dequantise_word_wide(words[i], scale, bias);
+      const f16x2 scale2 = {(_Float16)scale, (_Float16)scale}, bias2 = {(_Float16)bias, (_Float16)bias};
+      *(uint4 *)(bt) = dequantise_word(first, scale2, bias2);
+      *(uint4 *)(bt + 16) = dequantise_word(second, scale2, bias2);
     }
   };
 
@@ -218,7 +232,7 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   w_now[1] = w_next[1];
   affine_now = affine_next;
   fetch_w(1);
-  stage_b(0);
+  for (int part = 0; part < 4; ++part) stage_b(0, part);
   __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's rows have landed in LDS
   __syncthreads();
   const uint32_t swizzle = (l32 >> 1) & 7;
@@ -244,8 +258,8 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
+      stage_b(buffer ^ 1, s);   // a quarter of the next step's weights between the sub-steps
     }
-    stage_b(buffer ^ 1);
     __builtin_amdgcn_s_waitcnt(0x0f74);   // vmcnt(4): all but the four weight loads just issued
     __syncthreads();
   }
@@ -273,7 +287,8 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
 
 bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
   const uint64_t rows_bytes = ((uint64_t)p.rows * p.inner * 2 + 255) / 256 * 256;
-  char *ws = backend_workspace(backend, rows_bytes + (uint64_t)p.rows * sizeof(float));
+  const uint64_t unscale_bytes = ((uint64_t)p.rows * sizeof(float) + 255) / 256 * 256;
+  char *ws = backend_workspace(backend, rows_bytes + unscale_bytes + 256);
   if (!ws) return false;
   hipStream_t stream = backend_stream(backend);
   GemmArgs a{};
@@ -292,9 +307,13 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
   a.columns = p.columns;
   a.row_tiles = (p.rows + kBM - 1) / kBM;
   a.column_tiles = (p.columns + kBN - 1) / kBN;
+  uint32_t *flag = (uint32_t *)(ws + rows_bytes + unscale_bytes);
+  a.wide_flag = flag;
   static bool configured = false;   // raise the dynamic LDS limit once per process
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_gemm_kernel),
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_gemm_kernel<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_gemm_kernel<true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds) != hipSuccess)
       return false;
     configured = true;
@@ -305,7 +324,12 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
   prepare_rows_kernel<<<(p.rows + 3) / 4, 256, 0, stream>>>(
       (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, (uint16_t *)ws,
       (float *)(ws + rows_bytes));
-  qmm_gemm_kernel<<<grid, 256, kGemmLds, stream>>>(a);
+  launch_fill_u32(stream, flag, 1, 0);
+  const uint64_t affine_count = (uint64_t)p.columns * (p.inner / kBK);
+  check_affine_kernel<<<(uint32_t)((affine_count + 255) / 256), 256, 0, stream>>>(a.scales, a.biases,
+                                                                                 affine_count, flag);
+  qmm_gemm_kernel<false><<<grid, 256, kGemmLds, stream>>>(a);
+  qmm_gemm_kernel<true><<<grid, 256, kGemmLds, stream>>>(a);
   return true;
 }
 

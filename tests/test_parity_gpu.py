@@ -154,6 +154,35 @@ def test_quant_matmul(cpu, hip, rows, n, k, bits, group, dtype):
     differential(cpu, hip, build)
 
 
+def test_quant_gemm_with_scales_outside_the_fp16_range_and_huge_activations(cpu, hip):
+    """Prefill-sized product whose affine parameters are not fp16 normal numbers (tiny scales, a
+    zero bias, a large scale) and whose activations exceed the fp16 range in some rows: the
+    f32 dequantisation path and the per-row power-of-two scaling."""
+    rows, n, k = 300, 200, 512
+    weights = Quantised(61, 3, (n, k))
+    scales = orc.bf16_to_f32(weights.scales).copy()
+    biases = orc.bf16_to_f32(weights.biases).copy()
+    scales[::3, 0] = 3.0e-6
+    scales[1::7, 1] = 7000.0
+    biases[::5, 2] = 0.0
+    biases[2::5, 3] = 1.0e-7
+    weights.scales = orc.f32_to_bf16(scales.ravel()).reshape(scales.shape)
+    weights.biases = orc.f32_to_bf16(biases.ravel()).reshape(biases.shape)
+    x_values = orc.bf16_to_f32(normal_bf16(61, 9, (rows, k))).copy()
+    x_values[5] *= 3.0e6
+    x_values[17, 3] = 1.0e9
+    x_values[40] *= 1.0e-6
+
+    def build(backend):
+        x = upload(backend, x_values, DType.BF16)
+        packed, sc, bi = weights.upload(backend)
+        out = backend.alloc(DType.BF16, (rows, n))
+        commands = CommandList()
+        commands.dispatch(Op.quant_matmul(4, 64), [x, packed, sc, bi], out)
+        return commands, [out]
+    differential(cpu, hip, build)
+
+
 def test_quant_matmul_on_strided_views_with_bias_epilogue(cpu, hip):
     """Every operand sliced with step 2 (crates/forja-metal/tests/quant_matmul/shared.rs:95-107)
     plus a fused epilogue that adds a broadcast bias."""

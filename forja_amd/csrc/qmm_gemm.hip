@@ -21,13 +21,14 @@
 //     packed weights are requested two steps ahead (they are cold in HBM);
 //   * a thread dequantises one weight row of the tile per step (64 nibbles): two nibbles become
 //     the fp16 pair (1024+q) with one and-or, minus 1024 exactly, then one packed fused
-//     multiply-add gives scale*q+bias rounded once.  That needs every scale and bias to be an
-//     fp16 normal number (or zero); check_affine_kernel scans them first and raises a flag
+//     multiply-add gives scale*q+bias rounded once.  That needs every scale and bias to lie
+//     well inside the fp16 range; check_affine_kernel scans them first and raises a flag
 //     otherwise, and then a second instantiation of the kernel, which dequantises in f32, does
 //     the work instead (both are launched; the one whose turn it is not returns at once).  Every weight byte is read from HBM once per 256 rows and unpacked once per
 //     workgroup;
-//   * the workgroup -> tile map walks all row tiles of a column tile before moving on and keeps
-//     the walk of one XCD contiguous, so a weight tile is fetched into that XCD's L2 once.
+//   * the workgroup -> tile map gives the 32 workgroups that run together on one XCD a patch of
+//     about 4 row tiles x 8 column tiles, so that its L2 serves each activation tile to 8
+//     workgroups and each weight tile to 4, instead of every workgroup streaming its own.
 // Accumulation is f32.
 #include "fast_kernels.hpp"
 
@@ -41,6 +42,7 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int kBM = 256, kBN = 256, kBK = 64;
+constexpr int kBand = 8;   // column tiles per band of the tile numbering
 constexpr int kPitch = 2 * kBK + 16;              // bytes per staged weight row
 constexpr int kATileBytes = kBM * 2 * kBK;        // activation tile, swizzled, no padding
 constexpr int kBTileBytes = kBN * kPitch;         // weight tile
@@ -57,7 +59,7 @@ struct GemmArgs {
   uint32_t out_f32;
   uint32_t rows, inner, columns;
   uint32_t row_tiles, column_tiles;
-  const uint32_t *wide_flag;   // non-zero: some scale or bias is not an fp16 normal number
+  const uint32_t *wide_flag;   // non-zero: some scale or bias does not fit fp16
 };
 
 __device__ inline uint32_t pack2(float lo, float hi) {
@@ -97,9 +99,11 @@ __device__ inline uint4 dequantise_word_wide(uint32_t w, float scale, float bias
                     pack_f16(v[3], v[7]));
 }
 
-__device__ inline bool f16_exact(float value) {
-  const float magnitude = fabsf(value);
-  return magnitude == 0.0f || (magnitude >= 6.103515625e-05f && magnitude <= 4096.0f);
+// Scales and biases the fp16 form can take: finite and well inside the fp16 range (15 * scale +
+// bias must not overflow).  Magnitudes below the fp16 normal range become fp16 subnormals, an
+// absolute error under 2^-25 per weight, far below the rounding of the weight itself.
+__device__ inline bool f16_safe(float scale, float bias) {
+  return fabsf(scale) <= 2048.0f && fabsf(bias) <= 30000.0f;   // false for NaN too
 }
 
 // x bf16 [rows, inner] -> fp16 [rows, inner] (every 8 values stored as 0,4,1,5,2,6,3,7), each row
@@ -143,12 +147,12 @@ __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, ui
   }
 }
 
-// flag[0] = 1 if any scale or bias of the matrix is not exactly an fp16 normal number or zero.
+// flag[0] = 1 if any scale or bias of the matrix is too large for (or not a number in) fp16.
 __global__ void check_affine_kernel(const uint16_t *scales, const uint16_t *biases, uint64_t count,
                                     uint32_t *flag) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= count) return;
-  if (!f16_exact(bf16_bits_to_f32(scales[i])) || !f16_exact(bf16_bits_to_f32(biases[i]))) flag[0] = 1;
+  if (!f16_safe(bf16_bits_to_f32(scales[i]), bf16_bits_to_f32(biases[i]))) flag[0] = 1;
 }
 
 template <bool kWide>
@@ -161,13 +165,19 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   const uint32_t wm = wave >> 1, wn = wave & 1;
   const uint32_t l32 = lane & 31, kh = lane >> 5;
 
-  // workgroup -> tile: workgroups are dealt round-robin to the 8 XCDs; give each XCD a
-  // contiguous run of tiles, column tile major
-  const uint32_t tiles = a.row_tiles * a.column_tiles;
-  const uint32_t per_xcd = (tiles + 7) / 8;
-  const uint32_t tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (tile >= tiles) return;
-  const uint32_t bn = tile / a.row_tiles, bm = tile % a.row_tiles;
+  // workgroup -> tile.  Tiles are numbered band by band (a band = kBand column tiles), row
+  // tile major inside a band, so 32 consecutive numbers are a 4 x 8 patch of tiles sharing
+  // activation and weight tiles.  Workgroups are dealt round-robin to the 8 XCDs (workgroup b is
+  // the (b / 8)-th of XCD b % 8, and 32 consecutive ones of an XCD run together): each such
+  // group of 32 takes one patch, so the XCD's L2 serves an activation tile to 8 workgroups and
+  // a weight tile to 4.
+  const uint32_t xcd = blockIdx.x % 8, nth = blockIdx.x / 8;
+  const uint32_t tile = (nth / 32) * 256 + xcd * 32 + nth % 32;
+  if (tile >= a.row_tiles * a.column_tiles) return;
+  const uint32_t band = tile / (a.row_tiles * kBand);
+  const uint32_t band_width = min((uint32_t)kBand, a.column_tiles - band * kBand);
+  const uint32_t in_band = tile - band * a.row_tiles * kBand;
+  const uint32_t bm = in_band / band_width, bn = band * kBand + in_band % band_width;
   const uint32_t row0 = bm * kBM, col0 = bn * kBN;
 
   // Activation staging: a wave owns 64 rows of the tile; one instruction moves 8 rows (lane ->
@@ -202,19 +212,17 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
     w_next[1] = *(const uint4 *)(w_row + st * 8 + 4);
     affine_next = (uint32_t)s_row[st] | ((uint32_t)b_row[st] << 16);
   };
-  // quarter `part` of the weight row: two packed words = 16 values
+  // one packed word (8 values) of the weight row: `part` 0..7
   auto stage_b = [&](uint32_t buffer, int part) {
-    unsigned char *bt = b_tiles + buffer * kBTileBytes + tid * kPitch + 32 * part;
+    unsigned char *bt = b_tiles + buffer * kBTileBytes + tid * kPitch + 16 * part;
     const float scale = bf16_bits_to_f32(affine_now & 0xffffu), bias = bf16_bits_to_f32(affine_now >> 16);
-    const uint4 w = w_now[part / 2];
-    const uint32_t first = (part & 1) ? w.z : w.x, second = (part & 1) ? w.w : w.y;
+    const uint4 w = w_now[part / 4];
+    const uint32_t word = (part & 3) == 0 ? w.x : ((part & 3) == 1 ? w.y : ((part & 3) == 2 ? w.z : w.w));
     if (kWide) {
-      *(uint4 *)(bt) = dequantise_word_wide(first, scale, bias);
-      *(uint4 *)(bt + 16) = dequantise_word_wide(second, scale, bias);
+      *(uint4 *)(bt) = dequantise_word_wide(word, scale, bias);
     } else {
       const f16x2 scale2 = {(_Float16)scale, (_Float16)scale}, bias2 = {(_Float16)bias, (_Float16)bias};
-      *(uint4 *)(bt) = dequantise_word(first, scale2, bias2);
-      *(uint4 *)(bt + 16) = dequantise_word(second, scale2, bias2);
+      *(uint4 *)(bt) = dequantise_word(word, scale2, bias2);
     }
   };
 
@@ -232,7 +240,7 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   w_now[1] = w_next[1];
   affine_now = affine_next;
   fetch_w(1);
-  for (int part = 0; part < 4; ++part) stage_b(0, part);
+  for (int part = 0; part < 8; ++part) stage_b(0, part);
   __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's rows have landed in LDS
   __syncthreads();
   const uint32_t swizzle = (l32 >> 1) & 7;
@@ -245,20 +253,32 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
     fetch_w(step + 2);
     const unsigned char *at = a_tiles + buffer * kATileBytes + (128 * wm + l32) * 128;
     const unsigned char *bt = b_tiles + buffer * kBTileBytes + (128 * wn + l32) * kPitch + 16 * kh;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      f16x8 a_op[4], b_op[4];
+    // operand fragments are read one sub-step ahead of the MFMAs that use them
+    f16x8 a_op[2][4], b_op[2][4];
+    auto read_fragments = [&](int slot, int sub) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        a_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * 128 + 16 * ((2 * s + kh) ^ swizzle)));
-        b_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kPitch + 32 * s));
+        a_op[slot][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * 128 + 16 * ((2 * sub + kh) ^ swizzle)));
+        b_op[slot][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kPitch + 32 * sub));
       }
+    };
+    read_fragments(0, 0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+    for (int s = 0; s < 4; ++s) {
+      if (s < 3) read_fragments((s + 1) & 1, s + 1);
+      // eight MFMAs, then one word of the next step's weights, fenced so that the staging
+      // instructions issue in the shadow of the matrix pipe instead of after all sixteen
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
-      stage_b(buffer ^ 1, s);   // a quarter of the next step's weights between the sub-steps
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
+        if (i & 1) {
+          __builtin_amdgcn_sched_barrier(0);
+          stage_b(buffer ^ 1, 2 * s + (i >> 1));
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
     }
     __builtin_amdgcn_s_waitcnt(0x0f74);   // vmcnt(4): all but the four weight loads just issued
     __syncthreads();
@@ -318,8 +338,7 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
       return false;
     configured = true;
   }
-  const uint32_t tiles = a.row_tiles * a.column_tiles;
-  const uint32_t grid = ((tiles + 7) / 8) * 8;
+  const uint32_t grid = (a.row_tiles * a.column_tiles + 255) / 256 * 256;
   KernelTimer timer(backend, FH_KC_QMM_KERNEL);
   prepare_rows_kernel<<<(p.rows + 3) / 4, 256, 0, stream>>>(
       (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, (uint16_t *)ws,

@@ -229,6 +229,73 @@ def prefill_gemm_c4(backend, rows=8256, seed=91, repeats=3):
     }
 
 
+def prefill_attention_c4(backend, seed=93, repeats=3):
+    """Paged attention of one BASELINE config 4 layer: an 8192-token chunk packed from 6 prompts
+    (512..3072 tokens, from empty contexts) plus 64 decode rows (contexts uniform 128..4096), 40
+    query / 8 kv heads of 128, bf16 pools of 16-token pages behind shuffled block tables."""
+    from forja_amd.model import DENSE_27B
+    c = DENSE_27B
+    rng = np.random.default_rng(seed)
+    prompts = [512, 768, 1024, 1280, 1536, 3072]
+    contexts = [0] * len(prompts) + [int(v) for v in rng.integers(128, 4097, 64)]
+    counts = prompts + [1] * 64
+    lanes, tokens, pt = len(counts), sum(counts), c.page_tokens
+    pages_of = [(ctx + n + pt - 1) // pt for ctx, n in zip(contexts, counts)]
+    table_pages = max(pages_of)
+    physical = sum(pages_of) + 7
+    order = rng.permutation(physical)
+    tables = np.zeros((lanes, table_pages, 2), np.uint32)
+    tables[:, :, 1] = 0xffffffff
+    cursor = 0
+    for lane, n_pages in enumerate(pages_of):
+        pages = order[cursor:cursor + n_pages]
+        cursor += n_pages
+        tables[lane, :n_pages, 0] = pages
+        tables[lane, :n_pages, 1] = 11 + pages
+    generations = (11 + np.arange(physical)).astype(np.uint32)
+    cu = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+
+    def up(array, dtype, shape):
+        tensor = backend.alloc(dtype, shape)
+        backend.write(tensor, np.ascontiguousarray(array).tobytes())
+        return tensor
+    t_tables = up(tables, DType.U32, tables.shape)
+    t_generations = up(generations, DType.U32, (physical,))
+    t_cu = up(cu, DType.U32, (lanes + 1,))
+    t_starts = up(np.array(contexts, np.uint32), DType.U32, (lanes,))
+    t_activity = up(np.ones(lanes, np.uint32), DType.U32, (lanes,))
+    q = backend.alloc(DType.BF16, (tokens, c.q_heads, c.head_dim))
+    k_new = backend.alloc(DType.BF16, (tokens, c.kv_heads, c.head_dim))
+    v_new = backend.alloc(DType.BF16, (tokens, c.kv_heads, c.head_dim))
+    out = backend.alloc(DType.BF16, (tokens, c.q_heads, c.head_dim))
+    keys = backend.alloc(DType.BF16, (physical, pt, c.kv_heads, c.head_dim))
+    values = backend.alloc(DType.BF16, (physical, pt, c.kv_heads, c.head_dim))
+    fill = CommandList()
+    for stream, tensor in enumerate((q, k_new, v_new, keys, values)):
+        fill.dispatch(Op.fill_seeded(2, seed, 20 + stream), [], tensor)
+    backend.submit(fill).wait()
+    commands = CommandList()
+    commands.dispatch_many(Op.paged_attention_ragged(1.0 / math.sqrt(c.head_dim), pt),
+                           [q, k_new, v_new, t_tables, t_generations, t_cu, t_starts, t_activity],
+                           [out, keys, values])
+    encoded = backend.encode(commands)
+    backend.submit(encoded).wait()
+    backend.profile_enable(2)
+    backend.profile_reset()
+    for _ in range(repeats):
+        backend.submit(encoded).wait()
+    op_ns, _ = backend.profile_read(KC_ATTENTION)
+    kernel_ns, _ = backend.profile_read(KC_ATTENTION_KERNEL)
+    backend.profile_enable(0)
+    pairs = sum(n * ctx + n * (n + 1) // 2 for ctx, n in zip(contexts, counts))
+    flops = 2.0 * c.q_heads * pairs * 2 * c.head_dim
+    for tensor in (t_tables, t_generations, t_cu, t_starts, t_activity, q, k_new, v_new, out, keys, values):
+        backend.release(tensor)
+    return {"tokens": tokens, "lanes": lanes, "query_key_pairs": pairs, "flops": flops,
+            "us_op": op_ns / repeats / 1e3, "us_kernel": kernel_ns / repeats / 1e3,
+            "tflops": flops / (op_ns / repeats * 1e-9) / 1e12}
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -260,7 +327,9 @@ def main():
                           "kernel": "copy_kernel", "launches": 8}))
         return
     if args.prefill_only:
-        print(json.dumps(prefill_gemm_c4(HipBackend(0))))
+        backend = HipBackend(0)
+        print(json.dumps({"prefill_gemm_c4": prefill_gemm_c4(backend),
+                          "prefill_attention_c4": prefill_attention_c4(backend)}))
         return
     if args.gpus != 1:
         print("bench.py: this build runs the ragged forward step on ONE MI355X; collectives and "

@@ -200,6 +200,7 @@ constexpr uint32_t kTile = 32;          // tokens per inner step
 
 struct TokenPlan {
   uint32_t lane, attended, chunk, splits;  // splits == 0: token produces zeros
+  uint32_t leader, members;                // first token of this token's group, group size
 };
 
 struct FastRagged {
@@ -210,11 +211,14 @@ struct FastRagged {
   float2 *partial_ml;  // [T, S, Hq]
   uint32_t *bad;       // [T]
   TokenPlan *plans;    // [T]
-  uint2 *items;        // [T * S] (token, split) of every live split, compacted
+  uint2 *items;        // [T * S] (group leader token, split) of every live split, compacted
   uint32_t *item_count;
   uint64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h;
   uint32_t tokens, lanes, query_heads, kv_heads, group, page_tokens, physical_pages, table_pages,
       max_splits, split_tokens;
+  // Query tokens of one lane are processed `group_tokens` at a time by one wave per kv head (they
+  // share the lane's K/V stream): 1 for decode batches, 2 * (16 / group) for prefill.
+  uint32_t group_tokens;
   float scale_log2;
   // Single-lane form (Op::PagedSdpa / Op::PagedSdpaAppend): cu == nullptr, every token belongs
   // to lane 0 whose first query sits at `one_start`; `fixed_attended` != 0 disables the causal
@@ -222,30 +226,44 @@ struct FastRagged {
   uint32_t one_start, fixed_attended;
 };
 
-// Work decomposition of one token.  attended == 0 with splits == 0 and lane == 0xffffffff marks a
-// token whose context exceeds its table (reported as a bad page).
+// Work decomposition of one token.  Tokens of a lane are grouped `group_tokens` at a time; a
+// group shares its split layout, sized for its last (longest) member, and every member carries
+// its own causal limit in `attended`.  attended == 0 with splits == 0 and lane == 0xffffffff
+// marks a token whose context exceeds its table (reported as a bad page).
 __device__ inline TokenPlan plan_token(const FastRagged &p, uint32_t token, uint32_t split_tokens) {
-  TokenPlan plan{0, 0, 0, 0};
-  uint64_t attended;
+  TokenPlan plan{0, 0, 0, 0, token, 1};
+  uint64_t attended, first_of_lane, lane_tokens, start;
   if (p.cu == nullptr) {
     if (p.activity && p.activity[0] == 0) return plan;
-    attended = p.fixed_attended ? p.fixed_attended : (uint64_t)p.one_start + token + 1;
+    first_of_lane = 0;
+    lane_tokens = p.tokens;
+    start = p.one_start;
   } else {
     if (token < p.cu[0] || token >= p.cu[p.lanes]) return plan;
     plan.lane = find_lane(p.cu, p.lanes, token);
     if (p.activity && p.activity[plan.lane] == 0) return plan;
-    attended = (uint64_t)p.starts[plan.lane] + (token - p.cu[plan.lane]) + 1;
+    first_of_lane = p.cu[plan.lane];
+    lane_tokens = p.cu[plan.lane + 1] - first_of_lane;
+    start = p.starts[plan.lane];
   }
-  if (attended > (uint64_t)p.table_pages * p.page_tokens) {
+  const uint64_t index = token - first_of_lane;
+  const uint64_t leader = index - index % p.group_tokens;
+  const uint64_t last = min(leader + p.group_tokens, lane_tokens) - 1;
+  attended = p.fixed_attended ? p.fixed_attended : start + index + 1;
+  const uint64_t group_attended = p.fixed_attended ? p.fixed_attended : start + last + 1;
+  if (group_attended > (uint64_t)p.table_pages * p.page_tokens) {
     plan.lane = 0xffffffffu;
     return plan;
   }
+  plan.leader = (uint32_t)(first_of_lane + leader);
+  plan.members = (uint32_t)(last - leader + 1);
   plan.attended = (uint32_t)attended;
-  uint32_t want = (plan.attended + split_tokens - 1) / split_tokens;
+  const uint32_t longest = (uint32_t)group_attended;
+  uint32_t want = (longest + split_tokens - 1) / split_tokens;
   if (want > p.max_splits) want = p.max_splits;
-  uint32_t chunk = (plan.attended + want - 1) / want;
+  uint32_t chunk = (longest + want - 1) / want;
   plan.chunk = (chunk + kTile - 1) / kTile * kTile;
-  plan.splits = (plan.attended + plan.chunk - 1) / plan.chunk;
+  plan.splits = (longest + plan.chunk - 1) / plan.chunk;
   return plan;
 }
 
@@ -266,7 +284,7 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
   if (split_tokens == 0) {
     unsigned long long mine = 0;
     for (uint32_t token = threadIdx.x; token < p.tokens; token += 256)
-      mine += plan_token(p, token, 1u << 30).attended;
+      mine += plan_token(p, token, 1u << 30).attended / p.group_tokens;
     for (int offset = 32; offset > 0; offset >>= 1) mine += __shfl_xor(mine, offset, 64);
     if ((threadIdx.x & 63) == 0) atomicAdd(&total_attended, mine);
     __syncthreads();
@@ -277,7 +295,7 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
   }
   for (uint32_t base = 0; base < p.tokens; base += 256) {
     uint32_t token = base + threadIdx.x;
-    TokenPlan plan{0, 0, 0, 0};
+    TokenPlan plan{0, 0, 0, 0, 0, 1};
     if (token < p.tokens) {
       plan = plan_token(p, token, split_tokens);
       uint32_t bad = 0;
@@ -289,7 +307,9 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
       p.bad[token] = bad;
       p.plans[token] = plan;
     }
-    uint32_t inclusive = plan.splits;
+    // work items come from group leaders only
+    const uint32_t my_items = (token < p.tokens && plan.leader == token) ? plan.splits : 0;
+    uint32_t inclusive = my_items;
     for (int offset = 1; offset < 64; offset <<= 1) {
       uint32_t other = __shfl_up(inclusive, offset, 64);
       if ((int)(threadIdx.x & 63) >= offset) inclusive += other;
@@ -298,8 +318,8 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
     __syncthreads();
     uint32_t before = running;
     for (uint32_t w = 0; w < (threadIdx.x >> 6); ++w) before += wave_totals[w];
-    uint32_t first = before + inclusive - plan.splits;
-    for (uint32_t s = 0; s < plan.splits; ++s) p.items[first + s] = make_uint2(token, s);
+    uint32_t first = before + inclusive - my_items;
+    for (uint32_t s = 0; s < my_items; ++s) p.items[first + s] = make_uint2(token, s);
     __syncthreads();
     if (threadIdx.x == 255) running = before + inclusive;
     __syncthreads();
@@ -364,45 +384,55 @@ struct Softmax {
   float m, l;
 };
 
-// Scores, online softmax and the value product for one tile.
-template <bool kMasked>
-__device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[4], f32x4 (&o)[8],
-                                    Softmax &sm, uint32_t tile0, uint32_t end, float scale_log2,
-                                    uint32_t g) {
-  float s_val[8];
-  for (int sub = 0; sub < 2; ++sub) {
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int step = 0; step < 4; ++step)
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, cur.k[sub][step]),
-                                                    __builtin_bit_cast(bf16x8, q_reg[step]), acc, 0,
-                                                    0, 0);
-    for (int j = 0; j < 4; ++j) {
-      s_val[4 * sub + j] = acc[j] * scale_log2;
-      if (kMasked && tile0 + 16 * sub + 4 * g + j >= end) s_val[4 * sub + j] = -__builtin_inff();
+// Scores, online softmax and the value product for one tile of 32 keys against NT query tiles
+// (16 query rows each: this lane holds row hl of every tile).  `limit[nt]` is the first key the
+// lane's row of tile nt may NOT attend (0 for an unused row); with kMasked false every key of
+// the tile is below every limit.
+template <int NT, bool kMasked>
+__device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[NT][4],
+                                    f32x4 (&o)[NT][8], Softmax (&sm)[NT], uint32_t tile0,
+                                    const uint32_t (&limit)[NT], float scale_log2, uint32_t g) {
+  uint4 p_reg[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    float s_val[8];
+    for (int sub = 0; sub < 2; ++sub) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      for (int step = 0; step < 4; ++step)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, cur.k[sub][step]),
+                                                      __builtin_bit_cast(bf16x8, q_reg[nt][step]),
+                                                      acc, 0, 0, 0);
+      for (int j = 0; j < 4; ++j) {
+        s_val[4 * sub + j] = acc[j] * scale_log2;
+        if (kMasked && tile0 + 16 * sub + 4 * g + j >= limit[nt]) s_val[4 * sub + j] = -__builtin_inff();
+      }
     }
+    float tile_max = s_val[0];
+    for (int i = 1; i < 8; ++i) tile_max = fmaxf(tile_max, s_val[i]);
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    const float m_new = fmaxf(sm[nt].m, tile_max);
+    // a row with nothing to attend yet keeps m = -inf; subtract 0 instead so that exp2(-inf) = 0
+    const float m_safe = (kMasked && m_new == -__builtin_inff()) ? 0.0f : m_new;
+    float p_val[8], p_sum = 0.0f;
+    for (int i = 0; i < 8; ++i) {
+      p_val[i] = __builtin_amdgcn_exp2f(s_val[i] - m_safe);
+      p_sum += p_val[i];
+    }
+    // The running maximum settles after a few tiles; skip the rescale when no lane's moved.
+    if (__any(m_new != sm[nt].m)) {
+      const float alpha = __builtin_amdgcn_exp2f(sm[nt].m - m_safe);   // 0 while m is -inf
+      sm[nt].l *= alpha;
+      for (int mt = 0; mt < 8; ++mt)
+        for (int j = 0; j < 4; ++j) o[nt][mt][j] *= alpha;
+      sm[nt].m = m_new;
+    }
+    sm[nt].l += p_sum;
+    p_reg[nt] = make_uint4(pack_bf16(p_val[0], p_val[1]), pack_bf16(p_val[2], p_val[3]),
+                           pack_bf16(p_val[4], p_val[5]), pack_bf16(p_val[6], p_val[7]));
   }
-  float tile_max = s_val[0];
-  for (int i = 1; i < 8; ++i) tile_max = fmaxf(tile_max, s_val[i]);
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-  const float m_new = fmaxf(sm.m, tile_max);
-  float p_val[8], p_sum = 0.0f;
-  for (int i = 0; i < 8; ++i) {
-    p_val[i] = __builtin_amdgcn_exp2f(s_val[i] - m_new);
-    p_sum += p_val[i];
-  }
-  // The running maximum settles after a few tiles; skip the rescale when no lane's moved.
-  if (__any(m_new != sm.m)) {
-    const float alpha = __builtin_amdgcn_exp2f(sm.m - m_new);
-    sm.l *= alpha;
-    for (int mt = 0; mt < 8; ++mt)
-      for (int j = 0; j < 4; ++j) o[mt][j] *= alpha;
-    sm.m = m_new;
-  }
-  sm.l += p_sum;
-  const uint4 p_reg = make_uint4(pack_bf16(p_val[0], p_val[1]), pack_bf16(p_val[2], p_val[3]),
-                                 pack_bf16(p_val[4], p_val[5]), pack_bf16(p_val[6], p_val[7]));
-  // O^T += V^T . P^T.  Tile mt takes element mt of each of the lane's 8 token pieces.
+  // O^T += V^T . P^T.  Tile mt takes element mt of each of the lane's 8 token pieces; the
+  // transposed value operand serves all NT query tiles.
   for (int mt = 0; mt < 8; ++mt) {
     const uint32_t selector = (mt & 1) ? 0x07060302u : 0x05040100u;
     uint32_t a_words[4];
@@ -410,22 +440,30 @@ __device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[4]
       a_words[pair] = __builtin_amdgcn_perm(dword_of(cur.v[2 * pair + 1], mt >> 1),
                                             dword_of(cur.v[2 * pair], mt >> 1), selector);
     const uint4 a_reg = make_uint4(a_words[0], a_words[1], a_words[2], a_words[3]);
-    o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_reg),
-                                                   __builtin_bit_cast(bf16x8, p_reg), o[mt], 0, 0,
-                                                   0);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      o[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_reg),
+                                                         __builtin_bit_cast(bf16x8, p_reg[nt]),
+                                                         o[nt][mt], 0, 0, 0);
   }
 }
 
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void ragged_attention_mfma_kernel(
-    FastRagged p, ErrorSlot *error) {
+// NT query tiles of 16 rows per wave: row hl of tile nt is (query token nt * per_tile + hl / group
+// of the item's group, head hl % group of the kv head), per_tile = 16 / group.
+template <int NT>
+__device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *error) {
   const uint32_t lane = threadIdx.x, hl = lane & 15, g = lane >> 4;
   const uint32_t item = blockIdx.x / p.kv_heads, kv_head = blockIdx.x % p.kv_heads;
   if (item >= p.item_count[0]) return;
   const uint2 work = p.items[item];
-  const uint32_t token = work.x, split = work.y;
-  const TokenPlan plan = p.plans[token];
+  const uint32_t leader = work.x, split = work.y;
+  const TokenPlan plan = p.plans[leader];
+  const uint32_t members = NT == 1 ? 1 : plan.members;
+  // the group's split layout is sized for its last member
+  const uint32_t longest =
+      (NT == 1 || p.fixed_attended) ? plan.attended : plan.attended + members - 1;
   const uint32_t begin = split * plan.chunk;
-  const uint32_t end = min(plan.attended, begin + plan.chunk);
+  const uint32_t end = min(longest, begin + plan.chunk);
   const uint32_t pt = p.page_tokens;
   const uint32_t *table = p.tables + (uint64_t)plan.lane * p.table_pages * 2;
   LaneConst lc;
@@ -433,19 +471,37 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   lc.k_offset = (hl * p.kv_heads + kv_head) * 128 + 8 * g;
   lc.v_offset = (4 * g * p.kv_heads + kv_head) * 128 + 8 * hl;
 
-  // Query operand: head hl of this kv head's group (zero rows beyond the group).
-  uint4 q_reg[4];
-  {
-    const uint32_t head = kv_head * p.group + hl;
-    const uint16_t *q_row = p.q + (uint64_t)token * p.q_stride_t + (uint64_t)head * p.q_stride_h;
+  // Query operands and causal limits of this lane's rows.
+  const uint32_t per_tile = NT == 1 ? 1 : 16 / p.group;
+  uint4 q_reg[NT][4];
+  uint32_t limit[NT], member_of[NT];
+  const uint32_t head = kv_head * p.group + (NT == 1 ? hl : hl % p.group);
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    member_of[nt] = NT == 1 ? 0 : nt * per_tile + hl / p.group;
+    const bool used = hl < per_tile * p.group && member_of[nt] < members;
+    // (a decode row that is only padding keeps the uniform limit: its query is zero anyway)
+    limit[nt] = NT == 1 ? end
+                        : (!used ? 0
+                                 : min(end, p.fixed_attended ? plan.attended
+                                                             : plan.attended + member_of[nt]));
+    const uint16_t *q_row = p.q + (uint64_t)(leader + member_of[nt]) * p.q_stride_t +
+                            (uint64_t)head * p.q_stride_h;
     for (int step = 0; step < 4; ++step) {  // same head-dim slice per (step, g) as the K operand
-      q_reg[step] = make_uint4(0, 0, 0, 0);
-      if (hl < p.group) q_reg[step] = *(const uint4 *)(q_row + 32 * step + 8 * g);
+      q_reg[nt][step] = make_uint4(0, 0, 0, 0);
+      if (used) q_reg[nt][step] = *(const uint4 *)(q_row + 32 * step + 8 * g);
     }
+    if (NT > 1 && !used) member_of[nt] = 0xffffffffu;
   }
-  f32x4 o[8];
-  for (int mt = 0; mt < 8; ++mt) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  Softmax sm{-__builtin_inff(), 0.0f};
+  // keys below `unmasked_end` are attended by every used row
+  const uint32_t unmasked_end = NT == 1 ? end : min(end, plan.attended);
+  f32x4 o[NT][8];
+  Softmax sm[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    for (int mt = 0; mt < 8; ++mt) o[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    sm[nt] = Softmax{-__builtin_inff(), 0.0f};
+  }
 
   const uint32_t first_page = begin / pt, last_page = (end - 1) / pt;
   for (uint32_t page0 = first_page; page0 <= last_page; page0 += 64) {
@@ -461,56 +517,94 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     if (bad_mask) {
       if (lane == (uint32_t)__ffsll((long long)bad_mask) - 1) {
         report_error(error, my_page);
-        p.bad[token] = 1;
+        for (uint32_t member = 0; member < members; ++member) p.bad[leader + member] = 1;
       }
       return;
     }
     const uint32_t tok_lo = max(begin, page0 * pt);
     const uint32_t tok_hi = (uint32_t)min((uint64_t)end, ((uint64_t)page0 + 64) * pt);
-    // Full tiles first (no bounds logic at all), then at most one partial tile.
-    const uint32_t full_hi = tok_lo + (tok_hi - tok_lo) / kTile * kTile;
+    // Tiles wholly below unmasked_end need no bounds logic at all; the rest (at most a few
+    // around the causal diagonal and the end of the split) take the masked forms.
+    const uint32_t plain_keys = unmasked_end > tok_lo ? min(tok_hi, unmasked_end) - tok_lo : 0;
+    const uint32_t full_hi = tok_lo + plain_keys / kTile * kTile;
     TileRegs cur;
-    if (tok_lo < full_hi)
+    if (tok_lo + kTile <= tok_hi)
       load_tile<false>(p, cur, tok_lo, end, page0, physical, lc, hl, g);
     else
       load_tile<true>(p, cur, tok_lo, end, page0, physical, lc, hl, g);
-    for (uint32_t tile0 = tok_lo; tile0 < full_hi; tile0 += kTile) {
-      // Software pipeline: the next tile's loads are in flight while this one is consumed.
-      TileRegs nxt;
-      const uint32_t next0 = tile0 + kTile;
-      if (next0 < full_hi)
-        load_tile<false>(p, nxt, next0, end, page0, physical, lc, hl, g);
-      else if (next0 < tok_hi)
-        load_tile<true>(p, nxt, next0, end, page0, physical, lc, hl, g);
-      consume_tile<false>(cur, q_reg, o, sm, tile0, end, p.scale_log2, g);
-      if (next0 < tok_hi) cur = nxt;
+    // Software pipeline: the next tile's loads are in flight while this one is consumed.
+    if constexpr (NT == 1) {
+      // a decode split is plain tiles followed by at most one masked tile
+      for (uint32_t tile0 = tok_lo; tile0 < full_hi; tile0 += kTile) {
+        TileRegs nxt;
+        const uint32_t next0 = tile0 + kTile;
+        if (next0 < full_hi)
+          load_tile<false>(p, nxt, next0, end, page0, physical, lc, hl, g);
+        else if (next0 < tok_hi)
+          load_tile<true>(p, nxt, next0, end, page0, physical, lc, hl, g);
+        consume_tile<NT, false>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+        if (next0 < tok_hi) cur = nxt;
+      }
+      if (full_hi < tok_hi)
+        consume_tile<NT, true>(cur, q_reg, o, sm, full_hi, limit, p.scale_log2, g);
+    } else {
+      for (uint32_t tile0 = tok_lo; tile0 < tok_hi; tile0 += kTile) {
+        TileRegs nxt;
+        const uint32_t next0 = tile0 + kTile;
+        if (next0 + kTile <= tok_hi)
+          load_tile<false>(p, nxt, next0, end, page0, physical, lc, hl, g);
+        else if (next0 < tok_hi)
+          load_tile<true>(p, nxt, next0, end, page0, physical, lc, hl, g);
+        if (tile0 < full_hi)
+          consume_tile<NT, false>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+        else
+          consume_tile<NT, true>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+        if (next0 < tok_hi) cur = nxt;
+      }
     }
-    if (full_hi < tok_hi) consume_tile<true>(cur, q_reg, o, sm, full_hi, end, p.scale_log2, g);
   }
-  float m_run = sm.m, l_run = sm.l;
-  l_run += __shfl_xor(l_run, 16, 64);
-  l_run += __shfl_xor(l_run, 32, 64);
-  if (hl >= p.group) return;
-  // Lane (head hl, group g) holds value columns 32g + 8j + mt.
-  const uint32_t head = kv_head * p.group + hl;
-  if (plan.splits == 1) {
-    float inv = 1.0f / l_run;
-    uint16_t *out_row = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
+  // Lane (row hl, group g) holds value columns 32g + 8j + mt of its rows.
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    float m_run = sm[nt].m, l_run = sm[nt].l;
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (NT == 1 ? hl >= p.group : member_of[nt] == 0xffffffffu) continue;
+    const uint32_t token = leader + member_of[nt];
+    if (plan.splits == 1) {
+      float inv = 1.0f / l_run;
+      uint16_t *out_row = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
+      for (int j = 0; j < 4; ++j) {
+        uint2 lo = make_uint2(pack_bf16(o[nt][0][j] * inv, o[nt][1][j] * inv),
+                              pack_bf16(o[nt][2][j] * inv, o[nt][3][j] * inv));
+        uint2 hi = make_uint2(pack_bf16(o[nt][4][j] * inv, o[nt][5][j] * inv),
+                              pack_bf16(o[nt][6][j] * inv, o[nt][7][j] * inv));
+        *(uint2 *)(out_row + 32 * g + 8 * j) = lo;
+        *(uint2 *)(out_row + 32 * g + 8 * j + 4) = hi;
+      }
+      continue;
+    }
+    uint64_t slot = ((uint64_t)token * p.max_splits + split) * p.query_heads + head;
+    float *po = p.partial_o + slot * 128 + 32 * g;
     for (int j = 0; j < 4; ++j) {
-      uint2 lo = make_uint2(pack_bf16(o[0][j] * inv, o[1][j] * inv), pack_bf16(o[2][j] * inv, o[3][j] * inv));
-      uint2 hi = make_uint2(pack_bf16(o[4][j] * inv, o[5][j] * inv), pack_bf16(o[6][j] * inv, o[7][j] * inv));
-      *(uint2 *)(out_row + 32 * g + 8 * j) = lo;
-      *(uint2 *)(out_row + 32 * g + 8 * j + 4) = hi;
+      *(float4 *)(po + 8 * j) = make_float4(o[nt][0][j], o[nt][1][j], o[nt][2][j], o[nt][3][j]);
+      *(float4 *)(po + 8 * j + 4) = make_float4(o[nt][4][j], o[nt][5][j], o[nt][6][j], o[nt][7][j]);
     }
-    return;
+    if (g == 0) p.partial_ml[slot] = make_float2(m_run, l_run);
   }
-  uint64_t slot = ((uint64_t)token * p.max_splits + split) * p.query_heads + head;
-  float *po = p.partial_o + slot * 128 + 32 * g;
-  for (int j = 0; j < 4; ++j) {
-    *(float4 *)(po + 8 * j) = make_float4(o[0][j], o[1][j], o[2][j], o[3][j]);
-    *(float4 *)(po + 8 * j + 4) = make_float4(o[4][j], o[5][j], o[6][j], o[7][j]);
-  }
-  if (g == 0) p.partial_ml[slot] = make_float2(m_run, l_run);
+}
+
+// Decode batches: one query token per wave, two waves per SIMD to hide the K/V stream's latency.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void ragged_attention_mfma_kernel(
+    FastRagged p, ErrorSlot *error) {
+  ragged_attention_body<1>(p, error);
+}
+
+// Prefill chunks: two query tiles per wave share every K/V tile (one wave per SIMD, the whole
+// register file).
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void ragged_attention_prefill_kernel(
+    FastRagged p, ErrorSlot *error) {
+  ragged_attention_body<2>(p, error);
 }
 
 // Merges the per-split partials of one (token, head): out = sum_s O_s 2^(m_s-M) / sum_s l_s
@@ -620,10 +714,14 @@ void launch_plan(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
 }
 
 void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
-  uint64_t blocks = (uint64_t)f.tokens * f.max_splits * f.kv_heads;
+  uint64_t groups = f.group_tokens > 1 ? f.tokens / f.group_tokens + f.lanes : f.tokens;
+  uint64_t blocks = groups * f.max_splits * f.kv_heads;
   {
     KernelTimer timer(backend, FH_KC_ATTENTION_KERNEL);
-    ragged_attention_mfma_kernel<<<dim3((unsigned)blocks), 64, 0, stream>>>(f, error);
+    if (f.group_tokens > 1)
+      ragged_attention_prefill_kernel<<<dim3((unsigned)blocks), 64, 0, stream>>>(f, error);
+    else
+      ragged_attention_mfma_kernel<<<dim3((unsigned)blocks), 64, 0, stream>>>(f, error);
   }
   ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens), 64, 0, stream>>>(f);
 }
@@ -651,6 +749,7 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   f.physical_pages = lane.physical_pages;
   f.table_pages = lane.logical_pages;
   f.max_splits = splits_for(f.tokens);
+  f.group_tokens = f.tokens > 1 ? 2 * (16 / group) : 1;
   f.scale_log2 = lane.scale * 1.4426950408889634f;
   f.one_start = lane.query_start;
   f.fixed_attended = lane.causal ? 0 : lane.key_length;
@@ -703,6 +802,7 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     f.query_heads = p.query_heads;
     f.kv_heads = p.kv_heads;
     f.group = p.query_heads / p.kv_heads;
+    f.group_tokens = p.tokens > p.lanes ? 2 * (16 / f.group) : 1;
     f.page_tokens = p.page_tokens;
     f.physical_pages = p.physical_pages;
     f.table_pages = p.table_pages;

@@ -428,6 +428,9 @@ PAGED_CASES = [
     (4, 2, 5, 37, 32, True, DType.BF16, 16),
     (4, 4, 3, 33, 0, False, DType.F16, 16),
     (2, 1, 4, 20, 16, True, DType.F32, 4),
+    (40, 8, 77, 177, 100, True, DType.BF16, 16),     # prefill chunk through the single-lane op
+    (16, 8, 50, 90, 0, False, DType.BF16, 16),       # non-causal: every row attends key_length
+    (32, 4, 130, 130, 0, True, DType.BF16, 16),
 ]
 
 
@@ -559,6 +562,10 @@ RAGGED_CASES = [
     ([300, 1, 2047, 700, 15, 16, 0], [1, 1, 1, 1, 1, 1, 1], 32, 4, 16),
     ([40, 0, 100], [1, 5, 3], 8, 2, 16),                           # decode + prefill chunks
     ([100, 257], [1, 1], 32, 4, 64),                               # engine page size
+    ([0, 130, 33, 900], [70, 1, 45, 1], 40, 8, 16),                # prefill chunks of a 5-head group + decode rows
+    ([0, 64], [200, 37], 16, 8, 16),                               # 16 tokens per query group, ragged tails
+    ([500], [96], 32, 4, 16),                                      # a chunk continuing a long context
+    ([0, 5], [33, 31], 4, 4, 16),                                  # one head per kv head: 32 tokens per group
 ]
 
 

@@ -229,6 +229,27 @@ def prefill_gemm_c4(backend, rows=8256, seed=91, repeats=3):
     }
 
 
+def stream_read_rate(backend, rows=4096, width=1 << 20, repeats=3):
+    """What a plain read-only stream sustains on this device: a row-wise argmax over 8 GiB of
+    bf16 (16-byte loads, one workgroup per row).  The practical ceiling the HBM-bound kernels are
+    up against, next to the nominal one."""
+    source = backend.alloc(DType.BF16, (rows, width))
+    result = backend.alloc(DType.U32, (rows,))
+    commands = CommandList()
+    commands.dispatch(Op.argmax(), [source], result)
+    encoded = backend.encode(commands)
+    backend.submit(encoded).wait()
+    backend.profile_enable(2)
+    backend.profile_reset()
+    for _ in range(repeats):
+        backend.submit(encoded).wait()
+    ns, _ = backend.profile_read(0)
+    backend.profile_enable(0)
+    backend.release(source)
+    backend.release(result)
+    return 2.0 * rows * width * repeats / (ns * 1e-9) / 1e9
+
+
 def prefill_attention_c4(backend, seed=93, repeats=3):
     """Paged attention of one BASELINE config 4 layer: an 8192-token chunk packed from 6 prompts
     (512..3072 tokens, from empty contexts) plus 64 decode rows (contexts uniform 128..4096), 40
@@ -324,7 +345,7 @@ def main():
             commands.dispatch(Op.copy(), [source], target)
             backend.submit(commands).wait()
         print(json.dumps({"copy_bytes_read": elements * 4, "copy_bytes_written": elements * 4,
-                          "kernel": "copy_kernel", "launches": 8}))
+                          "kernel": "copy_flat_kernel", "launches": 8}))
         return
     if args.prefill_only:
         backend = HipBackend(0)
@@ -456,7 +477,11 @@ def main():
             breakdown[name] = class_ns / 1e6 / extra
         result["gpu_ms_per_step_by_op"] = breakdown
         backend.profile_enable(0)
-        result["secondary_workloads"] = {"prefill_gemm_c4": prefill_gemm_c4(backend)}
+        result["roofline"]["measured_stream_read_gbps"] = stream_read_rate(backend)
+        result["roofline"]["frac_of_measured_stream_read"] = (
+            result["roofline"]["achieved"] / result["roofline"]["measured_stream_read_gbps"])
+        result["secondary_workloads"] = {"prefill_gemm_c4": prefill_gemm_c4(backend),
+                                         "prefill_attention_c4": prefill_attention_c4(backend)}
         if config.moe:
             result["secondary_workloads"]["moe_block_c2"] = moe_block_c2(backend, workload.model)
     step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction

@@ -452,9 +452,11 @@ __device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[NT
 // of the item's group, head hl % group of the kv head), per_tile = 16 / group.
 template <int NT>
 __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *error) {
-  const uint32_t lane = threadIdx.x, hl = lane & 15, g = lane >> 4;
-  const uint32_t item = blockIdx.x / p.kv_heads, kv_head = blockIdx.x % p.kv_heads;
-  if (item >= p.item_count[0]) return;
+  // a workgroup is one work item; its waves take one kv head each, so the slices of a K/V page
+  // (one 256-byte piece of every token row per kv head) are requested close together in time
+  const uint32_t lane = threadIdx.x & 63, hl = lane & 15, g = lane >> 4;
+  const uint32_t item = blockIdx.x, kv_head = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= p.item_count[0] || kv_head >= p.kv_heads) return;
   const uint2 work = p.items[item];
   const uint32_t leader = work.x, split = work.y;
   const TokenPlan plan = p.plans[leader];
@@ -595,14 +597,14 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
 }
 
 // Decode batches: one query token per wave, two waves per SIMD to hide the K/V stream's latency.
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void ragged_attention_mfma_kernel(
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void ragged_attention_mfma_kernel(
     FastRagged p, ErrorSlot *error) {
   ragged_attention_body<1>(p, error);
 }
 
 // Prefill chunks: two query tiles per wave share every K/V tile (one wave per SIMD, the whole
 // register file).
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void ragged_attention_prefill_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void ragged_attention_prefill_kernel(
     FastRagged p, ErrorSlot *error) {
   ragged_attention_body<2>(p, error);
 }
@@ -715,13 +717,19 @@ void launch_plan(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
 
 void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
   uint64_t groups = f.group_tokens > 1 ? f.tokens / f.group_tokens + f.lanes : f.tokens;
-  uint64_t blocks = groups * f.max_splits * f.kv_heads;
+  uint64_t blocks = groups * f.max_splits;
   {
     KernelTimer timer(backend, FH_KC_ATTENTION_KERNEL);
-    if (f.group_tokens > 1)
-      ragged_attention_prefill_kernel<<<dim3((unsigned)blocks), 64, 0, stream>>>(f, error);
-    else
-      ragged_attention_mfma_kernel<<<dim3((unsigned)blocks), 64, 0, stream>>>(f, error);
+    // one workgroup per work item, up to 8 (decode) or 4 (prefill) kv heads of it per workgroup
+    if (f.group_tokens > 1) {
+      const uint32_t waves = f.kv_heads < 4 ? f.kv_heads : 4;
+      ragged_attention_prefill_kernel<<<dim3((unsigned)blocks, (f.kv_heads + waves - 1) / waves),
+                                        64 * waves, 0, stream>>>(f, error);
+    } else {
+      const uint32_t waves = f.kv_heads < 8 ? f.kv_heads : 8;
+      ragged_attention_mfma_kernel<<<dim3((unsigned)blocks, (f.kv_heads + waves - 1) / waves),
+                                     64 * waves, 0, stream>>>(f, error);
+    }
   }
   ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens), 64, 0, stream>>>(f);
 }

@@ -21,7 +21,12 @@
 //     packed weights are requested two steps ahead (they are cold in HBM);
 //   * a thread dequantises one weight row of the tile per step (64 nibbles): two nibbles become
 //     the fp16 pair (1024+q) with one and-or, minus 1024 exactly, then one packed fused
-//     multiply-add gives scale*q+bias rounded once.  That needs every scale and bias to lie
+//     multiply-add gives scale*q - c rounded once, with c ~ 7.5*scale the fp16 value that centres
+//     the group.  What the centring takes out, (bias + c) * sum of the group's activations, is
+//     added back exactly: the row sums per group come from prepare_rows_kernel in f32 and an f32
+//     MFMA adds the rank-2 update of every two groups to the same accumulators.  Centred values
+//     are half the magnitude of the weights and carry no bias, which keeps the fp16 rounding
+//     inside the tolerance at the deepest contractions (K = 17408).  That needs every scale and bias to lie
 //     well inside the fp16 range; check_affine_kernel scans them first and raises a flag
 //     otherwise, and then a second instantiation of the kernel, which dequantises in f32, does
 //     the work instead (both are launched; the one whose turn it is not returns at once).  Every weight byte is read from HBM once per 256 rows and unpacked once per
@@ -31,6 +36,8 @@
 //     workgroups and each weight tile to 4, instead of every workgroup streaming its own.
 // Accumulation is f32.
 #include "fast_kernels.hpp"
+
+#include <type_traits>
 
 namespace fh {
 
@@ -46,11 +53,13 @@ constexpr int kBand = 8;   // column tiles per band of the tile numbering
 constexpr int kPitch = 2 * kBK + 16;              // bytes per staged weight row
 constexpr int kATileBytes = kBM * 2 * kBK;        // activation tile, swizzled, no padding
 constexpr int kBTileBytes = kBN * kPitch;         // weight tile
-constexpr int kGemmLds = 2 * (kATileBytes + kBTileBytes);
+constexpr int kSideBytes = 4 * (kBM + kBN) * 4;  // row sums and column offsets of four groups, f32
+constexpr int kGemmLds = 2 * (kATileBytes + kBTileBytes) + kSideBytes;
 
 struct GemmArgs {
   const uint16_t *x;        // fp16 rows prepared by prepare_rows_kernel, stride = inner
   const float *row_unscale; // per row: multiply the result by this
+  const float *group_sums;  // [inner / 64][rows]: sums of the prepared rows per group
   uint64_t x_row_stride;
   const uint32_t *packed;
   const uint16_t *scales, *biases;
@@ -76,7 +85,7 @@ __device__ inline uint32_t pack_f16(float lo, float hi) {
 
 // Eight nibbles of `w`, dequantised to fp16, as the four pairs (0,4)(1,5)(2,6)(3,7).
 // Fast form: (1024+q) pairs by and-or, minus 1024 (exact), then fused scale*q+bias per pair.
-__device__ inline uint4 dequantise_word(uint32_t w, f16x2 scale2, f16x2 bias2) {
+__device__ inline uint4 dequantise_word(uint32_t w, f16x2 scale2, f16x2 shift2) {
   const uint32_t mask = 0x000f000fu, magic = 0x64006400u;
   const f16x2 offset = {(_Float16)1024.0f, (_Float16)1024.0f};
   uint32_t raw[4] = {(w & mask) | magic, ((w >> 4) & mask) | magic, ((w >> 8) & mask) | magic,
@@ -85,16 +94,16 @@ __device__ inline uint4 dequantise_word(uint32_t w, f16x2 scale2, f16x2 bias2) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const f16x2 q = __builtin_bit_cast(f16x2, raw[i]) - offset;
-    out[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(q, scale2, bias2));
+    out[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(q, scale2, shift2));
   }
   return make_uint4(out[0], out[1], out[2], out[3]);
 }
 
-// The same in f32 with one rounding to fp16, for scales or biases outside the fp16 normal range.
-__device__ inline uint4 dequantise_word_wide(uint32_t w, float scale, float bias) {
+// The same in f32 with one rounding to fp16, for scales or biases outside the fp16 range.
+__device__ inline uint4 dequantise_word_wide(uint32_t w, float scale, float shift) {
   float v[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(scale, (float)((w >> (4 * i)) & 15u), bias);
+  for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(scale, (float)((w >> (4 * i)) & 15u), shift);
   return make_uint4(pack_f16(v[0], v[4]), pack_f16(v[1], v[5]), pack_f16(v[2], v[6]),
                     pack_f16(v[3], v[7]));
 }
@@ -108,10 +117,12 @@ __device__ inline bool f16_safe(float scale, float bias) {
 
 // x bf16 [rows, inner] -> fp16 [rows, inner] (every 8 values stored as 0,4,1,5,2,6,3,7), each row
 // multiplied by a power of two that brings its largest magnitude under 2^15; unscale[row] is the
-// inverse.  One wave per row.
+// inverse; group_sums[g][row] is the f32 sum of the row's 64 prepared values of group g.
+// One wave per row.
 __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, uint64_t x_row_stride,
                                                            uint32_t rows, uint32_t inner,
-                                                           uint16_t *out, float *unscale) {
+                                                           uint16_t *out, float *unscale,
+                                                           float *group_sums) {
   const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= rows) return;
   const uint16_t *in_row = x + (uint64_t)row * x_row_stride;
@@ -144,6 +155,12 @@ __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, ui
     }
     *(uint4 *)(out_row + 8 * piece) = make_uint4(pack_f16(f[0], f[4]), pack_f16(f[1], f[5]),
                                                  pack_f16(f[2], f[6]), pack_f16(f[3], f[7]));
+    // eight consecutive pieces (= lanes) make one group; the scaled values are exact in f32
+    float sum = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    sum += __shfl_xor(sum, 4, 64);
+    if ((piece & 7) == 0) group_sums[(uint64_t)(piece >> 3) * rows + row] = sum;
   }
 }
 
@@ -161,6 +178,8 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
   unsigned char *a_tiles = gemm_lds;                      // [2][kBM][128], pieces swizzled
   unsigned char *b_tiles = gemm_lds + 2 * kATileBytes;    // [2][kBN][kPitch]
+  float *side_rows = (float *)(gemm_lds + 2 * (kATileBytes + kBTileBytes));   // [4][kBM], ring by group
+  float *side_cols = side_rows + 4 * kBM;                                     // [4][kBN]
   const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const uint32_t wm = wave >> 1, wn = wave & 1;
   const uint32_t l32 = lane & 31, kh = lane >> 5;
@@ -206,11 +225,22 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   const uint16_t *b_row = a.biases + (uint64_t)b_col * steps;
   uint4 w_now[2], w_next[2];
   uint32_t affine_now, affine_next;   // scale | bias << 16
+  float sum_now, sum_next;            // group sum of tile row `tid`
+  const float *sums_of_row = a.group_sums + min(row0 + tid, a.rows - 1);
   auto fetch_w = [&](uint32_t step) {
     const uint32_t st = min(step, steps - 1);
     w_next[0] = *(const uint4 *)(w_row + st * 8);
     w_next[1] = *(const uint4 *)(w_row + st * 8 + 4);
     affine_next = (uint32_t)s_row[st] | ((uint32_t)b_row[st] << 16);
+    sum_next = sums_of_row[(uint64_t)st * a.rows];
+  };
+  // The group's centre c (an fp16 value near 7.5 * scale) and what it leaves to add back per
+  // unit of activation sum: bias + c.
+  auto centre_of = [&](float scale) { return (float)(_Float16)(7.5f * scale); };
+  auto stage_side = [&](uint32_t step) {
+    const float scale = bf16_bits_to_f32(affine_now & 0xffffu), bias = bf16_bits_to_f32(affine_now >> 16);
+    side_rows[(step & 3) * kBM + tid] = sum_now;
+    side_cols[(step & 3) * kBN + tid] = bias + (kWide ? 7.5f * scale : centre_of(scale));
   };
   // one packed word (8 values) of the weight row: `part` 0..7
   auto stage_b = [&](uint32_t buffer, int part) {
@@ -218,11 +248,13 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
     const float scale = bf16_bits_to_f32(affine_now & 0xffffu), bias = bf16_bits_to_f32(affine_now >> 16);
     const uint4 w = w_now[part / 4];
     const uint32_t word = (part & 3) == 0 ? w.x : ((part & 3) == 1 ? w.y : ((part & 3) == 2 ? w.z : w.w));
+    (void)bias;
     if (kWide) {
-      *(uint4 *)(bt) = dequantise_word_wide(word, scale, bias);
+      *(uint4 *)(bt) = dequantise_word_wide(word, scale, -7.5f * scale);
     } else {
-      const f16x2 scale2 = {(_Float16)scale, (_Float16)scale}, bias2 = {(_Float16)bias, (_Float16)bias};
-      *(uint4 *)(bt) = dequantise_word(word, scale2, bias2);
+      const _Float16 shift = (_Float16)(-centre_of(scale));
+      const f16x2 scale2 = {(_Float16)scale, (_Float16)scale}, shift2 = {shift, shift};
+      *(uint4 *)(bt) = dequantise_word(word, scale2, shift2);
     }
   };
 
@@ -239,40 +271,40 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   w_now[0] = w_next[0];
   w_now[1] = w_next[1];
   affine_now = affine_next;
+  sum_now = sum_next;
   fetch_w(1);
   for (int part = 0; part < 8; ++part) stage_b(0, part);
+  stage_side(0);
   __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's rows have landed in LDS
   __syncthreads();
   const uint32_t swizzle = (l32 >> 1) & 7;
-  for (uint32_t step = 0; step < steps; ++step) {
-    const uint32_t buffer = step & 1;
+  // One K step on LDS buffer kBuffer (= step & 1); the loop below runs them in pairs so that the
+  // buffer, and the centring update after every second step, are fixed at compile time.
+  auto k_step = [&](uint32_t step, auto parity) {
+    constexpr uint32_t buffer = decltype(parity)::value;
     stage_a(buffer ^ 1, min(step + 1, steps - 1));
     w_now[0] = w_next[0];   // weights of step+1: requested a whole step ago
     w_now[1] = w_next[1];
     affine_now = affine_next;
+    sum_now = sum_next;
     fetch_w(step + 2);
     const unsigned char *at = a_tiles + buffer * kATileBytes + (128 * wm + l32) * 128;
     const unsigned char *bt = b_tiles + buffer * kBTileBytes + (128 * wn + l32) * kPitch + 16 * kh;
-    // operand fragments are read one sub-step ahead of the MFMAs that use them
-    f16x8 a_op[2][4], b_op[2][4];
-    auto read_fragments = [&](int slot, int sub) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        a_op[slot][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * 128 + 16 * ((2 * sub + kh) ^ swizzle)));
-        b_op[slot][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kPitch + 32 * sub));
-      }
-    };
-    read_fragments(0, 0);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      if (s < 3) read_fragments((s + 1) & 1, s + 1);
+      f16x8 a_op[4], b_op[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * 128 + 16 * ((2 * s + kh) ^ swizzle)));
+        b_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kPitch + 32 * s));
+      }
       // eight MFMAs, then one word of the next step's weights, fenced so that the staging
       // instructions issue in the shadow of the matrix pipe instead of after all sixteen
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
         if (i & 1) {
           __builtin_amdgcn_sched_barrier(0);
           stage_b(buffer ^ 1, 2 * s + (i >> 1));
@@ -280,8 +312,29 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
         }
       }
     }
-    __builtin_amdgcn_s_waitcnt(0x0f74);   // vmcnt(4): all but the four weight loads just issued
+    // after the second step of a pair: the centring terms of the two groups just multiplied,
+    // as one f32 MFMA per accumulator tile (lane half kh supplies group step - 1 + kh of both
+    // operands)
+    if (buffer == 1) {
+      float row_sum[4], column_offset[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        row_sum[i] = side_rows[((step - 1 + kh) & 3) * kBM + 128 * wm + 32 * i + l32];
+        column_offset[i] = side_cols[((step - 1 + kh) & 3) * kBN + 128 * wn + 32 * i + l32];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(row_sum[i], column_offset[j], acc[i][j], 0, 0, 0);
+    }
+    stage_side(step + 1);   // a ring slot nobody reads in this step
+    __builtin_amdgcn_s_waitcnt(0x0f75);   // vmcnt(5): all but the five loads of fetch_w just issued
     __syncthreads();
+  };
+  for (uint32_t step = 0; step < steps; step += 2) {   // K is a multiple of 256: steps is even
+    k_step(step, std::integral_constant<uint32_t, 0>{});
+    k_step(step + 1, std::integral_constant<uint32_t, 1>{});
   }
   // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile
 #pragma unroll
@@ -308,12 +361,14 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
 bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
   const uint64_t rows_bytes = ((uint64_t)p.rows * p.inner * 2 + 255) / 256 * 256;
   const uint64_t unscale_bytes = ((uint64_t)p.rows * sizeof(float) + 255) / 256 * 256;
-  char *ws = backend_workspace(backend, rows_bytes + unscale_bytes + 256);
+  const uint64_t sums_bytes = ((uint64_t)p.rows * (p.inner / kBK) * sizeof(float) + 255) / 256 * 256;
+  char *ws = backend_workspace(backend, rows_bytes + unscale_bytes + sums_bytes + 256);
   if (!ws) return false;
   hipStream_t stream = backend_stream(backend);
   GemmArgs a{};
   a.x = (const uint16_t *)ws;
   a.row_unscale = (const float *)(ws + rows_bytes);
+  a.group_sums = (const float *)(ws + rows_bytes + unscale_bytes);
   a.x_row_stride = p.inner;
   a.packed = (const uint32_t *)p.packed.base + p.packed.offset;
   a.scales = (const uint16_t *)p.scales.base + p.scales.offset;
@@ -327,7 +382,7 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
   a.columns = p.columns;
   a.row_tiles = (p.rows + kBM - 1) / kBM;
   a.column_tiles = (p.columns + kBN - 1) / kBN;
-  uint32_t *flag = (uint32_t *)(ws + rows_bytes + unscale_bytes);
+  uint32_t *flag = (uint32_t *)(ws + rows_bytes + unscale_bytes + sums_bytes);
   a.wide_flag = flag;
   static bool configured = false;   // raise the dynamic LDS limit once per process
   if (!configured) {
@@ -342,7 +397,7 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
   KernelTimer timer(backend, FH_KC_QMM_KERNEL);
   prepare_rows_kernel<<<(p.rows + 3) / 4, 256, 0, stream>>>(
       (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, (uint16_t *)ws,
-      (float *)(ws + rows_bytes));
+      (float *)(ws + rows_bytes), (float *)(ws + rows_bytes + unscale_bytes));
   launch_fill_u32(stream, flag, 1, 0);
   const uint64_t affine_count = (uint64_t)p.columns * (p.inner / kBK);
   check_affine_kernel<<<(uint32_t)((affine_count + 255) / 256), 256, 0, stream>>>(a.scales, a.biases,

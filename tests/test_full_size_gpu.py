@@ -1,0 +1,190 @@
+"""The BASELINE configurations at their full sizes, where the CPU oracle is out of reach.
+
+Each case runs the operation twice on the device with the same seeded data: once through the
+specialised bf16 kernels and once through the strided generic kernels (reached by giving the
+activations as f32; those kernels follow the oracle's arithmetic order and are checked against it
+at small sizes in test_parity_gpu.py).  The two are independent implementations, and they must
+agree to the stated bf16 bar, |a - b| <= 1e-2 + 1e-2 |b|.  Paging is checked through its
+round-trip property: rows appended through block tables read back bit for bit."""
+import math
+
+import numpy as np
+import pytest
+
+from forja_amd import programs
+from forja_amd.core import CommandList, DType, Op
+from tests.helpers import assert_close, to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def seeded(hip, dtype, shape, seed, stream, kind=2, lo=0.0, hi=0.0):
+    tensor = hip.alloc(dtype, shape)
+    commands = CommandList()
+    commands.dispatch(Op.fill_seeded(kind, seed, stream, lo=lo, hi=hi), [], tensor)
+    hip.submit(commands).wait()
+    return tensor
+
+
+def as_f32(hip, tensor):
+    wide = hip.alloc(DType.F32, tensor.shape)
+    commands = CommandList()
+    commands.dispatch(Op.copy(), [tensor], wide)
+    hip.submit(commands).wait()
+    return wide
+
+
+def quantised(hip, n, k, seed, experts=None):
+    lead = () if experts is None else (experts,)
+    packed = seeded(hip, DType.U32, lead + (n, k // 8), seed, 1, kind=0)
+    scales = seeded(hip, DType.BF16, lead + (n, k // 64), seed, 2, kind=1, lo=0.001, hi=0.02)
+    biases = seeded(hip, DType.BF16, lead + (n, k // 64), seed, 3, kind=1, lo=-0.1, hi=0.1)
+    return [packed, scales, biases]
+
+
+def run(hip, commands):
+    hip.submit(commands).wait()
+
+
+def release(hip, *tensors):
+    for tensor in tensors:
+        hip.release(tensor)
+
+
+@pytest.mark.parametrize("rows,n,k,note", [
+    (128, 5120, 2048, "config 3 stacked qkv"),
+    (128, 2048, 4096, "config 3 o_proj"),
+    (128, 128, 2048, "config 3 router"),
+    (128, 151936, 2048, "config 3 lm_head"),
+    (2048, 4096, 1024, "config 1 stacked qkv over the packed 2048-token batch"),
+    (8256, 512, 5120, "config 4 prefill rows, a 512-column slice of a projection"),
+    (8256, 256, 17408, "config 4 down projection depth, a 256-column slice"),
+])
+def test_quantised_projection_fast_and_generic_paths_agree(hip, rows, n, k, note):
+    weights = quantised(hip, n, k, seed=101)
+    x = seeded(hip, DType.BF16, (rows, k), 101, 4)
+    x_wide = as_f32(hip, x)
+    fast = hip.alloc(DType.BF16, (rows, n))
+    generic = hip.alloc(DType.F32, (rows, n))
+    commands = CommandList()
+    commands.dispatch(Op.quant_matmul(4, 64), [x, *weights], fast)
+    commands.dispatch(Op.quant_matmul(4, 64), [x_wide, *weights], generic)
+    run(hip, commands)
+    assert_close(to_f32(hip.read(fast), DType.BF16), to_f32(hip.read(generic), DType.F32), DType.BF16)
+    release(hip, x, x_wide, fast, generic, *weights)
+
+
+def test_config2_moe_block_fast_and_generic_paths_agree(hip):
+    """256 decode tokens, 128 experts, top-8 of N(0,1) router logits, expert SwiGLU 2048 x 768."""
+    tokens, hidden, experts, top_k, inner = 256, 2048, 128, 8, 768
+    gate, up = quantised(hip, inner, hidden, 201, experts), quantised(hip, inner, hidden, 202, experts)
+    down = quantised(hip, hidden, inner, 203, experts)
+    x = seeded(hip, DType.BF16, (tokens, hidden), 204, 1)
+    logits = seeded(hip, DType.BF16, (tokens, experts), 204, 2)
+    weights = hip.alloc(DType.BF16, (tokens, top_k))
+    indices = hip.alloc(DType.U32, (tokens, top_k))
+    swiglu = hip.prepare_epilogue(programs.silu_mul_elements())
+    activated = hip.alloc(DType.BF16, (tokens, top_k, inner))
+    out = hip.alloc(DType.BF16, (tokens, hidden))
+    gq = Op.gather_quant_matmul(4, 64)
+    commands = CommandList()
+    commands.dispatch_many(Op.top_k(top_k, True), [logits], [weights, indices])
+    commands.dispatch_epilogue(gq, [x, *gate, *up, indices], activated, swiglu, [])
+    commands.dispatch(gq, [activated, *down, indices, weights], out)
+    run(hip, commands)
+    chosen = np.frombuffer(hip.read(indices), np.uint32)
+    counts = np.bincount(chosen, minlength=experts)
+    assert counts.sum() == tokens * top_k and counts.max() <= 40 and len(np.unique(chosen)) > 120
+    # the same block through the generic kernels: f32 activations and route weights
+    x_wide, weights_wide, activated_from_fast = as_f32(hip, x), as_f32(hip, weights), as_f32(hip, activated)
+    activated_wide = hip.alloc(DType.F32, (tokens, top_k, inner))
+    out_wide = hip.alloc(DType.F32, (tokens, hidden))
+    commands = CommandList()
+    commands.dispatch_epilogue(gq, [x_wide, *gate, *up, indices], activated_wide, swiglu, [])
+    commands.dispatch(gq, [activated_from_fast, *down, indices, weights_wide], out_wide)
+    run(hip, commands)
+    assert_close(to_f32(hip.read(activated), DType.BF16), to_f32(hip.read(activated_wide), DType.F32),
+                 DType.BF16)
+    assert_close(to_f32(hip.read(out), DType.BF16), to_f32(hip.read(out_wide), DType.F32), DType.BF16)
+
+
+def ragged_batch(hip, contexts, counts, hq, hkv, pt, seed):
+    """Device-seeded ragged batch with shuffled block tables; returns the tensors by name."""
+    rng = np.random.default_rng(seed)
+    lanes = len(contexts)
+    pages_of = [(c + n + pt - 1) // pt for c, n in zip(contexts, counts)]
+    table_pages, physical = max(pages_of) + 1, sum(pages_of) + 3
+    order = rng.permutation(physical)
+    tables = np.zeros((lanes, table_pages, 2), np.uint32)
+    tables[:, :, 1] = 0xffffffff
+    cursor = 0
+    for lane, need in enumerate(pages_of):
+        pages = order[cursor:cursor + need]
+        cursor += need
+        tables[lane, :need, 0] = pages
+        tables[lane, :need, 1] = 11 + pages
+    total = sum(counts)
+
+    def up(array, shape):
+        tensor = hip.alloc(DType.U32, shape)
+        hip.write(tensor, np.ascontiguousarray(array, dtype=np.uint32).tobytes())
+        return tensor
+    return dict(
+        tables=up(tables, tables.shape), generations=up(11 + np.arange(physical), (physical,)),
+        cu=up(np.concatenate([[0], np.cumsum(counts)]), (lanes + 1,)), starts=up(contexts, (lanes,)),
+        activity=up(np.ones(lanes), (lanes,)),
+        q=seeded(hip, DType.BF16, (total, hq, 128), seed, 1),
+        k_new=seeded(hip, DType.BF16, (total, hkv, 128), seed, 2),
+        v_new=seeded(hip, DType.BF16, (total, hkv, 128), seed, 3),
+        keys=seeded(hip, DType.BF16, (physical, pt, hkv, 128), seed, 4),
+        values=seeded(hip, DType.BF16, (physical, pt, hkv, 128), seed, 5),
+        table_array=tables, total=total)
+
+
+def attention_both_ways(hip, contexts, counts, hq, hkv):
+    pt, scale = 16, 1.0 / math.sqrt(128)
+    t = ragged_batch(hip, contexts, counts, hq, hkv, pt, seed=301)
+    tail = [t["tables"], t["generations"], t["cu"], t["starts"], t["activity"]]
+    fast = hip.alloc(DType.BF16, (t["total"], hq, 128))
+    commands = CommandList()
+    commands.dispatch_many(Op.paged_attention_ragged(scale, pt), [t["q"], t["k_new"], t["v_new"], *tail],
+                           [fast, t["keys"], t["values"]])
+    run(hip, commands)
+    keys_after = hip.read(t["keys"])
+    wide = [as_f32(hip, t[name]) for name in ("q", "k_new", "v_new")]
+    generic = hip.alloc(DType.F32, (t["total"], hq, 128))
+    commands = CommandList()
+    commands.dispatch_many(Op.paged_attention_ragged(scale, pt), [*wide, *tail],
+                           [generic, t["keys"], t["values"]])
+    run(hip, commands)
+    assert hip.read(t["keys"]) == keys_after          # appending the same rows again changes nothing
+    assert_close(to_f32(hip.read(fast), DType.BF16), to_f32(hip.read(generic), DType.F32), DType.BF16)
+    # round trip of the appended rows of the longest lane through its block table
+    lane = int(np.argmax(np.array(contexts) + np.array(counts)))
+    first = int(np.cumsum([0] + list(counts))[lane])
+    new_rows = np.frombuffer(hip.read(t["k_new"]), np.uint16).reshape(t["total"], hkv * 128)
+    pool = np.frombuffer(keys_after, np.uint16).reshape(-1, pt, hkv * 128)
+    for offset in range(counts[lane]):
+        position = contexts[lane] + offset
+        page = int(t["table_array"][lane, position // pt, 0])
+        assert np.array_equal(pool[page, position % pt], new_rows[first + offset])
+
+
+def test_config3_decode_attention_full_batch(hip):
+    """128 decode lanes, contexts log-uniform over 256..32768, 32 query / 4 kv heads."""
+    rng = np.random.default_rng(7)
+    contexts = np.exp(rng.uniform(math.log(256), math.log(32768), 128)).astype(int).tolist()
+    attention_both_ways(hip, contexts, [1] * 128, 32, 4)
+
+
+def test_config1_packed_batch_attention(hip):
+    """48 decode lanes (contexts uniform 128..4096) and prefill chunks of 256, 384, 512 and 848
+    tokens packed into 2048 tokens, 16 query / 8 kv heads."""
+    rng = np.random.default_rng(8)
+    contexts = rng.integers(128, 4097, 48).tolist() + [0, 0, 0, 0]
+    attention_both_ways(hip, contexts, [1] * 48 + [256, 384, 512, 848], 16, 8)
+
+
+def test_config4_prefill_attention_largest_prompt(hip):
+    """The 3072-token prompt of the config 4 chunk plus decode rows, 40 query / 8 kv heads."""
+    attention_both_ways(hip, [0, 1500, 4000], [3072, 1, 1], 40, 8)

@@ -267,16 +267,16 @@ __device__ inline TokenPlan plan_token(const FastRagged &p, uint32_t token, uint
   return plan;
 }
 
-// One workgroup: plans every token, compacts the live (token, split) pairs and clears the
-// per-token failure flags.
+// One workgroup: plans every token, clears the per-token failure flags and lists the live
+// (group leader, split) work items longest first (by split length, 32-token classes), so that the
+// hardware, which starts workgroups in list order, ends the launch on its shortest items.
+constexpr uint32_t kSizeClasses = 65;   // split length / 32, clamped
+
 __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlot *error) {
-  __shared__ uint32_t wave_totals[4];
-  __shared__ uint32_t running;
+  __shared__ uint32_t class_items[kSizeClasses];   // items per class, then the class's cursor
   __shared__ unsigned long long total_attended;
-  if (threadIdx.x == 0) {
-    running = 0;
-    total_attended = 0;
-  }
+  for (uint32_t c = threadIdx.x; c < kSizeClasses; c += 256) class_items[c] = 0;
+  if (threadIdx.x == 0) total_attended = 0;
   __syncthreads();
   // Split length: long enough that a wave's fixed start-up cost (plan, table, query) is small
   // against its stream, short enough that the batch still yields ~kTargetItems work items.
@@ -293,38 +293,39 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
     if (split_tokens < kMinSplitTokens) split_tokens = kMinSplitTokens;
     if (split_tokens > kMaxSplitTokens) split_tokens = kMaxSplitTokens;
   }
-  for (uint32_t base = 0; base < p.tokens; base += 256) {
-    uint32_t token = base + threadIdx.x;
-    TokenPlan plan{0, 0, 0, 0, 0, 1};
-    if (token < p.tokens) {
-      plan = plan_token(p, token, split_tokens);
-      uint32_t bad = 0;
-      if (plan.lane == 0xffffffffu) {
-        report_error(error, p.table_pages);
-        bad = 1;
-        plan.lane = 0;
-      }
-      p.bad[token] = bad;
-      p.plans[token] = plan;
+  auto class_of = [](const TokenPlan &plan) {
+    const uint32_t c = plan.chunk / kTile;
+    return c < kSizeClasses ? c : kSizeClasses - 1;
+  };
+  for (uint32_t token = threadIdx.x; token < p.tokens; token += 256) {
+    TokenPlan plan = plan_token(p, token, split_tokens);
+    uint32_t bad = 0;
+    if (plan.lane == 0xffffffffu) {
+      report_error(error, p.table_pages);
+      bad = 1;
+      plan.lane = 0;
     }
-    // work items come from group leaders only
-    const uint32_t my_items = (token < p.tokens && plan.leader == token) ? plan.splits : 0;
-    uint32_t inclusive = my_items;
-    for (int offset = 1; offset < 64; offset <<= 1) {
-      uint32_t other = __shfl_up(inclusive, offset, 64);
-      if ((int)(threadIdx.x & 63) >= offset) inclusive += other;
-    }
-    if ((threadIdx.x & 63) == 63) wave_totals[threadIdx.x >> 6] = inclusive;
-    __syncthreads();
-    uint32_t before = running;
-    for (uint32_t w = 0; w < (threadIdx.x >> 6); ++w) before += wave_totals[w];
-    uint32_t first = before + inclusive - my_items;
-    for (uint32_t s = 0; s < my_items; ++s) p.items[first + s] = make_uint2(token, s);
-    __syncthreads();
-    if (threadIdx.x == 255) running = before + inclusive;
-    __syncthreads();
+    p.bad[token] = bad;
+    p.plans[token] = plan;
+    if (plan.leader == token && plan.splits) atomicAdd(&class_items[class_of(plan)], plan.splits);
   }
-  if (threadIdx.x == 0) p.item_count[0] = running;
+  __syncthreads();
+  if (threadIdx.x == 0) {   // class counts -> first item of each class, longest class first
+    uint32_t running = 0;
+    for (int c = (int)kSizeClasses - 1; c >= 0; --c) {
+      const uint32_t count = class_items[c];
+      class_items[c] = running;
+      running += count;
+    }
+    p.item_count[0] = running;
+  }
+  __syncthreads();
+  for (uint32_t token = threadIdx.x; token < p.tokens; token += 256) {
+    const TokenPlan plan = p.plans[token];
+    if (plan.leader != token || plan.splits == 0) continue;
+    const uint32_t first = atomicAdd(&class_items[class_of(plan)], plan.splits);
+    for (uint32_t s = 0; s < plan.splits; ++s) p.items[first + s] = make_uint2(token, s);
+  }
 }
 
 __device__ inline uint32_t pack_bf16(float lo, float hi) {

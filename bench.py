@@ -229,6 +229,36 @@ def prefill_gemm_c4(backend, rows=8256, seed=91, repeats=3):
     }
 
 
+def prefill_layer_c4(backend, seed=95, repeats=2):
+    """One whole BASELINE config 4 decoder layer over the packed batch (6 prompts of 512..3072
+    tokens summing to 8192, plus 64 decode rows): norms, stacked qkv, qk-norm + rope, paged
+    attention, o, gate/up, SwiGLU, down with residual.  Device time of the step from the
+    submission's events; flops = projections + attention."""
+    from forja_amd.model import DENSE_27B, Model, PackedStep
+    c = DENSE_27B
+    rng = np.random.default_rng(seed)
+    prompts = [512, 768, 1024, 1280, 1536, 3072]
+    contexts = [0] * len(prompts) + [int(v) for v in rng.integers(128, 4097, 64)]
+    counts = prompts + [1] * 64
+    model = Model(backend, c, seed=seed, layers=1)
+    step = PackedStep(model, contexts, counts, seed=seed, head=False)
+    step.run()
+    nanoseconds = 0
+    for _ in range(repeats):
+        nanoseconds += step.run().gpu_time_ns()
+    seconds = nanoseconds / repeats * 1e-9
+    rows = step.tokens
+    qkv_width = (c.q_heads + 2 * c.kv_heads) * c.head_dim
+    weights = qkv_width * c.hidden + c.hidden * c.q_heads * c.head_dim + 3 * c.intermediate * c.hidden
+    pairs = sum(n * ctx + n * (n + 1) // 2 for ctx, n in zip(contexts, counts))
+    flops = 2.0 * rows * weights + 2.0 * c.q_heads * pairs * 2 * c.head_dim
+    return {"rows": rows, "ms_per_layer": seconds * 1e3, "flops_per_layer": flops,
+            "roofline": {"bound": "mfma", "achieved": flops / seconds / 1e12,
+                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": flops / seconds / 1e12 / MFMA_BF16_PEAK_TFLOPS},
+            "prefill_tok_per_s_64_layers": rows / (seconds * c.layers)}
+
+
 def stream_read_rate(backend, rows=4096, width=1 << 20, repeats=3):
     """What a plain read-only stream sustains on this device: a row-wise argmax over 8 GiB of
     bf16 (16-byte loads, one workgroup per row).  The practical ceiling the HBM-bound kernels are
@@ -350,7 +380,8 @@ def main():
     if args.prefill_only:
         backend = HipBackend(0)
         print(json.dumps({"prefill_gemm_c4": prefill_gemm_c4(backend),
-                          "prefill_attention_c4": prefill_attention_c4(backend)}))
+                          "prefill_attention_c4": prefill_attention_c4(backend),
+                          "prefill_layer_c4": prefill_layer_c4(backend)}))
         return
     if args.gpus != 1:
         print("bench.py: this build runs the ragged forward step on ONE MI355X; collectives and "
@@ -481,7 +512,8 @@ def main():
         result["roofline"]["frac_of_measured_stream_read"] = (
             result["roofline"]["achieved"] / result["roofline"]["measured_stream_read_gbps"])
         result["secondary_workloads"] = {"prefill_gemm_c4": prefill_gemm_c4(backend),
-                                         "prefill_attention_c4": prefill_attention_c4(backend)}
+                                         "prefill_attention_c4": prefill_attention_c4(backend),
+                                         "prefill_layer_c4": prefill_layer_c4(backend)}
         if config.moe:
             result["secondary_workloads"]["moe_block_c2"] = moe_block_c2(backend, workload.model)
     step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction

@@ -230,7 +230,7 @@ class KvCache:
 class StepBuffers:
     """Activations and per-lane metadata of one packed batch of `tokens` rows over `lanes` lanes."""
 
-    def __init__(self, backend, config: ModelConfig, tokens: int, lanes: int):
+    def __init__(self, backend, config: ModelConfig, tokens: int, lanes: int, head: bool = True):
         c = config
         qkv_width = (c.q_heads + 2 * c.kv_heads) * c.head_dim
         a = lambda *shape: backend.alloc(DType.BF16, shape)
@@ -254,16 +254,17 @@ class StepBuffers:
         else:
             self.gate_up = a(tokens, 2 * c.intermediate)
             self.activated = a(tokens, c.intermediate)
-        self.logits = a(tokens, c.vocab)
+        self.logits = a(tokens, c.vocab) if head else None
         self.next_tokens = backend.alloc(DType.U32, (tokens,))
 
 
 def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: CommandList,
-                feed_back: bool = False, route_trace: Optional[Tensor] = None) -> None:
+                feed_back: bool = False, route_trace: Optional[Tensor] = None,
+                head: bool = True) -> None:
     """Appends one forward step over the packed batch to `commands`.  With `feed_back` the greedy
     tokens are copied into the id buffer for the next step (device to device).  `route_trace`
     (u32 [layers, tokens, top_k]) receives a copy of every layer's expert choices, for
-    diagnostics."""
+    diagnostics.  Without `head` the step stops after the last layer's norm (no lm_head)."""
     c, b = model.config, buffers
     tokens = b.tokens
     heads = c.q_heads + c.kv_heads
@@ -331,6 +332,8 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
             else model.final_norm
         commands.dispatch_kernel(model.rms_norm, [hidden, norm_weight(following)], [normalized_next])
         normalized, normalized_next = normalized_next, normalized
+    if not head:
+        return
     commands.dispatch(q4, [normalized, *model.lm_head.triple], b.logits)
     commands.dispatch(Op.argmax(), [b.logits], b.next_tokens)
     if feed_back:
@@ -416,3 +419,42 @@ class DecodeSession:
         """Algorithmic K/V bytes the next step's attention reads: (context+1) rows per lane."""
         return int((self.contexts + 1).sum()) * self.model.config.kv_bytes_per_token \
             * self.model.n_layers // self.model.config.layers
+
+
+class PackedStep:
+    """One forward step over a packed batch that mixes prefill chunks and decode rows: lane l has
+    `contexts[l]` cached tokens and contributes `counts[l]` new rows (BASELINE configs 1 and 4).
+    Owns the cache, the buffers and the recorded command list; `run()` executes it once."""
+
+    def __init__(self, model: Model, contexts, counts, seed: int = 7, head: bool = True,
+                 fill_pools: bool = True):
+        c, backend = model.config, model.backend
+        self.model = model
+        contexts = np.array(contexts, dtype=np.int64)
+        counts = np.array(counts, dtype=np.int64)
+        lanes, tokens, pt = len(contexts), int(counts.sum()), c.page_tokens
+        pages = (contexts + counts + pt - 1) // pt
+        self.cache = KvCache(backend, c, model.n_layers, lanes, int(pages.sum()) + 8,
+                             int(pages.max()) + 1, seed, fill_pools=fill_pools)
+        rng = np.random.default_rng(seed)
+        self.cache.shuffle_free(rng)
+        for lane in range(lanes):
+            self.cache.ensure(lane, int(contexts[lane] + counts[lane]))
+        self.cache.upload_tables()
+        self.buffers = b = StepBuffers(backend, c, tokens, lanes, head=head)
+        cu = np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32)
+        positions = np.concatenate([contexts[lane] + np.arange(counts[lane]) for lane in range(lanes)])
+        backend.write(b.cu_seqlens, cu.tobytes())
+        backend.write(b.activity, np.ones(lanes, dtype=np.uint32).tobytes())
+        backend.write(b.q_starts, contexts.astype(np.uint32).tobytes())
+        backend.write(b.positions, positions.astype(np.float32).tobytes())
+        backend.write(b.ids, rng.integers(0, c.vocab, tokens).astype(np.uint32).tobytes())
+        self.commands = CommandList()
+        record_step(model, self.cache, b, self.commands, head=head)
+        self.encoded = backend.encode(self.commands) if hasattr(backend, "encode") else self.commands
+        self.tokens, self.lanes = tokens, lanes
+
+    def run(self):
+        submission = self.model.backend.submit(self.encoded)
+        submission.wait()
+        return submission

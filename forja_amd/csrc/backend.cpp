@@ -105,6 +105,11 @@ struct fh_backend {
   uint64_t route_plan_bytes = 0;
   bool route_plan_valid = false;
   RoutePlanKey route_plan_key{};
+  // attention work plan kept between the layers of a step
+  char *attention_plan = nullptr;
+  uint64_t attention_plan_bytes = 0;
+  bool attention_plan_valid = false;
+  AttentionPlanKey attention_plan_key{};
   // profiling
   int profiling = 0;  // 0 off, 1 kernel-level timers, 2 also one timer per dispatch
   struct Timed {
@@ -128,6 +133,23 @@ struct fh_backend {
   uint64_t class_ns[FH_KC_COUNT] = {};
   uint64_t class_launches[FH_KC_COUNT] = {};
 
+  // f32 accumulators handed to an epilogue program; separate from `workspace` because the kernel
+  // that fills them may carve its own scratch out of the workspace.
+  char *accumulators = nullptr;
+  uint64_t accumulator_bytes = 0;
+  char *ensure_accumulators(uint64_t bytes) {
+    if (bytes <= accumulator_bytes) return accumulators;
+    (void)hipStreamSynchronize(stream);
+    if (accumulators) (void)hipFree(accumulators);
+    accumulators = nullptr;
+    accumulator_bytes = 0;
+    uint64_t want = std::max<uint64_t>(bytes, 16ull << 20);
+    void *ptr = nullptr;
+    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
+    accumulators = (char *)ptr;
+    accumulator_bytes = want;
+    return accumulators;
+  }
   char *ensure_workspace(uint64_t bytes) {
     if (bytes <= workspace_bytes) return workspace;
     (void)hipStreamSynchronize(stream);
@@ -530,8 +552,19 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
                                 inner, columns, d.bits, d.group_size);
     return FH_OK;
   }
+  // Recognised epilogue: out = accumulator + extra (the residual add after a dense projection).
+  auto prog = b->programs.find(d.epilogue);
+  FH_REQUIRE(prog != b->programs.end());
+  if (d.accumulator_count == 1 && d.n_extras == 1 &&
+      is_add_epilogue(prog->second.insts, prog->second.pairs) &&
+      shape_is(d.inputs[primitive], {rows, columns})) {
+    QmmProblem fused{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows, inner, columns,
+                     d.bits, d.group_size, &pl.in[primitive]};
+    if (try_fast_quant_matmul(b, fused)) return FH_OK;
+  }
+  // The accumulators live apart from the workspace, which the product kernels use themselves.
   uint64_t elements = (uint64_t)rows * columns;
-  char *acc = b->ensure_workspace(elements * 4);
+  char *acc = b->ensure_accumulators(elements * 4);
   if (!acc) return FH_ALLOCATION_FAILED;
   View acc_view = contiguous_view(acc, FH_F32, out);
   QmmProblem problem{pl.in[0], pl.in[1], pl.in[2], pl.in[3], acc_view, rows, inner, columns,
@@ -978,6 +1011,11 @@ fh_status plan_ragged(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
   problem.physical_pages = kp.shape[0];
   problem.table_pages = tables.shape[1];
   problem.scale = d.scale;
+  problem.metadata_buffers[0] = d.inputs[5].buffer;
+  problem.metadata_buffers[1] = d.inputs[6].buffer;
+  problem.metadata_buffers[2] = d.n_inputs == 8 ? d.inputs[7].buffer : 0;
+  problem.metadata_buffers[3] = d.inputs[3].buffer;
+  problem.metadata_buffers[4] = d.inputs[4].buffer;
   if (!run_ragged_attention(b, problem, error)) return FH_ALLOCATION_FAILED;
   return FH_OK;
 }
@@ -1164,7 +1202,9 @@ void fh_destroy(fh_backend *b) {
     for (auto &entry : b->programs)
       for (auto &typed : entry.second.typed) (void)hipFree(typed.second);
     if (b->workspace) (void)hipFree(b->workspace);
+    if (b->accumulators) (void)hipFree(b->accumulators);
     if (b->route_plan) (void)hipFree(b->route_plan);
+    if (b->attention_plan) (void)hipFree(b->attention_plan);
     for (auto &e : b->error_pool) {
       (void)hipFree(e.device);
       (void)hipHostFree(e.host);
@@ -1436,6 +1476,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   s->start = take_event(b);
   s->end = take_event(b);
   b->route_plan_valid = false;  // host writes between submissions are not tracked
+  b->attention_plan_valid = false;
   launch_init_errors(b->stream, s->device_errors, slots);
   (void)hipEventRecord(s->start, b->stream);
   fh_status status = FH_OK;
@@ -1451,6 +1492,11 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
     if (b->route_plan_valid)
       for (uint32_t o = 0; o < dispatches[i].n_outputs && o < FH_MAX_OUTPUTS; ++o)
         if (dispatches[i].outputs[o].buffer == b->route_plan_key.buffer) b->route_plan_valid = false;
+    if (b->attention_plan_valid)
+      for (uint32_t o = 0; o < dispatches[i].n_outputs && o < FH_MAX_OUTPUTS; ++o)
+        for (uint64_t watched : b->attention_plan_key.buffers)
+          if (watched != 0 && dispatches[i].outputs[o].buffer == watched)
+            b->attention_plan_valid = false;
     if (b->profiling >= 2) {
       (void)hipEventRecord(t1, b->stream);
       b->timed.push_back({t0, t1, kernel_class_of(dispatches[i].op)});
@@ -1660,6 +1706,27 @@ char *backend_route_plan(fh_backend *b, const RoutePlanKey &key, uint64_t bytes,
   b->route_plan_key = key;
   b->route_plan_valid = true;
   return b->route_plan;
+}
+char *backend_attention_plan(fh_backend *b, const AttentionPlanKey &key, uint64_t bytes,
+                             bool *reuse) {
+  *reuse = b->attention_plan_valid && bytes <= b->attention_plan_bytes &&
+           memcmp(&b->attention_plan_key, &key, sizeof(key)) == 0;
+  if (*reuse) return b->attention_plan;
+  b->attention_plan_valid = false;
+  if (bytes > b->attention_plan_bytes) {
+    (void)hipStreamSynchronize(b->stream);
+    if (b->attention_plan) (void)hipFree(b->attention_plan);
+    b->attention_plan = nullptr;
+    b->attention_plan_bytes = 0;
+    uint64_t want = std::max<uint64_t>(bytes, 1ull << 20);
+    void *ptr = nullptr;
+    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
+    b->attention_plan = (char *)ptr;
+    b->attention_plan_bytes = want;
+  }
+  b->attention_plan_key = key;
+  b->attention_plan_valid = true;
+  return b->attention_plan;
 }
 hipStream_t backend_stream(fh_backend *backend) { return backend->stream; }
 uint32_t backend_compute_units(fh_backend *backend) {

@@ -29,6 +29,18 @@ struct RoutePlanKey {
 // the same submission.  Null when allocation fails.
 char *backend_route_plan(fh_backend *backend, const RoutePlanKey &key, uint64_t bytes, bool *reuse);
 
+// Identity of an attention work plan: the metadata it was built from (allocation ids and device
+// addresses of cu_seqlens, q_starts, activity, tables and generations; the last two because the
+// per-token failure flags kept with the plan come from them) and every scalar it depends on.
+struct AttentionPlanKey {
+  uint64_t buffers[5], address[5];
+  uint32_t params[10];
+};
+// Like backend_route_plan, for the work plan the attention dispatches of one submission share:
+// every layer of a step attends with the same lanes, starts and tables.
+char *backend_attention_plan(fh_backend *backend, const AttentionPlanKey &key, uint64_t bytes,
+                             bool *reuse);
+
 // Brackets one kernel launch with HIP events when profiling is enabled.
 struct KernelTimer {
   fh_backend *backend;
@@ -42,11 +54,16 @@ struct KernelTimer {
 struct QmmProblem {
   View x, packed, scales, biases, out;
   uint32_t rows, inner, columns, bits, group;
+  // Optional [rows, columns] bf16 rows added to the f32 result before it is rounded (the dense
+  // residual-add epilogue); only honoured together with a bf16 `out`.
+  const View *residual = nullptr;
 };
 bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &problem);
-// Tiled GEMM with weights dequantised into LDS, for many rows; operands as checked by
-// try_fast_quant_matmul.  False when the launch could not be configured.
-bool launch_quant_gemm(fh_backend *backend, const QmmProblem &problem);
+// Dequantise-once tiled GEMM for many rows; operands as checked by try_fast_quant_matmul.  False
+// when the launch could not be configured.  On success `*refused` points at a device word the
+// launched kernels leave non-zero when some scale or bias is outside their fp16 scheme; they
+// have then written nothing and the caller must run a kernel conditioned on that word.
+bool launch_quant_gemm(fh_backend *backend, const QmmProblem &problem, const uint32_t **refused);
 
 struct GatherProblem {
   View x;           // projection: [R,K]; weighted sum: [R,k,K]
@@ -79,13 +96,18 @@ struct RaggedAttention {
   uint32_t tokens, lanes, query_heads, kv_heads, width, value_width, page_tokens, physical_pages,
       table_pages;
   float scale;
+  // allocation identities of cu_seqlens, q_starts, activity, tables, generations (0: none)
+  uint64_t metadata_buffers[5];
 };
 // Always handles the problem (specialised kernel when the layout allows, generic otherwise);
 // false only when workspace allocation fails.
 bool run_ragged_attention(fh_backend *backend, const RaggedAttention &problem, ErrorSlot *error);
 
 // Recognised guest row programs (by canonical expression) and their constants.
-enum ProgramKindFast { kProgramGeneric = 0, kProgramRmsNorm, kProgramResidualNorm, kProgramQkNormRope };
+enum ProgramKindFast {
+  kProgramGeneric = 0, kProgramRmsNorm, kProgramResidualNorm, kProgramQkNormRope,
+  kProgramSiluMul, kProgramAdd   // element-wise: in0 * sigmoid(in0) * in1, in0 + in1
+};
 struct ProgramClass {
   int kind;
   uint32_t axis;  // the axis the program's extent/index instruction names (must be the last)

@@ -88,6 +88,54 @@ __global__ void ragged_append_kernel(RaggedAttention p, ErrorSlot *error) {
   }
 }
 
+// The same append for bf16 rows and pools whose head rows are 16-byte aligned: a thread moves
+// eight elements.
+__global__ __launch_bounds__(256) void ragged_append_pieces_kernel(RaggedAttention p, ErrorSlot *error) {
+  const uint32_t key_pieces = p.kv_heads * p.width / 8, value_pieces = p.kv_heads * p.value_width / 8;
+  const uint32_t per_token = key_pieces + value_pieces;
+  const uint64_t flat = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (flat >= (uint64_t)p.tokens * per_token) return;
+  const uint32_t token = (uint32_t)(flat / per_token), piece = (uint32_t)(flat % per_token);
+  const uint32_t *cu = (const uint32_t *)p.cu_seqlens.base + p.cu_seqlens.offset;
+  if (token < cu[0] || token >= cu[p.lanes]) return;
+  const uint32_t lane = find_lane(cu, p.lanes, token);
+  if (p.activity.base && ((const uint32_t *)p.activity.base)[p.activity.offset + lane] == 0) return;
+  const uint64_t position =
+      (uint64_t)((const uint32_t *)p.q_starts.base)[p.q_starts.offset + lane] + (token - cu[lane]);
+  const uint32_t *table =
+      (const uint32_t *)p.tables.base + p.tables.offset + (uint64_t)lane * p.table_pages * 2;
+  const uint32_t *generations = (const uint32_t *)p.generations.base + p.generations.offset;
+  uint32_t physical;
+  const uint64_t logical_page = position / p.page_tokens;
+  if (logical_page >= p.table_pages ||
+      !entry_ok(table, generations, (uint32_t)logical_page, p.table_pages, p.physical_pages,
+                &physical)) {
+    if (piece == 0) report_error(error, logical_page > 0xffffffffull ? 0xffffffffu
+                                                                     : (uint32_t)logical_page);
+    return;
+  }
+  const uint64_t pool_row = (uint64_t)physical * p.page_tokens + position % p.page_tokens;
+  const bool key = piece < key_pieces;
+  const uint32_t local = key ? piece : piece - key_pieces;
+  const uint32_t row_width = key ? p.width : p.value_width;
+  const uint32_t head = 8 * local / row_width, c = 8 * local % row_width;
+  const View &src = key ? p.k_new : p.v_new;
+  const View &pool = key ? p.key_pool : p.value_pool;
+  const uint4 value = *(const uint4 *)((const uint16_t *)src.base + src.offset +
+                                       (uint64_t)token * src.stride[0] + head * src.stride[1] + c);
+  *(uint4 *)((uint16_t *)pool.base + pool.offset + pool_row * ((uint64_t)p.kv_heads * row_width) +
+             8 * local) = value;
+}
+
+bool append_by_pieces(const RaggedAttention &p) {
+  for (const View *v : {&p.k_new, &p.v_new})
+    if (v->dtype != FH_BF16 || v->stride[2] != 1 || v->stride[0] % 8 || v->stride[1] % 8 || v->offset % 8)
+      return false;
+  for (const View *v : {&p.key_pool, &p.value_pool})
+    if (v->dtype != FH_BF16 || v->offset % 8) return false;
+  return p.width % 8 == 0 && p.value_width % 8 == 0;
+}
+
 // Any dtype / width: one wave per (token, query head); per-lane online softmax merged at the end.
 template <int kMaxDv>
 __global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *error) {
@@ -612,42 +660,57 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
 // Merges the per-split partials of one (token, head): out = sum_s O_s 2^(m_s-M) / sum_s l_s
 // 2^(m_s-M).  Also writes the zero rows of inactive lanes, uncovered tokens and tokens whose page
-// table was refused.
-__global__ __launch_bounds__(64) void ragged_reduce_kernel(FastRagged p) {
+// table was refused.  Four waves: every wave finds M and the weights from one (m, l) load per
+// lane (a token has at most 64 splits), then wave w folds splits 2w+half, 2w+half+8, ... of its
+// lanes' four columns, all loads in flight at once, and the waves' sums meet in LDS.
+__global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
+  __shared__ float4 folded[3][32];
   const uint32_t head = blockIdx.x, token = blockIdx.y;
   const TokenPlan plan = p.plans[token];
   const bool zero = plan.splits == 0 || p.bad[token] != 0;
   if (!zero && plan.splits == 1) return;
-  const uint32_t lane = threadIdx.x, column = (lane & 31) * 4, half = lane >> 5;
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t column = (lane & 31) * 4, half = lane >> 5;
   uint16_t *dst = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
   if (zero) {
-    if (half == 0) *(uint2 *)dst = make_uint2(0, 0);
+    if (threadIdx.x < 32) *(uint2 *)dst = make_uint2(0, 0);
     return;
   }
   const uint64_t base = (uint64_t)token * p.max_splits * p.query_heads + head;
-  float m_all = -__builtin_inff();
-  for (uint32_t s = 0; s < plan.splits; ++s)
-    m_all = fmaxf(m_all, p.partial_ml[base + (uint64_t)s * p.query_heads].x);
-  float l_all = 0.0f;
+  float2 ml = make_float2(-__builtin_inff(), 0.0f);
+  if (lane < plan.splits) ml = p.partial_ml[base + (uint64_t)lane * p.query_heads];
+  const float m_all = wave_max(ml.x);
+  const float weight = lane < plan.splits ? exp2f(ml.x - m_all) : 0.0f;
+  const float l_all = wave_sum(ml.y * weight);
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (uint32_t s = half; s < plan.splits; s += 2) {
-    uint64_t at = base + (uint64_t)s * p.query_heads;
-    float2 ml = p.partial_ml[at];
-    float w = exp2f(ml.x - m_all);
-    l_all += ml.y * w;
-    float4 part = *(const float4 *)(p.partial_o + at * 128 + column);
-    acc.x += part.x * w;
-    acc.y += part.y * w;
-    acc.z += part.z * w;
-    acc.w += part.w * w;
+#pragma unroll
+  for (uint32_t i = 0; i < 8; ++i) {   // 64 splits / (4 waves * 2 halves)
+    const uint32_t s = 8 * i + 2 * wave + half;
+    const float w = __shfl(weight, (int)(s & 63), 64);
+    if (s < plan.splits) {
+      const float4 part =
+          *(const float4 *)(p.partial_o + (base + (uint64_t)s * p.query_heads) * 128 + column);
+      acc.x += part.x * w;
+      acc.y += part.y * w;
+      acc.z += part.z * w;
+      acc.w += part.w * w;
+    }
   }
-  l_all += __shfl_xor(l_all, 32, 64);
   acc.x += __shfl_xor(acc.x, 32, 64);
   acc.y += __shfl_xor(acc.y, 32, 64);
   acc.z += __shfl_xor(acc.z, 32, 64);
   acc.w += __shfl_xor(acc.w, 32, 64);
-  if (half == 0) {
-    float inv = 1.0f / l_all;
+  if (wave != 0 && half == 0) folded[wave - 1][lane] = acc;
+  __syncthreads();
+  if (threadIdx.x < 32) {
+    for (int other = 0; other < 3; ++other) {
+      const float4 part = folded[other][lane];
+      acc.x += part.x;
+      acc.y += part.y;
+      acc.z += part.z;
+      acc.w += part.w;
+    }
+    const float inv = 1.0f / l_all;
     *(uint2 *)dst = make_uint2(pack_bf16(acc.x * inv, acc.y * inv), pack_bf16(acc.z * inv, acc.w * inv));
   }
 }
@@ -679,33 +742,50 @@ uint32_t splits_for(uint32_t tokens) {
   return max_splits;
 }
 
-// Carves flags / plans / work items / (m,l) / O partial storage out of the backend workspace.
-bool carve_partials(fh_backend *backend, FastRagged *f) {
+uint32_t forced_split_tokens() {
   static const uint32_t split_tokens = [] {
     const char *env = getenv("FORJA_HIP_SPLIT_TOKENS");
     uint32_t value = env ? (uint32_t)atoi(env) : 0;
     return value >= 32 ? value / 32 * 32 : 0;  // 0 = chosen per launch from the batch
   }();
-  f->split_tokens = split_tokens;
-  auto round = [](uint64_t bytes) { return (bytes + 255) / 256 * 256; };
+  return split_tokens;
+}
+
+uint64_t round_256(uint64_t bytes) { return (bytes + 255) / 256 * 256; }
+
+// Flags, plans, work items and the item count: everything ragged_plan_kernel writes.
+uint64_t plan_storage_bytes(const FastRagged &f) {
+  uint64_t slots = (uint64_t)f.tokens * f.max_splits;
+  return round_256((uint64_t)f.tokens * 4) + round_256((uint64_t)f.tokens * sizeof(TokenPlan)) +
+         round_256(slots * sizeof(uint2)) + 256;
+}
+
+char *carve_plan(FastRagged *f, char *ws) {
   uint64_t slots = (uint64_t)f->tokens * f->max_splits;
-  uint64_t flags_bytes = round((uint64_t)f->tokens * 4);
-  uint64_t plan_bytes = round((uint64_t)f->tokens * sizeof(TokenPlan));
-  uint64_t item_bytes = round(slots * sizeof(uint2));
-  uint64_t count_bytes = 256;
-  uint64_t ml_bytes = round(slots * f->query_heads * sizeof(float2));
+  f->bad = (uint32_t *)ws;
+  ws += round_256((uint64_t)f->tokens * 4);
+  f->plans = (TokenPlan *)ws;
+  ws += round_256((uint64_t)f->tokens * sizeof(TokenPlan));
+  f->items = (uint2 *)ws;
+  ws += round_256(slots * sizeof(uint2));
+  f->item_count = (uint32_t *)ws;
+  return ws + 256;
+}
+
+// Carves the (m,l) and O partial storage out of the backend workspace, and the plan storage too
+// unless `plan_storage` already holds room for it.
+bool carve_partials(fh_backend *backend, FastRagged *f, char *plan_storage) {
+  f->split_tokens = forced_split_tokens();
+  uint64_t slots = (uint64_t)f->tokens * f->max_splits;
+  uint64_t ml_bytes = round_256(slots * f->query_heads * sizeof(float2));
   uint64_t o_bytes = slots * f->query_heads * 128 * sizeof(float);
   char *ws = backend_workspace(
-      backend, flags_bytes + plan_bytes + item_bytes + count_bytes + ml_bytes + o_bytes);
+      backend, (plan_storage ? 0 : plan_storage_bytes(*f)) + ml_bytes + o_bytes);
   if (!ws) return false;
-  f->bad = (uint32_t *)ws;
-  ws += flags_bytes;
-  f->plans = (TokenPlan *)ws;
-  ws += plan_bytes;
-  f->items = (uint2 *)ws;
-  ws += item_bytes;
-  f->item_count = (uint32_t *)ws;
-  ws += count_bytes;
+  if (plan_storage)
+    carve_plan(f, plan_storage);
+  else
+    ws = carve_plan(f, ws);
   f->partial_ml = (float2 *)ws;
   ws += ml_bytes;
   f->partial_o = (float *)ws;
@@ -732,7 +812,7 @@ void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, E
                                      64 * waves, 0, stream>>>(f, error);
     }
   }
-  ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens), 64, 0, stream>>>(f);
+  ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens), 256, 0, stream>>>(f);
 }
 
 }  // namespace
@@ -762,7 +842,7 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   f.scale_log2 = lane.scale * 1.4426950408889634f;
   f.one_start = lane.query_start;
   f.fixed_attended = lane.causal ? 0 : lane.key_length;
-  if (!carve_partials(backend, &f)) return false;
+  if (!carve_partials(backend, &f, nullptr)) return false;
   f.q = (const uint16_t *)lane.q.base + lane.q.offset;
   f.out = (uint16_t *)lane.out.base + lane.out.offset;
   f.key_pool = (const uint16_t *)lane.key_pool.base + lane.key_pool.offset;
@@ -790,23 +870,6 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
   FastRagged f{};
   if (fast) {
     f.tokens = p.tokens;
-    f.query_heads = p.query_heads;
-    f.max_splits = splits_for(p.tokens);
-    if (!carve_partials(backend, &f)) return false;
-    f.q = (const uint16_t *)p.q.base + p.q.offset;
-    f.out = (uint16_t *)p.out.base + p.out.offset;
-    f.key_pool = (const uint16_t *)p.key_pool.base + p.key_pool.offset;
-    f.value_pool = (const uint16_t *)p.value_pool.base + p.value_pool.offset;
-    f.tables = (const uint32_t *)p.tables.base + p.tables.offset;
-    f.generations = (const uint32_t *)p.generations.base + p.generations.offset;
-    f.cu = (const uint32_t *)p.cu_seqlens.base + p.cu_seqlens.offset;
-    f.starts = (const uint32_t *)p.q_starts.base + p.q_starts.offset;
-    f.activity = p.activity.base ? (const uint32_t *)p.activity.base + p.activity.offset : nullptr;
-    f.q_stride_t = p.q.stride[0];
-    f.q_stride_h = p.q.stride[1];
-    f.out_stride_t = p.out.stride[0];
-    f.out_stride_h = p.out.stride[1];
-    f.tokens = p.tokens;
     f.lanes = p.lanes;
     f.query_heads = p.query_heads;
     f.kv_heads = p.kv_heads;
@@ -815,12 +878,46 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     f.page_tokens = p.page_tokens;
     f.physical_pages = p.physical_pages;
     f.table_pages = p.table_pages;
+    f.max_splits = splits_for(p.tokens);
     f.scale_log2 = p.scale * 1.4426950408889634f;
-    launch_plan(stream, f, error);
+    f.tables = (const uint32_t *)p.tables.base + p.tables.offset;
+    f.generations = (const uint32_t *)p.generations.base + p.generations.offset;
+    f.cu = (const uint32_t *)p.cu_seqlens.base + p.cu_seqlens.offset;
+    f.starts = (const uint32_t *)p.q_starts.base + p.q_starts.offset;
+    f.activity = p.activity.base ? (const uint32_t *)p.activity.base + p.activity.offset : nullptr;
+    // The plan depends on the lane metadata only, which every layer of a step shares: it is built
+    // by the first attention dispatch of a submission and reused until that metadata is written.
+    AttentionPlanKey key{};
+    for (int i = 0; i < 5; ++i) key.buffers[i] = p.metadata_buffers[i];
+    key.address[0] = (uint64_t)f.cu;
+    key.address[1] = (uint64_t)f.starts;
+    key.address[2] = (uint64_t)f.activity;
+    key.address[3] = (uint64_t)f.tables;
+    key.address[4] = (uint64_t)f.generations;
+    const uint32_t params[10] = {f.tokens, f.lanes, f.group_tokens, f.page_tokens, f.physical_pages,
+                                 f.table_pages, f.max_splits, forced_split_tokens(), f.kv_heads,
+                                 f.query_heads};
+    for (int i = 0; i < 10; ++i) key.params[i] = params[i];
+    bool reuse = false;
+    char *plan_storage = backend_attention_plan(backend, key, plan_storage_bytes(f), &reuse);
+    if (!plan_storage || !carve_partials(backend, &f, plan_storage)) return false;
+    f.q = (const uint16_t *)p.q.base + p.q.offset;
+    f.out = (uint16_t *)p.out.base + p.out.offset;
+    f.key_pool = (const uint16_t *)p.key_pool.base + p.key_pool.offset;
+    f.value_pool = (const uint16_t *)p.value_pool.base + p.value_pool.offset;
+    f.q_stride_t = p.q.stride[0];
+    f.q_stride_h = p.q.stride[1];
+    f.out_stride_t = p.out.stride[0];
+    f.out_stride_h = p.out.stride[1];
+    if (!reuse) launch_plan(stream, f, error);
   }
   uint64_t append_work =
       (uint64_t)p.tokens * (p.kv_heads * p.width + p.kv_heads * p.value_width);
-  ragged_append_kernel<<<dim3((unsigned)((append_work + 255) / 256)), 256, 0, stream>>>(p, error);
+  if (append_by_pieces(p))
+    ragged_append_pieces_kernel<<<dim3((unsigned)((append_work / 8 + 255) / 256)), 256, 0, stream>>>(
+        p, error);
+  else
+    ragged_append_kernel<<<dim3((unsigned)((append_work + 255) / 256)), 256, 0, stream>>>(p, error);
   if (fast) {
     launch_fast(backend, stream, f, error);
     return true;

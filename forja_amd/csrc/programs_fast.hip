@@ -1,10 +1,11 @@
-// Fused kernels for the guest row programs every engine dispatches around the matmuls
-// (crates/forja-sdk/src/nn/blocks.rs:380-443): rms_norm_rows, residual_norm_rows and
-// qk_norm_rope_rows.  A program is recognised by its canonical expression (commutative operands
+// Fused kernels for the guest programs every engine dispatches around the matmuls
+// (crates/forja-sdk/src/nn/blocks.rs:380-443): the row programs rms_norm_rows, residual_norm_rows
+// and qk_norm_rope_rows, and the element-wise silu_mul_elements and add_elements.  A program is recognised by its canonical expression (commutative operands
 // sorted, constants captured), never by name, so any instruction order the SDK emits matches;
 // everything else runs on the generic interpreter.  bf16 rows, innermost axis contiguous.
 #include "fast_kernels.hpp"
 
+#include <algorithm>
 #include <regex>
 #include <string>
 
@@ -130,6 +131,40 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(QkArgs a) {
   a.out_hi[row * a.ohi_s[0] + head * a.ohi_s[1] + lane] = (uint16_t)(pack2(r_hi, 0.0f) & 0xffffu);
 }
 
+struct PairArgs {
+  const uint16_t *a, *b;
+  uint16_t *out;
+  uint64_t a_stride, b_stride, out_stride;   // elements between rows
+  uint32_t rows, pieces_per_row;             // 8-element pieces
+};
+
+// out = a * sigmoid(a) * b (kSilu) or a + b, eight bf16 values per thread and trip; the
+// arithmetic is the interpreter's: f32 throughout, sigmoid(x) = 1 / (1 + exp(-x)), one rounding.
+template <bool kSilu>
+__global__ __launch_bounds__(256) void map_pair_kernel(PairArgs p) {
+  const uint64_t pieces = (uint64_t)p.rows * p.pieces_per_row;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t piece = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; piece < pieces;
+       piece += stride) {
+    const uint64_t row = piece / p.pieces_per_row, at = 8 * (piece % p.pieces_per_row);
+    const uint4 av = *(const uint4 *)(p.a + row * p.a_stride + at);
+    const uint4 bv = *(const uint4 *)(p.b + row * p.b_stride + at);
+    const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a_lo = lo_f32(aw[i]), a_hi = hi_f32(aw[i]);
+      const float b_lo = lo_f32(bw[i]), b_hi = hi_f32(bw[i]);
+      if (kSilu)
+        ow[i] = pack2(a_lo * (1.0f / (1.0f + expf(-a_lo))) * b_lo,
+                      a_hi * (1.0f / (1.0f + expf(-a_hi))) * b_hi);
+      else
+        ow[i] = pack2(a_lo + b_lo, a_hi + b_hi);
+    }
+    *(uint4 *)(p.out + row * p.out_stride + at) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  }
+}
+
 // Canonical expression of value v: commutative operands sorted; constants carry their bits.
 std::string canonical(const fh_inst *insts, uint32_t count, uint32_t v, int depth = 0) {
   if (v >= count || depth > 24) return "?";
@@ -181,6 +216,13 @@ ProgramClass classify_program(uint32_t kind, const fh_inst *insts, uint32_t n_in
                               const uint32_t *pairs, uint32_t n_pairs) {
   ProgramClass result{};
   result.kind = kProgramGeneric;
+  if (kind == 0) {   // element-wise programs with one output
+    if (n_pairs != 1 || pairs[0] != 0) return result;
+    const std::string e = canonical(insts, n_insts, pairs[1]);
+    if (e == "b2(b2(in0,u9(in0)),in1)") result.kind = kProgramSiluMul;
+    if (e == "b0(in0,in1)") result.kind = kProgramAdd;
+    return result;
+  }
   if (kind != 1) return result;
   std::smatch m;
   auto value_of = [&](uint32_t slot) -> std::string {
@@ -257,7 +299,6 @@ bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const Program
                       uint64_t elements) {
   if (cls.kind == kProgramGeneric || elements == 0) return false;
   const uint32_t rank = p.rank;
-  if (cls.axis != rank - 1) return false;
   auto ptr = [](const View &v) { return (uint16_t *)v.base + v.offset; };
   auto aligned = [&](const View &v) {
     if (v.offset % 8) return false;
@@ -265,6 +306,21 @@ bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const Program
       if (v.stride[axis] % 8) return false;
     return true;
   };
+  if (cls.kind == kProgramSiluMul || cls.kind == kProgramAdd) {
+    if (rank != 2 || p.n_inputs != 2 || p.shape[1] % 8 != 0) return false;
+    for (const View *v : {&p.inputs[0], &p.inputs[1], &p.outputs[0]})
+      if (!bf16_rows(*v, 2) || !aligned(*v)) return false;
+    PairArgs a{ptr(p.inputs[0]), ptr(p.inputs[1]), ptr(p.outputs[0]), p.inputs[0].stride[0],
+               p.inputs[1].stride[0], p.outputs[0].stride[0], p.shape[0], p.shape[1] / 8};
+    const uint64_t pieces = (uint64_t)a.rows * a.pieces_per_row;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((pieces + 255) / 256, 256 * 16);
+    if (cls.kind == kProgramSiluMul)
+      map_pair_kernel<true><<<blocks, 256, 0, stream>>>(a);
+    else
+      map_pair_kernel<false><<<blocks, 256, 0, stream>>>(a);
+    return true;
+  }
+  if (cls.axis != rank - 1) return false;
   if (cls.kind == kProgramRmsNorm || cls.kind == kProgramResidualNorm) {
     const bool residual = cls.kind == kProgramResidualNorm;
     if (rank != 2 || p.n_inputs != (residual ? 3u : 2u)) return false;

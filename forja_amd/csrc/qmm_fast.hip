@@ -50,6 +50,10 @@ struct QmmArgs {
   // routed form
   const uint32_t *sorted_routes, *blocks, *n_blocks;
   uint32_t route_div;       // input row = route / route_div
+  // dense form only
+  const uint32_t *run_if_set;   // when not null: do nothing unless this device word is non-zero
+  const uint16_t *residual;     // optional bf16 rows added to the result before it is rounded
+  uint64_t residual_row_stride;
 };
 
 __device__ inline uint32_t pack2(float lo, float hi) {
@@ -74,6 +78,7 @@ __device__ inline bf16x8 unpack_word(uint32_t w) {
 // workgroup share the staged activations and own 32 output columns each.
 template <int MT, bool kPair, bool kRouted>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qmm_mfma_kernel(QmmArgs a) {
+  if (!kRouted && a.run_if_set && a.run_if_set[0] == 0) return;
   constexpr int NW = kWaves;
   constexpr int kThreads = 64 * NW;
   constexpr int KC = 512 / MT;  // 33 KB of LDS either way: two workgroups per CU overlap staging
@@ -267,6 +272,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
       const uint64_t out_row = kRouted ? row_ids[row] : first + row;
       const uint64_t at = out_row * a.out_row_stride + column;
+      if (!kRouted && a.residual)
+        value += bf16_bits_to_f32(a.residual[out_row * a.residual_row_stride + column]);
       if (a.out_f32)
         ((float *)a.out)[at] = value;
       else
@@ -638,7 +645,8 @@ __global__ __launch_bounds__(kSlabThreads) void qmm_slab_kernel(SlabArgs a) {
 // four consecutive columns (the host guarantees columns % 4 == 0 and aligned output rows).
 __global__ void sum_slabs_kernel(const float *partials, uint32_t slabs, uint32_t rows,
                                  uint32_t columns, void *out, uint64_t out_row_stride,
-                                 uint32_t out_f32) {
+                                 uint32_t out_f32, const uint16_t *residual,
+                                 uint64_t residual_row_stride) {
   const uint64_t flat = 4 * ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x);
   const uint64_t plane = (uint64_t)rows * columns;
   if (flat >= plane) return;
@@ -651,6 +659,13 @@ __global__ void sum_slabs_kernel(const float *partials, uint32_t slabs, uint32_t
     total.w += v.w;
   }
   const uint64_t at = (flat / columns) * out_row_stride + flat % columns;
+  if (residual) {   // four bf16 values, added before the result is rounded
+    const uint2 r = *(const uint2 *)(residual + (flat / columns) * residual_row_stride + flat % columns);
+    total.x += __uint_as_float(r.x << 16);
+    total.y += __uint_as_float(r.x & 0xffff0000u);
+    total.z += __uint_as_float(r.y << 16);
+    total.w += __uint_as_float(r.y & 0xffff0000u);
+  }
   if (out_f32) {
     *(float4 *)((float *)out + at) = total;
   } else {
@@ -730,7 +745,8 @@ void launch_slab(hipStream_t stream, const SlabArgs &s, dim3 grid) {
   qmm_slab_kernel<MT><<<grid, kSlabThreads, slab_lds_bytes<MT>(), stream>>>(s);
 }
 
-bool launch_skinny(fh_backend *backend, const QmmArgs &q) {
+bool launch_skinny(fh_backend *backend, const QmmArgs &q, const uint16_t *residual,
+                   uint64_t residual_row_stride) {
   hipStream_t stream = backend_stream(backend);
   const uint32_t slabs = q.inner / kSlabK;
   const uint64_t plane = (uint64_t)q.rows * q.columns;
@@ -760,7 +776,8 @@ bool launch_skinny(fh_backend *backend, const QmmArgs &q) {
     launch_slab<4>(stream, s, grid);
   if (slabs > 1)
     sum_slabs_kernel<<<(uint32_t)((plane / 4 + 255) / 256), 256, 0, stream>>>(
-        s.partials, slabs, q.rows, q.columns, q.out, q.out_row_stride, q.out_f32);
+        s.partials, slabs, q.rows, q.columns, q.out, q.out_row_stride, q.out_f32, residual,
+        residual_row_stride);
   return true;
 }
 
@@ -789,15 +806,31 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
   a.rows = p.rows;
   a.inner = p.inner;
   a.columns = p.columns;
+  const uint16_t *residual = nullptr;
+  uint64_t residual_row_stride = 0;
+  if (p.residual) {
+    const View &r = *p.residual;
+    if (r.dtype != FH_BF16 || p.out.dtype != FH_BF16 || r.stride[1] != 1 || r.stride[0] % 4 != 0 ||
+        r.offset % 4 != 0)
+      return false;
+    residual = u16_ptr(r);
+    residual_row_stride = r.stride[0];
+  }
   if (p.rows <= 128 && p.columns <= 16384 && p.columns % 4 == 0 && p.out.stride[0] % 4 == 0 &&
-      p.out.offset % 4 == 0) {
-    if (!launch_skinny(backend, a)) return false;
+      p.out.offset % 4 == 0 && (!residual || p.inner > kSlabK)) {
+    if (!launch_skinny(backend, a, residual, residual_row_stride)) return false;
     return true;
   }
-  if (p.rows > 128 && launch_quant_gemm(backend, p)) return true;
+  a.residual = residual;
+  a.residual_row_stride = residual_row_stride;
+  KernelTimer timer(backend, FH_KC_QMM_KERNEL);
+  if (p.rows > 128) {
+    // the tiled GEMM, followed by the any-range kernel conditioned on the GEMM's refusal
+    const uint32_t *refused = nullptr;
+    if (launch_quant_gemm(backend, p, &refused)) a.run_if_set = refused;
+  }
   int mt = p.rows <= 32 ? 1 : 2;
   uint32_t row_blocks = (p.rows + 32 * mt - 1) / (32 * mt);
-  KernelTimer timer(backend, FH_KC_QMM_KERNEL);
   launch_qmm<false, false>(stream, a, row_blocks, mt);
   return true;
 }

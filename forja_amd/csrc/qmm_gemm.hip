@@ -1,43 +1,39 @@
-// MLX-4bit quantised matmul for many activation rows (prefill chunks): a tiled f16 MFMA GEMM
-// whose weight tiles are dequantised on their way into LDS.
+// MLX-4bit quantised matmul for many activation rows (prefill chunks): the weights are
+// dequantised to fp16 once per product and a plain tiled f16 MFMA GEMM does the rest.
 //
 // y[m,n] = sum_k x[m,k] * (scale[n,k/64] * q[n,k] + bias[n,k/64])   (affine_quant_dot,
-// crates/forja-cpu/src/lib.rs:1277-1310).  With hundreds of rows per weight the work is bound by
-// the matrix cores, not by HBM, so the kernel is a classic GEMM:
-//   * operands are fp16, not bf16: a dequantised weight scale*q+bias rounded to bf16 (8
-//     significant bits) is too coarse for the stated tolerance on outputs that cancel, fp16 (11
-//     bits) is not, and the matrix cores run both at the same rate.  bf16 activations convert to
-//     fp16 exactly; prepare_rows_kernel does that once per product (scaling a row by a power of
-//     two first if it holds values beyond the fp16 range, undone exactly in the epilogue) and
-//     stores every 8 values in the order (0,4,1,5,2,6,3,7) in which nibbles unpack pairwise;
-//   * workgroup tile 256 rows x 256 columns, K step 64 (one quantisation group); four waves in
-//     a 2 x 2 arrangement, each owning 128 x 128 outputs = 16 accumulator tiles of
-//     v_mfma_f32_32x32x16_f16 (256 accumulator registers);
-//   * both operand tiles live in LDS, double buffered.  The activation tile goes from memory
-//     straight into LDS (global_load_lds, no registers), its 16-byte pieces XOR-swizzled inside
-//     each 128-byte row so that operand reads are bank-conflict free without padding; the weight
-//     tile passes through registers to be dequantised and is stored in rows padded to 144 bytes.
-//     The next K step is staged while the current one is multiplied, one barrier per step;
-//     packed weights are requested two steps ahead (they are cold in HBM);
-//   * a thread dequantises one weight row of the tile per step (64 nibbles): two nibbles become
-//     the fp16 pair (1024+q) with one and-or, minus 1024 exactly, then one packed fused
-//     multiply-add gives scale*q - c rounded once, with c ~ 7.5*scale the fp16 value that centres
-//     the group.  What the centring takes out, (bias + c) * sum of the group's activations, is
-//     added back exactly: the row sums per group come from prepare_rows_kernel in f32 and an f32
-//     MFMA adds the rank-2 update of every two groups to the same accumulators.  Centred values
-//     are half the magnitude of the weights and carry no bias, which keeps the fp16 rounding
-//     inside the tolerance at the deepest contractions (K = 17408).  That needs every scale and bias to lie
-//     well inside the fp16 range; check_affine_kernel scans them first and raises a flag
-//     otherwise, and then a second instantiation of the kernel, which dequantises in f32, does
-//     the work instead (both are launched; the one whose turn it is not returns at once).  Every weight byte is read from HBM once per 256 rows and unpacked once per
-//     workgroup;
-//   * the workgroup -> tile map gives the 32 workgroups that run together on one XCD a patch of
+// crates/forja-cpu/src/lib.rs:1277-1310).  With thousands of rows per weight the work is bound
+// by the matrix cores, not by HBM: writing the dequantised matrix (4 bytes per weight, written and
+// read back) costs a few percent of the product's time and takes every unpacking instruction,
+// strided weight load and register-staged tile out of the GEMM loop.
+//   * Operands are fp16, not bf16: a dequantised weight rounded to bf16 (8 significant bits) is
+//     too coarse for the stated tolerance on outputs that cancel, fp16 (11 bits) is not, and the
+//     matrix cores run both at the same rate.  bf16 activations convert to fp16 exactly once a row
+//     is scaled by a power of two into the fp16 range (undone exactly when the result is stored).
+//   * Weights are centred: w = scale * q - c with c = 7.5 * scale, which halves their magnitude
+//     and so their rounding error; at the deepest contraction (K = 17408) the uncentred form does
+//     not meet the tolerance.  What centring takes out, (bias + c) * sum of the group's
+//     activations, is put back through the same GEMM: both operand matrices get three more
+//     columns per quantisation group, holding S/64 and 64 * (bias + c) each split in an fp16
+//     head and tail (head*head + tail*head + head*tail, about 22 significant bits), so the
+//     kernel needs no side channel for it.  The contraction grows by 3/64.
+//   * prepare_rows_kernel and prepare_weights_kernel write the two operand matrices
+//     [rows, Kt] and [N, Kt], Kt = K + 3K/64 rounded up to the K step, every 8 values in the
+//     order (0,4,1,5,2,6,3,7) in which nibbles unpack pairwise.  prepare_weights_kernel also
+//     raises a flag when some scale or bias does not fit this scheme's fp16 range; the GEMM
+//     kernel then returns at once and the caller runs its any-range kernel instead.
+//   * GEMM: workgroup tile 256 rows x 256 columns, K step 64; four waves in a 2 x 2
+//     arrangement, each owning 128 x 128 outputs = 16 accumulator tiles of
+//     v_mfma_f32_32x32x16_f16 (256 accumulator registers).  Both operand tiles go from memory
+//     straight into LDS (global_load_lds, no registers), double buffered, their 16-byte pieces
+//     XOR-swizzled inside each 128-byte row so that operand reads are bank-conflict free
+//     without padding; one barrier per step.  Operand registers are double buffered too: the
+//     reads of a sub-step are issued before the previous sub-step's MFMAs.
+//   * The workgroup -> tile map gives the 32 workgroups that run together on one XCD a patch of
 //     about 4 row tiles x 8 column tiles, so that its L2 serves each activation tile to 8
 //     workgroups and each weight tile to 4, instead of every workgroup streaming its own.
 // Accumulation is f32.
 #include "fast_kernels.hpp"
-
-#include <type_traits>
 
 namespace fh {
 
@@ -48,27 +44,33 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-constexpr int kBM = 256, kBN = 256, kBK = 64;
+constexpr int kBM = 256, kBN = 256;
+constexpr int kPadK = 64;   // operand rows are padded to a multiple of this (every K step divides it)
+// K step and LDS stages of the GEMM.  Steps of 32 with three or four stages measured the same
+// (the kernel is bound by what the matrix cores and the L2 -> LDS path sustain, not by latency).
+constexpr int kGemmK = 64, kGemmStages = 2;
+constexpr int kGemmLds = kGemmStages * 2 * kBM * 2 * kGemmK;   // both operand tiles of every stage
 constexpr int kBand = 8;   // column tiles per band of the tile numbering
-constexpr int kPitch = 2 * kBK + 16;              // bytes per staged weight row
-constexpr int kATileBytes = kBM * 2 * kBK;        // activation tile, swizzled, no padding
-constexpr int kBTileBytes = kBN * kPitch;         // weight tile
-constexpr int kSideBytes = 4 * (kBM + kBN) * 4;  // row sums and column offsets of four groups, f32
-constexpr int kGemmLds = 2 * (kATileBytes + kBTileBytes) + kSideBytes;
+constexpr uint32_t kMaxGroups = 512;              // quantisation groups per row the row kernel holds
+
+// Columns of the operand matrices: K values, then 3 per group, rounded up to the K step.
+inline uint32_t padded_inner(uint32_t inner) {
+  const uint32_t with_sums = inner + 3 * (inner / 64);
+  return (with_sums + kPadK - 1) / kPadK * kPadK;
+}
 
 struct GemmArgs {
-  const uint16_t *x;        // fp16 rows prepared by prepare_rows_kernel, stride = inner
+  const uint16_t *a, *b;    // fp16 operand matrices [rows, kt] and [columns, kt]
   const float *row_unscale; // per row: multiply the result by this
-  const float *group_sums;  // [inner / 64][rows]: sums of the prepared rows per group
-  uint64_t x_row_stride;
-  const uint32_t *packed;
-  const uint16_t *scales, *biases;
+  uint32_t kt;
   void *out;
   uint64_t out_row_stride;
   uint32_t out_f32;
-  uint32_t rows, inner, columns;
+  uint32_t rows, columns;
   uint32_t row_tiles, column_tiles;
-  const uint32_t *wide_flag;   // non-zero: some scale or bias does not fit fp16
+  const uint32_t *refused;     // non-zero: some scale or bias is out of range, do nothing
+  const uint16_t *residual;    // optional bf16 rows added before rounding
+  uint64_t residual_row_stride;
 };
 
 __device__ inline uint32_t pack2(float lo, float hi) {
@@ -83,48 +85,28 @@ __device__ inline uint32_t pack_f16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-// Eight nibbles of `w`, dequantised to fp16, as the four pairs (0,4)(1,5)(2,6)(3,7).
-// Fast form: (1024+q) pairs by and-or, minus 1024 (exact), then fused scale*q+bias per pair.
-__device__ inline uint4 dequantise_word(uint32_t w, f16x2 scale2, f16x2 shift2) {
-  const uint32_t mask = 0x000f000fu, magic = 0x64006400u;
-  const f16x2 offset = {(_Float16)1024.0f, (_Float16)1024.0f};
-  uint32_t raw[4] = {(w & mask) | magic, ((w >> 4) & mask) | magic, ((w >> 8) & mask) | magic,
-                     ((w >> 12) & mask) | magic};
-  uint32_t out[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const f16x2 q = __builtin_bit_cast(f16x2, raw[i]) - offset;
-    out[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(q, scale2, shift2));
-  }
-  return make_uint4(out[0], out[1], out[2], out[3]);
+__device__ inline uint16_t f16_bits(float v) {
+  return __builtin_bit_cast(uint16_t, (_Float16)v);
 }
 
-// The same in f32 with one rounding to fp16, for scales or biases outside the fp16 range.
-__device__ inline uint4 dequantise_word_wide(uint32_t w, float scale, float shift) {
-  float v[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(scale, (float)((w >> (4 * i)) & 15u), shift);
-  return make_uint4(pack_f16(v[0], v[4]), pack_f16(v[1], v[5]), pack_f16(v[2], v[6]),
-                    pack_f16(v[3], v[7]));
+// Head and tail of v in fp16: v ~ head + tail.
+__device__ inline void split_f16(float v, float *head, float *tail) {
+  *head = (float)(_Float16)v;
+  *tail = (float)(_Float16)(v - *head);
 }
 
-// Scales and biases the fp16 form can take: finite and well inside the fp16 range (15 * scale +
-// bias must not overflow).  Magnitudes below the fp16 normal range become fp16 subnormals, an
-// absolute error under 2^-25 per weight, far below the rounding of the weight itself.
-__device__ inline bool f16_safe(float scale, float bias) {
-  return fabsf(scale) <= 2048.0f && fabsf(bias) <= 30000.0f;   // false for NaN too
-}
-
-// x bf16 [rows, inner] -> fp16 [rows, inner] (every 8 values stored as 0,4,1,5,2,6,3,7), each row
-// multiplied by a power of two that brings its largest magnitude under 2^15; unscale[row] is the
-// inverse; group_sums[g][row] is the f32 sum of the row's 64 prepared values of group g.
+// x bf16 [rows, inner] -> fp16 [rows, kt].  Each row is multiplied by the power of two that
+// brings its largest magnitude into [2^14, 2^15) (unscale[row] is the inverse); every 8 values are
+// stored in the order (0,4,1,5,2,6,3,7); after the inner values come, for every group g of 64,
+// (head, tail, head) of S_g / 64 with S_g the f32 sum of the group's scaled values, then zeros.
 // One wave per row.
 __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, uint64_t x_row_stride,
-                                                           uint32_t rows, uint32_t inner,
-                                                           uint16_t *out, float *unscale,
-                                                           float *group_sums) {
-  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (row >= rows) return;
+                                                           uint32_t rows, uint32_t inner, uint32_t kt,
+                                                           uint16_t *out, float *unscale) {
+  __shared__ float sums[4][kMaxGroups];
+  const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * 4 + wave;
+  if (row >= rows) return;   // no workgroup-wide barrier below
   const uint16_t *in_row = x + (uint64_t)row * x_row_stride;
   uint32_t top = 0;   // largest magnitude bits (bf16 without sign) in the row
   for (uint32_t piece = lane; piece < inner / 8; piece += 64) {
@@ -140,10 +122,11 @@ __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, ui
   }
   for (int offset = 32; offset > 0; offset >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, offset, 64));
   const int exponent = (int)(top >> 7) - 127;                    // floor(log2(max |x|))
-  const int down = exponent > 14 ? exponent - 14 : 0;            // scale by 2^-down
+  int down = exponent - 14;                                      // scale by 2^-down
+  if (down < -100) down = -100;                                  // rows of zeros and denormals
   const float scale = __uint_as_float((uint32_t)(127 - down) << 23);
   if (lane == 0) unscale[row] = __uint_as_float((uint32_t)(127 + down) << 23);
-  uint16_t *out_row = out + (uint64_t)row * inner;
+  uint16_t *out_row = out + (uint64_t)row * kt;
   for (uint32_t piece = lane; piece < inner / 8; piece += 64) {
     const uint4 v = *(const uint4 *)(in_row + 8 * piece);
     const uint32_t words[4] = {v.x, v.y, v.z, v.w};
@@ -160,29 +143,99 @@ __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, ui
     sum += __shfl_xor(sum, 1, 64);
     sum += __shfl_xor(sum, 2, 64);
     sum += __shfl_xor(sum, 4, 64);
-    if ((piece & 7) == 0) group_sums[(uint64_t)(piece >> 3) * rows + row] = sum;
+    if ((piece & 7) == 0) sums[wave][piece >> 3] = sum;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const uint32_t groups = inner / 64;
+  for (uint32_t extra = lane; extra < kt - inner; extra += 64) {
+    const uint32_t group = extra / 3, kind = extra % 3;
+    float value = 0.0f;
+    if (group < groups) {
+      float head, tail;
+      split_f16(sums[wave][group] * (1.0f / 64.0f), &head, &tail);
+      value = kind == 1 ? tail : head;
+    }
+    out_row[inner + extra] = f16_bits(value);
   }
 }
 
-// flag[0] = 1 if any scale or bias of the matrix is too large for (or not a number in) fp16.
-__global__ void check_affine_kernel(const uint16_t *scales, const uint16_t *biases, uint64_t count,
-                                    uint32_t *flag) {
-  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= count) return;
-  if (!f16_safe(bf16_bits_to_f32(scales[i]), bf16_bits_to_f32(biases[i]))) flag[0] = 1;
+// Scales and biases this scheme can take: every centred weight and 64 * (bias + centre) must
+// stay inside the fp16 range.  False for NaN too.
+__device__ inline bool f16_safe(float scale, float bias) {
+  return fabsf(scale) <= 4000.0f && fabsf(bias + 7.5f * scale) <= 900.0f;
 }
 
-template <bool kWide>
-__global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
-  if ((a.wide_flag[0] != 0) != kWide) return;
+// packed/scales/biases [columns, inner] -> fp16 [columns, kt]: scale * q - 7.5 * scale (one
+// rounding, from f32) in the order (0,4,1,5,2,6,3,7) inside every 8, then per group (head, head,
+// tail) of 64 * (bias + 7.5 * scale), then zeros.  Eight threads per 64-value chunk, one packed
+// word each; refused[0] is set when a group is out of range.
+__global__ __launch_bounds__(256) void prepare_weights_kernel(const uint32_t *packed,
+                                                              const uint16_t *scales,
+                                                              const uint16_t *biases, uint32_t columns,
+                                                              uint32_t inner, uint32_t kt,
+                                                              uint16_t *out, uint32_t *refused) {
+  const uint64_t flat = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t part = (uint32_t)(flat & 7);
+  const uint32_t chunks = kt / 64, groups = inner / 64;
+  const uint64_t chunk_flat = flat >> 3;
+  if (chunk_flat >= (uint64_t)columns * chunks) return;
+  const uint32_t column = (uint32_t)(chunk_flat / chunks), chunk = (uint32_t)(chunk_flat % chunks);
+  uint16_t *to = out + (uint64_t)column * kt + 64 * chunk + 8 * part;
+  const uint16_t *s_row = scales + (uint64_t)column * groups, *b_row = biases + (uint64_t)column * groups;
+  if (chunk < groups) {
+    const float scale = bf16_bits_to_f32(s_row[chunk]), bias = bf16_bits_to_f32(b_row[chunk]);
+    if (part == 0 && !f16_safe(scale, bias)) refused[0] = 1;
+    const uint32_t w = packed[(uint64_t)column * (inner / 8) + 8 * chunk + part];
+    const float centre = 7.5f * scale;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(scale, (float)((w >> (4 * i)) & 15u), -centre);
+    *(uint4 *)to = make_uint4(pack_f16(v[0], v[4]), pack_f16(v[1], v[5]), pack_f16(v[2], v[6]),
+                              pack_f16(v[3], v[7]));
+    return;
+  }
+  uint16_t values[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t extra = 64 * (chunk - groups) + 8 * part + i;
+    const uint32_t group = extra / 3, kind = extra % 3;
+    float value = 0.0f;
+    if (group < groups) {
+      const float scale = bf16_bits_to_f32(s_row[group]), bias = bf16_bits_to_f32(b_row[group]);
+      float head, tail;
+      split_f16(64.0f * (bias + 7.5f * scale), &head, &tail);
+      value = kind == 2 ? tail : head;
+    }
+    values[i] = f16_bits(value);
+  }
+  *(uint4 *)to = make_uint4(values[0] | ((uint32_t)values[1] << 16), values[2] | ((uint32_t)values[3] << 16),
+                            values[4] | ((uint32_t)values[5] << 16), values[6] | ((uint32_t)values[7] << 16));
+}
+
+constexpr uint32_t wait_vmcnt(uint32_t n) {   // s_waitcnt immediate: vmcnt(n) only
+  return (n & 15u) | ((n >> 4) << 14) | 0x0f70u;
+}
+
+template <int kBK, int kStages>
+__global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
+  if (a.refused[0] != 0) return;
+  constexpr int kSub = kBK / 16;                 // MFMA sub-steps per K step
+  constexpr int kRowBytes = 2 * kBK;             // one tile row in LDS
+  constexpr int kTile = kBM * kRowBytes;         // one operand tile of one stage
+  constexpr int kSlots = kRowBytes / 16;         // 16-byte pieces per row
+  constexpr int kRowsPerLoad = 64 / kSlots;      // rows one wave-wide load instruction covers
+  constexpr int kLoads = 64 / kRowsPerLoad;      // instructions per wave, operand and stage
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
-  unsigned char *a_tiles = gemm_lds;                      // [2][kBM][128], pieces swizzled
-  unsigned char *b_tiles = gemm_lds + 2 * kATileBytes;    // [2][kBN][kPitch]
-  float *side_rows = (float *)(gemm_lds + 2 * (kATileBytes + kBTileBytes));   // [4][kBM], ring by group
-  float *side_cols = side_rows + 4 * kBM;                                     // [4][kBN]
+  unsigned char *a_tiles = gemm_lds;                      // [kStages][kBM][kRowBytes], pieces swizzled
+  unsigned char *b_tiles = gemm_lds + kStages * kTile;    // [kStages][kBN][kRowBytes]
   const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const uint32_t wm = wave >> 1, wn = wave & 1;
   const uint32_t l32 = lane & 31, kh = lane >> 5;
+  // A row's piece p sits in slot p ^ swizzle(row), which spreads the 32 rows a wave reads at once
+  // over all LDS banks.
+  auto swizzle_of = [](uint32_t row) { return kBK == 64 ? (row >> 1) & 7u : (row >> 2) & 3u; };
 
   // workgroup -> tile.  Tiles are numbered band by band (a band = kBand column tiles), row
   // tile major inside a band, so 32 consecutive numbers are a 4 x 8 patch of tiles sharing
@@ -199,62 +252,31 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
   const uint32_t bm = in_band / band_width, bn = band * kBand + in_band % band_width;
   const uint32_t row0 = bm * kBM, col0 = bn * kBN;
 
-  // Activation staging: a wave owns 64 rows of the tile; one instruction moves 8 rows (lane ->
-  // row lane/8, LDS slot lane%8), and the piece a lane fetches is its slot XOR ((row >> 1) & 7).
-  const uint16_t *a_src[8];
+  // Staging: a wave owns 64 rows of each operand tile; one instruction moves kRowsPerLoad rows
+  // (lane -> row lane / kSlots, LDS slot lane % kSlots) and the piece a lane fetches is its slot
+  // XOR the row's swizzle.  Rows past the end of a matrix reload its last row; what they produce
+  // is never stored.
+  const uint16_t *a_src[kLoads], *b_src[kLoads];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const uint32_t in_tile = 64 * wave + 8 * i + lane / 8;
-    const uint32_t row = min(row0 + in_tile, a.rows - 1);   // tail rows reload the last row; never stored
-    const uint32_t piece = (lane % 8) ^ ((in_tile >> 1) & 7);
-    a_src[i] = a.x + (uint64_t)row * a.x_row_stride + 8 * piece;
+  for (int i = 0; i < kLoads; ++i) {
+    const uint32_t in_tile = 64 * wave + kRowsPerLoad * i + lane / kSlots;
+    const uint32_t piece = (lane % kSlots) ^ swizzle_of(in_tile);
+    a_src[i] = a.a + (uint64_t)min(row0 + in_tile, a.rows - 1) * a.kt + 8 * piece;
+    b_src[i] = a.b + (uint64_t)min(col0 + in_tile, a.columns - 1) * a.kt + 8 * piece;
   }
-  auto stage_a = [&](uint32_t buffer, uint32_t step) {
-    unsigned char *to = a_tiles + buffer * kATileBytes + 64 * wave * 128;
+  const uint32_t steps = a.kt / kBK;
+  auto stage = [&](uint32_t buffer, uint32_t step) {
+    const uint32_t st = min(step, steps - 1);   // past the end: reload the last step, never used
+    unsigned char *to_a = a_tiles + buffer * kTile + 64 * wave * kRowBytes;
+    unsigned char *to_b = b_tiles + buffer * kTile + 64 * wave * kRowBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < kLoads; ++i) {
       __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void *)(a_src[i] + step * kBK),
-          (__attribute__((address_space(3))) void *)(to + 8 * i * 128), 16, 0, 0);
-  };
-  // Weight staging: thread t dequantises row t of the tile.
-  const uint32_t b_col = min(col0 + tid, a.columns - 1);
-  const uint32_t steps = a.inner / kBK;
-  const uint32_t *w_row = a.packed + (uint64_t)b_col * (a.inner / 8);
-  const uint16_t *s_row = a.scales + (uint64_t)b_col * steps;
-  const uint16_t *b_row = a.biases + (uint64_t)b_col * steps;
-  uint4 w_now[2], w_next[2];
-  uint32_t affine_now, affine_next;   // scale | bias << 16
-  float sum_now, sum_next;            // group sum of tile row `tid`
-  const float *sums_of_row = a.group_sums + min(row0 + tid, a.rows - 1);
-  auto fetch_w = [&](uint32_t step) {
-    const uint32_t st = min(step, steps - 1);
-    w_next[0] = *(const uint4 *)(w_row + st * 8);
-    w_next[1] = *(const uint4 *)(w_row + st * 8 + 4);
-    affine_next = (uint32_t)s_row[st] | ((uint32_t)b_row[st] << 16);
-    sum_next = sums_of_row[(uint64_t)st * a.rows];
-  };
-  // The group's centre c (an fp16 value near 7.5 * scale) and what it leaves to add back per
-  // unit of activation sum: bias + c.
-  auto centre_of = [&](float scale) { return (float)(_Float16)(7.5f * scale); };
-  auto stage_side = [&](uint32_t step) {
-    const float scale = bf16_bits_to_f32(affine_now & 0xffffu), bias = bf16_bits_to_f32(affine_now >> 16);
-    side_rows[(step & 3) * kBM + tid] = sum_now;
-    side_cols[(step & 3) * kBN + tid] = bias + (kWide ? 7.5f * scale : centre_of(scale));
-  };
-  // one packed word (8 values) of the weight row: `part` 0..7
-  auto stage_b = [&](uint32_t buffer, int part) {
-    unsigned char *bt = b_tiles + buffer * kBTileBytes + tid * kPitch + 16 * part;
-    const float scale = bf16_bits_to_f32(affine_now & 0xffffu), bias = bf16_bits_to_f32(affine_now >> 16);
-    const uint4 w = w_now[part / 4];
-    const uint32_t word = (part & 3) == 0 ? w.x : ((part & 3) == 1 ? w.y : ((part & 3) == 2 ? w.z : w.w));
-    (void)bias;
-    if (kWide) {
-      *(uint4 *)(bt) = dequantise_word_wide(word, scale, -7.5f * scale);
-    } else {
-      const _Float16 shift = (_Float16)(-centre_of(scale));
-      const f16x2 scale2 = {(_Float16)scale, (_Float16)scale}, shift2 = {shift, shift};
-      *(uint4 *)(bt) = dequantise_word(word, scale2, shift2);
+          (const __attribute__((address_space(1))) void *)(a_src[i] + st * kBK),
+          (__attribute__((address_space(3))) void *)(to_a + kRowsPerLoad * i * kRowBytes), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void *)(b_src[i] + st * kBK),
+          (__attribute__((address_space(3))) void *)(to_b + kRowsPerLoad * i * kRowBytes), 16, 0, 0);
     }
   };
 
@@ -265,76 +287,57 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
     for (int j = 0; j < 4; ++j)
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  // prologue: step 0 staged, weights of step 1 in flight
-  stage_a(0, 0);
-  fetch_w(0);
-  w_now[0] = w_next[0];
-  w_now[1] = w_next[1];
-  affine_now = affine_next;
-  sum_now = sum_next;
-  fetch_w(1);
-  for (int part = 0; part < 8; ++part) stage_b(0, part);
-  stage_side(0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's rows have landed in LDS
-  __syncthreads();
-  const uint32_t swizzle = (l32 >> 1) & 7;
-  // One K step on LDS buffer kBuffer (= step & 1); the loop below runs them in pairs so that the
-  // buffer, and the centring update after every second step, are fixed at compile time.
-  auto k_step = [&](uint32_t step, auto parity) {
-    constexpr uint32_t buffer = decltype(parity)::value;
-    stage_a(buffer ^ 1, min(step + 1, steps - 1));
-    w_now[0] = w_next[0];   // weights of step+1: requested a whole step ago
-    w_now[1] = w_next[1];
-    affine_now = affine_next;
-    sum_now = sum_next;
-    fetch_w(step + 2);
-    const unsigned char *at = a_tiles + buffer * kATileBytes + (128 * wm + l32) * 128;
-    const unsigned char *bt = b_tiles + buffer * kBTileBytes + (128 * wn + l32) * kPitch + 16 * kh;
+  // Operand registers, two sets: the set for the next sub-step is read from LDS while the matrix
+  // pipe works on the current one.  The last sub-step of a K step is multiplied after the
+  // step's barrier, behind the first read of the next step.
+  f16x8 a_op[2][4], b_op[2][4];
+  const uint32_t swizzle = swizzle_of(l32);
+  auto read_operands = [&](uint32_t buffer, int s, int set) {
+    const unsigned char *at = a_tiles + buffer * kTile + (128 * wm + l32) * kRowBytes;
+    const unsigned char *bt = b_tiles + buffer * kTile + (128 * wn + l32) * kRowBytes;
+    const uint32_t piece = 16 * ((2 * s + kh) ^ swizzle);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      f16x8 a_op[4], b_op[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        a_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * 128 + 16 * ((2 * s + kh) ^ swizzle)));
-        b_op[i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kPitch + 32 * s));
-      }
-      // eight MFMAs, then one word of the next step's weights, fenced so that the staging
-      // instructions issue in the shadow of the matrix pipe instead of after all sixteen
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[i], b_op[j], acc[i][j], 0, 0, 0);
-        if (i & 1) {
-          __builtin_amdgcn_sched_barrier(0);
-          stage_b(buffer ^ 1, 2 * s + (i >> 1));
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
+    for (int i = 0; i < 4; ++i) {
+      a_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * kRowBytes + piece));
+      b_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kRowBytes + piece));
     }
-    // after the second step of a pair: the centring terms of the two groups just multiplied,
-    // as one f32 MFMA per accumulator tile (lane half kh supplies group step - 1 + kh of both
-    // operands)
-    if (buffer == 1) {
-      float row_sum[4], column_offset[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        row_sum[i] = side_rows[((step - 1 + kh) & 3) * kBM + 128 * wm + 32 * i + l32];
-        column_offset[i] = side_cols[((step - 1 + kh) & 3) * kBN + 128 * wn + 32 * i + l32];
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(row_sum[i], column_offset[j], acc[i][j], 0, 0, 0);
-    }
-    stage_side(step + 1);   // a ring slot nobody reads in this step
-    __builtin_amdgcn_s_waitcnt(0x0f75);   // vmcnt(5): all but the five loads of fetch_w just issued
-    __syncthreads();
   };
-  for (uint32_t step = 0; step < steps; step += 2) {   // K is a multiple of 256: steps is even
-    k_step(step, std::integral_constant<uint32_t, 0>{});
-    k_step(step + 1, std::integral_constant<uint32_t, 1>{});
+  auto multiply = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[set][i], b_op[set][j], acc[i][j], 0, 0, 0);
+  };
+
+  // Stages 0 .. kStages-1 are requested up front; from then on the buffer a step frees is
+  // refilled with the step kStages ahead, so kStages-1 steps of loads are always in flight.
+#pragma unroll
+  for (int p = 0; p < kStages; ++p) stage(p, p);
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt((kStages - 1) * 2 * kLoads));   // step 0 has landed
+  __syncthreads();
+  read_operands(0, 0, 0);
+  uint32_t buffer = 0;
+  for (uint32_t step = 0; step < steps; ++step) {
+    const uint32_t next_buffer = buffer + 1 == kStages ? 0 : buffer + 1;
+#pragma unroll
+    for (int s = 0; s < kSub; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 1 < kSub) {
+        read_operands(buffer, s + 1, (s + 1) & 1);
+      } else {
+        // every read of this buffer has been issued: once they have landed, and the next step's
+        // tiles too, the workgroup meets and the buffer is refilled
+        __builtin_amdgcn_s_waitcnt(0xc07f);                                   // lgkmcnt(0)
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt((kStages - 2) * 2 * kLoads));   // step + 1 has landed
+        __syncthreads();
+        stage(buffer, step + kStages);
+        read_operands(next_buffer, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(s & 1);
+    }
+    buffer = next_buffer;
   }
   // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile
 #pragma unroll
@@ -347,7 +350,9 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
         const uint32_t row = row0 + 128 * wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
         if (row >= a.rows) continue;
         const uint64_t at_out = (uint64_t)row * a.out_row_stride + column;
-        const float value = acc[i][j][r] * a.row_unscale[row];
+        float value = acc[i][j][r] * a.row_unscale[row];
+        if (a.residual)
+          value += __uint_as_float((uint32_t)a.residual[(uint64_t)row * a.residual_row_stride + column] << 16);
         if (a.out_f32)
           ((float *)a.out)[at_out] = value;
         else
@@ -358,52 +363,54 @@ __global__ __launch_bounds__(256) void qmm_gemm_kernel(GemmArgs a) {
 
 }  // namespace
 
-bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p) {
-  const uint64_t rows_bytes = ((uint64_t)p.rows * p.inner * 2 + 255) / 256 * 256;
+bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t **refused) {
+  if (p.inner / 64 > kMaxGroups) return false;
+  const uint32_t kt = padded_inner(p.inner);
+  const uint64_t a_bytes = ((uint64_t)p.rows * kt * 2 + 255) / 256 * 256;
+  const uint64_t b_bytes = ((uint64_t)p.columns * kt * 2 + 255) / 256 * 256;
   const uint64_t unscale_bytes = ((uint64_t)p.rows * sizeof(float) + 255) / 256 * 256;
-  const uint64_t sums_bytes = ((uint64_t)p.rows * (p.inner / kBK) * sizeof(float) + 255) / 256 * 256;
-  char *ws = backend_workspace(backend, rows_bytes + unscale_bytes + sums_bytes + 256);
+  char *ws = backend_workspace(backend, a_bytes + b_bytes + unscale_bytes + 256);
   if (!ws) return false;
   hipStream_t stream = backend_stream(backend);
+  uint32_t *flag = (uint32_t *)(ws + a_bytes + b_bytes + unscale_bytes);
   GemmArgs a{};
-  a.x = (const uint16_t *)ws;
-  a.row_unscale = (const float *)(ws + rows_bytes);
-  a.group_sums = (const float *)(ws + rows_bytes + unscale_bytes);
-  a.x_row_stride = p.inner;
-  a.packed = (const uint32_t *)p.packed.base + p.packed.offset;
-  a.scales = (const uint16_t *)p.scales.base + p.scales.offset;
-  a.biases = (const uint16_t *)p.biases.base + p.biases.offset;
+  a.a = (const uint16_t *)ws;
+  a.b = (const uint16_t *)(ws + a_bytes);
+  a.row_unscale = (const float *)(ws + a_bytes + b_bytes);
+  a.kt = kt;
   a.out = p.out.dtype == FH_F32 ? (void *)((float *)p.out.base + p.out.offset)
                                 : (void *)((uint16_t *)p.out.base + p.out.offset);
   a.out_row_stride = p.out.stride[0];
   a.out_f32 = p.out.dtype == FH_F32;
+  if (p.residual) {
+    a.residual = (const uint16_t *)p.residual->base + p.residual->offset;
+    a.residual_row_stride = p.residual->stride[0];
+  }
   a.rows = p.rows;
-  a.inner = p.inner;
   a.columns = p.columns;
   a.row_tiles = (p.rows + kBM - 1) / kBM;
   a.column_tiles = (p.columns + kBN - 1) / kBN;
-  uint32_t *flag = (uint32_t *)(ws + rows_bytes + unscale_bytes + sums_bytes);
-  a.wide_flag = flag;
+  a.refused = flag;
   static bool configured = false;   // raise the dynamic LDS limit once per process
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_gemm_kernel<false>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void *>(&qmm_gemm_kernel<true>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds) != hipSuccess)
       return false;
     configured = true;
   }
   const uint32_t grid = (a.row_tiles * a.column_tiles + 255) / 256 * 256;
-  KernelTimer timer(backend, FH_KC_QMM_KERNEL);
-  prepare_rows_kernel<<<(p.rows + 3) / 4, 256, 0, stream>>>(
-      (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, (uint16_t *)ws,
-      (float *)(ws + rows_bytes), (float *)(ws + rows_bytes + unscale_bytes));
   launch_fill_u32(stream, flag, 1, 0);
-  const uint64_t affine_count = (uint64_t)p.columns * (p.inner / kBK);
-  check_affine_kernel<<<(uint32_t)((affine_count + 255) / 256), 256, 0, stream>>>(a.scales, a.biases,
-                                                                                 affine_count, flag);
-  qmm_gemm_kernel<false><<<grid, 256, kGemmLds, stream>>>(a);
-  qmm_gemm_kernel<true><<<grid, 256, kGemmLds, stream>>>(a);
+  prepare_rows_kernel<<<(p.rows + 3) / 4, 256, 0, stream>>>(
+      (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, kt, (uint16_t *)ws,
+      (float *)(ws + a_bytes + b_bytes));
+  const uint64_t weight_threads = (uint64_t)p.columns * (kt / 64) * 8;
+  prepare_weights_kernel<<<(uint32_t)((weight_threads + 255) / 256), 256, 0, stream>>>(
+      (const uint32_t *)p.packed.base + p.packed.offset,
+      (const uint16_t *)p.scales.base + p.scales.offset,
+      (const uint16_t *)p.biases.base + p.biases.offset, p.columns, p.inner, kt,
+      (uint16_t *)(ws + a_bytes), flag);
+  gemm_f16_kernel<kGemmK, kGemmStages><<<grid, 256, kGemmLds, stream>>>(a);
+  *refused = flag;
   return true;
 }
 

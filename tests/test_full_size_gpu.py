@@ -74,6 +74,26 @@ def test_quantised_projection_fast_and_generic_paths_agree(hip, rows, n, k, note
     release(hip, x, x_wide, fast, generic, *weights)
 
 
+@pytest.mark.parametrize("rows,n,k,note", [
+    (8256, 1024, 2048, "config 4 prefill rows: residual add joined to the tiled GEMM"),
+    (128, 5120, 17408, "config 4 decode rows: residual add joined to the slab sum"),
+])
+def test_projection_with_residual_add_fast_and_generic_paths_agree(hip, rows, n, k, note):
+    weights = quantised(hip, n, k, seed=111)
+    x = seeded(hip, DType.BF16, (rows, k), 111, 4)
+    residual = seeded(hip, DType.BF16, (rows, n), 111, 5)
+    x_wide = as_f32(hip, x)
+    add = hip.prepare_epilogue(programs.add_elements())
+    fast = hip.alloc(DType.BF16, (rows, n))
+    generic = hip.alloc(DType.F32, (rows, n))
+    commands = CommandList()
+    commands.dispatch_epilogue(Op.quant_matmul(4, 64), [x, *weights], fast, add, [residual])
+    commands.dispatch_epilogue(Op.quant_matmul(4, 64), [x_wide, *weights], generic, add, [residual])
+    run(hip, commands)
+    assert_close(to_f32(hip.read(fast), DType.BF16), to_f32(hip.read(generic), DType.F32), DType.BF16)
+    release(hip, x, x_wide, residual, fast, generic, *weights)
+
+
 def test_config2_moe_block_fast_and_generic_paths_agree(hip):
     """256 decode tokens, 128 experts, top-8 of N(0,1) router logits, expert SwiGLU 2048 x 768."""
     tokens, hidden, experts, top_k, inner = 256, 2048, 128, 8, 768

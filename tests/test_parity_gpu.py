@@ -207,6 +207,39 @@ def test_quant_matmul_on_strided_views_with_bias_epilogue(cpu, hip):
     differential(cpu, hip, build)
 
 
+@pytest.mark.parametrize("rows,n,k,kind", [
+    (128, 256, 1024, "add"),    # decode rows: the add joins the slab sum
+    (8, 64, 256, "add"),        # a single K slab: accumulators + epilogue program
+    (300, 520, 512, "add"),     # prefill rows: the add joins the tiled GEMM's store
+    (300, 130, 512, "add"),     # residual rows not 8-byte aligned: accumulators + epilogue program
+    (700, 768, 1024, "mul"),    # unrecognised epilogue over a GEMM of several tiles
+    (96, 512, 2048, "mul"),     # unrecognised epilogue over the slab kernels
+])
+def test_quant_matmul_with_elementwise_epilogue(cpu, hip, rows, n, k, kind):
+    """out = epilogue(f32 accumulator, extra) with a full [rows, N] extra operand: the residual add
+    after the dense down projection (crates/forja-sdk/src/nn/blocks.rs:408-411) and a product."""
+    weights = Quantised(23, n + k, (n, k))
+    x_values = normal_bf16(23, 1, (rows, k))
+    extra_values = normal_bf16(23, 2, (rows, n))
+
+    def build(backend):
+        x = upload(backend, x_values, DType.BF16)
+        extra = upload(backend, extra_values, DType.BF16)
+        out = backend.alloc(DType.BF16, (rows, n))
+        if kind == "add":
+            program = programs.add_elements()
+        else:
+            b = ProgramBuilder(ProgramKind.MAP)
+            b.output(0, b.mul(b.input(0), b.input(1)))
+            program = b.finish()
+        epilogue = backend.prepare_epilogue(program)
+        commands = CommandList()
+        commands.dispatch_epilogue(Op.quant_matmul(4, 64), [x, *weights.upload(backend)], out, epilogue,
+                                   [extra])
+        return commands, [out]
+    differential(cpu, hip, build)
+
+
 # ------------------------------------------------------------------ routed projections
 
 def routed_case(seed, rows, k, experts, n, inner, bad=()):
@@ -583,6 +616,33 @@ def test_ragged_attention_equals_the_per_lane_sequence(cpu, hip, contexts, count
     assert cpu.read(cpu_out[1]) == hip.read(hip_out[1]) and cpu.read(cpu_out[2]) == hip.read(hip_out[2])
 
 
+@pytest.mark.parametrize("contexts,counts,hq,hkv", [([300, 40, 2047, 700], [1, 1, 1, 1], 32, 4),
+                                                    ([0, 130, 33], [70, 1, 45], 16, 8)])
+def test_ragged_attention_layers_share_metadata_until_it_is_rewritten(cpu, hip, contexts, counts, hq, hkv):
+    """One command list the way a model step records it: two layers (their own pools) attend with
+    the same tables, starts and cu_seqlens, then the starts are overwritten on the device and a third
+    dispatch must follow the new values."""
+    scale, pt = 1.0 / math.sqrt(128), 16
+    moved = [max(0, c - 5) for c in contexts]
+
+    def build(backend):
+        t, inputs = ragged_case(backend, contexts, counts, hq, hkv, pt, seed=64)
+        physical = t["keys"].shape[0]
+        other_k = upload(backend, normal_bf16(64, 8, (physical, pt, hkv, 128)), DType.BF16)
+        other_v = upload(backend, normal_bf16(64, 9, (physical, pt, hkv, 128)), DType.BF16)
+        out2, out3 = (backend.alloc(DType.BF16, t["out"].shape) for _ in range(2))
+        new_starts = upload(backend, np.array(moved), DType.U32)
+        op = Op.paged_attention_ragged(scale, pt)
+        commands = CommandList()
+        commands.dispatch_many(op, inputs, [t["out"], t["keys"], t["values"]])
+        commands.dispatch_many(op, inputs, [out2, other_k, other_v])
+        commands.dispatch(Op.copy(), [new_starts], t["starts"])
+        commands.dispatch_many(op, inputs, [out3, t["keys"], t["values"]])
+        return commands, [t["out"], out2, out3, t["keys"], other_k]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    assert cpu.read(cpu_out[3]) == hip.read(hip_out[3]) and cpu.read(cpu_out[4]) == hip.read(hip_out[4])
+
+
 def test_ragged_attention_skips_inactive_lanes(cpu, hip):
     def build(backend):
         t, inputs = ragged_case(backend, [33, 70, 5], [1, 1, 1], 8, 4, 16, seed=62, activity=[1, 0, 1])
@@ -636,6 +696,27 @@ def test_engine_row_programs(cpu, hip):
             [rotated.narrow(2, 0, half), rotated.narrow(2, half, half)])
         return commands, [normed, hidden_out, normed2, rotated]
     differential(cpu, hip, build, abs_=2e-2)
+
+
+@pytest.mark.parametrize("rows,width", [(5, 64), (130, 1024), (3, 20)])
+def test_engine_element_programs_on_the_halves_of_a_stacked_projection(cpu, hip, rows, width):
+    """silu_mul_elements over the gate and up halves of one [rows, 2 * width] tensor and
+    add_elements (crates/forja-sdk/src/nn/blocks.rs:408-416); the last width is not a multiple of
+    eight."""
+    stacked_values = 3.0 * normal_bf16(72, 1, (rows, 2 * width))
+    residual_values = normal_bf16(72, 2, (rows, width))
+
+    def build(backend):
+        stacked = upload(backend, stacked_values, DType.BF16)
+        residual = upload(backend, residual_values, DType.BF16)
+        activated, summed = (backend.alloc(DType.BF16, (rows, width)) for _ in range(2))
+        commands = CommandList()
+        commands.dispatch_kernel(backend.prepare_program(programs.silu_mul_elements()),
+                                 [stacked.narrow(1, 0, width), stacked.narrow(1, width, width)], [activated])
+        commands.dispatch_kernel(backend.prepare_program(programs.add_elements()), [residual, activated],
+                                 [summed])
+        return commands, [activated, summed]
+    differential(cpu, hip, build)
 
 
 def test_map_programs_casts_index_select(cpu, hip):

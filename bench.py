@@ -224,7 +224,7 @@ def prefill_gemm_c4(backend, rows=8256, seed=91, repeats=3):
                      f"64 decode rows), hidden {c.hidden}, intermediate {c.intermediate}, MLX-4bit"),
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "kernel": "qmm_gemm_kernel"},
+                     "kernel": "gemm_f16_kernel, with prepare_rows_kernel and prepare_weights_kernel"},
         "ms_per_layer_projections": total_ns / 1e6, "products": products,
     }
 
@@ -278,6 +278,22 @@ def stream_read_rate(backend, rows=4096, width=1 << 20, repeats=3):
     backend.release(source)
     backend.release(result)
     return 2.0 * rows * width * repeats / (ns * 1e-9) / 1e9
+
+
+def mfma_sustained_rates():
+    """What the matrix cores sustain from registers on this device (v_mfma_f32_32x32x16_f16, one
+    wave per SIMD, ~60 ms): with all-zero operands and with random ones.  The second is the
+    practical ceiling of the prefill GEMM: operand bits that toggle cost power, and the device
+    lowers its clock to stay inside its limit.  None when the probe library is not built."""
+    import ctypes
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "forja_amd", "libforja_probes.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.fh_probe_mfma_f16_tflops.restype = ctypes.c_double
+    lib.fh_probe_mfma_f16_tflops.argtypes = [ctypes.c_int, ctypes.c_int]
+    return {"zeros_tflops": lib.fh_probe_mfma_f16_tflops(200000, 0),
+            "random_tflops": lib.fh_probe_mfma_f16_tflops(200000, 1)}
 
 
 def prefill_attention_c4(backend, seed=93, repeats=3):
@@ -379,7 +395,8 @@ def main():
         return
     if args.prefill_only:
         backend = HipBackend(0)
-        print(json.dumps({"prefill_gemm_c4": prefill_gemm_c4(backend),
+        print(json.dumps({"mfma_f16_sustained": mfma_sustained_rates(),
+                          "prefill_gemm_c4": prefill_gemm_c4(backend),
                           "prefill_attention_c4": prefill_attention_c4(backend),
                           "prefill_layer_c4": prefill_layer_c4(backend)}))
         return
@@ -511,7 +528,13 @@ def main():
         result["roofline"]["measured_stream_read_gbps"] = stream_read_rate(backend)
         result["roofline"]["frac_of_measured_stream_read"] = (
             result["roofline"]["achieved"] / result["roofline"]["measured_stream_read_gbps"])
-        result["secondary_workloads"] = {"prefill_gemm_c4": prefill_gemm_c4(backend),
+        sustained = mfma_sustained_rates()
+        gemm = prefill_gemm_c4(backend)
+        if sustained:
+            gemm["roofline"]["measured_mfma_f16"] = sustained
+            gemm["roofline"]["frac_of_measured_random_data_mfma"] = (
+                gemm["roofline"]["achieved"] / sustained["random_tflops"])
+        result["secondary_workloads"] = {"prefill_gemm_c4": gemm,
                                          "prefill_attention_c4": prefill_attention_c4(backend),
                                          "prefill_layer_c4": prefill_layer_c4(backend)}
         if config.moe:

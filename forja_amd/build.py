@@ -6,6 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libforja_hip.so")
+PROBES = os.path.join(HERE, "libforja_probes.so")
 CONFORMANCE = os.path.join(HERE, "host", "conformance")
 
 SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "qmm_gemm.hip", "programs_fast.hip"]
@@ -45,8 +46,20 @@ def build(verbose=False, jobs=8):
         raise RuntimeError("hipcc failed")
     link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objects
     subprocess.run(link, check=True)
+    build_probes()
     build_host()
     return LIB
+
+
+def build_probes():
+    """bench.py's measurement probes (sustained MFMA rate): a library of their own."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "-x", "hip", os.path.join(CSRC, "bench_probes.hip"), "-shared", "-o", PROBES] + COMMON
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if out.returncode != 0:
+        print(out.stdout, file=sys.stderr)
+        raise RuntimeError("hipcc failed on bench_probes.hip")
+    return PROBES
 
 
 def build_host():

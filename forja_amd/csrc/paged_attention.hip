@@ -665,53 +665,58 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 // lanes' four columns, all loads in flight at once, and the waves' sums meet in LDS.
 __global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
   __shared__ float4 folded[3][32];
-  const uint32_t head = blockIdx.x, token = blockIdx.y;
+  const uint32_t token = blockIdx.y;
   const TokenPlan plan = p.plans[token];
   const bool zero = plan.splits == 0 || p.bad[token] != 0;
   if (!zero && plan.splits == 1) return;
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t column = (lane & 31) * 4, half = lane >> 5;
-  uint16_t *dst = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
-  if (zero) {
-    if (threadIdx.x < 32) *(uint2 *)dst = make_uint2(0, 0);
-    return;
-  }
-  const uint64_t base = (uint64_t)token * p.max_splits * p.query_heads + head;
-  float2 ml = make_float2(-__builtin_inff(), 0.0f);
-  if (lane < plan.splits) ml = p.partial_ml[base + (uint64_t)lane * p.query_heads];
-  const float m_all = wave_max(ml.x);
-  const float weight = lane < plan.splits ? exp2f(ml.x - m_all) : 0.0f;
-  const float l_all = wave_sum(ml.y * weight);
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  // gridDim.x is the head count for decode batches and 1 for long prefill batches, where most
+  // tokens have a single split and leave at once
+  for (uint32_t head = blockIdx.x; head < p.query_heads; head += gridDim.x) {
+    uint16_t *dst = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
+    if (zero) {
+      if (threadIdx.x < 32) *(uint2 *)dst = make_uint2(0, 0);
+      continue;
+    }
+    const uint64_t base = (uint64_t)token * p.max_splits * p.query_heads + head;
+    float2 ml = make_float2(-__builtin_inff(), 0.0f);
+    if (lane < plan.splits) ml = p.partial_ml[base + (uint64_t)lane * p.query_heads];
+    const float m_all = wave_max(ml.x);
+    const float weight = lane < plan.splits ? exp2f(ml.x - m_all) : 0.0f;
+    const float l_all = wave_sum(ml.y * weight);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-  for (uint32_t i = 0; i < 8; ++i) {   // 64 splits / (4 waves * 2 halves)
-    const uint32_t s = 8 * i + 2 * wave + half;
-    const float w = __shfl(weight, (int)(s & 63), 64);
-    if (s < plan.splits) {
-      const float4 part =
-          *(const float4 *)(p.partial_o + (base + (uint64_t)s * p.query_heads) * 128 + column);
-      acc.x += part.x * w;
-      acc.y += part.y * w;
-      acc.z += part.z * w;
-      acc.w += part.w * w;
+    for (uint32_t i = 0; i < 8; ++i) {   // 64 splits / (4 waves * 2 halves)
+      const uint32_t s = 8 * i + 2 * wave + half;
+      const float w = __shfl(weight, (int)(s & 63), 64);
+      if (s < plan.splits) {
+        const float4 part =
+            *(const float4 *)(p.partial_o + (base + (uint64_t)s * p.query_heads) * 128 + column);
+        acc.x += part.x * w;
+        acc.y += part.y * w;
+        acc.z += part.z * w;
+        acc.w += part.w * w;
+      }
     }
-  }
-  acc.x += __shfl_xor(acc.x, 32, 64);
-  acc.y += __shfl_xor(acc.y, 32, 64);
-  acc.z += __shfl_xor(acc.z, 32, 64);
-  acc.w += __shfl_xor(acc.w, 32, 64);
-  if (wave != 0 && half == 0) folded[wave - 1][lane] = acc;
-  __syncthreads();
-  if (threadIdx.x < 32) {
-    for (int other = 0; other < 3; ++other) {
-      const float4 part = folded[other][lane];
-      acc.x += part.x;
-      acc.y += part.y;
-      acc.z += part.z;
-      acc.w += part.w;
+    acc.x += __shfl_xor(acc.x, 32, 64);
+    acc.y += __shfl_xor(acc.y, 32, 64);
+    acc.z += __shfl_xor(acc.z, 32, 64);
+    acc.w += __shfl_xor(acc.w, 32, 64);
+    __syncthreads();   // the previous head's sums have been read
+    if (wave != 0 && half == 0) folded[wave - 1][lane] = acc;
+    __syncthreads();
+    if (threadIdx.x < 32) {
+      for (int other = 0; other < 3; ++other) {
+        const float4 part = folded[other][lane];
+        acc.x += part.x;
+        acc.y += part.y;
+        acc.z += part.z;
+        acc.w += part.w;
+      }
+      const float inv = 1.0f / l_all;
+      *(uint2 *)dst = make_uint2(pack_bf16(acc.x * inv, acc.y * inv), pack_bf16(acc.z * inv, acc.w * inv));
     }
-    const float inv = 1.0f / l_all;
-    *(uint2 *)dst = make_uint2(pack_bf16(acc.x * inv, acc.y * inv), pack_bf16(acc.z * inv, acc.w * inv));
   }
 }
 
@@ -812,7 +817,7 @@ void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, E
                                      64 * waves, 0, stream>>>(f, error);
     }
   }
-  ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens), 256, 0, stream>>>(f);
+  ragged_reduce_kernel<<<dim3(f.tokens <= 1024 ? f.query_heads : 1, f.tokens), 256, 0, stream>>>(f);
 }
 
 }  // namespace

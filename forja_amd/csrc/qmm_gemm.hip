@@ -49,7 +49,10 @@ constexpr int kPadK = 64;   // operand rows are padded to a multiple of this (ev
 // K step and LDS stages of the GEMM.  Steps of 32 with three or four stages measured the same
 // (the kernel is bound by what the matrix cores and the L2 -> LDS path sustain, not by latency).
 constexpr int kGemmK = 64, kGemmStages = 2;
-constexpr int kGemmLds = kGemmStages * 2 * kBM * 2 * kGemmK;   // both operand tiles of every stage
+constexpr int kOutPitch = 2 * 128 + 16;           // bytes per row of a wave's staged output quadrant
+constexpr int kGemmPipelineLds = kGemmStages * 2 * kBM * 2 * kGemmK;   // both operand tiles of every stage
+constexpr int kGemmOutputLds = 4 * (128 * kOutPitch + 512);            // four quadrants of bf16 rows + row factors
+constexpr int kGemmLds = kGemmPipelineLds > kGemmOutputLds ? kGemmPipelineLds : kGemmOutputLds;
 constexpr int kBand = 8;   // column tiles per band of the tile numbering
 constexpr uint32_t kMaxGroups = 512;              // quantisation groups per row the row kernel holds
 
@@ -71,6 +74,7 @@ struct GemmArgs {
   const uint32_t *refused;     // non-zero: some scale or bias is out of range, do nothing
   const uint16_t *residual;    // optional bf16 rows added before rounding
   uint64_t residual_row_stride;
+  uint32_t row_stores;         // bf16 output (and residual) rows are 16-byte aligned, columns % 8 == 0
 };
 
 __device__ inline uint32_t pack2(float lo, float hi) {
@@ -230,7 +234,8 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
   unsigned char *a_tiles = gemm_lds;                      // [kStages][kBM][kRowBytes], pieces swizzled
   unsigned char *b_tiles = gemm_lds + kStages * kTile;    // [kStages][kBN][kRowBytes]
-  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const uint32_t tid = threadIdx.x, lane = tid & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: LDS bases stay scalar
   const uint32_t wm = wave >> 1, wn = wave & 1;
   const uint32_t l32 = lane & 31, kh = lane >> 5;
   // A row's piece p sits in slot p ^ swizzle(row), which spreads the 32 rows a wave reads at once
@@ -255,29 +260,28 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   // Staging: a wave owns 64 rows of each operand tile; one instruction moves kRowsPerLoad rows
   // (lane -> row lane / kSlots, LDS slot lane % kSlots) and the piece a lane fetches is its slot
   // XOR the row's swizzle.  Rows past the end of a matrix reload its last row; what they produce
-  // is never stored.
-  const uint16_t *a_src[kLoads], *b_src[kLoads];
+  // is never stored.  Addresses are a wave-uniform base that advances with the K step plus a
+  // 32-bit per-lane offset that never changes (both matrices are far below 4 GiB).
+  uint32_t a_off[kLoads], b_off[kLoads];
 #pragma unroll
   for (int i = 0; i < kLoads; ++i) {
     const uint32_t in_tile = 64 * wave + kRowsPerLoad * i + lane / kSlots;
     const uint32_t piece = (lane % kSlots) ^ swizzle_of(in_tile);
-    a_src[i] = a.a + (uint64_t)min(row0 + in_tile, a.rows - 1) * a.kt + 8 * piece;
-    b_src[i] = a.b + (uint64_t)min(col0 + in_tile, a.columns - 1) * a.kt + 8 * piece;
+    a_off[i] = (min(row0 + in_tile, a.rows - 1) * a.kt + 8 * piece) * 2;
+    b_off[i] = (min(col0 + in_tile, a.columns - 1) * a.kt + 8 * piece) * 2;
   }
   const uint32_t steps = a.kt / kBK;
-  auto stage = [&](uint32_t buffer, uint32_t step) {
+  // one pair of load instructions (activation rows and weight rows) of stage `step`
+  auto stage_pair = [&](uint32_t buffer, uint32_t step, int i) {
     const uint32_t st = min(step, steps - 1);   // past the end: reload the last step, never used
-    unsigned char *to_a = a_tiles + buffer * kTile + 64 * wave * kRowBytes;
-    unsigned char *to_b = b_tiles + buffer * kTile + 64 * wave * kRowBytes;
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void *)(a_src[i] + st * kBK),
-          (__attribute__((address_space(3))) void *)(to_a + kRowsPerLoad * i * kRowBytes), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void *)(b_src[i] + st * kBK),
-          (__attribute__((address_space(3))) void *)(to_b + kRowsPerLoad * i * kRowBytes), 16, 0, 0);
-    }
+    const unsigned char *from_a = (const unsigned char *)a.a + (uint64_t)st * (kBK * 2);
+    const unsigned char *from_b = (const unsigned char *)a.b + (uint64_t)st * (kBK * 2);
+    unsigned char *to_a = a_tiles + buffer * kTile + (64 * wave + kRowsPerLoad * i) * kRowBytes;
+    unsigned char *to_b = b_tiles + buffer * kTile + (64 * wave + kRowsPerLoad * i) * kRowBytes;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from_a + a_off[i]),
+                                     (__attribute__((address_space(3))) void *)to_a, 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from_b + b_off[i]),
+                                     (__attribute__((address_space(3))) void *)to_b, 16, 0, 0);
   };
 
   f32x16 acc[4][4];
@@ -288,8 +292,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   // Operand registers, two sets: the set for the next sub-step is read from LDS while the matrix
-  // pipe works on the current one.  The last sub-step of a K step is multiplied after the
-  // step's barrier, behind the first read of the next step.
+  // pipe works on the current one.
   f16x8 a_op[2][4], b_op[2][4];
   const uint32_t swizzle = swizzle_of(l32);
   auto read_operands = [&](uint32_t buffer, int s, int set) {
@@ -302,42 +305,101 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
       b_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kRowBytes + piece));
     }
   };
-  auto multiply = [&](int set) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[set][i], b_op[set][j], acc[i][j], 0, 0, 0);
-  };
 
-  // Stages 0 .. kStages-1 are requested up front; from then on the buffer a step frees is
-  // refilled with the step kStages ahead, so kStages-1 steps of loads are always in flight.
+  // K pipeline over kStages LDS buffers.  During step t the loads of step t + kStages - 1 are
+  // issued into the buffer step t - 1 has just freed, one pair of instructions behind every
+  // fourth MFMA so that they issue in the shadow of the matrix pipe; at the end of step t the
+  // loads of step t + 1 must have landed.
 #pragma unroll
-  for (int p = 0; p < kStages; ++p) stage(p, p);
-  __builtin_amdgcn_s_waitcnt(wait_vmcnt((kStages - 1) * 2 * kLoads));   // step 0 has landed
+  for (int p = 0; p < kStages - 1; ++p)
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) stage_pair(p, p, i);
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt((kStages - 2) * 2 * kLoads));   // step 0 has landed
   __syncthreads();
-  read_operands(0, 0, 0);
-  uint32_t buffer = 0;
+  uint32_t buffer = 0, refill = kStages - 1;
   for (uint32_t step = 0; step < steps; ++step) {
-    const uint32_t next_buffer = buffer + 1 == kStages ? 0 : buffer + 1;
+    read_operands(buffer, 0, 0);
+    int issued = 0;
 #pragma unroll
     for (int s = 0; s < kSub; ++s) {
       __builtin_amdgcn_sched_barrier(0);
-      if (s + 1 < kSub) {
-        read_operands(buffer, s + 1, (s + 1) & 1);
-      } else {
-        // every read of this buffer has been issued: once they have landed, and the next step's
-        // tiles too, the workgroup meets and the buffer is refilled
-        __builtin_amdgcn_s_waitcnt(0xc07f);                                   // lgkmcnt(0)
-        __builtin_amdgcn_s_waitcnt(wait_vmcnt((kStages - 2) * 2 * kLoads));   // step + 1 has landed
-        __syncthreads();
-        stage(buffer, step + kStages);
-        read_operands(next_buffer, 0, 0);
-      }
+      if (s + 1 < kSub) read_operands(buffer, s + 1, (s + 1) & 1);
       __builtin_amdgcn_sched_barrier(0);
-      multiply(s & 1);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
+        if (issued < kLoads) {
+          __builtin_amdgcn_sched_barrier(0);
+          stage_pair(refill, step + kStages - 1, issued);
+          ++issued;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
     }
-    buffer = next_buffer;
+    static_assert(kLoads <= 4 * kSub, "one load pair per MFMA row at most");
+    __builtin_amdgcn_s_waitcnt(0xc07f);                                   // lgkmcnt(0): reads done
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt((kStages - 2) * 2 * kLoads));   // step + 1 has landed
+    __syncthreads();
+    refill = buffer;
+    buffer = buffer + 1 == kStages ? 0 : buffer + 1;
+  }
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));   // nothing is on its way into LDS any more
+  __syncthreads();
+  // Lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile: a column
+  // per lane, the wrong way round for memory.  When the output rows allow 16-byte stores, every
+  // wave turns its 128 x 128 quadrant round through its own piece of LDS: the residual rows (if
+  // any) are staged there first, every lane then replaces "its" elements by the finished bf16
+  // result (f32 sum, one rounding), and the rows leave with one 16-byte store per lane, 256
+  // contiguous bytes per row.  Only wave-local ordering is needed: nobody else touches the piece.
+  if (a.row_stores) {
+    unsigned char *mine = gemm_lds + wave * (128 * kOutPitch + 512);
+    float *unscale_of = (float *)(mine + 128 * kOutPitch);   // the quadrant's 128 row factors
+    const uint32_t quad_row0 = row0 + 128 * wm, quad_col0 = col0 + 128 * wn;
+    const uint32_t piece_row = lane >> 4, piece_col = 8 * (lane & 15);
+    unscale_of[lane] = a.row_unscale[min(quad_row0 + lane, a.rows - 1)];
+    unscale_of[64 + lane] = a.row_unscale[min(quad_row0 + 64 + lane, a.rows - 1)];
+    if (a.residual) {
+#pragma unroll 4
+      for (int it = 0; it < 32; ++it) {
+        const uint32_t row = 4 * it + piece_row;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
+          v = *(const uint4 *)(a.residual + (uint64_t)(quad_row0 + row) * a.residual_row_stride +
+                               quad_col0 + piece_col);
+        *(uint4 *)(mine + row * kOutPitch + 2 * piece_col) = v;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+        const float unscale = unscale_of[row];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint16_t *slot = (uint16_t *)(mine + row * kOutPitch) + 32 * j + l32;
+          float value = acc[i][j][r] * unscale;
+          if (a.residual) value += bf16_bits_to_f32(*slot);
+          *slot = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+        }
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    uint16_t *out = (uint16_t *)a.out;
+#pragma unroll 4
+    for (int it = 0; it < 32; ++it) {
+      const uint32_t row = 4 * it + piece_row;
+      const uint4 v = *(const uint4 *)(mine + row * kOutPitch + 2 * piece_col);
+      if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
+        *(uint4 *)(out + (uint64_t)(quad_row0 + row) * a.out_row_stride + quad_col0 + piece_col) = v;
+    }
+    return;
   }
   // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile
 #pragma unroll
@@ -386,6 +448,8 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
     a.residual = (const uint16_t *)p.residual->base + p.residual->offset;
     a.residual_row_stride = p.residual->stride[0];
   }
+  a.row_stores = !a.out_f32 && p.columns % 8 == 0 && p.out.stride[0] % 8 == 0 && p.out.offset % 8 == 0 &&
+                 (!p.residual || (p.residual->stride[0] % 8 == 0 && p.residual->offset % 8 == 0));
   a.rows = p.rows;
   a.columns = p.columns;
   a.row_tiles = (p.rows + kBM - 1) / kBM;

@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 # hardware counters: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over the same launches, each
 # scaled by what the counter reads for a 1 GiB copy (FETCH_SIZE counts half of it, WRITE_SIZE all
 # of it); figures and commands in profiles/c3_decode_step_hbm_traffic.txt.
-ATTENTION_TRAFFIC_RATIO = 1.022
+ATTENTION_TRAFFIC_RATIO = 1.019
 KC_ATTENTION, KC_MOE, KC_QMM = 3, 2, 1
 KC_ATTENTION_KERNEL, KC_MOE_KERNEL, KC_QMM_KERNEL = 4, 5, 6
 

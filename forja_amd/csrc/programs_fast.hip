@@ -103,32 +103,44 @@ struct QkArgs {
   float head_dim, eps, theta, exponent_scale;
 };
 
-// One wave per (row, head): RMS-normalise the head over both halves, scale, rotate the
-// (lo, hi) pair by angle = position * theta^(i * exponent_scale).
+// One workgroup per row, its four waves taking the heads in turn: RMS-normalise the head over both
+// halves, scale, rotate the (lo, hi) pair by angle = position * theta^(i * exponent_scale).  The
+// rotation is the same for every head of a row when the positions do not vary along the head
+// axis (the usual broadcast view), and is then computed once per wave.
 __global__ __launch_bounds__(256) void qk_norm_rope_kernel(QkArgs a) {
-  const uint32_t lane = threadIdx.x & 63;
-  const uint64_t item = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= (uint64_t)a.rows * a.heads) return;
-  const uint32_t row = (uint32_t)(item / a.heads), head = (uint32_t)(item % a.heads);
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t row = blockIdx.x;
   const bool live = lane < a.width;
-  float lo = 0.0f, hi = 0.0f;
-  if (live) {
-    lo = __uint_as_float((uint32_t)a.lo[row * a.lo_s[0] + head * a.lo_s[1] + lane] << 16);
-    hi = __uint_as_float((uint32_t)a.hi[row * a.hi_s[0] + head * a.hi_s[1] + lane] << 16);
+  const bool shared_angle = a.pos_s[1] == 0;
+  float c = 1.0f, s = 0.0f;
+  const float frequency = powf(a.theta, (float)lane * a.exponent_scale);
+  if (shared_angle && live) {
+    const float angle = a.positions[row * a.pos_s[0] + lane * a.pos_s[2]] * frequency;
+    c = cosf(angle);
+    s = sinf(angle);
   }
-  float square_sum = lo * lo + hi * hi;
-  for (int offset = 32; offset > 0; offset >>= 1) square_sum += __shfl_xor(square_sum, offset, 64);
-  if (!live) return;
-  const float inverse = 1.0f / sqrtf(square_sum / a.head_dim + a.eps);
-  const float w_lo = __uint_as_float((uint32_t)a.w_lo[row * a.wlo_s[0] + head * a.wlo_s[1] + lane] << 16);
-  const float w_hi = __uint_as_float((uint32_t)a.w_hi[row * a.whi_s[0] + head * a.whi_s[1] + lane] << 16);
-  const float n_lo = lo * inverse * w_lo, n_hi = hi * inverse * w_hi;
-  const float position = a.positions[row * a.pos_s[0] + head * a.pos_s[1] + lane * a.pos_s[2]];
-  const float angle = position * powf(a.theta, (float)lane * a.exponent_scale);
-  const float c = cosf(angle), s = sinf(angle);
-  const float r_lo = n_lo * c - n_hi * s, r_hi = n_hi * c + n_lo * s;
-  a.out_lo[row * a.olo_s[0] + head * a.olo_s[1] + lane] = (uint16_t)(pack2(r_lo, 0.0f) & 0xffffu);
-  a.out_hi[row * a.ohi_s[0] + head * a.ohi_s[1] + lane] = (uint16_t)(pack2(r_hi, 0.0f) & 0xffffu);
+  for (uint32_t head = wave; head < a.heads; head += 4) {
+    float lo = 0.0f, hi = 0.0f;
+    if (live) {
+      lo = __uint_as_float((uint32_t)a.lo[row * a.lo_s[0] + head * a.lo_s[1] + lane] << 16);
+      hi = __uint_as_float((uint32_t)a.hi[row * a.hi_s[0] + head * a.hi_s[1] + lane] << 16);
+    }
+    float square_sum = lo * lo + hi * hi;
+    for (int offset = 32; offset > 0; offset >>= 1) square_sum += __shfl_xor(square_sum, offset, 64);
+    if (!live) continue;
+    const float inverse = 1.0f / sqrtf(square_sum / a.head_dim + a.eps);
+    const float w_lo = __uint_as_float((uint32_t)a.w_lo[row * a.wlo_s[0] + head * a.wlo_s[1] + lane] << 16);
+    const float w_hi = __uint_as_float((uint32_t)a.w_hi[row * a.whi_s[0] + head * a.whi_s[1] + lane] << 16);
+    const float n_lo = lo * inverse * w_lo, n_hi = hi * inverse * w_hi;
+    if (!shared_angle) {
+      const float angle = a.positions[row * a.pos_s[0] + head * a.pos_s[1] + lane * a.pos_s[2]] * frequency;
+      c = cosf(angle);
+      s = sinf(angle);
+    }
+    const float r_lo = n_lo * c - n_hi * s, r_hi = n_hi * c + n_lo * s;
+    a.out_lo[row * a.olo_s[0] + head * a.olo_s[1] + lane] = (uint16_t)(pack2(r_lo, 0.0f) & 0xffffu);
+    a.out_hi[row * a.ohi_s[0] + head * a.ohi_s[1] + lane] = (uint16_t)(pack2(r_hi, 0.0f) & 0xffffu);
+  }
 }
 
 struct PairArgs {
@@ -389,8 +401,7 @@ bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const Program
     a.eps = cls.c[1];
     a.theta = cls.c[2];
     a.exponent_scale = cls.c[3];
-    uint64_t items = (uint64_t)a.rows * a.heads;
-    qk_norm_rope_kernel<<<dim3((unsigned)((items + 3) / 4)), 256, 0, stream>>>(a);
+    qk_norm_rope_kernel<<<dim3(a.rows), 256, 0, stream>>>(a);
     return true;
   }
   return false;

@@ -208,9 +208,10 @@ typedef enum fh_kernel_class {
   FH_KC_MOE = 2,       /* FH_OP_GATHER_QUANT_MATMUL (packing + grouped matmul + combine) */
   FH_KC_ATTENTION = 3, /* paged attention ops (plan + append + attention + merge) */
   /* single kernels: the launch that dominates each class */
-  FH_KC_ATTENTION_KERNEL = 4, /* ragged_attention_mfma_kernel */
-  FH_KC_MOE_KERNEL = 5,       /* routed qmm_mfma_kernel */
-  FH_KC_QMM_KERNEL = 6,       /* dense qmm_mfma_kernel */
+  FH_KC_ATTENTION_KERNEL = 4, /* the ragged attention kernel (decode or prefill form) */
+  FH_KC_MOE_KERNEL = 5,       /* the routed quantised-matmul kernel of a gather dispatch */
+  FH_KC_QMM_KERNEL = 6,       /* the kernels of one dense quantised product: slab + sum (decode rows),
+                                 operand preparation + GEMM (prefill rows), or the streaming kernel */
   FH_KC_COUNT = 7
 } fh_kernel_class;
 FH_API fh_status fh_profile_enable(fh_backend *backend, int enabled);

@@ -1400,7 +1400,22 @@ fh_status fh_prepare_program(fh_backend *b, uint32_t kind, const fh_inst *insts,
   p.n_outputs = max_output + 1;
   for (uint32_t slot = 0; slot < p.n_outputs; ++slot)
     if (!seen[slot]) return FH_INVALID_INPUT;
-  // Structural check with every input assumed f32; u32 bindings are re-typed at dispatch.
+  // validate_structure (program.rs:1052-1094): operands defined earlier, reductions only in row
+  // programs and at most four.  These do not depend on how the inputs are bound.
+  {
+    uint32_t reductions = 0;
+    for (uint32_t i = 0; i < n_insts; ++i) {
+      const fh_inst &inst = p.insts[i];
+      const uint32_t operands = inst.kind == 4 || inst.kind == 7 || inst.kind == 8 ? 1
+                                : inst.kind == 5 ? 2 : inst.kind == 6 ? 3 : 0;
+      const uint32_t values[3] = {inst.a, inst.b, inst.c};
+      for (uint32_t o = 0; o < operands; ++o)
+        if (values[o] >= i) return FH_INVALID_INPUT;
+      if (inst.kind == 8 && (kind != 1 || ++reductions > (uint32_t)kMaxReductions))
+        return FH_INVALID_INPUT;
+    }
+  }
+  // Typing check with every input assumed f32; u32 bindings are re-typed at dispatch.
   std::vector<DInst> typed;
   fh_status status = type_program(p, 0, FH_MAX_RANK, &typed);
   if (status != FH_OK) {

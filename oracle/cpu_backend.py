@@ -209,6 +209,25 @@ class CpuBackend:
             raise BackendError(Status.INVALID_INPUT)
 
     def prepare_program(self, program: Program):
+        """The structural limits of validate_structure (crates/forja-core/src/program.rs:25-31,
+        1052-1094): at most 256 instructions, 8 input slots, 4 outputs and 4 reductions, operands
+        defined earlier, no reduction in a map program.  Typing is checked when the program runs."""
+        if len(program.insts) > 256 or not program.outputs:
+            raise BackendError(Status.INVALID_INPUT)
+        reductions = 0
+        for index, inst in enumerate(program.insts):
+            if inst.kind == 0 and inst.a >= 8:
+                raise BackendError(Status.INVALID_INPUT)
+            if inst.kind == 8:
+                reductions += 1
+                if int(program.kind) == 0 or reductions > 4:
+                    raise BackendError(Status.INVALID_INPUT)
+            operands = {4: (inst.a,), 5: (inst.a, inst.b), 6: (inst.a, inst.b, inst.c), 7: (inst.a,),
+                        8: (inst.a,)}.get(inst.kind, ())
+            if any(operand >= index for operand in operands):
+                raise BackendError(Status.INVALID_INPUT)
+        if any(slot >= 4 for slot, _ in program.outputs):
+            raise BackendError(Status.INVALID_INPUT)
         return program
 
     prepare_epilogue = prepare_program

@@ -743,6 +743,110 @@ def test_map_programs_casts_index_select(cpu, hip):
         assert cpu.read(a) == hip.read(b_)
 
 
+def random_program(rng, kind, inputs, length, exact):
+    """A typed random SSA program over `inputs` = [ValueType of input slot ...]: every operand is
+    drawn from earlier values of the right type, the way the reference's proptest generator does
+    (crates/forja-metal/tests/map_programs.rs).  `exact` keeps to operations IEEE fixes bit for bit
+    (no division, roots or transcendentals, no sum reduction)."""
+    b = ProgramBuilder(kind)
+    of_type = {ValueType.F32: [], ValueType.U32: [], ValueType.BOOL: []}
+    for slot, value_type in enumerate(inputs):
+        of_type[value_type].append(b.input(slot))
+    of_type[ValueType.F32].append(b.const(float(rng.choice([0.0, -1.5, 2.0, 0.3, 1e-3]))))
+    of_type[ValueType.U32].append(b.index(1))
+    of_type[ValueType.U32].append(b.extent(1))
+    pick = lambda t: int(rng.choice(of_type[t]))
+    reductions = 0
+    exact_unary = [UnOp.NEG, UnOp.ABS, UnOp.FLOOR]
+    loose_unary = [UnOp.NEG, UnOp.ABS, UnOp.TANH, UnOp.SIGMOID, UnOp.SIN, UnOp.COS]
+    exact_binary = [BinOp.ADD, BinOp.SUB, BinOp.MUL, BinOp.MIN, BinOp.MAX]
+    compare = [BinOp.LT, BinOp.LE, BinOp.EQ, BinOp.NE, BinOp.GE, BinOp.GT]
+    for _ in range(length):
+        # the loose set stays with continuous operations: a comparison, floor or integer cast of a
+        # value that differs in its last bit may legitimately take the other branch
+        choice = int(rng.integers(0, 9)) if exact else int(rng.choice([0, 1, 2, 7, 8]))
+        if choice == 0:
+            of_type[ValueType.F32].append(b.unary(rng.choice(exact_unary if exact else loose_unary),
+                                                  pick(ValueType.F32)))
+        elif choice in (1, 2):
+            ops = exact_binary
+            of_type[ValueType.F32].append(b.binary(rng.choice(ops), pick(ValueType.F32), pick(ValueType.F32)))
+        elif choice == 3:
+            of_type[ValueType.U32].append(b.binary(rng.choice(exact_binary), pick(ValueType.U32),
+                                                   pick(ValueType.U32)))
+        elif choice == 4:
+            operand = ValueType.F32 if rng.integers(0, 2) else ValueType.U32
+            of_type[ValueType.BOOL].append(b.binary(rng.choice(compare), pick(operand), pick(operand)))
+        elif choice == 5 and of_type[ValueType.BOOL]:
+            chosen = ValueType.F32 if rng.integers(0, 2) else ValueType.U32
+            of_type[chosen].append(b.select(pick(ValueType.BOOL), pick(chosen), pick(chosen)))
+        elif choice == 6:
+            source = [t for t in of_type if of_type[t]][int(rng.integers(0, sum(1 for t in of_type if of_type[t])))]
+            target = ValueType(int(rng.integers(0, 3)))
+            of_type[target].append(b.cast(target, pick(source)))
+        elif choice == 7 and kind == ProgramKind.ROW and reductions < 4:   # MAX_REDUCTIONS, program.rs:27
+            reductions += 1
+            ops = [RedOp.MAX, RedOp.MIN] if exact else [RedOp.MAX, RedOp.MIN, RedOp.SUM]
+            of_type[ValueType.F32].append(b.reduce(rng.choice(ops), pick(ValueType.F32)))
+        else:
+            of_type[ValueType.F32].append(b.cast(ValueType.F32, pick(ValueType.U32)))
+    for slot in range(2):
+        b.output(slot, int(of_type[ValueType.F32][-1 - slot]))
+    return b.finish()
+
+
+@pytest.mark.parametrize("kind", [ProgramKind.MAP, ProgramKind.ROW])
+@pytest.mark.parametrize("exact", [True, False])
+def test_random_typed_programs_agree_with_the_interpreter(cpu, hip, kind, exact):
+    """25 seeded random programs per case over a broadcast row, a strided view and an integer
+    tensor: bit for bit where IEEE fixes the result, to 1e-5 where libm or the order of a sum does
+    not."""
+    rows, width = 5, 37
+    rng = np.random.default_rng(1234 + 2 * int(kind) + int(exact))
+    first = orc.fill_normal_f32(73, 1, rows * width).reshape(rows, width)
+    second = orc.fill_normal_f32(73, 2, 2 * width).reshape(1, 2 * width)
+    for case in range(25):
+        program = random_program(rng, kind, [ValueType.F32, ValueType.F32, ValueType.U32],
+                                 length=int(rng.integers(4, 24)), exact=exact)
+
+        def build(backend):
+            x = upload(backend, first, DType.F32)
+            y = upload(backend, second, DType.F32).slice([Slice(0, 1), Slice(1, width, 2)]).broadcast(
+                (rows, width))
+            ids = upload(backend, (np.arange(rows * width) * 7919) % 1000, DType.U32).reshape((rows, width))
+            outs = [backend.alloc(DType.F32, (rows, width)) for _ in range(2)]
+            commands = CommandList()
+            commands.dispatch_kernel(backend.prepare_program(program), [x, y, ids], outs)
+            return commands, outs
+        try:
+            if exact:
+                (cpu_out, _), (hip_out, _) = differential(cpu, hip, build, rel=0.0, abs_=0.0, norm_tol=0.0)
+                for a, b_ in zip(cpu_out, hip_out):
+                    assert cpu.read(a) == hip.read(b_), (case, program)
+            else:
+                differential(cpu, hip, build, rel=1e-5, abs_=1e-6, norm_tol=1e-5)
+        except AssertionError as error:
+            raise AssertionError(f"program {case}: {program}") from error
+
+
+def test_program_limits_are_refused_when_prepared(cpu, hip):
+    """Five reductions, a reduction in a map program, an operand that is not earlier
+    (validate_structure, crates/forja-core/src/program.rs:1052-1094)."""
+    five = ProgramBuilder(ProgramKind.ROW)
+    value = five.input(0)
+    for _ in range(5):
+        value = five.reduce(RedOp.MAX, value)
+    five.output(0, value)
+    in_map = ProgramBuilder(ProgramKind.MAP)
+    in_map.output(0, in_map.reduce(RedOp.SUM, in_map.input(0)))
+    forward = Program(ProgramKind.MAP, [Inst.input(0), Inst.unary(UnOp.NEG, 2), Inst.const(1.0)], [(0, 1)])
+    for backend in (cpu, hip):
+        for program in (five.finish(), in_map.finish(), forward):
+            with pytest.raises(BackendError) as info:
+                backend.prepare_program(program)
+            assert info.value.status == Status.INVALID_INPUT
+
+
 def test_softmax_row_program_with_max_and_sum_reductions(cpu, hip):
     b = ProgramBuilder(ProgramKind.ROW)
     x = b.input(0)

@@ -665,6 +665,31 @@ def test_ragged_attention_reports_a_stale_page(hip):
     assert not out[1].any() and out[0].any() and out[2].any()
 
 
+def test_empty_batches_are_accepted_and_change_nothing(cpu, hip):
+    """Zero rows through the projections, the router and a program, and a ragged batch whose lanes
+    bring no query tokens: both backends accept them, write nothing and report nothing."""
+    weights = Quantised(81, 1, (64, 128))
+    stacked = Quantised(81, 2, (64, 128), experts=4)
+
+    def build(backend):
+        x = backend.alloc(DType.BF16, (0, 128))
+        out = backend.alloc(DType.BF16, (0, 64))
+        logits = backend.alloc(DType.BF16, (0, 4))
+        route_weights, route_ids = backend.alloc(DType.BF16, (0, 2)), backend.alloc(DType.U32, (0, 2))
+        routed = backend.alloc(DType.BF16, (0, 2, 64))
+        t, inputs = ragged_case(backend, [5, 9], [0, 0], 8, 4, 16, seed=82)
+        commands = CommandList()
+        commands.dispatch(Op.quant_matmul(4, 64), [x, *weights.upload(backend)], out)
+        commands.dispatch_many(Op.top_k(2, True), [logits], [route_weights, route_ids])
+        commands.dispatch(Op.gather_quant_matmul(4, 64), [x, *stacked.upload(backend), route_ids], routed)
+        commands.dispatch_kernel(backend.prepare_program(programs.add_elements()), [out, out],
+                                 [backend.alloc(DType.BF16, (0, 64))])
+        commands.dispatch_many(Op.paged_attention_ragged(0.1, 16), inputs, [t["out"], t["keys"], t["values"]])
+        return commands, [t["keys"], t["values"]]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    assert cpu.read(cpu_out[0]) == hip.read(hip_out[0]) and cpu.read(cpu_out[1]) == hip.read(hip_out[1])
+
+
 # ------------------------------------------------------------------ programs and glue
 
 def test_engine_row_programs(cpu, hip):

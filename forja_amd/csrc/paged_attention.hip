@@ -264,8 +264,9 @@ struct FastRagged {
   uint64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h;
   uint32_t tokens, lanes, query_heads, kv_heads, group, page_tokens, physical_pages, table_pages,
       max_splits, split_tokens;
-  // Query tokens of one lane are processed `group_tokens` at a time by one wave per kv head (they
-  // share the lane's K/V stream): 1 for decode batches, 2 * (16 / group) for prefill.
+  // Query tokens of one lane are processed `group_tokens` at a time (they share the lane's K/V
+  // stream): 1 for decode batches (a wave per kv head), kSharedWaves * kSharedTiles * (16 / group)
+  // for prefill batches (a workgroup per kv head).
   uint32_t group_tokens;
   float scale_log2;
   // Single-lane form (Op::PagedSdpa / Op::PagedSdpaAppend): cu == nullptr, every token belongs
@@ -645,17 +646,186 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
   }
 }
 
+// ---- prefill: K/V tiles staged in LDS and shared by the four waves of a workgroup -------------
+//
+// A work item of a prefill batch is (up to kSharedWaves * kSharedTiles * (16 / group) consecutive query
+// tokens of a lane, split); blockIdx.y is the kv head.  Wave w owns the w-th slice of those tokens
+// (one 16-row query tile: 16 / group tokens x group heads) and all waves walk the same keys, so a
+// K/V tile is fetched from memory once per workgroup: each wave moves its share of the tile
+// straight into LDS (global_load_lds), double buffered, one barrier per tile.  The softmax is
+// vector-ALU and latency heavy, so the kernel is built for occupancy rather than for long
+// software pipelines: one query tile per wave keeps it at 168 registers, three waves per SIMD
+// (three workgroups per CU).  Rows are 256 bytes (one head of one
+// token); the 16-byte piece p of row r sits in slot p ^ (r & 15), which keeps both operand read
+// patterns (a K row piece per lane, a V column piece of eight tokens per lane) free of bank
+// conflicts.  Keys past the end of the split are staged from its last valid token and masked.
+constexpr uint32_t kSharedWaves = 4;    // waves of a prefill workgroup
+constexpr int kSharedTiles = 1;          // 16-row query tiles per wave
+
+struct SharedTiles {
+  uint4 rows[2][2][kTile][16];   // [buffer][K, V][token][slot]
+};
+
+__device__ inline void stage_tile(const FastRagged &p, SharedTiles &lds, uint32_t buffer,
+                                  uint32_t tile0, uint32_t end, uint32_t page0, uint32_t physical,
+                                  uint32_t kv_head, uint32_t wave, uint32_t lane) {
+  const uint32_t pt = p.page_tokens;
+  constexpr int kPerWave = kTile / 4 / kSharedWaves;   // instructions per wave and operand
+#pragma unroll
+  for (int j = 0; j < kPerWave; ++j) {
+    const uint32_t row = 4 * kPerWave * wave + 4 * j + (lane >> 4);
+    const uint32_t token = min(tile0 + row, end - 1);
+    const uint32_t page = (uint32_t)__shfl((int)physical, (int)(token / pt - page0), 64);
+    const uint64_t element = (((uint64_t)page * pt + token % pt) * p.kv_heads + kv_head) * 128 +
+                             8 * ((lane & 15) ^ (row & 15));
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void *)(p.key_pool + element),
+        (__attribute__((address_space(3))) void *)&lds.rows[buffer][0][4 * kPerWave * wave + 4 * j][0], 16, 0, 0);
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void *)(p.value_pool + element),
+        (__attribute__((address_space(3))) void *)&lds.rows[buffer][1][4 * kPerWave * wave + 4 * j][0], 16, 0, 0);
+  }
+}
+
+// The register image load_tile would have produced, read from the staged tile.
+__device__ inline void read_tile(const SharedTiles &lds, uint32_t buffer, TileRegs &r, uint32_t hl,
+                                 uint32_t g) {
+#pragma unroll
+  for (int sub = 0; sub < 2; ++sub) {
+    const uint32_t k_row = 16 * sub + hl;
+#pragma unroll
+    for (int step = 0; step < 4; ++step) r.k[sub][step] = lds.rows[buffer][0][k_row][(4 * step + g) ^ hl];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t v_row = 16 * sub + 4 * g + i;
+      r.v[4 * sub + i] = lds.rows[buffer][1][v_row][hl ^ (v_row & 15)];
+    }
+  }
+}
+
+__global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_eu(3, 3))) void ragged_attention_prefill_kernel(
+    FastRagged p, ErrorSlot *error) {
+  constexpr int NT = kSharedTiles;
+  __shared__ SharedTiles lds;
+  const uint32_t lane = threadIdx.x & 63, hl = lane & 15, g = lane >> 4;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t item = blockIdx.x, kv_head = blockIdx.y;
+  if (item >= p.item_count[0]) return;
+  const uint2 work = p.items[item];
+  const uint32_t leader = work.x, split = work.y;
+  const TokenPlan plan = p.plans[leader];
+  const uint32_t per_tile = 16 / p.group, per_wave = NT * per_tile;
+  const uint32_t first = wave * per_wave;                       // this wave's first member
+  const uint32_t members = plan.members > first ? min(plan.members - first, per_wave) : 0;
+  // the item's split layout is sized for its last member; a wave stops at its own last member
+  const uint32_t longest = p.fixed_attended ? plan.attended : plan.attended + plan.members - 1;
+  const uint32_t begin = split * plan.chunk;
+  const uint32_t end = min(longest, begin + plan.chunk);
+  const uint32_t own_end =
+      members == 0 ? begin : min(end, p.fixed_attended ? plan.attended : plan.attended + first + members - 1);
+  const uint32_t pt = p.page_tokens;
+  const uint32_t *table = p.tables + (uint64_t)plan.lane * p.table_pages * 2;
+
+  uint4 q_reg[NT][4];
+  uint32_t limit[NT], member_of[NT];
+  const uint32_t head = kv_head * p.group + hl % p.group;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    member_of[nt] = first + nt * per_tile + hl / p.group;
+    const bool used = hl < per_tile * p.group && member_of[nt] < plan.members;
+    limit[nt] = !used ? 0 : min(end, p.fixed_attended ? plan.attended : plan.attended + member_of[nt]);
+    const uint16_t *q_row = p.q + (uint64_t)(leader + (used ? member_of[nt] : 0)) * p.q_stride_t +
+                            (uint64_t)head * p.q_stride_h;
+    for (int step = 0; step < 4; ++step) {
+      q_reg[nt][step] = make_uint4(0, 0, 0, 0);
+      if (used) q_reg[nt][step] = *(const uint4 *)(q_row + 32 * step + 8 * g);
+    }
+    if (!used) member_of[nt] = 0xffffffffu;
+  }
+  // keys below `unmasked_end` are attended by every used row of this wave
+  const uint32_t unmasked_end = min(own_end, p.fixed_attended ? plan.attended : plan.attended + first);
+  f32x4 o[NT][8];
+  Softmax sm[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    for (int mt = 0; mt < 8; ++mt) o[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    sm[nt] = Softmax{-__builtin_inff(), 0.0f};
+  }
+
+  const uint32_t first_page = begin / pt, last_page = (end - 1) / pt;
+  for (uint32_t page0 = first_page; page0 <= last_page; page0 += 64) {
+    // Authenticate up to 64 table entries at once (every wave for itself: same entries, same
+    // verdict); nothing is dereferenced through a bad one.
+    uint32_t my_page = page0 + lane, physical = 0;
+    bool mine = my_page <= last_page, ok = true;
+    if (mine) {
+      uint32_t page = table[2 * (uint64_t)my_page], generation = table[2 * (uint64_t)my_page + 1];
+      ok = page < p.physical_pages && p.generations[page] == generation;
+      physical = page;
+    }
+    unsigned long long bad_mask = __ballot(mine && !ok);
+    if (bad_mask) {
+      if (wave == 0 && lane == (uint32_t)__ffsll((long long)bad_mask) - 1) {
+        report_error(error, my_page);
+        for (uint32_t member = 0; member < plan.members; ++member) p.bad[leader + member] = 1;
+      }
+      return;
+    }
+    const uint32_t tok_lo = max(begin, page0 * pt);
+    const uint32_t tok_hi = (uint32_t)min((uint64_t)end, ((uint64_t)page0 + 64) * pt);
+    stage_tile(p, lds, 0, tok_lo, end, page0, physical, kv_head, wave, lane);
+    uint32_t buffer = 0;
+    for (uint32_t tile0 = tok_lo; tile0 < tok_hi; tile0 += kTile, buffer ^= 1) {
+      __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's share of the tile has landed
+      __syncthreads();                      // everybody's has, and the other buffer is free
+      if (tile0 + kTile < tok_hi)
+        stage_tile(p, lds, buffer ^ 1, tile0 + kTile, end, page0, physical, kv_head, wave, lane);
+      if (tile0 < own_end) {
+        TileRegs cur;
+        read_tile(lds, buffer, cur, hl, g);
+        if (tile0 + kTile <= unmasked_end)
+          consume_tile<NT, false>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+        else
+          consume_tile<NT, true>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();   // the next group's first tile goes into buffer 0
+  }
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    float m_run = sm[nt].m, l_run = sm[nt].l;
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (member_of[nt] == 0xffffffffu) continue;
+    const uint32_t token = leader + member_of[nt];
+    if (plan.splits == 1) {
+      float inv = 1.0f / l_run;
+      uint16_t *out_row = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
+      for (int j = 0; j < 4; ++j) {
+        uint2 lo = make_uint2(pack_bf16(o[nt][0][j] * inv, o[nt][1][j] * inv),
+                              pack_bf16(o[nt][2][j] * inv, o[nt][3][j] * inv));
+        uint2 hi = make_uint2(pack_bf16(o[nt][4][j] * inv, o[nt][5][j] * inv),
+                              pack_bf16(o[nt][6][j] * inv, o[nt][7][j] * inv));
+        *(uint2 *)(out_row + 32 * g + 8 * j) = lo;
+        *(uint2 *)(out_row + 32 * g + 8 * j + 4) = hi;
+      }
+      continue;
+    }
+    uint64_t slot = ((uint64_t)token * p.max_splits + split) * p.query_heads + head;
+    float *po = p.partial_o + slot * 128 + 32 * g;
+    for (int j = 0; j < 4; ++j) {
+      *(float4 *)(po + 8 * j) = make_float4(o[nt][0][j], o[nt][1][j], o[nt][2][j], o[nt][3][j]);
+      *(float4 *)(po + 8 * j + 4) = make_float4(o[nt][4][j], o[nt][5][j], o[nt][6][j], o[nt][7][j]);
+    }
+    if (g == 0) p.partial_ml[slot] = make_float2(m_run, l_run);
+  }
+}
+
 // Decode batches: one query token per wave, two waves per SIMD to hide the K/V stream's latency.
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void ragged_attention_mfma_kernel(
     FastRagged p, ErrorSlot *error) {
   ragged_attention_body<1>(p, error);
-}
-
-// Prefill chunks: two query tiles per wave share every K/V tile (one wave per SIMD, the whole
-// register file).
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void ragged_attention_prefill_kernel(
-    FastRagged p, ErrorSlot *error) {
-  ragged_attention_body<2>(p, error);
 }
 
 // Merges the per-split partials of one (token, head): out = sum_s O_s 2^(m_s-M) / sum_s l_s
@@ -808,9 +978,8 @@ void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, E
     KernelTimer timer(backend, FH_KC_ATTENTION_KERNEL);
     // one workgroup per work item, up to 8 (decode) or 4 (prefill) kv heads of it per workgroup
     if (f.group_tokens > 1) {
-      const uint32_t waves = f.kv_heads < 4 ? f.kv_heads : 4;
-      ragged_attention_prefill_kernel<<<dim3((unsigned)blocks, (f.kv_heads + waves - 1) / waves),
-                                        64 * waves, 0, stream>>>(f, error);
+      ragged_attention_prefill_kernel<<<dim3((unsigned)blocks, f.kv_heads), 64 * kSharedWaves, 0,
+                                        stream>>>(f, error);
     } else {
       const uint32_t waves = f.kv_heads < 8 ? f.kv_heads : 8;
       ragged_attention_mfma_kernel<<<dim3((unsigned)blocks, (f.kv_heads + waves - 1) / waves),
@@ -843,7 +1012,7 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   f.physical_pages = lane.physical_pages;
   f.table_pages = lane.logical_pages;
   f.max_splits = splits_for(f.tokens);
-  f.group_tokens = f.tokens > 1 ? 2 * (16 / group) : 1;
+  f.group_tokens = f.tokens > 1 ? kSharedWaves * kSharedTiles * (16 / group) : 1;
   f.scale_log2 = lane.scale * 1.4426950408889634f;
   f.one_start = lane.query_start;
   f.fixed_attended = lane.causal ? 0 : lane.key_length;
@@ -879,7 +1048,7 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     f.query_heads = p.query_heads;
     f.kv_heads = p.kv_heads;
     f.group = p.query_heads / p.kv_heads;
-    f.group_tokens = p.tokens > p.lanes ? 2 * (16 / f.group) : 1;
+    f.group_tokens = p.tokens > p.lanes ? kSharedWaves * kSharedTiles * (16 / f.group) : 1;
     f.page_tokens = p.page_tokens;
     f.physical_pages = p.physical_pages;
     f.table_pages = p.table_pages;

@@ -88,6 +88,7 @@ void launch_init_errors(hipStream_t s, ErrorSlot *slots, uint32_t count);
 void launch_route_pack(hipStream_t s, const View &indices, uint32_t rows, uint32_t k,
                        uint32_t experts, uint32_t tile_rows, uint32_t *counts, uint32_t *offsets,
                        uint32_t *sorted_routes, uint32_t *blocks, uint32_t max_blocks,
-                       uint32_t *n_blocks, ErrorSlot *error);
+                       uint32_t *n_blocks, ErrorSlot *error, uint32_t *zero_rows = nullptr,
+                       uint32_t zero_row_words = 0);
 
 }  // namespace fh

@@ -19,7 +19,7 @@ constexpr uint32_t kPackThreads = 1024, kPackWaves = kPackThreads / 64;
 __global__ __launch_bounds__(1024) void route_pack_kernel(
     View indices, uint32_t rows, uint32_t k, uint32_t experts, uint32_t tile_rows, uint32_t *counts,
     uint32_t *offsets, uint32_t *sorted_routes, uint32_t *blocks, uint32_t max_blocks,
-    uint32_t *n_blocks, ErrorSlot *error) {
+    uint32_t *n_blocks, uint32_t *zero_rows, uint32_t zero_row_words, ErrorSlot *error) {
   extern __shared__ uint32_t lds[];
   uint32_t *lds_counts = lds;                    // [experts]
   uint32_t *lds_cursor = lds + experts;          // [experts] next free position per expert
@@ -37,9 +37,12 @@ __global__ __launch_bounds__(1024) void route_pack_kernel(
   const uint32_t first_expert = tid < routes ? expert_of(tid) : 0xffffffffu;
   for (uint32_t route = tid; route < routes; route += kPackThreads) {
     const uint32_t expert = route == tid ? first_expert : expert_of(route);
-    if (expert >= experts)
+    if (expert >= experts) {
       report_error(error, expert);
-    else
+      // a bad route is never packed: its output row (if the caller has one) is cleared here
+      if (zero_rows)
+        for (uint32_t w = 0; w < zero_row_words; ++w) zero_rows[(uint64_t)route * zero_row_words + w] = 0;
+    } else
       atomicAdd(&lds_counts[expert], 1u);
   }
   __syncthreads();
@@ -140,10 +143,12 @@ __global__ __launch_bounds__(1024) void route_pack_kernel(
 void launch_route_pack(hipStream_t s, const View &indices, uint32_t rows, uint32_t k,
                        uint32_t experts, uint32_t tile_rows, uint32_t *counts, uint32_t *offsets,
                        uint32_t *sorted_routes, uint32_t *blocks, uint32_t max_blocks,
-                       uint32_t *n_blocks, ErrorSlot *error) {
+                       uint32_t *n_blocks, ErrorSlot *error, uint32_t *zero_rows,
+                       uint32_t zero_row_words) {
   size_t lds = ((size_t)experts * (2 + kPackWaves) + 2 * (kPackWaves + 1)) * sizeof(uint32_t);
   route_pack_kernel<<<dim3(1), kPackThreads, lds, s>>>(indices, rows, k, experts, tile_rows, counts, offsets,
-                                             sorted_routes, blocks, max_blocks, n_blocks, error);
+                                             sorted_routes, blocks, max_blocks, n_blocks, zero_rows,
+                                             zero_row_words, error);
 }
 
 }  // namespace fh

@@ -700,6 +700,52 @@ __global__ void combine_routes_kernel(const float *partial, View indices, View w
   store_float_at(out, out.offset + row * out.stride[0] + column * out.stride[1], value);
 }
 
+// The same sum for bf16 rows with 8-byte aligned columns: a thread owns four consecutive columns
+// of a row, fetches the row's (expert, weight) pairs first and then all its partial rows at once
+// (at most kMax routes), and adds them in ascending slot order.
+template <int kMax>
+__global__ __launch_bounds__(256) void combine_routes_rows_kernel(
+    const float *partial, View indices, View weights, const uint16_t *residual,
+    uint64_t residual_row_stride, uint16_t *out, uint64_t out_row_stride, uint32_t rows,
+    uint32_t routes, uint32_t columns, uint32_t experts) {
+  const uint64_t flat = 4 * ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x);
+  if (flat >= (uint64_t)rows * columns) return;
+  const uint32_t row = (uint32_t)(flat / columns), column = (uint32_t)(flat % columns);
+  float weight[kMax];
+  float4 part[kMax];
+#pragma unroll
+  for (int slot = 0; slot < kMax; ++slot) {
+    weight[slot] = 0.0f;
+    part[slot] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if ((uint32_t)slot < routes) {
+      const uint32_t expert = load_u32_at(indices, indices.offset + row * indices.stride[0] +
+                                                       slot * indices.stride[1]);
+      if (expert < experts) {
+        weight[slot] = load_float_at(weights, weights.offset + row * weights.stride[0] +
+                                                  slot * weights.stride[1]);
+        part[slot] = *(const float4 *)(partial + ((uint64_t)row * routes + slot) * columns + column);
+      }
+    }
+  }
+  float4 value = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+  for (int slot = 0; slot < kMax; ++slot) {   // a skipped route adds +0 * 0: no effect
+    value.x += weight[slot] * part[slot].x;
+    value.y += weight[slot] * part[slot].y;
+    value.z += weight[slot] * part[slot].z;
+    value.w += weight[slot] * part[slot].w;
+  }
+  if (residual) {
+    const uint2 r = *(const uint2 *)(residual + (uint64_t)row * residual_row_stride + column);
+    value.x += bf16_bits_to_f32(r.x & 0xffffu);
+    value.y += bf16_bits_to_f32(r.x >> 16);
+    value.z += bf16_bits_to_f32(r.y & 0xffffu);
+    value.w += bf16_bits_to_f32(r.y >> 16);
+  }
+  *(uint2 *)(out + (uint64_t)row * out_row_stride + column) =
+      make_uint2(pack2(value.x, value.y), pack2(value.z, value.w));
+}
+
 bool rows_contiguous(const View &v, uint32_t rank) {
   // innermost axis contiguous and every outer stride the dense product (weights, scales)
   uint64_t expected = 1;
@@ -843,12 +889,13 @@ struct RoutePlan {
   uint32_t *counts, *offsets, *sorted_routes, *blocks, *n_blocks;
   uint32_t max_blocks;
   char *rest;  // workspace after the plan
+  bool reused; // nothing was packed for this call
 };
 
 // Packs the routes on the device (or reuses the plan the previous routed projection packed from
 // the same indices); `extra` bytes of ordinary workspace are returned in plan->rest.
 bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, ErrorSlot *error,
-                 RoutePlan *plan) {
+                 RoutePlan *plan, uint32_t *zero_rows = nullptr, uint32_t zero_row_words = 0) {
   uint64_t routes = (uint64_t)p.rows * p.k;
   plan->max_blocks = p.experts + (uint32_t)(routes / kRouteTile) + 1;
   auto round = [](uint64_t bytes) { return (bytes + 255) / 256 * 256; };
@@ -873,10 +920,11 @@ bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, Er
   plan->blocks = (uint32_t *)ws;
   ws += blocks_b;
   plan->n_blocks = (uint32_t *)ws;
+  plan->reused = reuse;
   if (!reuse)
     launch_route_pack(backend_stream(backend), p.indices, p.rows, p.k, p.experts, kRouteTile,
                       plan->counts, plan->offsets, plan->sorted_routes, plan->blocks,
-                      plan->max_blocks, plan->n_blocks, error);
+                      plan->max_blocks, plan->n_blocks, error, zero_rows, zero_row_words);
   return true;
 }
 
@@ -920,12 +968,19 @@ bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int
   if (p.out.stride[2] != 1 || p.out.stride[1] != p.columns ||
       p.out.stride[0] != (uint64_t)p.k * p.columns)
     return false;
+  // Rows of bad routes must read zero and bad routes are never packed: the packing kernel clears
+  // them as it meets them (a row = `columns` bf16); when the plan is reused instead, nothing
+  // packs, and the whole output is cleared first.
   RoutePlan plan;
-  if (!plan_routes(backend, p, 0, error, &plan)) return false;
+  const bool row_words = p.columns % 2 == 0 && p.out.offset % 2 == 0;
+  if (!plan_routes(backend, p, 0, error, &plan,
+                   row_words ? (uint32_t *)((uint16_t *)p.out.base + p.out.offset) : nullptr,
+                   p.columns / 2))
+    return false;
   hipStream_t stream = backend_stream(backend);
-  // Rows of bad routes stay zero: clear the output first (bad routes are never packed).
-  launch_fill_u32(stream, (uint32_t *)((uint16_t *)p.out.base + p.out.offset),
-                  (uint64_t)p.rows * p.k * p.columns / 2, 0);
+  if (plan.reused || !row_words)
+    launch_fill_u32(stream, (uint32_t *)((uint16_t *)p.out.base + p.out.offset),
+                    (uint64_t)p.rows * p.k * p.columns / 2, 0);
   QmmArgs a{};
   a.x = u16_ptr(p.x);
   a.x_row_stride = p.x.stride[0];
@@ -989,6 +1044,24 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
     launch_routed<false>(stream, a, plan.max_blocks);
   }
   uint64_t work = (uint64_t)p.rows * p.columns;
+  auto row_view = [&](const View &v) {   // bf16 [rows, columns], 8-byte aligned row pieces
+    return v.dtype == FH_BF16 && v.stride[1] == 1 && v.stride[0] % 4 == 0 && v.offset % 4 == 0;
+  };
+  if (p.columns % 4 == 0 && p.k <= 16 && row_view(p.out) && (!residual || row_view(*residual))) {
+    const uint16_t *res = residual ? (const uint16_t *)residual->base + residual->offset : nullptr;
+    const uint64_t res_stride = residual ? residual->stride[0] : 0;
+    uint16_t *out = (uint16_t *)p.out.base + p.out.offset;
+    const dim3 grid((unsigned)((work / 4 + 255) / 256));
+    if (p.k <= 8)
+      combine_routes_rows_kernel<8><<<grid, 256, 0, stream>>>(partial, p.indices, p.weights, res, res_stride,
+                                                             out, p.out.stride[0], p.rows, p.k,
+                                                             p.columns, p.experts);
+    else
+      combine_routes_rows_kernel<16><<<grid, 256, 0, stream>>>(partial, p.indices, p.weights, res, res_stride,
+                                                              out, p.out.stride[0], p.rows, p.k,
+                                                              p.columns, p.experts);
+    return true;
+  }
   View none{};
   none.base = nullptr;
   combine_routes_kernel<<<dim3((unsigned)((work + 255) / 256)), 256, 0, stream>>>(

@@ -419,48 +419,37 @@ __global__ void top_k_registers_kernel(View in, View values, View indices, uint3
   __shared__ float selected[64 * kPer];
   const uint32_t row = blockIdx.x, lane = threadIdx.x;
   const uint64_t in_row = in.offset + (uint64_t)row * in.stride[0];
-  int32_t keys[kPer];
-  bool live[kPer];
+  // A candidate is one 64-bit word that orders like (key descending, index ascending): the key
+  // mapped to unsigned order in the high half, the complemented index in the low half; 0 stands
+  // for "none" (no element has index 0xffffffff).  A selection is then a 64-bit maximum.
+  unsigned long long word[kPer];
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
     const uint32_t index = lane + 64 * i;
-    live[i] = index < width;
-    keys[i] = live[i] ? total_key(load_float_at(in, in_row + (uint64_t)index * in.stride[1]))
-                      : (int32_t)0x80000000;
+    word[i] = 0;
+    if (index < width) {
+      const int32_t key = total_key(load_float_at(in, in_row + (uint64_t)index * in.stride[1]));
+      word[i] = ((unsigned long long)((uint32_t)key ^ 0x80000000u) << 32) | (uint32_t)~index;
+    }
   }
   for (uint32_t slot = 0; slot < k; ++slot) {
-    Candidate best = {(int32_t)0x80000000, 0xffffffffu};
-    bool have = false;
-    int mine = -1;
+    unsigned long long best = word[0];
 #pragma unroll
-    for (int i = 0; i < kPer; ++i) {
-      Candidate c = {keys[i], lane + 64 * i};
-      if (live[i] && (!have || before(c, best))) {
-        best = c;
-        have = true;
-        mine = i;
-      }
-    }
-    const uint32_t my_index = best.index;
+    for (int i = 1; i < kPer; ++i) best = word[i] > best ? word[i] : best;
     for (int offset = 32; offset > 0; offset >>= 1) {
-      Candidate other;
-      other.key = __shfl_xor(best.key, offset, 64);
-      other.index = __shfl_xor(best.index, offset, 64);
-      int other_have = __shfl_xor((int)have, offset, 64);
-      if (other_have && (!have || before(other, best))) {
-        best = other;
-        have = true;
-      }
+      const unsigned long long other = __shfl_xor(best, offset, 64);
+      best = other > best ? other : best;
     }
     // the owner retires the selected element
 #pragma unroll
     for (int i = 0; i < kPer; ++i)
-      if (mine == i && my_index == best.index) live[i] = false;
+      if (word[i] == best) word[i] = 0;
     if (lane == 0) {
-      const int32_t bits = best.key ^ (int32_t)(((uint32_t)(best.key >> 31)) >> 1);
+      const int32_t key = (int32_t)((uint32_t)(best >> 32) ^ 0x80000000u);
+      const int32_t bits = key ^ (int32_t)(((uint32_t)(key >> 31)) >> 1);
       selected[slot] = __uint_as_float((uint32_t)bits);
       ((uint32_t *)indices.base)[indices.offset + (uint64_t)row * indices.stride[0] +
-                                 (uint64_t)slot * indices.stride[1]] = best.index;
+                                 (uint64_t)slot * indices.stride[1]] = ~(uint32_t)best;
     }
   }
   if (lane == 0) {

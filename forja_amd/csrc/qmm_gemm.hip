@@ -428,6 +428,9 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
 bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t **refused) {
   if (p.inner / 64 > kMaxGroups) return false;
   const uint32_t kt = padded_inner(p.inner);
+  // the GEMM addresses its operand matrices with 32-bit byte offsets
+  if ((uint64_t)p.rows * kt * 2 >= (1ull << 32) || (uint64_t)p.columns * kt * 2 >= (1ull << 32))
+    return false;
   const uint64_t a_bytes = ((uint64_t)p.rows * kt * 2 + 255) / 256 * 256;
   const uint64_t b_bytes = ((uint64_t)p.columns * kt * 2 + 255) / 256 * 256;
   const uint64_t unscale_bytes = ((uint64_t)p.rows * sizeof(float) + 255) / 256 * 256;

@@ -778,6 +778,168 @@ void launch_qmm(hipStream_t stream, const QmmArgs &a, uint32_t row_blocks, int m
     qmm_mfma_kernel<2, kPair, kRouted><<<grid, 256, 0, stream>>>(a);
 }
 
+// ---- decode-sized dense products, one kernel, no partial tiles in memory ----------------------
+//
+// A workgroup owns one 32 x 32 output tile (32 rows, 32 columns) for the whole of K and splits K
+// over its waves in 256-value pieces (one 128-byte line of every packed weight row, so each line
+// is fetched once).  Nothing is staged: a lane loads the 16-byte activation pieces of "its" row
+// and K half straight into MFMA operand registers (permuted in registers to the order in which
+// nibbles unpack) and sums them per group for the bias term.  The waves' 32 x 32 sums meet in LDS
+// and wave 0 adds them in wave order (fixed: results do not depend on scheduling), adds the
+// optional residual and stores.  Activations are re-read from L2 by every column tile and
+// weights by every row tile; at decode sizes that is cheaper than writing f32 partial tiles to
+// memory and summing them in a second launch.
+struct TileProductArgs {
+  const uint16_t *x;
+  uint64_t x_row_stride;
+  const uint32_t *packed;
+  const uint16_t *scales, *biases;
+  void *out;
+  uint64_t out_row_stride;
+  uint32_t out_f32;
+  const uint16_t *residual;
+  uint64_t residual_row_stride;
+  uint32_t rows, inner, columns;
+};
+
+constexpr int kTileProductWaves = 8;
+
+template <int kCols>   // 32-column tiles per wave: they share the wave's activation registers
+__global__ __launch_bounds__(64 * kTileProductWaves) void qmm_tile_product_kernel(TileProductArgs a) {
+  __shared__ float handed[kTileProductWaves - 1][kCols][16][64];
+  const uint32_t tid = threadIdx.x, lane = tid & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
+  const uint32_t nl = lane & 31, h = lane >> 5;
+  const uint32_t row = blockIdx.y * 32 + nl;
+  const bool row_live = row < a.rows;
+  const uint32_t quads = a.inner / 256, groups_per_row = a.inner / kGroup;
+  uint32_t column[kCols];
+  const uint32_t *w_row[kCols];
+  const uint16_t *s_row[kCols], *b_row[kCols];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) {
+    column[c] = (blockIdx.x * kCols + c) * 32 + nl;
+    const uint32_t column_c = min(column[c], a.columns - 1);
+    w_row[c] = a.packed + (uint64_t)column_c * (a.inner / 8) + 4 * h;
+    s_row[c] = a.scales + (uint64_t)column_c * groups_per_row;
+    b_row[c] = a.biases + (uint64_t)column_c * groups_per_row;
+  }
+  const uint16_t *x_row = a.x + (uint64_t)min(row, a.rows - 1) * a.x_row_stride + 32 * h;
+  f32x16 acc[kCols];
+  for (int c = 0; c < kCols; ++c)
+    for (int j = 0; j < 16; ++j) acc[c][j] = 0.0f;
+  for (uint32_t quad = wave; quad < quads; quad += waves) {
+    uint4 wq[kCols][4], xq[4][4];
+    uint2 scale4[kCols], bias4[kCols];
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) wq[c][i] = *(const uint4 *)(w_row[c] + (uint64_t)(4 * quad + i) * 8);
+      scale4[c] = *(const uint2 *)(s_row[c] + 4 * quad);
+      bias4[c] = *(const uint2 *)(b_row[c] + 4 * quad);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int step = 0; step < 4; ++step) {
+        xq[i][step] = make_uint4(0, 0, 0, 0);
+        if (row_live) xq[i][step] = *(const uint4 *)(x_row + 256 * quad + 64 * i + 8 * step);
+      }
+    float group_sum[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float half_sum = 0.0f;
+#pragma unroll
+      for (int step = 0; step < 4; ++step) {
+        const uint4 v = xq[i][step];
+        half_sum += bf16_bits_to_f32(v.x & 0xffffu) + bf16_bits_to_f32(v.x >> 16) +
+                    bf16_bits_to_f32(v.y & 0xffffu) + bf16_bits_to_f32(v.y >> 16) +
+                    bf16_bits_to_f32(v.z & 0xffffu) + bf16_bits_to_f32(v.z >> 16) +
+                    bf16_bits_to_f32(v.w & 0xffffu) + bf16_bits_to_f32(v.w >> 16);
+        // the operand order in which nibbles unpack: (x0,x4)(x1,x5)(x2,x6)(x3,x7)
+        uint4 permuted;
+        permuted.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+        permuted.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+        permuted.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+        permuted.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+        xq[i][step] = permuted;
+      }
+      group_sum[i] = half_sum + __shfl_xor(half_sum, 32, 64);   // both K halves of the group
+    }
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+      float shift[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t s_bits = (i < 2 ? scale4[c].x : scale4[c].y) >> (16 * (i & 1)) & 0xffffu;
+        const uint32_t b_bits = (i < 2 ? bias4[c].x : bias4[c].y) >> (16 * (i & 1)) & 0xffffu;
+        const float scale = bf16_bits_to_f32(s_bits);
+        shift[i] = bf16_bits_to_f32(b_bits) - 16.0f * scale;
+        f32x16 part;
+        for (int j = 0; j < 16; ++j) part[j] = 0.0f;
+#pragma unroll
+        for (int step = 0; step < 4; ++step) {
+          const uint4 w = wq[c][i];
+          const uint32_t word = step == 0 ? w.x : (step == 1 ? w.y : (step == 2 ? w.z : w.w));
+          part = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xq[i][step]),
+                                                         unpack_word(word), part, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[c][j] += scale * part[j];
+      }
+      // bias term of the four groups: two f32 MFMAs, lane half h supplying group 2p + h
+#pragma unroll
+      for (int p2 = 0; p2 < 2; ++p2)
+        acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(h ? group_sum[2 * p2 + 1] : group_sum[2 * p2],
+                                                      h ? shift[2 * p2 + 1] : shift[2 * p2], acc[c], 0, 0, 0);
+    }
+  }
+  if (wave != 0)
+    for (int c = 0; c < kCols; ++c)
+      for (int j = 0; j < 16; ++j) handed[wave - 1][c][j][lane] = acc[c][j];
+  __syncthreads();
+  if (wave != 0) return;
+  for (int c = 0; c < kCols; ++c) {
+    if (column[c] >= a.columns) continue;
+    for (uint32_t other = 0; other + 1 < waves; ++other)
+      for (int j = 0; j < 16; ++j) acc[c][j] += handed[other][c][j][lane];
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t out_row = blockIdx.y * 32 + 8 * (j / 4) + 4 * h + (j % 4);
+      if (out_row >= a.rows) continue;
+      float value = acc[c][j];
+      if (a.residual)
+        value += bf16_bits_to_f32(a.residual[(uint64_t)out_row * a.residual_row_stride + column[c]]);
+      const uint64_t at = (uint64_t)out_row * a.out_row_stride + column[c];
+      if (a.out_f32)
+        ((float *)a.out)[at] = value;
+      else
+        ((uint16_t *)a.out)[at] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+    }
+  }
+}
+
+void launch_tile_product(fh_backend *backend, const QmmArgs &q, const uint16_t *residual,
+                         uint64_t residual_row_stride) {
+  TileProductArgs t{};
+  t.x = q.x;
+  t.x_row_stride = q.x_row_stride;
+  t.packed = q.packed[0];
+  t.scales = q.scales[0];
+  t.biases = q.biases[0];
+  t.out = q.out;
+  t.out_row_stride = q.out_row_stride;
+  t.out_f32 = q.out_f32;
+  t.residual = residual;
+  t.residual_row_stride = residual_row_stride;
+  t.rows = q.rows;
+  t.inner = q.inner;
+  t.columns = q.columns;
+  const uint32_t quads = q.inner / 256, column_tiles = (q.columns + 31) / 32, row_tiles = (q.rows + 31) / 32;
+  const uint32_t waves = quads < (uint32_t)kTileProductWaves ? quads : (uint32_t)kTileProductWaves;
+  KernelTimer timer(backend, FH_KC_QMM_KERNEL);
+  qmm_tile_product_kernel<1><<<dim3(column_tiles, row_tiles), 64 * waves, 0, backend_stream(backend)>>>(t);
+}
+
 // Decode-sized dense product through the slab kernels; false when workspace is short.
 template <int MT>
 void launch_slab(hipStream_t stream, const SlabArgs &s, dim3 grid) {
@@ -861,6 +1023,13 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
       return false;
     residual = u16_ptr(r);
     residual_row_stride = r.stride[0];
+  }
+  // Decode rows.  When one workgroup per compute unit covers the output, the single-kernel tile
+  // product; wider outputs go through the K slabs.
+  if (p.rows <= 128 &&
+      (uint64_t)((p.columns + 31) / 32) * ((p.rows + 31) / 32) <= backend_compute_units(backend)) {
+    launch_tile_product(backend, a, residual, residual_row_stride);
+    return true;
   }
   if (p.rows <= 128 && p.columns <= 16384 && p.columns % 4 == 0 && p.out.stride[0] % 4 == 0 &&
       p.out.offset % 4 == 0 && (!residual || p.inner > kSlabK)) {

@@ -103,10 +103,11 @@ struct QkArgs {
   float head_dim, eps, theta, exponent_scale;
 };
 
-// One workgroup per row, its four waves taking the heads in turn: RMS-normalise the head over both
-// halves, scale, rotate the (lo, hi) pair by angle = position * theta^(i * exponent_scale).  The
-// rotation is the same for every head of a row when the positions do not vary along the head
-// axis (the usual broadcast view), and is then computed once per wave.
+// blockIdx.x is the row; the waves of its gridDim.y workgroups take the heads in turn (one head per
+// wave for small batches, many for long ones): RMS-normalise the head over both halves, scale,
+// rotate the (lo, hi) pair by angle = position * theta^(i * exponent_scale).  The rotation is the
+// same for every head of a row when the positions do not vary along the head axis (the usual
+// broadcast view), and is then computed once per wave.
 __global__ __launch_bounds__(256) void qk_norm_rope_kernel(QkArgs a) {
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t row = blockIdx.x;
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(QkArgs a) {
     c = cosf(angle);
     s = sinf(angle);
   }
-  for (uint32_t head = wave; head < a.heads; head += 4) {
+  for (uint32_t head = blockIdx.y * 4 + wave; head < a.heads; head += 4 * gridDim.y) {
     float lo = 0.0f, hi = 0.0f;
     if (live) {
       lo = __uint_as_float((uint32_t)a.lo[row * a.lo_s[0] + head * a.lo_s[1] + lane] << 16);
@@ -401,7 +402,11 @@ bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const Program
     a.eps = cls.c[1];
     a.theta = cls.c[2];
     a.exponent_scale = cls.c[3];
-    qk_norm_rope_kernel<<<dim3(a.rows), 256, 0, stream>>>(a);
+    // enough workgroups to fill the device for small batches, one per row for long ones
+    const uint32_t head_blocks = (a.heads + 3) / 4;
+    uint32_t per_row = 4096 / a.rows;
+    per_row = per_row < 1 ? 1 : (per_row > head_blocks ? head_blocks : per_row);
+    qk_norm_rope_kernel<<<dim3(a.rows, per_row), 256, 0, stream>>>(a);
     return true;
   }
   return false;

@@ -426,6 +426,8 @@ def main():
         submission.free()
     backend.synchronize()
     if not args.no_profile:
+        # inside the timed region only the dominant kernel is timed (two event records per launch)
+        backend.profile_select(1 << KC_ATTENTION_KERNEL)
         backend.profile_enable(1)
         backend.profile_reset()
 
@@ -473,8 +475,15 @@ def main():
             "kernel": "ragged_attention_mfma_kernel", "launches": launches,
             "avg_launch_us": average * 1e6, "algorithmic_bytes_per_launch": kernel_bytes,
         }
-        # Secondary kernels over the same region, then a per-op breakdown from a few extra steps
-        # (every dispatch timed; not part of `value`).
+        # Secondary kernels from a few extra steps with every kernel class timed, then a per-op
+        # breakdown with every dispatch timed (neither is part of `value`).
+        secondary_steps = 4
+        backend.profile_select(0xffffffff)
+        backend.profile_reset()
+        for _ in range(secondary_steps):
+            submission, _ = run_step()
+            submission.wait()
+            submission.free()
         moe_ns, moe_launches = backend.profile_read(KC_MOE_KERNEL)
         qmm_ns, qmm_launches = backend.profile_read(KC_QMM_KERNEL)
         secondary = {}
@@ -493,7 +502,7 @@ def main():
                 workload.model.n_layers, args.lanes * config.top_k)
             distinct = np.array([len(np.unique(layer)) for layer in chosen])
             fraction = float(distinct.mean()) / config.experts
-            moe_bytes = weights["routed_all_experts"] * fraction * args.steps / moe_launches
+            moe_bytes = weights["routed_all_experts"] * fraction * secondary_steps / moe_launches
             secondary["routed_qmm_mfma_kernel"] = {
                 "avg_launch_us": moe_ns / moe_launches / 1e3,
                 "achieved_gbps": moe_bytes / (moe_ns / moe_launches * 1e-9) / 1e9,
@@ -505,7 +514,7 @@ def main():
                          "one traced step), per projection launch")}
             routed_fraction = fraction
         if qmm_launches:
-            qmm_bytes = weights["dense"] * args.steps / qmm_launches
+            qmm_bytes = weights["dense"] * secondary_steps / qmm_launches
             secondary["dense_qmm_mfma_kernel"] = {
                 "avg_launch_us": qmm_ns / qmm_launches / 1e3,
                 "achieved_gbps": qmm_bytes / (qmm_ns / qmm_launches * 1e-9) / 1e9,

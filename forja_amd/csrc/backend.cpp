@@ -112,6 +112,7 @@ struct fh_backend {
   AttentionPlanKey attention_plan_key{};
   // profiling
   int profiling = 0;  // 0 off, 1 kernel-level timers, 2 also one timer per dispatch
+  uint32_t profile_mask = 0xffffffffu;  // kernel classes the kernel-level timers cover
   struct Timed {
     hipEvent_t start, end;
     uint32_t kernel_class;
@@ -1670,6 +1671,16 @@ fh_status fh_profile_enable(fh_backend *b, int enabled) {
   return FH_OK;
 }
 
+fh_status fh_profile_select(fh_backend *b, uint32_t class_mask) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  (void)hipStreamSynchronize(b->stream);
+  drain_profile(b);
+  b->profile_mask = class_mask;
+  return FH_OK;
+}
+
 fh_status fh_profile_reset(fh_backend *b) {
   if (!b) return FH_INVALID_INPUT;
   std::lock_guard<std::mutex> lock(b->mutex);
@@ -1749,6 +1760,7 @@ uint32_t backend_compute_units(fh_backend *backend) {
 }
 void backend_profile_begin(fh_backend *backend, uint32_t kernel_class) {
   if (!backend->profiling || kernel_class >= FH_KC_COUNT) return;
+  if (!((backend->profile_mask >> kernel_class) & 1u)) return;
   hipEvent_t event = nullptr;
   if (!backend->event_pool.empty()) {
     event = backend->event_pool.back();

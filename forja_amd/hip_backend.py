@@ -58,7 +58,8 @@ EXPORTS = [
     "fh_create", "fh_destroy", "fh_alloc", "fh_release", "fh_import", "fh_write", "fh_read",
     "fh_read_tensor", "fh_prepare_program", "fh_release_program", "fh_submit", "fh_wait",
     "fh_gpu_time_ns", "fh_submission_free", "fh_device_info_get", "fh_memory_usage",
-    "fh_synchronize", "fh_profile_enable", "fh_profile_reset", "fh_profile_read", "fh_version",
+    "fh_synchronize", "fh_profile_enable", "fh_profile_select", "fh_profile_reset", "fh_profile_read",
+    "fh_version",
 ]
 
 _lib = None
@@ -97,6 +98,7 @@ def load_library():
     lib.fh_synchronize.argtypes = [vp]
     lib.fh_profile_enable.argtypes = [vp, C.c_int]
     lib.fh_profile_reset.argtypes = [vp]
+    lib.fh_profile_select.argtypes = [vp, u32]
     lib.fh_profile_read.argtypes = [vp, u32, C.POINTER(u64), C.POINTER(u64)]
     lib.fh_version.restype = C.c_char_p
     _lib = lib
@@ -313,6 +315,10 @@ class HipBackend:
     def profile_enable(self, level: int):
         """0 off, 1 single-kernel timers, 2 also one timer per dispatch."""
         _check(self._lib.fh_profile_enable(self._handle, int(level)))
+
+    def profile_select(self, class_mask: int):
+        """Kernel classes (bit i = class i) the kernel-level timers cover; all by default."""
+        _check(self._lib.fh_profile_select(self._handle, int(class_mask) & 0xffffffff))
 
     def profile_reset(self):
         _check(self._lib.fh_profile_reset(self._handle))

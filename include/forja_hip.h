@@ -215,6 +215,10 @@ typedef enum fh_kernel_class {
   FH_KC_COUNT = 7
 } fh_kernel_class;
 FH_API fh_status fh_profile_enable(fh_backend *backend, int enabled);
+/* Restricts the kernel-level timers to the classes whose bit is set (bit i = fh_kernel_class i;
+ * all classes by default): every timed launch costs two event records on the stream, so a
+ * throughput measurement times only the kernel it reports on. */
+FH_API fh_status fh_profile_select(fh_backend *backend, uint32_t class_mask);
 FH_API fh_status fh_profile_reset(fh_backend *backend);
 FH_API fh_status fh_profile_read(fh_backend *backend, uint32_t kernel_class, uint64_t *nanoseconds,
                           uint64_t *launches);

@@ -63,14 +63,24 @@ __device__ inline uint32_t pack2(float lo, float hi) {
 
 __device__ inline float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
-// Eight nibbles of `w` as bf16 (16+q), in slot order (0,4)(1,5)(2,6)(3,7).
+// (x & mask) | magic in one instruction.  The compiler splits the expression in two when both
+// constants are literals (a VOP3 instruction reads one scalar operand at most); with the mask in a
+// scalar register and the other constant in a vector register it is a single v_and_or_b32.
+__device__ inline uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
+  return r;
+}
+
+// Eight nibbles of `w` as bf16 (16+q), in slot order (0,4)(1,5)(2,6)(3,7): two instructions per
+// pair of nibbles.
 __device__ inline bf16x8 unpack_word(uint32_t w) {
   const uint32_t mask = 0x00780078u, magic = 0x41804180u;
   uint4 r;
-  r.x = ((w << 3) & mask) | magic;
-  r.y = ((w >> 1) & mask) | magic;
-  r.z = ((w >> 5) & mask) | magic;
-  r.w = ((w >> 9) & mask) | magic;
+  r.x = and_or(w << 3, mask, magic);
+  r.y = and_or(w >> 1, mask, magic);
+  r.z = and_or(w >> 5, mask, magic);
+  r.w = and_or(w >> 9, mask, magic);
   return __builtin_bit_cast(bf16x8, r);
 }
 
@@ -238,7 +248,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
         for (int j = 0; j < 16; ++j)
-          acc[pj][mt][j] += scale0 * part[0][pj][mt][j] + scale1 * part[1][pj][mt][j];
+          acc[pj][mt][j] = __builtin_fmaf(scale1, part[1][pj][mt][j],
+                                          __builtin_fmaf(scale0, part[0][pj][mt][j], acc[pj][mt][j]));
         acc[pj][mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(
             xsum[(gi + h) * kRows + mt * 32 + nl], shift, acc[pj][mt], 0, 0, 0);
       }
@@ -406,7 +417,7 @@ __global__ __launch_bounds__(512) void qmm_routed_tile_kernel(QmmArgs a) {
       const float shift1 = bf16_bits_to_f32(bias_bits >> 16) - 16.0f * scale1;
 #pragma unroll
       for (int j = 0; j < 16; ++j)
-        acc[pj][j] += scale0 * part[0][pj][j] + scale1 * part[1][pj][j];
+        acc[pj][j] = __builtin_fmaf(scale1, part[1][pj][j], __builtin_fmaf(scale0, part[0][pj][j], acc[pj][j]));
       acc[pj] = __builtin_amdgcn_mfma_f32_32x32x2f32(xsum[(group + h) * kRows + nl],
                                                      h ? shift1 : shift0, acc[pj], 0, 0, 0);
     }

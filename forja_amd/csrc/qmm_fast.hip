@@ -1038,7 +1038,7 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
   // Decode rows.  When one workgroup per compute unit covers the output, the single-kernel tile
   // product; wider outputs go through the K slabs.
   if (p.rows <= 128 &&
-      (uint64_t)((p.columns + 31) / 32) * ((p.rows + 31) / 32) <= backend_compute_units(backend)) {
+      (uint64_t)((p.columns + 31) / 32) * ((p.rows + 31) / 32) <= 3 * backend_compute_units(backend)) {
     launch_tile_product(backend, a, residual, residual_row_stride);
     return true;
   }

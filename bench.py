@@ -259,6 +259,28 @@ def prefill_layer_c4(backend, seed=95, repeats=2):
             "prefill_tok_per_s_64_layers": rows / (seconds * c.layers)}
 
 
+def packed_step_c1(backend, seed=97, repeats=3):
+    """BASELINE config 1: the whole Qwen3-0.6B-shaped model (28 layers, vocabulary 151936) over a
+    packed 2048-token batch of 48 decode rows (contexts uniform 128..4096) and prefill chunks of
+    256, 384, 512 and 848 tokens; logits and greedy tokens for every row.  Device time of the
+    step from the submission's events."""
+    from forja_amd.model import PackedStep
+    c = QWEN3_0_6B
+    rng = np.random.default_rng(seed)
+    contexts = [int(v) for v in rng.integers(128, 4097, 48)] + [0, 0, 0, 0]
+    counts = [1] * 48 + [256, 384, 512, 848]
+    model = Model(backend, c, seed=seed)
+    step = PackedStep(model, contexts, counts, seed=seed, head=True)
+    step.run()
+    nanoseconds = 0
+    for _ in range(repeats):
+        nanoseconds += step.run().gpu_time_ns()
+    seconds = nanoseconds / repeats * 1e-9
+    return {"workload": "BASELINE config 1: 28 layers, 48 decode rows + prefill chunks 256/384/512/848 "
+                        "packed into 2048 tokens, lm_head and argmax on every row",
+            "tokens": step.tokens, "ms_per_step": seconds * 1e3, "tok_per_s": step.tokens / seconds}
+
+
 def stream_read_rate(backend, rows=4096, width=1 << 20, repeats=3):
     """What a plain read-only stream sustains on this device: a row-wise argmax over 8 GiB of
     bf16 (16-byte loads, one workgroup per row).  The practical ceiling the HBM-bound kernels are
@@ -398,7 +420,8 @@ def main():
         print(json.dumps({"mfma_f16_sustained": mfma_sustained_rates(),
                           "prefill_gemm_c4": prefill_gemm_c4(backend),
                           "prefill_attention_c4": prefill_attention_c4(backend),
-                          "prefill_layer_c4": prefill_layer_c4(backend)}))
+                          "prefill_layer_c4": prefill_layer_c4(backend),
+                          "packed_step_c1": packed_step_c1(backend)}))
         return
     if args.gpus != 1:
         print("bench.py: this build runs the ragged forward step on ONE MI355X; collectives and "
@@ -545,7 +568,8 @@ def main():
                 gemm["roofline"]["achieved"] / sustained["random_tflops"])
         result["secondary_workloads"] = {"prefill_gemm_c4": gemm,
                                          "prefill_attention_c4": prefill_attention_c4(backend),
-                                         "prefill_layer_c4": prefill_layer_c4(backend)}
+                                         "prefill_layer_c4": prefill_layer_c4(backend),
+                                         "packed_step_c1": packed_step_c1(backend)}
         if config.moe:
             result["secondary_workloads"]["moe_block_c2"] = moe_block_c2(backend, workload.model)
     step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction

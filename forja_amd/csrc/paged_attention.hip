@@ -243,6 +243,9 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr uint32_t kMinSplitTokens = 128, kMaxSplitTokens = 1024;  // split length bounds
+// Groups of several query tokens (prefill) are many and each split of theirs costs a merge of
+// `members x heads` partial rows: they are split only beyond this many keys.
+constexpr uint32_t kPrefillSplitTokens = 2048;
 constexpr uint32_t kTargetItems = 1024;  // (token, split) items wanted per launch
 constexpr uint32_t kTile = 32;          // tokens per inner step
 
@@ -260,7 +263,8 @@ struct FastRagged {
   uint32_t *bad;       // [T]
   TokenPlan *plans;    // [T]
   uint2 *items;        // [T * S] (group leader token, split) of every live split, compacted
-  uint32_t *item_count;
+  uint32_t *item_count;   // [0] work items, [1] tokens the merge kernel has work for
+  uint32_t *merge_tokens; // [T] those tokens (several splits, or a zero row to write)
   uint64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h;
   uint32_t tokens, lanes, query_heads, kv_heads, group, page_tokens, physical_pages, table_pages,
       max_splits, split_tokens;
@@ -308,6 +312,7 @@ __device__ inline TokenPlan plan_token(const FastRagged &p, uint32_t token, uint
   plan.members = (uint32_t)(last - leader + 1);
   plan.attended = (uint32_t)attended;
   const uint32_t longest = (uint32_t)group_attended;
+  if (plan.members > 1 && split_tokens < kPrefillSplitTokens) split_tokens = kPrefillSplitTokens;
   uint32_t want = (longest + split_tokens - 1) / split_tokens;
   if (want > p.max_splits) want = p.max_splits;
   uint32_t chunk = (longest + want - 1) / want;
@@ -324,8 +329,12 @@ constexpr uint32_t kSizeClasses = 65;   // split length / 32, clamped
 __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlot *error) {
   __shared__ uint32_t class_items[kSizeClasses];   // items per class, then the class's cursor
   __shared__ unsigned long long total_attended;
+  __shared__ uint32_t merge_count;
   for (uint32_t c = threadIdx.x; c < kSizeClasses; c += 256) class_items[c] = 0;
-  if (threadIdx.x == 0) total_attended = 0;
+  if (threadIdx.x == 0) {
+    total_attended = 0;
+    merge_count = 0;
+  }
   __syncthreads();
   // Split length: long enough that a wave's fixed start-up cost (plan, table, query) is small
   // against its stream, short enough that the batch still yields ~kTargetItems work items.
@@ -357,6 +366,8 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
     p.bad[token] = bad;
     p.plans[token] = plan;
     if (plan.leader == token && plan.splits) atomicAdd(&class_items[class_of(plan)], plan.splits);
+    // tokens with a single split are finished by the attention kernel itself
+    if (plan.splits != 1 || bad) p.merge_tokens[atomicAdd(&merge_count, 1u)] = token;
   }
   __syncthreads();
   if (threadIdx.x == 0) {   // class counts -> first item of each class, longest class first
@@ -367,6 +378,7 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
       running += count;
     }
     p.item_count[0] = running;
+    p.item_count[1] = merge_count;
   }
   __syncthreads();
   for (uint32_t token = threadIdx.x; token < p.tokens; token += 256) {
@@ -384,6 +396,16 @@ __device__ inline uint32_t pack_bf16(float lo, float hi) {
 
 __device__ inline uint32_t dword_of(const uint4 &v, int index) {
   return index == 0 ? v.x : (index == 1 ? v.y : (index == 2 ? v.z : v.w));
+}
+
+// Zero output rows of `count` tokens from `first` for the query heads of one kv head (a wave's
+// duty when it refuses a page and no merge will follow: the token has a single split).
+__device__ inline void zero_head_rows(const FastRagged &p, uint32_t first, uint32_t count,
+                                      uint32_t kv_head, uint32_t lane) {
+  for (uint32_t member = 0; member < count; ++member)
+    for (uint32_t head = kv_head * p.group; head < (kv_head + 1) * p.group; ++head)
+      *(uint32_t *)(p.out + (uint64_t)(first + member) * p.out_stride_t + (uint64_t)head * p.out_stride_h +
+                    2 * lane) = 0;
 }
 
 struct TileRegs {
@@ -571,6 +593,7 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
         report_error(error, my_page);
         for (uint32_t member = 0; member < members; ++member) p.bad[leader + member] = 1;
       }
+      if (plan.splits == 1) zero_head_rows(p, leader, members, kv_head, lane);
       return;
     }
     const uint32_t tok_lo = max(begin, page0 * pt);
@@ -769,6 +792,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_
         report_error(error, my_page);
         for (uint32_t member = 0; member < plan.members; ++member) p.bad[leader + member] = 1;
       }
+      if (plan.splits == 1) zero_head_rows(p, leader + first, members, kv_head, lane);
       return;
     }
     const uint32_t tok_lo = max(begin, page0 * pt);
@@ -835,15 +859,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // lanes' four columns, all loads in flight at once, and the waves' sums meet in LDS.
 __global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
   __shared__ float4 folded[3][32];
-  const uint32_t token = blockIdx.y;
-  const TokenPlan plan = p.plans[token];
-  const bool zero = plan.splits == 0 || p.bad[token] != 0;
-  if (!zero && plan.splits == 1) return;
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t column = (lane & 31) * 4, half = lane >> 5;
-  // gridDim.x is the head count for decode batches and 1 for long prefill batches, where most
-  // tokens have a single split and leave at once
-  for (uint32_t head = blockIdx.x; head < p.query_heads; head += gridDim.x) {
+  const uint32_t head = blockIdx.x, listed = p.item_count[1];
+  // blockIdx.y walks the list of tokens that need the merge (the plan kernel compiled it; the
+  // bad-page flags an attention wave may have raised since are re-read here)
+  for (uint32_t entry = blockIdx.y; entry < listed; entry += gridDim.y) {
+    const uint32_t token = p.merge_tokens[entry];
+    const TokenPlan plan = p.plans[token];
+    const bool zero = plan.splits == 0 || p.bad[token] != 0;
     uint16_t *dst = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
     if (zero) {
       if (threadIdx.x < 32) *(uint2 *)dst = make_uint2(0, 0);
@@ -873,7 +897,7 @@ __global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
     acc.y += __shfl_xor(acc.y, 32, 64);
     acc.z += __shfl_xor(acc.z, 32, 64);
     acc.w += __shfl_xor(acc.w, 32, 64);
-    __syncthreads();   // the previous head's sums have been read
+    __syncthreads();   // the previous entry's sums have been read
     if (wave != 0 && half == 0) folded[wave - 1][lane] = acc;
     __syncthreads();
     if (threadIdx.x < 32) {
@@ -931,13 +955,15 @@ uint64_t round_256(uint64_t bytes) { return (bytes + 255) / 256 * 256; }
 // Flags, plans, work items and the item count: everything ragged_plan_kernel writes.
 uint64_t plan_storage_bytes(const FastRagged &f) {
   uint64_t slots = (uint64_t)f.tokens * f.max_splits;
-  return round_256((uint64_t)f.tokens * 4) + round_256((uint64_t)f.tokens * sizeof(TokenPlan)) +
+  return 2 * round_256((uint64_t)f.tokens * 4) + round_256((uint64_t)f.tokens * sizeof(TokenPlan)) +
          round_256(slots * sizeof(uint2)) + 256;
 }
 
 char *carve_plan(FastRagged *f, char *ws) {
   uint64_t slots = (uint64_t)f->tokens * f->max_splits;
   f->bad = (uint32_t *)ws;
+  ws += round_256((uint64_t)f->tokens * 4);
+  f->merge_tokens = (uint32_t *)ws;
   ws += round_256((uint64_t)f->tokens * 4);
   f->plans = (TokenPlan *)ws;
   ws += round_256((uint64_t)f->tokens * sizeof(TokenPlan));
@@ -986,7 +1012,7 @@ void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, E
                                      64 * waves, 0, stream>>>(f, error);
     }
   }
-  ragged_reduce_kernel<<<dim3(f.tokens <= 1024 ? f.query_heads : 1, f.tokens), 256, 0, stream>>>(f);
+  ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens < 1024 ? f.tokens : 1024), 256, 0, stream>>>(f);
 }
 
 }  // namespace

@@ -106,10 +106,13 @@ __device__ inline void split_f16(float v, float *head, float *tail) {
 // One wave per row.
 __global__ __launch_bounds__(256) void prepare_rows_kernel(const uint16_t *x, uint64_t x_row_stride,
                                                            uint32_t rows, uint32_t inner, uint32_t kt,
-                                                           uint16_t *out, float *unscale) {
+                                                           uint16_t *out, float *unscale,
+                                                           uint32_t *refused) {
   __shared__ float sums[4][kMaxGroups];
   const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint32_t row = blockIdx.x * 4 + wave;
+  // the refusal flag of this product starts clear (prepare_weights_kernel, launched next, sets it)
+  if (blockIdx.x == 0 && threadIdx.x == 0) refused[0] = 0;
   if (row >= rows) return;   // no workgroup-wide barrier below
   const uint16_t *in_row = x + (uint64_t)row * x_row_stride;
   uint32_t top = 0;   // largest magnitude bits (bf16 without sign) in the row
@@ -466,10 +469,9 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
     configured = true;
   }
   const uint32_t grid = (a.row_tiles * a.column_tiles + 255) / 256 * 256;
-  launch_fill_u32(stream, flag, 1, 0);
   prepare_rows_kernel<<<(p.rows + 3) / 4, 256, 0, stream>>>(
       (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, kt, (uint16_t *)ws,
-      (float *)(ws + a_bytes + b_bytes));
+      (float *)(ws + a_bytes + b_bytes), flag);
   const uint64_t weight_threads = (uint64_t)p.columns * (kt / 64) * 8;
   prepare_weights_kernel<<<(uint32_t)((weight_threads + 255) / 256), 256, 0, stream>>>(
       (const uint32_t *)p.packed.base + p.packed.offset,

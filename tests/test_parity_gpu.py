@@ -109,6 +109,27 @@ def test_seeded_fill_matches_the_host_generator_bit_for_bit(cpu, hip):
         assert cpu.read(a) == hip.read(b)
 
 
+def test_kernel_timers_follow_the_selected_classes(hip):
+    """fh_profile_select: only the selected kernel classes are timed (class 6 = the kernels of a
+    dense quantised product)."""
+    weights = Quantised(20, 1, (64, 256))
+    x = upload(hip, normal_bf16(20, 2, (8, 256)), DType.BF16)
+    out = hip.alloc(DType.BF16, (8, 64))
+    commands = CommandList()
+    commands.dispatch(Op.quant_matmul(4, 64), [x, *weights.upload(hip)], out)
+    try:
+        hip.profile_enable(1)
+        for mask, expected in ((1 << 4, 0), (1 << 6, 1), (0xffffffff, 1)):
+            hip.profile_select(mask)
+            hip.profile_reset()
+            run(hip, commands)
+            nanoseconds, launches = hip.profile_read(6)
+            assert launches == expected and (nanoseconds > 0) == (expected > 0)
+    finally:
+        hip.profile_select(0xffffffff)
+        hip.profile_enable(0)
+
+
 # ------------------------------------------------------------------ quantised matmul
 
 QMM_CASES = [

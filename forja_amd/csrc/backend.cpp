@@ -12,6 +12,7 @@
 #include <set>
 #include <thread>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "fast_kernels.hpp"
@@ -133,6 +134,31 @@ struct fh_backend {
   uint64_t ring_bytes = 0, ring_head = 0;
   uint64_t class_ns[FH_KC_COUNT] = {};
   uint64_t class_launches[FH_KC_COUNT] = {};
+
+  // Fusion of runs of per-lane attention dispatches: gathered lane metadata followed by the
+  // attended rows, kept between the layers of a step (every layer names the same lanes).
+  bool lane_fusion = true;
+  char *lane_scratch = nullptr;
+  uint64_t lane_scratch_bytes = 0;
+  bool lane_metadata_valid = false;
+  std::vector<uint64_t> lane_metadata_key;          // what the gathered metadata was built from
+  std::unordered_set<uint64_t> lane_metadata_watch; // allocations whose writes invalidate it
+  uint64_t fused_runs = 0, fused_dispatches = 0;
+  char *ensure_lane_scratch(uint64_t bytes) {
+    if (bytes <= lane_scratch_bytes) return lane_scratch;
+    (void)hipStreamSynchronize(stream);
+    if (lane_scratch) (void)hipFree(lane_scratch);
+    lane_scratch = nullptr;
+    lane_scratch_bytes = 0;
+    lane_metadata_valid = false;
+    attention_plan_valid = false;
+    uint64_t want = std::max<uint64_t>(bytes, 4ull << 20);
+    void *ptr = nullptr;
+    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
+    lane_scratch = (char *)ptr;
+    lane_scratch_bytes = want;
+    return lane_scratch;
+  }
 
   // f32 accumulators handed to an epilogue program; separate from `workspace` because the kernel
   // that fills them may carve its own scratch out of the workspace.
@@ -1115,6 +1141,276 @@ fh_status process(fh_backend *b, const fh_dispatch &d, ErrorSlot *error, bool ex
   }
 }
 
+// ---------------------------------------------------------------- fusion of per-lane attention
+//
+// The engines record a decode batch lane by lane (engines/qwen3-coder/src/lib.rs:917-935): for
+// every lane one Op::PagedSdpaAppend on narrowed rows of the packed q/k/v activations, with the
+// lane's own block-table allocation and a freshly allocated output row
+// (crates/forja-sdk/src/paged.rs:525-528), followed by the Op::Copy of that row into the packed
+// `attended` activation.  Executed one by one that is hundreds of tiny launches per layer.  A run
+// of such dispatches is recognised here and executed as: one gather of the lanes' metadata (kept
+// for the other layers of the submission), one ragged attention launch into scratch rows, one
+// scatter of the rows to the places the dispatches named.  The result is what serial execution
+// gives as long as no member reads what another member writes, which the checks below establish
+// from the tensors alone (allocation identities and element spans); a run that fails any check
+// is executed serially.  One thing is taken from the host rather than proved: a lane's appended
+// slot lies outside every other lane's attended range (pages are copy-on-write,
+// crates/forja-host/src/lib.rs:5408-5470), which also makes the key/value writes of different
+// members independent.
+
+struct LaneRun {
+  uint32_t items = 0;    // attention dispatches
+  uint32_t step = 1;     // dispatches per lane: 2 when each is followed by the copy of its row
+  int64_t delta[3] = {0, 0, 0};  // element distance between consecutive members' q, k_new, v_new
+};
+
+bool same_layout(const fh_tensor &a, const fh_tensor &b) {
+  if (a.dtype != b.dtype || a.rank != b.rank) return false;
+  for (uint32_t axis = 0; axis < a.rank; ++axis)
+    if (a.shape[axis] != b.shape[axis] || a.stride[axis] != b.stride[axis]) return false;
+  return true;
+}
+
+bool same_tensor(const fh_tensor &a, const fh_tensor &b) {
+  return a.buffer == b.buffer && a.offset == b.offset && same_layout(a, b);
+}
+
+// The [heads, 1, width] attention output as one dense row of heads * width elements.
+bool dense_head_rows(const fh_tensor &out) {
+  return out.rank == 3 && out.shape[1] == 1 && out.stride[2] == 1 && out.stride[0] == out.shape[2];
+}
+
+// `copy` moves exactly the row `attention` produced, unconverted, into a dense destination.
+bool copies_attended_row(const fh_dispatch &attention, const fh_dispatch &copy) {
+  if (copy.op != FH_OP_COPY || copy.n_inputs != 1 || copy.n_outputs != 1) return false;
+  const fh_tensor &row = attention.outputs[0], &in = copy.inputs[0], &out = copy.outputs[0];
+  return in.buffer == row.buffer && in.offset == row.offset && in.dtype == row.dtype &&
+         out.dtype == row.dtype && is_contiguous(in) && is_contiguous(out) &&
+         element_count(in) == (uint64_t)row.shape[0] * row.shape[2] &&
+         element_count(out) == element_count(in);
+}
+
+bool same_attention_shape(const fh_dispatch &a, const fh_dispatch &b) {
+  if (b.op != a.op || b.n_inputs != a.n_inputs || b.n_outputs != a.n_outputs) return false;
+  if (memcmp(&a.scale, &b.scale, sizeof(float)) != 0 || a.page_tokens != b.page_tokens) return false;
+  for (uint32_t i = 0; i < 3; ++i)
+    if (a.inputs[i].buffer != b.inputs[i].buffer || !same_layout(a.inputs[i], b.inputs[i])) return false;
+  if (!same_layout(a.inputs[3], b.inputs[3]) || !same_tensor(a.inputs[4], b.inputs[4])) return false;
+  if (a.n_inputs == 6 && !same_layout(a.inputs[5], b.inputs[5])) return false;
+  return same_layout(a.outputs[0], b.outputs[0]) && same_tensor(a.outputs[1], b.outputs[1]) &&
+         same_tensor(a.outputs[2], b.outputs[2]);
+}
+
+// Longest fusable run of per-lane attention dispatches starting at `first`; false when there is
+// none of at least two lanes.  `run` then still says how many dispatches were examined, so that
+// the caller does not examine the tail of a refused run again.
+bool find_lane_run(const fh_dispatch *d, uint32_t count, uint32_t first, LaneRun *run) {
+  const fh_dispatch &d0 = d[first];
+  *run = LaneRun{};
+  run->items = 1;
+  if (d0.op != FH_OP_PAGED_SDPA_APPEND || d0.n_outputs != 3 ||
+      (d0.n_inputs != 5 && d0.n_inputs != 6))
+    return false;
+  if (!dense_head_rows(d0.outputs[0]) || !is_contiguous(d0.inputs[3])) return false;
+  if (d0.n_inputs == 6 && element_count(d0.inputs[5]) != 1) return false;
+  LaneRun r;
+  r.step = first + 1 < count && copies_attended_row(d0, d[first + 1]) ? 2 : 1;
+  r.items = 1;
+  for (;;) {
+    uint64_t at = (uint64_t)first + (uint64_t)r.items * r.step;
+    if (at + r.step > count) break;
+    const fh_dispatch &m = d[at];
+    if (!same_attention_shape(d0, m)) break;
+    if (r.step == 2 && !(copies_attended_row(m, d[at + 1]) &&
+                         same_layout(d[first + 1].outputs[0], d[at + 1].outputs[0])))
+      break;
+    bool regular = true;
+    for (uint32_t i = 0; i < 3; ++i) {
+      int64_t distance = (int64_t)m.inputs[i].offset - (int64_t)d0.inputs[i].offset;
+      if (r.items == 1) {
+        if (distance <= 0) regular = false;
+        r.delta[i] = distance;
+      } else if (distance != r.delta[i] * (int64_t)r.items) {
+        regular = false;
+      }
+    }
+    if (!regular) break;
+    ++r.items;
+  }
+  *run = r;
+  if (r.items < 2) return false;
+  // Nothing a member writes may be something another member reads or writes.
+  std::unordered_set<uint64_t> read;
+  for (uint32_t i = 0; i < 3; ++i) read.insert(d0.inputs[i].buffer);
+  read.insert(d0.inputs[4].buffer);
+  read.insert(d0.outputs[1].buffer);
+  read.insert(d0.outputs[2].buffer);
+  struct Span {
+    uint64_t buffer, lo, hi;
+  };
+  std::vector<Span> written;
+  written.reserve((size_t)r.items * r.step);
+  for (uint32_t item = 0; item < r.items; ++item) {
+    const fh_dispatch &m = d[first + item * r.step];
+    read.insert(m.inputs[3].buffer);
+    if (m.n_inputs == 6) read.insert(m.inputs[5].buffer);
+    uint64_t row = (uint64_t)m.outputs[0].shape[0] * m.outputs[0].shape[2];
+    written.push_back({m.outputs[0].buffer, m.outputs[0].offset, m.outputs[0].offset + row});
+    if (r.step == 2) {
+      const fh_tensor &target = d[first + item * r.step + 1].outputs[0];
+      written.push_back({target.buffer, target.offset, target.offset + row});
+    }
+  }
+  for (const Span &span : written)
+    if (read.count(span.buffer)) return false;
+  std::sort(written.begin(), written.end(), [](const Span &a, const Span &b) {
+    return a.buffer != b.buffer ? a.buffer < b.buffer : a.lo < b.lo;
+  });
+  for (size_t i = 1; i < written.size(); ++i)
+    if (written[i].buffer == written[i - 1].buffer && written[i].lo < written[i - 1].hi) return false;
+  return true;
+}
+
+// Executes the run found by find_lane_run.  `errors` is the first member's record; member i's is
+// errors[i * run.step].
+fh_status run_lane_group(fh_backend *b, const fh_dispatch *d, uint32_t first, const LaneRun &run,
+                         ErrorSlot *errors) {
+  const fh_dispatch &d0 = d[first];
+  const fh_tensor &q0 = d0.inputs[0], &out0 = d0.outputs[0], &kp = d0.outputs[1],
+                  &vp = d0.outputs[2], &table0 = d0.inputs[3];
+  const uint32_t lanes = run.items, heads = q0.shape[0];
+  const uint32_t table_pages = table0.shape[0], table_words = table_pages * 2;
+  const uint64_t row_bytes = (uint64_t)heads * out0.shape[2] * dtype_size(out0.dtype);
+  FH_REQUIRE(row_bytes < (1ull << 31));
+  const uint64_t metadata_words = (uint64_t)lanes * table_words + 3ull * lanes + 1;
+  const uint64_t rows_at = (metadata_words * 4 + 255) / 256 * 256;
+  char *scratch = b->ensure_lane_scratch(rows_at + lanes * row_bytes);
+  if (!scratch) return FH_ALLOCATION_FAILED;
+  uint32_t *tables = (uint32_t *)scratch;
+  uint32_t *activity = tables + (uint64_t)lanes * table_words;
+  uint32_t *starts = activity + lanes;
+  uint32_t *cu = starts + lanes;
+  char *rows = scratch + rows_at;
+
+  // What the gathered metadata depends on; equal keys mean the gather of an earlier layer holds.
+  std::vector<uint64_t> key;
+  key.reserve(5ull * lanes + 2);
+  key.push_back(lanes);
+  key.push_back(table_words);
+  for (uint32_t item = 0; item < lanes; ++item) {
+    const fh_dispatch &m = d[first + item * run.step];
+    key.push_back(m.inputs[3].buffer);
+    key.push_back(m.inputs[3].offset);
+    key.push_back(m.n_inputs == 6 ? m.inputs[5].buffer : 0);
+    key.push_back(m.n_inputs == 6 ? m.inputs[5].offset : 0);
+    key.push_back(m.q_start);
+  }
+  if (!(b->lane_metadata_valid && key == b->lane_metadata_key)) {
+    b->lane_metadata_valid = false;
+    b->attention_plan_valid = false;  // the plan was built from the metadata replaced here
+    b->lane_metadata_watch.clear();
+    for (uint32_t base = 0; base < lanes; base += kLaneChunk) {
+      uint32_t chunk = std::min<uint32_t>(kLaneChunk, lanes - base);
+      LaneSources sources{};
+      for (uint32_t local = 0; local < chunk; ++local) {
+        const fh_dispatch &m = d[first + (base + local) * run.step];
+        View table, flag;
+        fh_status status = make_view(b, m.inputs[3], false, &table);
+        if (status != FH_OK) return status;
+        sources.table[local] = (const uint32_t *)table.base + table.offset;
+        b->lane_metadata_watch.insert(m.inputs[3].buffer);
+        if (m.n_inputs == 6) {
+          status = make_view(b, m.inputs[5], false, &flag);
+          if (status != FH_OK) return status;
+          sources.activity[local] = (const uint32_t *)flag.base + flag.offset;
+          b->lane_metadata_watch.insert(m.inputs[5].buffer);
+        }
+        sources.start[local] = m.q_start;
+      }
+      launch_gather_lane_metadata(b->stream, sources, base, chunk, lanes, table_words, tables,
+                                  activity, starts, cu);
+    }
+    b->lane_metadata_key = std::move(key);
+    b->lane_metadata_valid = true;
+  }
+
+  auto device_view = [](char *base, uint32_t dtype, std::initializer_list<uint32_t> shape) {
+    View v{};
+    v.base = base;
+    v.dtype = dtype;
+    v.rank = (uint32_t)shape.size();
+    for (uint32_t axis = 0; axis < FH_MAX_RANK; ++axis) {
+      v.shape[axis] = 1;
+      v.stride[axis] = 0;
+    }
+    uint32_t axis = 0;
+    for (uint32_t extent : shape) v.shape[axis++] = extent;
+    uint64_t stride = 1;
+    for (int at = (int)v.rank - 1; at >= 0; --at) {
+      v.stride[at] = stride;
+      stride *= v.shape[at];
+    }
+    return v;
+  };
+  RaggedAttention problem{};
+  // q [heads, 1, D] per member -> [lanes, heads, D]; k_new / v_new [1, Hkv, D] -> [lanes, Hkv, D].
+  fh_status status = make_view(b, q0, false, &problem.q);
+  if (status != FH_OK) return status;
+  problem.q.shape[0] = lanes;
+  problem.q.shape[1] = heads;
+  problem.q.stride[0] = (uint64_t)run.delta[0];
+  problem.q.stride[1] = q0.stride[0];
+  View *appended[2] = {&problem.k_new, &problem.v_new};
+  for (uint32_t i = 0; i < 2; ++i) {
+    status = make_view(b, d0.inputs[1 + i], false, appended[i]);
+    if (status != FH_OK) return status;
+    appended[i]->shape[0] = lanes;
+    appended[i]->stride[0] = (uint64_t)run.delta[1 + i];
+  }
+  if ((status = make_view(b, d0.inputs[4], false, &problem.generations)) != FH_OK) return status;
+  if ((status = make_view(b, kp, true, &problem.key_pool)) != FH_OK) return status;
+  if ((status = make_view(b, vp, true, &problem.value_pool)) != FH_OK) return status;
+  problem.tables = device_view((char *)tables, FH_U32, {lanes, table_pages, 2});
+  problem.activity = device_view((char *)activity, FH_U32, {lanes});
+  problem.q_starts = device_view((char *)starts, FH_U32, {lanes});
+  problem.cu_seqlens = device_view((char *)cu, FH_U32, {lanes + 1});
+  problem.out = device_view(rows, out0.dtype, {lanes, heads, out0.shape[2]});
+  problem.tokens = lanes;
+  problem.lanes = lanes;
+  problem.query_heads = heads;
+  problem.kv_heads = kp.shape[2];
+  problem.width = q0.shape[2];
+  problem.value_width = vp.shape[3];
+  problem.page_tokens = d0.page_tokens;
+  problem.physical_pages = kp.shape[0];
+  problem.table_pages = table_pages;
+  problem.scale = d0.scale;
+  problem.metadata_buffers[4] = d0.inputs[4].buffer;  // the rest is watched through the gather
+  problem.error_stride = run.step;
+  // The last query row of a member sits at q_start; serial execution refuses a start at the
+  // sentinel before anything runs, and validation has done the same here.
+  if (!run_ragged_attention(b, problem, errors)) return FH_ALLOCATION_FAILED;
+
+  for (uint32_t base = 0; base < lanes; base += kLaneChunk) {
+    uint32_t chunk = std::min<uint32_t>(kLaneChunk, lanes - base);
+    LaneRows targets{};
+    for (uint32_t local = 0; local < chunk; ++local) {
+      uint32_t at = first + (base + local) * run.step;
+      View row;
+      if ((status = make_view(b, d[at].outputs[0], true, &row)) != FH_OK) return status;
+      targets.first[local] = row.base + row.offset * dtype_size(row.dtype);
+      if (run.step == 2) {
+        if ((status = make_view(b, d[at + 1].outputs[0], true, &row)) != FH_OK) return status;
+        targets.second[local] = row.base + row.offset * dtype_size(row.dtype);
+      }
+    }
+    launch_scatter_lane_rows(b->stream, targets, rows, base, chunk, (uint32_t)row_bytes);
+  }
+  b->fused_runs += 1;
+  b->fused_dispatches += (uint64_t)run.items * run.step;
+  return FH_OK;
+}
+
 hipEvent_t take_event(fh_backend *b) {
   if (!b->event_pool.empty()) {
     hipEvent_t e = b->event_pool.back();
@@ -1204,6 +1500,7 @@ void fh_destroy(fh_backend *b) {
       for (auto &typed : entry.second.typed) (void)hipFree(typed.second);
     if (b->workspace) (void)hipFree(b->workspace);
     if (b->accumulators) (void)hipFree(b->accumulators);
+    if (b->lane_scratch) (void)hipFree(b->lane_scratch);
     if (b->route_plan) (void)hipFree(b->route_plan);
     if (b->attention_plan) (void)hipFree(b->attention_plan);
     for (auto &e : b->error_pool) {
@@ -1495,28 +1792,47 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   b->attention_plan_valid = false;
   launch_init_errors(b->stream, s->device_errors, slots);
   (void)hipEventRecord(s->start, b->stream);
+  b->lane_metadata_valid = false;
+  // Plans and gathered metadata kept between dispatches die when a dispatch writes their source.
+  auto note_outputs = [b](const fh_dispatch &d) {
+    for (uint32_t o = 0; o < d.n_outputs && o < FH_MAX_OUTPUTS; ++o) {
+      uint64_t written = d.outputs[o].buffer;
+      if (b->route_plan_valid && written == b->route_plan_key.buffer) b->route_plan_valid = false;
+      if (b->attention_plan_valid)
+        for (uint64_t watched : b->attention_plan_key.buffers)
+          if (watched != 0 && written == watched) b->attention_plan_valid = false;
+      if (b->lane_metadata_valid && b->lane_metadata_watch.count(written))
+        b->lane_metadata_valid = false;
+    }
+  };
   fh_status status = FH_OK;
-  for (uint32_t i = 0; i < count && status == FH_OK; ++i) {
-    s->ops[i] = dispatches[i].op;
+  uint32_t no_run_before = 0;  // dispatches already examined as part of a run that was refused
+  for (uint32_t i = 0; i < count && status == FH_OK;) {
+    uint32_t consumed = 1;
+    LaneRun run;
+    bool fused = b->lane_fusion && dispatches[i].op == FH_OP_PAGED_SDPA_APPEND &&
+                 i >= no_run_before && find_lane_run(dispatches, count, i, &run);
+    if (fused)
+      consumed = run.items * run.step;
+    else if (run.items > 1)
+      no_run_before = i + run.items * run.step;
+    for (uint32_t member = 0; member < consumed; ++member) s->ops[i + member] = dispatches[i + member].op;
     hipEvent_t t0 = nullptr, t1 = nullptr;
     if (b->profiling >= 2) {
       t0 = take_event(b);
       t1 = take_event(b);
       (void)hipEventRecord(t0, b->stream);
     }
-    status = process(b, dispatches[i], &s->device_errors[i], true);
-    if (b->route_plan_valid)
-      for (uint32_t o = 0; o < dispatches[i].n_outputs && o < FH_MAX_OUTPUTS; ++o)
-        if (dispatches[i].outputs[o].buffer == b->route_plan_key.buffer) b->route_plan_valid = false;
-    if (b->attention_plan_valid)
-      for (uint32_t o = 0; o < dispatches[i].n_outputs && o < FH_MAX_OUTPUTS; ++o)
-        for (uint64_t watched : b->attention_plan_key.buffers)
-          if (watched != 0 && dispatches[i].outputs[o].buffer == watched)
-            b->attention_plan_valid = false;
+    if (fused)
+      status = run_lane_group(b, dispatches, i, run, &s->device_errors[i]);
+    else
+      status = process(b, dispatches[i], &s->device_errors[i], true);
+    for (uint32_t member = 0; member < consumed; ++member) note_outputs(dispatches[i + member]);
     if (b->profiling >= 2) {
       (void)hipEventRecord(t1, b->stream);
       b->timed.push_back({t0, t1, kernel_class_of(dispatches[i].op)});
     }
+    i += consumed;
   }
   (void)hipEventRecord(s->end, b->stream);
   (void)hipMemcpyAsync(s->host_errors, s->device_errors, slots * sizeof(ErrorSlot),
@@ -1678,6 +1994,21 @@ fh_status fh_profile_select(fh_backend *b, uint32_t class_mask) {
   (void)hipStreamSynchronize(b->stream);
   drain_profile(b);
   b->profile_mask = class_mask;
+  return FH_OK;
+}
+
+fh_status fh_fusion_enable(fh_backend *b, int enabled) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  b->lane_fusion = enabled != 0;
+  return FH_OK;
+}
+
+fh_status fh_fusion_stats(fh_backend *b, uint64_t *runs, uint64_t *dispatches) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  if (runs) *runs = b->fused_runs;
+  if (dispatches) *dispatches = b->fused_dispatches;
   return FH_OK;
 }
 

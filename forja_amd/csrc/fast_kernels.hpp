@@ -98,6 +98,9 @@ struct RaggedAttention {
   float scale;
   // allocation identities of cu_seqlens, q_starts, activity, tables, generations (0: none)
   uint64_t metadata_buffers[5];
+  // A failure of query token t is recorded in error[t * error_stride]: 0 for one dispatch, the
+  // distance between the member dispatches' records when a run of per-lane dispatches is fused.
+  uint32_t error_stride;
 };
 // Always handles the problem (specialised kernel when the layout allows, generic otherwise);
 // false only when workspace allocation fails.

@@ -91,4 +91,27 @@ void launch_route_pack(hipStream_t s, const View &indices, uint32_t rows, uint32
                        uint32_t *n_blocks, ErrorSlot *error, uint32_t *zero_rows = nullptr,
                        uint32_t zero_row_words = 0);
 
+
+// ---- lane_fusion.hip: glue for a run of per-lane attention dispatches executed as one launch ----
+// Addresses of up to kLaneChunk lanes, passed by value as kernel arguments.
+constexpr uint32_t kLaneChunk = 128;
+struct LaneSources {
+  const uint32_t *table[kLaneChunk];     // the lane's block table, `table_words` words
+  const uint32_t *activity[kLaneChunk];  // the lane's activity word; null: always active
+  uint32_t start[kLaneChunk];            // position of the lane's query row
+};
+struct LaneRows {
+  void *first[kLaneChunk];   // where the lane's attended row goes
+  void *second[kLaneChunk];  // a second copy of it, or null
+};
+// Lanes [first, first + count) of `lanes`: tables [lanes, table_words], activity/starts [lanes],
+// cu [lanes + 1] (one query row per lane).
+void launch_gather_lane_metadata(hipStream_t s, const LaneSources &sources, uint32_t first,
+                                 uint32_t count, uint32_t lanes, uint32_t table_words,
+                                 uint32_t *tables, uint32_t *activity, uint32_t *starts,
+                                 uint32_t *cu);
+// rows: [lanes, row_bytes] contiguous.
+void launch_scatter_lane_rows(hipStream_t s, const LaneRows &targets, const void *rows,
+                              uint32_t first, uint32_t count, uint32_t row_bytes);
+
 }  // namespace fh

@@ -69,7 +69,7 @@ __global__ void ragged_append_kernel(RaggedAttention p, ErrorSlot *error) {
   if (logical_page >= p.table_pages ||
       !entry_ok(table, generations, (uint32_t)logical_page, p.table_pages, p.physical_pages,
                 &physical)) {
-    if (element == 0) report_error(error, logical_page > 0xffffffffull ? 0xffffffffu
+    if (element == 0) report_error(error + (uint64_t)token * p.error_stride, logical_page > 0xffffffffull ? 0xffffffffu
                                                                        : (uint32_t)logical_page);
     return;
   }
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void ragged_append_pieces_kernel(RaggedAttenti
   if (logical_page >= p.table_pages ||
       !entry_ok(table, generations, (uint32_t)logical_page, p.table_pages, p.physical_pages,
                 &physical)) {
-    if (piece == 0) report_error(error, logical_page > 0xffffffffull ? 0xffffffffu
+    if (piece == 0) report_error(error + (uint64_t)token * p.error_stride, logical_page > 0xffffffffull ? 0xffffffffu
                                                                      : (uint32_t)logical_page);
     return;
   }
@@ -165,7 +165,7 @@ __global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *er
   uint64_t pages = (attended64 + p.page_tokens - 1) / p.page_tokens;
   if (pages > p.table_pages) {
     if (lane_id == 0) {
-      report_error(error, p.table_pages);
+      report_error(error + (uint64_t)token * p.error_stride, p.table_pages);
       bad = 1;
     }
     pages = p.table_pages;
@@ -173,7 +173,7 @@ __global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *er
   for (uint32_t page = lane_id; page < pages; page += 64) {
     uint32_t physical;
     if (!entry_ok(table, generations, page, p.table_pages, p.physical_pages, &physical)) {
-      report_error(error, page);
+      report_error(error + (uint64_t)token * p.error_stride, page);
       bad = 1;
     }
   }
@@ -277,6 +277,7 @@ struct FastRagged {
   // to lane 0 whose first query sits at `one_start`; `fixed_attended` != 0 disables the causal
   // limit (every row attends exactly that many keys).
   uint32_t one_start, fixed_attended;
+  uint32_t error_stride;  // failures of token t go to error[t * error_stride]
 };
 
 // Work decomposition of one token.  Tokens of a lane are grouped `group_tokens` at a time; a
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
     TokenPlan plan = plan_token(p, token, split_tokens);
     uint32_t bad = 0;
     if (plan.lane == 0xffffffffu) {
-      report_error(error, p.table_pages);
+      report_error(error + (uint64_t)token * p.error_stride, p.table_pages);
       bad = 1;
       plan.lane = 0;
     }
@@ -590,7 +591,7 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
     unsigned long long bad_mask = __ballot(mine && !ok);
     if (bad_mask) {
       if (lane == (uint32_t)__ffsll((long long)bad_mask) - 1) {
-        report_error(error, my_page);
+        report_error(error + (uint64_t)leader * p.error_stride, my_page);
         for (uint32_t member = 0; member < members; ++member) p.bad[leader + member] = 1;
       }
       if (plan.splits == 1) zero_head_rows(p, leader, members, kv_head, lane);
@@ -789,7 +790,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_
     unsigned long long bad_mask = __ballot(mine && !ok);
     if (bad_mask) {
       if (wave == 0 && lane == (uint32_t)__ffsll((long long)bad_mask) - 1) {
-        report_error(error, my_page);
+        report_error(error + (uint64_t)leader * p.error_stride, my_page);
         for (uint32_t member = 0; member < plan.members; ++member) p.bad[leader + member] = 1;
       }
       if (plan.splits == 1) zero_head_rows(p, leader + first, members, kv_head, lane);
@@ -1079,6 +1080,7 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     f.physical_pages = p.physical_pages;
     f.table_pages = p.table_pages;
     f.max_splits = splits_for(p.tokens);
+    f.error_stride = p.error_stride;
     f.scale_log2 = p.scale * 1.4426950408889634f;
     f.tables = (const uint32_t *)p.tables.base + p.tables.offset;
     f.generations = (const uint32_t *)p.generations.base + p.generations.offset;

@@ -10,6 +10,8 @@ import ctypes as C
 import os
 from typing import List, Optional, Sequence
 
+import numpy as np
+
 from .core import (BackendError, CommandList, DType, Dispatch, Layout, Program, Slice, Status,
                    Tensor)
 
@@ -59,7 +61,7 @@ EXPORTS = [
     "fh_read_tensor", "fh_prepare_program", "fh_release_program", "fh_submit", "fh_wait",
     "fh_gpu_time_ns", "fh_submission_free", "fh_device_info_get", "fh_memory_usage",
     "fh_synchronize", "fh_profile_enable", "fh_profile_select", "fh_profile_reset", "fh_profile_read",
-    "fh_version",
+    "fh_fusion_enable", "fh_fusion_stats", "fh_version",
 ]
 
 _lib = None
@@ -100,6 +102,8 @@ def load_library():
     lib.fh_profile_reset.argtypes = [vp]
     lib.fh_profile_select.argtypes = [vp, u32]
     lib.fh_profile_read.argtypes = [vp, u32, C.POINTER(u64), C.POINTER(u64)]
+    lib.fh_fusion_enable.argtypes = [vp, C.c_int]
+    lib.fh_fusion_stats.argtypes = [vp, C.POINTER(u64), C.POINTER(u64)]
     lib.fh_version.restype = C.c_char_p
     _lib = lib
     return lib
@@ -290,6 +294,14 @@ class HipBackend:
         for i, t in enumerate(d.outputs):
             to_fh_tensor(t, out.outputs[i])
 
+    @staticmethod
+    def patch_query_starts(encoded: EncodedCommands, dispatch_indices, starts):
+        """Rewrites the q_start attribute of the named dispatches of an encoded list in place."""
+        raw = np.frombuffer(encoded.array, dtype=np.uint8).reshape(-1, C.sizeof(FhDispatch))
+        at = FhDispatch.q_start.offset
+        field = raw[:, at:at + 4].view(np.uint32)
+        field[np.asarray(dispatch_indices), 0] = np.asarray(starts, dtype=np.uint32)
+
     def submit(self, commands) -> HipSubmission:
         encoded = commands if isinstance(commands, EncodedCommands) else self.encode(commands)
         handle = C.c_void_p()
@@ -319,6 +331,16 @@ class HipBackend:
     def profile_select(self, class_mask: int):
         """Kernel classes (bit i = class i) the kernel-level timers cover; all by default."""
         _check(self._lib.fh_profile_select(self._handle, int(class_mask) & 0xffffffff))
+
+    def fusion_enable(self, enabled: bool):
+        """Whether runs of per-lane attention dispatches are executed as one ragged launch."""
+        _check(self._lib.fh_fusion_enable(self._handle, 1 if enabled else 0))
+
+    def fusion_stats(self):
+        """(runs fused, dispatches they replaced) since the backend was created."""
+        runs, dispatches = C.c_uint64(), C.c_uint64()
+        _check(self._lib.fh_fusion_stats(self._handle, C.byref(runs), C.byref(dispatches)))
+        return runs.value, dispatches.value
 
     def profile_reset(self):
         _check(self._lib.fh_profile_reset(self._handle))

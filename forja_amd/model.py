@@ -260,11 +260,18 @@ class StepBuffers:
 
 def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: CommandList,
                 feed_back: bool = False, route_trace: Optional[Tensor] = None,
-                head: bool = True) -> None:
+                head: bool = True, lane_starts=None, lane_sites: Optional[list] = None) -> None:
     """Appends one forward step over the packed batch to `commands`.  With `feed_back` the greedy
     tokens are copied into the id buffer for the next step (device to device).  `route_trace`
     (u32 [layers, tokens, top_k]) receives a copy of every layer's expert choices, for
-    diagnostics.  Without `head` the step stops after the last layer's norm (no lm_head)."""
+    diagnostics.  Without `head` the step stops after the last layer's norm (no lm_head).
+
+    With `lane_starts` (one cached-token count per lane, one query row per lane) attention is
+    recorded the way the engines record a decode batch (engines/qwen3-coder/src/lib.rs:917-935):
+    per lane one Op::PagedSdpaAppend on the lane's rows of q/k/v with the lane's table and a row of
+    its own for the result, followed by the Op::Copy of that row into the packed activation.  The
+    start is an attribute of the op; `lane_sites` receives (dispatch index, lane) of every such
+    dispatch so that a replay can patch it."""
     c, b = model.config, buffers
     tokens = b.tokens
     heads = c.q_heads + c.kv_heads
@@ -298,9 +305,25 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
             [qk_in.narrow(2, 0, half), qk_in.narrow(2, half, half), qk_weight.narrow(2, 0, half),
              qk_weight.narrow(2, half, half), positions],
             [b.qk.narrow(2, 0, half), b.qk.narrow(2, half, half)])
-        commands.dispatch_many(Op.paged_attention_ragged(scale, c.page_tokens),
-                               [q, k_new, v_new, *attention_inputs_tail],
-                               [b.attended, cache.keys[index], cache.values[index]])
+        if lane_starts is None:
+            commands.dispatch_many(Op.paged_attention_ragged(scale, c.page_tokens),
+                                   [q, k_new, v_new, *attention_inputs_tail],
+                                   [b.attended, cache.keys[index], cache.values[index]])
+        else:
+            table_pages = cache.tables.shape[1]
+            for lane in range(tokens):
+                row = b.lane_rows.narrow(0, lane, 1)
+                if lane_sites is not None:
+                    lane_sites.append((len(commands), lane))
+                commands.dispatch_many(
+                    Op.paged_sdpa_append(scale, int(lane_starts[lane]), c.page_tokens),
+                    [q.narrow(0, lane, 1).permute([1, 0, 2]), k_new.narrow(0, lane, 1),
+                     v_new.narrow(0, lane, 1),
+                     cache.tables.narrow(0, lane, 1).reshape((table_pages, 2)), cache.generations,
+                     b.activity.narrow(0, lane, 1)],
+                    [row.permute([1, 0, 2]), cache.keys[index], cache.values[index]])
+                commands.dispatch(Op.copy(), [row.reshape((1, c.q_heads * c.head_dim))],
+                                  b.attended.narrow(0, lane, 1).reshape((1, c.q_heads * c.head_dim)))
         commands.dispatch(q4, [b.attended.reshape((tokens, c.q_heads * c.head_dim)),
                                *layer.o_proj.triple], b.projected)
         commands.dispatch_kernel(model.residual_norm,
@@ -347,7 +370,7 @@ class DecodeSession:
 
     def __init__(self, model: Model, contexts, seed: int = 7, headroom_tokens: int = 64,
                  physical_pages: Optional[int] = None, table_pages: Optional[int] = None,
-                 fill_pools: bool = True):
+                 fill_pools: bool = True, lane_by_lane: bool = False):
         c = model.config
         backend = model.backend
         self.model = model
@@ -377,6 +400,40 @@ class DecodeSession:
         self.commands = commands
         self.encoded = backend.encode(commands) if hasattr(backend, "encode") else commands
         self.dispatches = len(commands)
+        self.lane_commands = self.lane_encoded = None
+        if lane_by_lane:
+            self.record_lane_by_lane()
+
+    def record_lane_by_lane(self):
+        """Records the same step lane by lane, as the engines record it, on the same storage."""
+        if self.lane_encoded is not None:
+            return
+        c, b, backend = self.model.config, self.buffers, self.model.backend
+        b.lane_rows = backend.alloc(DType.BF16, (len(self.contexts), c.q_heads, c.head_dim))
+        self.lane_sites = []
+        self.lane_commands = CommandList()
+        record_step(self.model, self.cache, b, self.lane_commands, feed_back=True,
+                    lane_starts=self.contexts, lane_sites=self.lane_sites)
+        self.lane_encoded = backend.encode(self.lane_commands) if hasattr(backend, "encode") \
+            else self.lane_commands
+        self._site_index = np.array([site for site, _ in self.lane_sites])
+        self._site_lane = np.array([lane for _, lane in self.lane_sites])
+
+    def submit_lane_step(self):
+        """Like submit_step, through the lane-by-lane recording: the query starts are attributes of
+        the per-lane dispatches, patched into the encoded list before it is submitted."""
+        self.prepare_step()
+        backend = self.model.backend
+        if hasattr(backend, "patch_query_starts"):
+            backend.patch_query_starts(self.lane_encoded, self._site_index,
+                                       self.contexts[self._site_lane])
+        else:   # a backend without an encoded form: record the step again with this step's starts
+            self.lane_encoded = CommandList()
+            record_step(self.model, self.cache, self.buffers, self.lane_encoded, feed_back=True,
+                        lane_starts=self.contexts)
+        submission = backend.submit(self.lane_encoded)
+        self.contexts += 1
+        return submission
 
     def upload_positions(self):
         b, backend = self.buffers, self.model.backend
@@ -402,8 +459,8 @@ class DecodeSession:
         self.contexts += 1
         return submission
 
-    def step(self) -> np.ndarray:
-        submission = self.submit_step()
+    def step(self, lane_by_lane: bool = False) -> np.ndarray:
+        submission = self.submit_lane_step() if lane_by_lane else self.submit_step()
         submission.wait()
         raw = self.model.backend.read(self.buffers.next_tokens)
         return np.frombuffer(raw, dtype=np.uint32).copy()

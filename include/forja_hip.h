@@ -223,6 +223,17 @@ FH_API fh_status fh_profile_reset(fh_backend *backend);
 FH_API fh_status fh_profile_read(fh_backend *backend, uint32_t kernel_class, uint64_t *nanoseconds,
                           uint64_t *launches);
 
+/* Fusion of per-lane attention dispatches.  The engines record a decode batch as one
+ * Op::PagedSdpaAppend per lane and layer, each followed by the Op::Copy of its output row into the
+ * packed activation (engines/qwen3-coder/src/lib.rs:917-935).  fh_submit recognises such a run and
+ * executes it as one ragged attention launch with the result serial execution gives; a run it
+ * cannot prove independent is executed dispatch by dispatch.  On by default.  The Backend trait
+ * has no switch for this (the Metal backend fuses in its encoder,
+ * crates/forja-metal/src/encoding.rs): these two calls exist for tests and measurements.
+ * fh_fusion_stats reports the runs fused and the dispatches they replaced since creation. */
+FH_API fh_status fh_fusion_enable(fh_backend *backend, int enabled);
+FH_API fh_status fh_fusion_stats(fh_backend *backend, uint64_t *runs, uint64_t *dispatches);
+
 FH_API const char *fh_version(void);
 
 #ifdef __cplusplus

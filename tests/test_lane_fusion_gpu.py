@@ -1,0 +1,207 @@
+"""A decode batch recorded the way the engines record it (engines/qwen3-coder/src/lib.rs:917-935):
+per lane one Op::PagedSdpaAppend on narrowed rows of the packed q/k/v, with the lane's own table
+allocation (crates/forja-host/src/lib.rs:4466-4480) and a fresh output row
+(crates/forja-sdk/src/paged.rs:525-528), each followed by the Op::Copy of that row into the packed
+activation.  The library executes such a run as one ragged launch; these tests hold the result to
+the CPU oracle's serial execution and to the library's own dispatch-by-dispatch execution."""
+import math
+
+import numpy as np
+import pytest
+
+from forja_amd.core import BackendError, CommandList, DType, Op, Status
+from oracle import cpu_backend as orc
+from tests.helpers import assert_close, normal_bf16, to_f32, upload
+
+pytestmark = pytest.mark.gpu
+
+WIDTH = 128
+
+
+def run(backend, commands):
+    backend.submit(commands).wait()
+
+
+class LaneBatch:
+    """Storage of a decode batch: packed q/k/v rows, one table allocation per lane, shared
+    generations and activity, `layers` pairs of pools."""
+
+    def __init__(self, backend, contexts, hq, hkv, pt, seed, layers=1, activity=None, corrupt=None,
+                 dtype=DType.BF16):
+        self.backend, self.contexts, self.hq, self.hkv, self.pt = backend, list(contexts), hq, hkv, pt
+        lanes = len(contexts)
+        pages_needed = [(c + 1 + pt - 1) // pt for c in contexts]
+        self.table_pages = max(pages_needed) + 2
+        physical = sum(pages_needed) + 3
+        rng = np.random.default_rng(seed)
+        free = list(rng.permutation(physical))
+        self.tables, self.host_tables = [], []
+        for lane, need in enumerate(pages_needed):
+            table = np.zeros((self.table_pages, 2), np.uint32)
+            table[:, 1] = 0xffffffff
+            for logical in range(need):
+                page = free.pop()
+                table[logical] = (page, 11 + page)
+            if corrupt is not None and corrupt[0] == lane:
+                table[corrupt[1], 1] += 1
+            self.tables.append(upload(backend, table, DType.U32))
+            self.host_tables.append(table)
+        self.spare_pages = free
+        self.generations = upload(backend, 11 + np.arange(physical), DType.U32)
+        self.activity = None if activity is None else upload(backend, np.array(activity), DType.U32)
+        self.q = upload(backend, normal_bf16(seed, 3, (lanes, hq, WIDTH)), dtype)
+        self.k = upload(backend, normal_bf16(seed, 4, (lanes, hkv, WIDTH)), dtype)
+        self.v = upload(backend, normal_bf16(seed, 5, (lanes, hkv, WIDTH)), dtype)
+        self.pools = []
+        for layer in range(layers):
+            keys = upload(backend, normal_bf16(seed, 10 + 2 * layer, (physical, pt, hkv, WIDTH)), dtype)
+            values = upload(backend, normal_bf16(seed, 11 + 2 * layer, (physical, pt, hkv, WIDTH)), dtype)
+            self.pools.append((keys, values))
+        self.dtype = dtype
+        self.lanes = lanes
+
+    def record_layer(self, commands, layer, starts=None, copy_rows=True, lanes=None):
+        """Appends the per-lane dispatches of one layer; returns (packed attended, lane rows)."""
+        backend, hq = self.backend, self.hq
+        starts = self.contexts if starts is None else starts
+        scale = 1.0 / math.sqrt(WIDTH)
+        attended = backend.alloc(self.dtype, (self.lanes, hq * WIDTH))
+        rows = []
+        keys, values = self.pools[layer]
+        for lane in (range(self.lanes) if lanes is None else lanes):
+            row = backend.alloc(self.dtype, (1, hq, WIDTH))
+            inputs = [self.q.narrow(0, lane, 1).permute([1, 0, 2]), self.k.narrow(0, lane, 1),
+                      self.v.narrow(0, lane, 1), self.tables[lane], self.generations]
+            if self.activity is not None:
+                inputs.append(self.activity.narrow(0, lane, 1))
+            commands.dispatch_many(Op.paged_sdpa_append(scale, starts[lane], self.pt), inputs,
+                                   [row.permute([1, 0, 2]), keys, values])
+            if copy_rows:
+                commands.dispatch(Op.copy(), [row.reshape((1, hq * WIDTH))], attended.narrow(0, lane, 1))
+            rows.append(row)
+        return attended, rows
+
+
+def check(cpu, hip, cpu_tensors, hip_tensors, exact=()):
+    for index, (a, b) in enumerate(zip(cpu_tensors, hip_tensors)):
+        if index in exact:
+            assert cpu.read(a) == hip.read(b)
+        else:
+            assert_close(to_f32(hip.read(b), b.dtype), to_f32(cpu.read(a), a.dtype), b.dtype)
+
+
+CASES = [
+    # contexts, hq, hkv, page_tokens
+    ([17, 64, 130, 511], 16, 8, 16),                        # BASELINE config 0
+    ([300, 1, 2047, 700, 15, 16, 0], 32, 4, 16),
+    ([100, 257, 31], 32, 4, 64),                            # engine page size
+    ([3 + (5 * lane) % 28 for lane in range(131)], 16, 2, 16),  # 131 lanes: more than one argument block
+]
+
+
+@pytest.mark.parametrize("contexts,hq,hkv,pt", CASES)
+def test_lane_by_lane_batch_equals_serial_execution(cpu, hip, contexts, hq, hkv, pt):
+    """Two layers on the same lanes (the second reuses the gathered metadata), fused on the
+    device, serial on the oracle; pools bit for bit, attention rows to the float bar; then the
+    library's own serial execution of the same list."""
+    outputs = {}
+    for name, backend in (("cpu", cpu), ("fused", hip), ("serial", hip)):
+        if backend is hip:
+            hip.fusion_enable(name == "fused")
+        before = hip.fusion_stats()
+        batch = LaneBatch(backend, contexts, hq, hkv, pt, seed=71, layers=2)
+        commands = CommandList()
+        kept = []
+        for layer in range(2):
+            attended, rows = batch.record_layer(commands, layer)
+            kept += [attended, rows[0], rows[-1], *batch.pools[layer]]
+        run(backend, commands)
+        outputs[name] = (backend, kept)
+        runs, dispatches = (after - start for after, start in zip(hip.fusion_stats(), before))
+        if name == "fused":
+            assert (runs, dispatches) == (2, 2 * 2 * len(contexts))
+        else:
+            assert (runs, dispatches) == (0, 0)
+    hip.fusion_enable(True)
+    pools = (3, 4, 8, 9)
+    check(cpu, hip, outputs["cpu"][1], outputs["fused"][1], exact=pools)
+    check(cpu, hip, outputs["cpu"][1], outputs["serial"][1], exact=pools)
+    check(hip, hip, outputs["serial"][1], outputs["fused"][1], exact=pools)
+
+
+def test_runs_without_row_copies_and_with_inactive_lanes(cpu, hip):
+    results = []
+    for backend in (cpu, hip):
+        before = hip.fusion_stats()
+        batch = LaneBatch(backend, [33, 70, 5, 129], 8, 4, 16, seed=72, activity=[1, 0, 1, 1])
+        commands = CommandList()
+        _, rows = batch.record_layer(commands, 0, copy_rows=False)
+        run(backend, commands)
+        results.append(rows + list(batch.pools[0]))
+        if backend is hip:
+            assert hip.fusion_stats()[0] - before[0] == 1
+    check(cpu, hip, results[0], results[1], exact=(4, 5))
+    assert not to_f32(hip.read(results[1][1]), DType.BF16).any()
+
+
+def test_gathered_metadata_follows_a_table_rewritten_between_layers(cpu, hip):
+    """Layer 0 and 1 share the gathered tables; then lane 1's table is overwritten on the device
+    (its first page moves to a spare physical page) and it gets a new start: the third run must
+    see both."""
+    contexts = [40, 90, 200, 7]
+    results = []
+    for backend in (cpu, hip):
+        batch = LaneBatch(backend, contexts, 16, 8, 16, seed=73, layers=2)
+        commands = CommandList()
+        first, _ = batch.record_layer(commands, 0)
+        second, _ = batch.record_layer(commands, 1)
+        replacement = batch.host_tables[1].copy()
+        spare = batch.spare_pages[0]
+        replacement[0] = (spare, 11 + spare)
+        commands.dispatch(Op.copy(), [upload(backend, replacement, DType.U32)], batch.tables[1])
+        moved = list(contexts)
+        moved[1] = 70
+        third, _ = batch.record_layer(commands, 0, starts=moved)
+        run(backend, commands)
+        results.append([first, second, third, *batch.pools[0], *batch.pools[1]])
+    check(cpu, hip, results[0], results[1], exact=(3, 4, 5, 6))
+
+
+def test_a_stale_page_is_reported_for_the_lane_that_holds_it(hip):
+    indices = []
+    for fused in (True, False):
+        hip.fusion_enable(fused)
+        batch = LaneBatch(hip, [33, 70, 50, 5], 8, 4, 16, seed=74, corrupt=(2, 1))
+        commands = CommandList()
+        attended, rows = batch.record_layer(commands, 0)
+        with pytest.raises(BackendError) as info:
+            run(hip, commands)
+        assert info.value.status == Status.DEVICE_ERROR_FLAG
+        indices.append((info.value.dispatch, info.value.index))
+    hip.fusion_enable(True)
+    assert indices[0] == indices[1] == (4, 1)      # lane 2's attention dispatch, logical page 1
+
+
+def test_runs_that_cannot_be_proved_independent_are_executed_serially(cpu, hip):
+    """Lane rows that overlap each other, and an output row inside the packed q allocation: the
+    list is valid dispatch by dispatch, so it runs, but not fused."""
+    contexts = [20, 45, 9]
+    results = []
+    for backend in (cpu, hip):
+        before = hip.fusion_stats()
+        batch = LaneBatch(backend, contexts, 8, 4, 16, seed=75)
+        commands = CommandList()
+        scale = 1.0 / math.sqrt(WIDTH)
+        shared = backend.alloc(DType.BF16, (1, 8, WIDTH))     # every lane writes the same row
+        keys, values = batch.pools[0]
+        for lane in range(3):
+            commands.dispatch_many(
+                Op.paged_sdpa_append(scale, contexts[lane], 16),
+                [batch.q.narrow(0, lane, 1).permute([1, 0, 2]), batch.k.narrow(0, lane, 1),
+                 batch.v.narrow(0, lane, 1), batch.tables[lane], batch.generations],
+                [shared.permute([1, 0, 2]), keys, values])
+        run(backend, commands)
+        results.append([shared, keys, values])
+        if backend is hip:
+            assert hip.fusion_stats() == before
+    check(cpu, hip, results[0], results[1], exact=(1, 2))

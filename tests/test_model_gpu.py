@@ -65,6 +65,33 @@ SMALL_DENSE = ModelConfig("small-dense", hidden=512, layers=2, q_heads=8, kv_hea
                           vocab=2000, intermediate=1024)
 
 
+def test_lane_by_lane_recording_gives_the_packed_recording(cpu, hip):
+    """The step recorded the way the engines record it (per lane one PagedSdpaAppend and one Copy
+    per layer, engines/qwen3-coder/src/lib.rs:917-935) against the packed recording: on the device
+    the fused runs feed the same attention kernel the same lanes, so tokens and logits are
+    identical; the oracle executes the per-lane dispatches one by one."""
+    contexts = [5, 40, 300, 77, 16, 15]
+    packed, by_lane = (DecodeSession(Model(hip, TINY_MOE, seed=14, layers=2), contexts, seed=14)
+                       for _ in range(2))
+    reference = DecodeSession(Model(cpu, TINY_MOE, seed=14, layers=2), contexts, seed=14)
+    by_lane.record_lane_by_lane()
+    reference.record_lane_by_lane()
+    before = hip.fusion_stats()
+    packed_tokens = np.stack([packed.step() for _ in range(20)])
+    lane_tokens = np.stack([by_lane.step(lane_by_lane=True) for _ in range(20)])
+    assert hip.fusion_stats()[0] - before[0] == 20 * 2          # one run per layer and step
+    assert packed_tokens.tolist() == lane_tokens.tolist()
+    assert hip.read(packed.buffers.logits) == hip.read(by_lane.buffers.logits)
+    reference_tokens = np.stack([reference.step(lane_by_lane=True) for _ in range(8)])
+    assert reference_tokens.tolist() == lane_tokens[:8].tolist()
+    hip.fusion_enable(False)
+    serial = DecodeSession(Model(hip, TINY_MOE, seed=14, layers=2), contexts, seed=14)
+    serial.record_lane_by_lane()
+    serial_tokens = np.stack([serial.step(lane_by_lane=True) for _ in range(8)])
+    hip.fusion_enable(True)
+    assert serial_tokens.tolist() == lane_tokens[:8].tolist()
+
+
 @pytest.mark.parametrize("config,contexts,counts", [
     (SMALL_DENSE, [40, 0, 300, 0, 7], [1, 150, 1, 37, 1]),      # BASELINE config 1 in miniature
     (TINY_MOE, [0, 64, 10], [140, 1, 1]),                       # prefill rows through the routed path

@@ -330,6 +330,8 @@ class OpKind(enum.IntEnum):
     GATHER_QUANT_MATMUL = 11
     PAGED_SDPA_APPEND = 12
     PAGED_SDPA = 13
+    SAMPLE = 14
+    SAMPLE_MASKED = 15
     PAGED_ATTENTION_RAGGED = 32
     ROUTE_PACK = 33
     FILL_SEEDED = 34
@@ -371,6 +373,12 @@ class Op:
 
     @staticmethod
     def top_k(k, normalize): return Op(OpKind.TOP_K, k=k, normalize=normalize)
+
+    @staticmethod
+    def sample(position): return Op(OpKind.SAMPLE, start=position)
+
+    @staticmethod
+    def sample_masked(position): return Op(OpKind.SAMPLE_MASKED, start=position)
 
     @staticmethod
     def rope(theta): return Op(OpKind.ROPE, theta=theta)

@@ -789,6 +789,38 @@ fh_status plan_argmax(fh_backend *b, const Planned &pl, bool execute) {
   return FH_OK;
 }
 
+// check_sample / check_sample_masked (crates/forja-core/src/ops.rs:1546-1592).
+fh_status plan_sample(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
+  const fh_dispatch &d = *pl.d;
+  const bool masked = d.op == FH_OP_SAMPLE_MASKED;
+  FH_REQUIRE(d.n_inputs == (masked ? 3u : 2u) && d.n_outputs == 1);
+  const fh_tensor &in = d.inputs[0], &params = d.inputs[1], &out = d.outputs[0];
+  FH_REQUIRE(is_float(in.dtype) && out.dtype == FH_U32);
+  FH_REQUIRE(params.dtype == FH_U32 && shape_is(params, {5}));
+  FH_REQUIRE(in.rank >= 1 && in.rank <= 2 && in.shape[in.rank - 1] != 0);
+  const uint32_t rows = in.rank == 2 ? in.shape[0] : 1, width = in.shape[in.rank - 1];
+  FH_REQUIRE(element_count(out) == rows);
+  if (masked) {
+    const fh_tensor &allow = d.inputs[2];
+    FH_REQUIRE(allow.dtype == FH_U32 && shape_is(allow, {(width + 31) / 32}) &&
+               is_contiguous(allow));
+  }
+  if (!execute || rows == 0) return FH_OK;
+  View in_v = pl.in[0];
+  if (in.rank == 1) {
+    in_v.stride[1] = in_v.stride[0];
+    in_v.shape[1] = in_v.shape[0];
+    in_v.stride[0] = 0;
+    in_v.shape[0] = 1;
+    in_v.rank = 2;
+  }
+  char *scratch = b->ensure_workspace(sample_scratch_bytes(rows, width));
+  if (!scratch) return FH_ALLOCATION_FAILED;
+  launch_sample(b->stream, in_v, pl.in[1], masked ? &pl.in[2] : nullptr, pl.out[0], rows, width,
+                d.start, scratch, error);
+  return FH_OK;
+}
+
 fh_status plan_quant_embed(fh_backend *b, const Planned &pl, ErrorSlot *error, bool execute) {
   const fh_dispatch &d = *pl.d;
   FH_REQUIRE(d.n_inputs == 4 && d.n_outputs == 1);
@@ -1126,6 +1158,8 @@ fh_status process(fh_backend *b, const fh_dispatch &d, ErrorSlot *error, bool ex
   case FH_OP_PAGED_COPY: return plan_paged_copy(b, pl, error, execute);
   case FH_OP_RMS_NORM: return plan_rms_norm(b, pl, execute);
   case FH_OP_ARGMAX: return plan_argmax(b, pl, execute);
+  case FH_OP_SAMPLE:
+  case FH_OP_SAMPLE_MASKED: return plan_sample(b, pl, error, execute);
   case FH_OP_TOP_K: return plan_top_k(b, pl, execute);
   case FH_OP_ROPE: return plan_rope(b, pl, execute);
   case FH_OP_QUANT_EMBED: return plan_quant_embed(b, pl, error, execute);
@@ -1909,7 +1943,10 @@ fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
         uint32_t op = s->ops[i];
         bool index_error = op == FH_OP_GATHER_QUANT_MATMUL || op == FH_OP_QUANT_EMBED ||
                            op == FH_OP_ROUTE_PACK;
-        s->result = index_error ? FH_INDEX_OUT_OF_RANGE : FH_DEVICE_ERROR_FLAG;
+        // Sampling refuses its live parameters or mask as InvalidInput (lib.rs:1560-1567, 1639-1652).
+        bool refused_input = op == FH_OP_SAMPLE || op == FH_OP_SAMPLE_MASKED;
+        s->result = refused_input ? FH_INVALID_INPUT
+                                  : (index_error ? FH_INDEX_OUT_OF_RANGE : FH_DEVICE_ERROR_FLAG);
         s->error.code = s->result;
         s->error.dispatch = i;
         s->error.submission = s->serial;

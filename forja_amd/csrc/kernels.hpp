@@ -92,6 +92,16 @@ void launch_route_pack(hipStream_t s, const View &indices, uint32_t rows, uint32
                        uint32_t zero_row_words = 0);
 
 
+// ---- sampling.hip: Op::Sample / Op::SampleMasked ----
+// Rows are processed by at most kSampleGrid workgroups, each with scratch for one row.
+constexpr uint32_t kSampleGrid = 128;
+uint64_t sample_scratch_bytes(uint32_t rows, uint32_t width);
+// logits [rows, width] (rank-2 view), params u32 [5], allow u32 [ceil(width/32)] contiguous or
+// null, out u32 with `rows` elements.  Refused parameters or mask set the error slot.
+void launch_sample(hipStream_t s, const View &logits, const View &params, const View *allow,
+                   const View &out, uint32_t rows, uint32_t width, uint32_t position,
+                   void *scratch, ErrorSlot *error);
+
 // ---- lane_fusion.hip: glue for a run of per-lane attention dispatches executed as one launch ----
 // Addresses of up to kLaneChunk lanes, passed by value as kernel arguments.
 constexpr uint32_t kLaneChunk = 128;

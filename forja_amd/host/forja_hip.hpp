@@ -155,6 +155,18 @@ struct Op {
     op.record.theta = theta;
     return op;
   }
+  // Op::Sample / Op::SampleMasked: the position travels in `start`; the Metal tuning attributes
+  // (chunk_width, fast_top_k, ...) stay on the host side of the boundary.
+  static Op sample(uint32_t position) {
+    Op op = of(FH_OP_SAMPLE);
+    op.record.start = position;
+    return op;
+  }
+  static Op sample_masked(uint32_t position) {
+    Op op = of(FH_OP_SAMPLE_MASKED);
+    op.record.start = position;
+    return op;
+  }
   static Op top_k(uint32_t k, bool normalize) {
     Op op = of(FH_OP_TOP_K);
     op.record.k = k;

@@ -69,6 +69,17 @@ typedef enum fh_op_kind {
   FH_OP_GATHER_QUANT_MATMUL = 11, /* Op::GatherQuantMatmul: 5, 8 (pair) or 6 (weighted sum) inputs */
   FH_OP_PAGED_SDPA_APPEND = 12,  /* Op::PagedSdpaAppend{scale,q_start,page_tokens} */
   FH_OP_PAGED_SDPA = 13,         /* Op::PagedSdpa{scale,causal,q_start,key_length,page_tokens} */
+  /* Op::Sample{position,..} (crates/forja-core/src/ops.rs:202-220; executed as
+   * crates/forja-cpu/src/lib.rs:610-642, 1577-1700): inputs logits [.., width] (float) and params
+   * u32 [5] = temperature bits, top_k, top_p bits, seed low, seed high, read when the dispatch
+   * runs; output u32 with one index per row.  `start` carries the position.  The op's
+   * chunk_width / fast_top_k / fast_max_chunks / rejection_rounds are tuning attributes of the
+   * Metal kernels, checked by forja-core before a backend sees the dispatch, and do not cross
+   * this boundary.  Refused live parameters make fh_wait return FH_INVALID_INPUT. */
+  FH_OP_SAMPLE = 14,
+  /* Op::SampleMasked (ops.rs:221-236; lib.rs:644-678): a third input allow u32
+   * [ceil(width/32)], one bit per column; an empty mask or set padding bits are refused. */
+  FH_OP_SAMPLE_MASKED = 15,
   /* --- fused forms with no single-dispatch counterpart in the reference --- */
   /* Packed ragged batch of lanes: append each lane's new K/V rows at its q_start, then causal
    * attention through them.  As-if-serial equivalent of, per lane, two Op::PagedCopy{IntoPages}

@@ -82,6 +82,41 @@ _NP = {DType.F32: np.float32, DType.F16: np.uint16, DType.BF16: np.uint16, DType
        DType.U32: np.uint32}
 
 
+def sampling_words(temperature: float, top_k: int, top_p: float, seed: int) -> np.ndarray:
+    """The five parameter words of Op::Sample (SamplingParameters::from_words, lib.rs:1553-1575)."""
+    bits = np.array([temperature, top_p], dtype=np.float32).view(np.uint32)
+    return np.array([bits[0], top_k, bits[1], seed & 0xffffffff, (seed >> 32) & 0xffffffff],
+                    dtype=np.uint32)
+
+
+def sample_rows(values: np.ndarray, params: np.ndarray, position: int, allow=None) -> np.ndarray:
+    """sample_row / sample_row_masked (lib.rs:1577-1597) over the rows of a 2-D f32 array."""
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    rows, width = values.shape
+    out = np.empty(rows, dtype=np.uint32)
+    params = np.ascontiguousarray(params, dtype=np.uint32)
+    if allow is not None:
+        allow = np.ascontiguousarray(allow, dtype=np.uint32)
+    _ok(lib().orc_sample(_p(values), _sz(rows), _sz(width), _p(params), C.c_uint32(position),
+                         _p(allow) if allow is not None else None, _p(out)))
+    return out
+
+
+def top_p_keep(row: np.ndarray, temperature: float, top_p: float) -> int:
+    """Candidates truncate_top_p (lib.rs:1654-1679) keeps out of a whole row."""
+    row = np.ascontiguousarray(row, dtype=np.float32)
+    keep = C.c_size_t()
+    _ok(lib().orc_top_p_keep(_p(row), _sz(row.size), C.c_float(temperature), C.c_float(top_p),
+                             C.byref(keep)))
+    return keep.value
+
+
+def validate_allow_mask(allow, width: int) -> bool:
+    """validate_allow_mask (lib.rs:1639-1652): True when accepted."""
+    allow = np.ascontiguousarray(allow, dtype=np.uint32)
+    return lib().orc_validate_allow_mask(_p(allow), _sz(allow.size), _sz(width)) == 0
+
+
 def decode(raw: np.ndarray, dtype: DType) -> np.ndarray:
     """lib.rs:1790-1809"""
     count = raw.size // dtype.byte_size
@@ -301,6 +336,7 @@ class CpuBackend:
             OpKind.PROGRAM: self._program, OpKind.COPY: self._copy,
             OpKind.PAGED_COPY: self._paged_copy_op, OpKind.RMS_NORM: self._rms_norm,
             OpKind.ARGMAX: self._argmax, OpKind.TOP_K: self._top_k, OpKind.ROPE: self._rope,
+            OpKind.SAMPLE: self._sample, OpKind.SAMPLE_MASKED: self._sample,
             OpKind.QUANT_EMBED: self._quant_embed, OpKind.MATMUL: self._matmul,
             OpKind.QUANT_MATMUL: self._quant_matmul,
             OpKind.GATHER_QUANT_MATMUL: self._gather_quant,
@@ -445,6 +481,21 @@ class CpuBackend:
         out = np.empty(rows, dtype=np.uint32)
         xs = self._floats(src)
         _ok(lib().orc_argmax(_p(xs), _sz(rows), _sz(width), _p(out)))
+        self._scatter(d.outputs[0], out)
+
+    def _sample(self, d):
+        """execute_sample / execute_sample_masked (crates/forja-cpu/src/lib.rs:610-678)."""
+        src = d.inputs[0]
+        width = src.shape[-1]
+        rows = src.layout.element_count // width
+        xs = self._floats(src)
+        params = np.ascontiguousarray(self._gather(d.inputs[1]).view(np.uint32))
+        allow = None
+        if d.op.kind == OpKind.SAMPLE_MASKED:
+            allow = np.ascontiguousarray(self._gather(d.inputs[2]).view(np.uint32))
+        out = np.empty(rows, dtype=np.uint32)
+        _ok(lib().orc_sample(_p(xs), _sz(rows), _sz(width), _p(params), C.c_uint32(d.op.start),
+                             _p(allow) if allow is not None else None, _p(out)))
         self._scatter(d.outputs[0], out)
 
     def _rms_norm(self, d):

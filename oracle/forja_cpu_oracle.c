@@ -343,6 +343,195 @@ static int topk_compare(const void *left, const void *right) {
   return l->index < r->index ? -1 : (l->index > r->index ? 1 : 0);
 }
 
+/* ---- Op::Sample / Op::SampleMasked (crates/forja-cpu/src/lib.rs:1545-1700) ----
+ * Pinned by the reference's own tests restated in tests/test_oracle_golden.py: the chi-squared
+ * checks against known probabilities (lib.rs:2636-2662, 3283-3306), the exact truncation sets of
+ * top_k / top_p, masks in every mode, the all-allowed mask, mask refusals, the 1025-candidate
+ * nucleus, counter determinism and the parameter refusals; plus the closed form P(i) =
+ * softmax(logits / T) at other temperatures and the max_by tie rule.
+ * PARITY UNPINNED: the token drawn for a given seed.  The reference holds no token vectors and
+ * does not promise tokens across builds or backends (crates/forja-core/src/ops.rs:206-208); a
+ * slip in the counter formula that keeps the noise uniform would pass every check above. */
+
+/* SamplingParameters::from_words (lib.rs:1553-1575). */
+static int sampling_parameters(const uint32_t words[5], float *temperature, uint32_t *top_k,
+                               float *top_p, uint64_t *seed) {
+  memcpy(temperature, &words[0], 4);
+  memcpy(top_p, &words[2], 4);
+  if (!isfinite(*temperature) || *temperature < 0.0f || !isfinite(*top_p) ||
+      !(*top_p >= 0.0f && *top_p <= 1.0f) || *top_p == 0.0f)
+    return ORC_INVALID_INPUT;
+  *top_k = words[1];
+  *seed = (uint64_t)words[3] | ((uint64_t)words[4] << 32);
+  return ORC_OK;
+}
+
+/* validate_allow_mask (lib.rs:1639-1652). */
+int orc_validate_allow_mask(const uint32_t *allow, size_t words, size_t width) {
+  size_t remainder = width % 32;
+  if (remainder != 0 &&
+      (words == 0 || (allow[words - 1] & ~((1u << remainder) - 1u)) != 0))
+    return ORC_INVALID_INPUT;
+  for (size_t word = 0; word < words; ++word)
+    if (allow[word] != 0) return ORC_OK;
+  return ORC_INVALID_INPUT;
+}
+
+/* f32::ln and f32::exp go to the platform's libm, whose f32 routines are not correctly rounded
+ * and differ between platforms in the last place (the reference says as much: tokens are not
+ * promised across builds, ops.rs:206-208).  The restatement uses the correctly rounded value
+ * (f64 evaluation rounded once), the function those routines approximate. */
+static float ln_f32(float value) { return (float)log((double)value); }
+static float exp_f32(float value) { return (float)exp((double)value); }
+
+/* sampled_score (lib.rs:1681-1692): Gumbel-max noise from a counter-based stream. */
+static float sampled_score(float logit, float temperature, uint64_t seed, uint32_t position,
+                           size_t index) {
+  if (!isfinite(logit)) return logit;
+  uint64_t counter = seed ^ ((uint64_t)position << 32) ^ (uint64_t)index;
+  uint64_t random = orc_splitmix64(counter);
+  uint32_t mantissa = (uint32_t)(random >> 40);
+  float uniform = ((float)mantissa + 0.5f) * (1.0f / 16777216.0f);
+  return logit / temperature - ln_f32(-ln_f32(uniform));
+}
+
+typedef struct {
+  int32_t key;
+  uint32_t index;
+} sample_item;
+
+/* sort_unstable_by(row[right].total_cmp(row[left]).then(right.cmp(left))) (lib.rs:1616-1620):
+ * descending value, ties by descending index; the order is total, so stability is moot. */
+static int sample_compare(const void *left, const void *right) {
+  const sample_item *l = (const sample_item *)left, *r = (const sample_item *)right;
+  if (l->key != r->key) return l->key > r->key ? -1 : 1;
+  return l->index > r->index ? -1 : (l->index < r->index ? 1 : 0);
+}
+
+/* truncate_top_p (lib.rs:1654-1679): number of leading candidates kept. */
+static size_t top_p_keep(const float *row, const sample_item *sorted, size_t count,
+                         float temperature, float top_p, float *weights) {
+  if (count == 0) return 0;
+  float maximum = row[sorted[0].index];
+  float total = 0.0f;
+  for (size_t i = 0; i < count; ++i) {
+    weights[i] = exp_f32((row[sorted[i].index] - maximum) / temperature);
+    total += weights[i];
+  }
+  if (!(isfinite(total) && total > 0.0f)) return 1;
+  float cumulative = 0.0f;
+  for (size_t i = 0; i < count; ++i) {
+    cumulative += weights[i] / total;
+    if (cumulative >= top_p) return i + 1;
+  }
+  return count;
+}
+
+/* The candidates truncate_top_p keeps out of a whole row (for the reference's own test of it). */
+int orc_top_p_keep(const float *row, size_t width, float temperature, float top_p, size_t *keep) {
+  sample_item *items = (sample_item *)malloc((width + 1) * sizeof(sample_item));
+  float *weights = (float *)malloc((width + 1) * sizeof(float));
+  if (!items || !weights) {
+    free(items);
+    free(weights);
+    return ORC_EXECUTION_FAILED;
+  }
+  for (size_t i = 0; i < width; ++i) {
+    items[i].key = total_key(row[i]);
+    items[i].index = (uint32_t)i;
+  }
+  qsort(items, width, sizeof(sample_item), sample_compare);
+  *keep = top_p_keep(row, items, width, temperature, top_p, weights);
+  free(items);
+  free(weights);
+  return ORC_OK;
+}
+
+/* sample_allowed (lib.rs:1599-1637) over the indices `allow` permits (all when null). */
+int orc_sample_row(const float *row, size_t width, const uint32_t params[5], uint32_t position,
+                   const uint32_t *allow, uint32_t *out) {
+  float temperature, top_p;
+  uint32_t top_k;
+  uint64_t seed;
+  int status = sampling_parameters(params, &temperature, &top_k, &top_p, &seed);
+  if (status != ORC_OK) return status;
+  sample_item *items = (sample_item *)malloc((width + 1) * sizeof(sample_item));
+  float *weights = (float *)malloc((width + 1) * sizeof(float));
+  if (!items || !weights) {
+    free(items);
+    free(weights);
+    return ORC_EXECUTION_FAILED;
+  }
+  size_t count = 0;
+  for (size_t i = 0; i < width; ++i) {
+    if (allow && !(allow[i / 32] & (1u << (i % 32)))) continue;
+    items[count].key = total_key(row[i]);
+    items[count].index = (uint32_t)i;
+    ++count;
+  }
+  status = ORC_OK;
+  if (temperature == 0.0f || top_k == 1) {
+    /* max_by(total_cmp.then(index)): the largest value, the largest index among equals */
+    if (count == 0) {
+      status = ORC_INVALID_INPUT;
+    } else {
+      size_t best = 0;
+      for (size_t i = 1; i < count; ++i)
+        if (items[i].key >= items[best].key) best = i;
+      *out = items[best].index;
+    }
+  } else {
+    qsort(items, count, sizeof(sample_item), sample_compare);
+    size_t cap = top_k == 0 ? count : (size_t)top_k;
+    if (cap < count) count = cap;
+    if (top_p < 1.0f) {
+      size_t keep = top_p_keep(row, items, count, temperature, top_p, weights);
+      if (count == 0) status = ORC_EXECUTION_FAILED;
+      if (keep < 1) keep = 1;
+      if (keep < count) count = keep;
+    }
+    if (count == 0) {
+      if (status == ORC_OK) status = ORC_EXECUTION_FAILED;
+    } else {
+      size_t best = 0;
+      int32_t best_key = 0;
+      for (size_t i = 0; i < count; ++i) {
+        int32_t key = total_key(sampled_score(row[items[i].index], temperature, seed, position,
+                                              items[i].index));
+        if (i == 0 || key > best_key ||
+            (key == best_key && items[i].index > items[best].index)) {
+          best = i;
+          best_key = key;
+        }
+      }
+      *out = items[best].index;
+    }
+  }
+  free(items);
+  free(weights);
+  return status;
+}
+
+/* execute_sample / execute_sample_masked (lib.rs:610-678): one parameter block for all rows. */
+int orc_sample(const float *values, size_t rows, size_t width, const uint32_t params[5],
+               uint32_t position, const uint32_t *allow, uint32_t *out) {
+  if (width == 0) return ORC_EXECUTION_FAILED;
+  float temperature, top_p;
+  uint32_t top_k;
+  uint64_t seed;
+  int status = sampling_parameters(params, &temperature, &top_k, &top_p, &seed);
+  if (status != ORC_OK) return status;
+  if (allow) {
+    status = orc_validate_allow_mask(allow, (width + 31) / 32, width);
+    if (status != ORC_OK) return status;
+  }
+  for (size_t row = 0; row < rows; ++row) {
+    status = orc_sample_row(values + row * width, width, params, position, allow, &out[row]);
+    if (status != ORC_OK) return status;
+  }
+  return ORC_OK;
+}
+
 /* execute_top_k (lib.rs:552-608). */
 int orc_top_k(const float *values, size_t rows, size_t width, size_t k, int normalize,
               float *out_values, uint32_t *out_indices) {

@@ -73,6 +73,14 @@ int orc_gather_quant_weighted_sum(const float *x, const uint32_t *packed, const 
 
 /* ---- selection (lib.rs:519-608) ---- */
 int orc_argmax(const float *values, size_t rows, size_t width, uint32_t *out);
+/* Op::Sample / Op::SampleMasked (crates/forja-cpu/src/lib.rs:610-678, 1545-1700).  params:
+ * temperature bits, top_k, top_p bits, seed low, seed high.  allow: one bit per column, or null. */
+int orc_validate_allow_mask(const uint32_t *allow, size_t words, size_t width);
+int orc_top_p_keep(const float *row, size_t width, float temperature, float top_p, size_t *keep);
+int orc_sample_row(const float *row, size_t width, const uint32_t params[5], uint32_t position,
+                   const uint32_t *allow, uint32_t *out);
+int orc_sample(const float *values, size_t rows, size_t width, const uint32_t params[5],
+               uint32_t position, const uint32_t *allow, uint32_t *out);
 int orc_top_k(const float *values, size_t rows, size_t width, size_t k, int normalize,
               float *out_values, uint32_t *out_indices);
 

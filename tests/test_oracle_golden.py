@@ -575,3 +575,101 @@ def test_seeded_generators_have_the_stated_distributions():
     assert np.all(np.abs(np.bincount(nibbles.ravel(), minlength=16) / nibbles.size - 1 / 16) < 0.002)
     # counter-based: a window equals the same indices of the full stream
     assert np.array_equal(orc.fill_words(1234, 7, 100, first=500), words[500:600])
+
+
+# ------------------------------------------------------------------ sampling
+# The reference's own tests of Op::Sample (crates/forja-cpu/src/lib.rs:2520-2690, 3283-3306),
+# restated on the oracle, plus the closed form Gumbel-max sampling has to reproduce.
+
+def _sample(row, temperature, top_k, top_p, seed, position, allow=None):
+    words = orc.sampling_words(temperature, top_k, top_p, seed)
+    return int(orc.sample_rows(np.array([row], dtype=np.float32), words, position, allow)[0])
+
+
+def _chi_squared(row, temperature, top_k, top_p, seed, expected, trials=20_000):
+    counts = np.zeros(len(row))
+    for position in range(trials):
+        counts[_sample(row, temperature, top_k, top_p, seed, position)] += 1
+    expected = np.asarray(expected, dtype=np.float64)
+    live = expected > 0
+    statistic = (((counts - expected * trials) ** 2)[live] / (expected * trials)[live]).sum()
+    assert statistic < 16.3, statistic               # the reference's bound (lib.rs:3300)
+    assert not counts[~live].any()
+
+
+def test_sampled_tokens_are_counter_deterministic():
+    row = [0.1, -0.3, 1.2, 0.7, 0.0, 0.9, -1.0]
+    first = [_sample(row, 0.7, 0, 1.0, 0xfeedbeefdeadcafe, p) for p in range(128)]
+    second = [_sample(row, 0.7, 0, 1.0, 0xfeedbeefdeadcafe, p) for p in range(128)]
+    assert first == second and len(set(first)) > 1
+
+
+def test_sampling_top_k_and_top_p_keep_only_the_exact_allowed_set():
+    row = [10.0, 9.0, 8.0, 1.0, 0.0, -1.0, -2.0]
+    for position in range(4096):
+        assert _sample(row, 1.0, 3, 1.0, 11, position) <= 2
+        assert _sample(row, 1.0, 0, 0.7, 11, position) <= 1
+        assert _sample(row, 1.0, 2, 0.999, 11, position) <= 1
+
+
+def test_masked_sampling_conditions_every_sampling_mode():
+    row = [10.0, 9.0, 8.0, 7.0, 6.0, 5.0, 4.0]
+    allow = [0b01010010]
+    for temperature, top_k, top_p, seed in [(0.0, 0, 1.0, 11), (1.0, 2, 1.0, 12), (1.0, 0, 0.8, 13),
+                                            (0.7, 0, 1.0, 14)]:
+        for position in range(256):
+            assert _sample(row, temperature, top_k, top_p, seed, position, allow) in (1, 4, 6)
+
+
+def test_all_allowed_mask_preserves_unconstrained_sampling():
+    row = [index / 7.0 for index in range(33)]
+    for position in range(512):
+        assert _sample(row, 0.7, 7, 0.9, 0xfeedbeef, position, [0xffffffff, 1]) == \
+            _sample(row, 0.7, 7, 0.9, 0xfeedbeef, position)
+
+
+def test_masked_sampling_refuses_empty_and_padding_bits():
+    assert not orc.validate_allow_mask([0], 7)
+    assert not orc.validate_allow_mask([1 << 7], 7)
+    assert orc.validate_allow_mask([1 << 6], 7)
+
+
+def test_top_p_uses_the_full_candidate_set_beyond_1024_values():
+    assert orc.top_p_keep(np.zeros(1025), 1.0, 0.9995) == 1025
+
+
+def test_sampling_distributions_match_known_probabilities():
+    _chi_squared([0.0, 0.0, 0.0, 0.0], 1.0, 0, 1.0, 91, [0.25] * 4)
+    _chi_squared([2.0, 1.0, 0.0], 1.0, 2, 1.0, 92, [0.7310586, 0.2689414, 0.0])
+    _chi_squared([2.0, 1.0, 0.0], 1.0, 0, 0.8, 93, [0.7310586, 0.2689414, 0.0])
+    _chi_squared([2.0, 1.0, 0.0, -1.0], 1.0, 3, 0.95, 94, [0.66524094, 0.24472848, 0.09003057, 0.0])
+
+
+def test_gumbel_max_reproduces_the_softmax_at_other_temperatures():
+    """Closed form the noise term has to give: P(i) = softmax(logits / T)_i."""
+    row = np.array([0.3, -1.2, 2.0, 0.9, 0.0])
+    for temperature, seed in ((0.5, 95), (2.5, 96)):
+        expected = np.exp(row / temperature)
+        _chi_squared(list(row), temperature, 0, 1.0, seed, expected / expected.sum())
+
+
+def test_greedy_sampling_takes_the_largest_value_and_the_last_of_equals():
+    row = [1.0, 5.0, -2.0, 5.0, 3.0, float("-inf")]
+    assert _sample(row, 0.0, 0, 1.0, 7, 3) == 3           # temperature 0
+    assert _sample(row, 1.3, 1, 0.5, 7, 3) == 3           # top_k 1
+    assert _sample(row, 0.0, 0, 1.0, 7, 3, [0b010111]) == 1
+    assert _sample([float("nan"), 2.0, float("inf")], 0.0, 0, 1.0, 1, 0) == 0   # total order: NaN above inf
+
+
+def test_sample_refuses_invalid_live_parameters(cpu):
+    logits = upload(cpu, np.zeros(7), DType.F32)
+    output = cpu.alloc(DType.U32, ())
+    for words in ([np.float32("nan").view(np.uint32), 0, np.float32(1.0).view(np.uint32), 0, 0],
+                  list(orc.sampling_words(-1.0, 0, 1.0, 0)), list(orc.sampling_words(1.0, 0, 0.0, 0)),
+                  list(orc.sampling_words(1.0, 0, 1.5, 0))):
+        params = upload(cpu, np.array(words, dtype=np.uint32), DType.U32)
+        commands = CommandList()
+        commands.dispatch(Op.sample(0), [logits, params], output)
+        with pytest.raises(orc.BackendError) as info:
+            run(cpu, commands)
+        assert info.value.status == orc.Status.INVALID_INPUT

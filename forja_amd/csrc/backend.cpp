@@ -1192,9 +1192,22 @@ fh_status process(fh_backend *b, const fh_dispatch &d, ErrorSlot *error, bool ex
 // crates/forja-host/src/lib.rs:5408-5470), which also makes the key/value writes of different
 // members independent.
 
+// One lane's share of a run, whichever way it was recorded.
+struct LaneMember {
+  fh_tensor q, k_new, v_new;  // [heads, 1, D]; [1, kv heads, D] twice
+  fh_tensor table, generations, activity, out, key_pool, value_pool;  // pools as [P, pt, Hkv, D]
+  bool has_activity = false;
+  bool has_copy = false;      // an Op::Copy of the output row follows
+  fh_tensor copy_target{};
+  uint32_t q_start = 0, page_tokens = 0;
+  float scale = 0.0f;
+  uint32_t dispatches = 0;    // dispatches of the member, the copy included
+  uint32_t attention_at = 0;  // which of them is the attention (its failures are recorded there)
+};
+
 struct LaneRun {
-  uint32_t items = 0;    // attention dispatches
-  uint32_t step = 1;     // dispatches per lane: 2 when each is followed by the copy of its row
+  std::vector<LaneMember> members;
+  uint32_t dispatches = 0;       // examined (and, when fused, replaced)
   int64_t delta[3] = {0, 0, 0};  // element distance between consecutive members' q, k_new, v_new
 };
 
@@ -1214,86 +1227,174 @@ bool dense_head_rows(const fh_tensor &out) {
   return out.rank == 3 && out.shape[1] == 1 && out.stride[2] == 1 && out.stride[0] == out.shape[2];
 }
 
-// `copy` moves exactly the row `attention` produced, unconverted, into a dense destination.
-bool copies_attended_row(const fh_dispatch &attention, const fh_dispatch &copy) {
+// `copy` moves exactly the row `out`, unconverted, into a dense destination.
+bool copies_attended_row(const fh_tensor &row, const fh_dispatch &copy) {
   if (copy.op != FH_OP_COPY || copy.n_inputs != 1 || copy.n_outputs != 1) return false;
-  const fh_tensor &row = attention.outputs[0], &in = copy.inputs[0], &out = copy.outputs[0];
+  const fh_tensor &in = copy.inputs[0], &out = copy.outputs[0];
   return in.buffer == row.buffer && in.offset == row.offset && in.dtype == row.dtype &&
          out.dtype == row.dtype && is_contiguous(in) && is_contiguous(out) &&
          element_count(in) == (uint64_t)row.shape[0] * row.shape[2] &&
          element_count(out) == element_count(in);
 }
 
-bool same_attention_shape(const fh_dispatch &a, const fh_dispatch &b) {
-  if (b.op != a.op || b.n_inputs != a.n_inputs || b.n_outputs != a.n_outputs) return false;
-  if (memcmp(&a.scale, &b.scale, sizeof(float)) != 0 || a.page_tokens != b.page_tokens) return false;
-  for (uint32_t i = 0; i < 3; ++i)
-    if (a.inputs[i].buffer != b.inputs[i].buffer || !same_layout(a.inputs[i], b.inputs[i])) return false;
-  if (!same_layout(a.inputs[3], b.inputs[3]) || !same_tensor(a.inputs[4], b.inputs[4])) return false;
-  if (a.n_inputs == 6 && !same_layout(a.inputs[5], b.inputs[5])) return false;
-  return same_layout(a.outputs[0], b.outputs[0]) && same_tensor(a.outputs[1], b.outputs[1]) &&
-         same_tensor(a.outputs[2], b.outputs[2]);
+// A [1, ...] row of `heads * width` contiguous elements as the tensor [1, heads, width].
+bool as_head_rows(const fh_tensor &row, uint32_t heads, uint32_t width, fh_tensor *out) {
+  if (row.rank < 2 || row.shape[0] != 1 || !is_contiguous(row)) return false;
+  if (element_count(row) != (uint64_t)heads * width) return false;
+  *out = row;
+  out->rank = 3;
+  out->shape[0] = 1;
+  out->shape[1] = heads;
+  out->shape[2] = width;
+  out->stride[0] = (uint64_t)heads * width;
+  out->stride[1] = width;
+  out->stride[2] = 1;
+  return true;
 }
 
-// Longest fusable run of per-lane attention dispatches starting at `first`; false when there is
-// none of at least two lanes.  `run` then still says how many dispatches were examined, so that
+// Reads the lane recorded at `at` in either idiom: Op::PagedSdpaAppend
+// (engines/qwen3-coder/src/lib.rs:917-935), or two Op::PagedCopy{IntoPages} of the lane's key and
+// value row followed by Op::PagedSdpa over one query row
+// (engines/qwen38/src/attention/batch.rs:37-53); each optionally followed by the row's Op::Copy.
+// Every dispatch has passed its own validation before this is called.
+bool lane_member_at(const fh_dispatch *d, uint32_t count, uint32_t at, LaneMember *m) {
+  const fh_dispatch &first = d[at];
+  *m = LaneMember{};
+  if (first.op == FH_OP_PAGED_SDPA_APPEND) {
+    if (first.n_outputs != 3 || (first.n_inputs != 5 && first.n_inputs != 6)) return false;
+    m->q = first.inputs[0];
+    m->k_new = first.inputs[1];
+    m->v_new = first.inputs[2];
+    m->table = first.inputs[3];
+    m->generations = first.inputs[4];
+    m->has_activity = first.n_inputs == 6;
+    if (m->has_activity) m->activity = first.inputs[5];
+    m->out = first.outputs[0];
+    m->key_pool = first.outputs[1];
+    m->value_pool = first.outputs[2];
+    m->q_start = first.q_start;
+    m->page_tokens = first.page_tokens;
+    m->scale = first.scale;
+    m->dispatches = 1;
+    m->attention_at = 0;
+  } else if (first.op == FH_OP_PAGED_COPY) {
+    if (at + 2 >= count) return false;
+    const fh_dispatch &second = d[at + 1], &attention = d[at + 2];
+    if (second.op != FH_OP_PAGED_COPY || attention.op != FH_OP_PAGED_SDPA) return false;
+    if (first.direction != 0 || second.direction != 0) return false;
+    if (first.n_inputs != second.n_inputs || attention.n_inputs != first.n_inputs + 2) return false;
+    if (attention.n_outputs != 1 || attention.inputs[0].shape[1] != 1) return false;
+    const fh_tensor &kp = attention.inputs[1], &vp = attention.inputs[2];
+    // both copies write the pools the attention reads, one row at its query position
+    if (first.outputs[0].buffer != kp.buffer || first.outputs[0].offset != kp.offset ||
+        first.outputs[0].dtype != kp.dtype || second.outputs[0].buffer != vp.buffer ||
+        second.outputs[0].offset != vp.offset || second.outputs[0].dtype != vp.dtype)
+      return false;
+    if (first.start != attention.q_start || second.start != attention.q_start ||
+        attention.key_length != attention.q_start + 1 || first.page_tokens != attention.page_tokens ||
+        second.page_tokens != attention.page_tokens)
+      return false;
+    for (const fh_dispatch *copy : {&first, &second}) {
+      if (!same_tensor(copy->inputs[1], attention.inputs[3]) ||
+          !same_tensor(copy->inputs[2], attention.inputs[4]))
+        return false;
+      if (copy->n_inputs == 4 && !same_tensor(copy->inputs[3], attention.inputs[5])) return false;
+    }
+    if (!as_head_rows(first.inputs[0], kp.shape[2], kp.shape[3], &m->k_new) ||
+        !as_head_rows(second.inputs[0], vp.shape[2], vp.shape[3], &m->v_new))
+      return false;
+    m->q = attention.inputs[0];
+    m->table = attention.inputs[3];
+    m->generations = attention.inputs[4];
+    m->has_activity = attention.n_inputs == 6;
+    if (m->has_activity) m->activity = attention.inputs[5];
+    m->out = attention.outputs[0];
+    m->key_pool = kp;
+    m->value_pool = vp;
+    m->q_start = attention.q_start;
+    m->page_tokens = attention.page_tokens;
+    m->scale = attention.scale;
+    m->dispatches = 3;
+    m->attention_at = 2;
+  } else {
+    return false;
+  }
+  if (m->k_new.dtype != m->q.dtype || m->v_new.dtype != m->q.dtype) return false;
+  if (!dense_head_rows(m->out) || !is_contiguous(m->table)) return false;
+  if (m->has_activity && element_count(m->activity) != 1) return false;
+  if (at + m->dispatches < count && copies_attended_row(m->out, d[at + m->dispatches])) {
+    m->has_copy = true;
+    m->copy_target = d[at + m->dispatches].outputs[0];
+    m->dispatches += 1;
+  }
+  return true;
+}
+
+bool same_lane_shape(const LaneMember &a, const LaneMember &b) {
+  if (a.dispatches != b.dispatches || a.attention_at != b.attention_at ||
+      a.has_activity != b.has_activity || a.has_copy != b.has_copy)
+    return false;
+  if (memcmp(&a.scale, &b.scale, sizeof(float)) != 0 || a.page_tokens != b.page_tokens) return false;
+  const fh_tensor *left[3] = {&a.q, &a.k_new, &a.v_new}, *right[3] = {&b.q, &b.k_new, &b.v_new};
+  for (uint32_t i = 0; i < 3; ++i)
+    if (left[i]->buffer != right[i]->buffer || !same_layout(*left[i], *right[i])) return false;
+  if (!same_layout(a.table, b.table) || !same_tensor(a.generations, b.generations)) return false;
+  if (a.has_activity && !same_layout(a.activity, b.activity)) return false;
+  if (a.has_copy && !same_layout(a.copy_target, b.copy_target)) return false;
+  return same_layout(a.out, b.out) && same_tensor(a.key_pool, b.key_pool) &&
+         same_tensor(a.value_pool, b.value_pool);
+}
+
+// Longest fusable run of per-lane attention starting at `first`; false when there is none of at
+// least two lanes.  `run->dispatches` then still says how many dispatches were examined, so that
 // the caller does not examine the tail of a refused run again.
 bool find_lane_run(const fh_dispatch *d, uint32_t count, uint32_t first, LaneRun *run) {
-  const fh_dispatch &d0 = d[first];
   *run = LaneRun{};
-  run->items = 1;
-  if (d0.op != FH_OP_PAGED_SDPA_APPEND || d0.n_outputs != 3 ||
-      (d0.n_inputs != 5 && d0.n_inputs != 6))
-    return false;
-  if (!dense_head_rows(d0.outputs[0]) || !is_contiguous(d0.inputs[3])) return false;
-  if (d0.n_inputs == 6 && element_count(d0.inputs[5]) != 1) return false;
-  LaneRun r;
-  r.step = first + 1 < count && copies_attended_row(d0, d[first + 1]) ? 2 : 1;
-  r.items = 1;
+  LaneMember member;
+  if (!lane_member_at(d, count, first, &member)) return false;
+  run->members.push_back(member);
+  run->dispatches = member.dispatches;
   for (;;) {
-    uint64_t at = (uint64_t)first + (uint64_t)r.items * r.step;
-    if (at + r.step > count) break;
-    const fh_dispatch &m = d[at];
-    if (!same_attention_shape(d0, m)) break;
-    if (r.step == 2 && !(copies_attended_row(m, d[at + 1]) &&
-                         same_layout(d[first + 1].outputs[0], d[at + 1].outputs[0])))
-      break;
+    const uint32_t at = first + run->dispatches;
+    if (at >= count || !lane_member_at(d, count, at, &member)) break;
+    const LaneMember &head = run->members[0];
+    if (!same_lane_shape(head, member)) break;
+    const fh_tensor *mine[3] = {&member.q, &member.k_new, &member.v_new};
+    const fh_tensor *heads[3] = {&head.q, &head.k_new, &head.v_new};
     bool regular = true;
+    const int64_t index = (int64_t)run->members.size();
     for (uint32_t i = 0; i < 3; ++i) {
-      int64_t distance = (int64_t)m.inputs[i].offset - (int64_t)d0.inputs[i].offset;
-      if (r.items == 1) {
+      int64_t distance = (int64_t)mine[i]->offset - (int64_t)heads[i]->offset;
+      if (index == 1) {
         if (distance <= 0) regular = false;
-        r.delta[i] = distance;
-      } else if (distance != r.delta[i] * (int64_t)r.items) {
+        run->delta[i] = distance;
+      } else if (distance != run->delta[i] * index) {
         regular = false;
       }
     }
     if (!regular) break;
-    ++r.items;
+    run->members.push_back(member);
+    run->dispatches += member.dispatches;
   }
-  *run = r;
-  if (r.items < 2) return false;
+  if (run->members.size() < 2) return false;
   // Nothing a member writes may be something another member reads or writes.
+  const LaneMember &head = run->members[0];
   std::unordered_set<uint64_t> read;
-  for (uint32_t i = 0; i < 3; ++i) read.insert(d0.inputs[i].buffer);
-  read.insert(d0.inputs[4].buffer);
-  read.insert(d0.outputs[1].buffer);
-  read.insert(d0.outputs[2].buffer);
+  for (const fh_tensor *t : {&head.q, &head.k_new, &head.v_new, &head.generations, &head.key_pool,
+                             &head.value_pool})
+    read.insert(t->buffer);
   struct Span {
     uint64_t buffer, lo, hi;
   };
   std::vector<Span> written;
-  written.reserve((size_t)r.items * r.step);
-  for (uint32_t item = 0; item < r.items; ++item) {
-    const fh_dispatch &m = d[first + item * r.step];
-    read.insert(m.inputs[3].buffer);
-    if (m.n_inputs == 6) read.insert(m.inputs[5].buffer);
-    uint64_t row = (uint64_t)m.outputs[0].shape[0] * m.outputs[0].shape[2];
-    written.push_back({m.outputs[0].buffer, m.outputs[0].offset, m.outputs[0].offset + row});
-    if (r.step == 2) {
-      const fh_tensor &target = d[first + item * r.step + 1].outputs[0];
-      written.push_back({target.buffer, target.offset, target.offset + row});
-    }
+  written.reserve(run->members.size() * 2);
+  for (const LaneMember &m : run->members) {
+    read.insert(m.table.buffer);
+    if (m.has_activity) read.insert(m.activity.buffer);
+    const uint64_t row = (uint64_t)m.out.shape[0] * m.out.shape[2];
+    written.push_back({m.out.buffer, m.out.offset, m.out.offset + row});
+    if (m.has_copy)
+      written.push_back({m.copy_target.buffer, m.copy_target.offset, m.copy_target.offset + row});
   }
   for (const Span &span : written)
     if (read.count(span.buffer)) return false;
@@ -1305,15 +1406,13 @@ bool find_lane_run(const fh_dispatch *d, uint32_t count, uint32_t first, LaneRun
   return true;
 }
 
-// Executes the run found by find_lane_run.  `errors` is the first member's record; member i's is
-// errors[i * run.step].
-fh_status run_lane_group(fh_backend *b, const fh_dispatch *d, uint32_t first, const LaneRun &run,
-                         ErrorSlot *errors) {
-  const fh_dispatch &d0 = d[first];
-  const fh_tensor &q0 = d0.inputs[0], &out0 = d0.outputs[0], &kp = d0.outputs[1],
-                  &vp = d0.outputs[2], &table0 = d0.inputs[3];
-  const uint32_t lanes = run.items, heads = q0.shape[0];
-  const uint32_t table_pages = table0.shape[0], table_words = table_pages * 2;
+// Executes the run found by find_lane_run.  `errors` is the record of the run's first dispatch;
+// member i's records start at errors[i * dispatches per member].
+fh_status run_lane_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors) {
+  const LaneMember &head = run.members[0];
+  const fh_tensor &q0 = head.q, &out0 = head.out, &kp = head.key_pool, &vp = head.value_pool;
+  const uint32_t lanes = (uint32_t)run.members.size(), heads = q0.shape[0];
+  const uint32_t table_pages = head.table.shape[0], table_words = table_pages * 2;
   const uint64_t row_bytes = (uint64_t)heads * out0.shape[2] * dtype_size(out0.dtype);
   FH_REQUIRE(row_bytes < (1ull << 31));
   const uint64_t metadata_words = (uint64_t)lanes * table_words + 3ull * lanes + 1;
@@ -1331,14 +1430,14 @@ fh_status run_lane_group(fh_backend *b, const fh_dispatch *d, uint32_t first, co
   key.reserve(5ull * lanes + 2);
   key.push_back(lanes);
   key.push_back(table_words);
-  for (uint32_t item = 0; item < lanes; ++item) {
-    const fh_dispatch &m = d[first + item * run.step];
-    key.push_back(m.inputs[3].buffer);
-    key.push_back(m.inputs[3].offset);
-    key.push_back(m.n_inputs == 6 ? m.inputs[5].buffer : 0);
-    key.push_back(m.n_inputs == 6 ? m.inputs[5].offset : 0);
+  for (const LaneMember &m : run.members) {
+    key.push_back(m.table.buffer);
+    key.push_back(m.table.offset);
+    key.push_back(m.has_activity ? m.activity.buffer : 0);
+    key.push_back(m.has_activity ? m.activity.offset : 0);
     key.push_back(m.q_start);
   }
+  fh_status status;
   if (!(b->lane_metadata_valid && key == b->lane_metadata_key)) {
     b->lane_metadata_valid = false;
     b->attention_plan_valid = false;  // the plan was built from the metadata replaced here
@@ -1347,17 +1446,15 @@ fh_status run_lane_group(fh_backend *b, const fh_dispatch *d, uint32_t first, co
       uint32_t chunk = std::min<uint32_t>(kLaneChunk, lanes - base);
       LaneSources sources{};
       for (uint32_t local = 0; local < chunk; ++local) {
-        const fh_dispatch &m = d[first + (base + local) * run.step];
+        const LaneMember &m = run.members[base + local];
         View table, flag;
-        fh_status status = make_view(b, m.inputs[3], false, &table);
-        if (status != FH_OK) return status;
+        if ((status = make_view(b, m.table, false, &table)) != FH_OK) return status;
         sources.table[local] = (const uint32_t *)table.base + table.offset;
-        b->lane_metadata_watch.insert(m.inputs[3].buffer);
-        if (m.n_inputs == 6) {
-          status = make_view(b, m.inputs[5], false, &flag);
-          if (status != FH_OK) return status;
+        b->lane_metadata_watch.insert(m.table.buffer);
+        if (m.has_activity) {
+          if ((status = make_view(b, m.activity, false, &flag)) != FH_OK) return status;
           sources.activity[local] = (const uint32_t *)flag.base + flag.offset;
-          b->lane_metadata_watch.insert(m.inputs[5].buffer);
+          b->lane_metadata_watch.insert(m.activity.buffer);
         }
         sources.start[local] = m.q_start;
       }
@@ -1388,20 +1485,19 @@ fh_status run_lane_group(fh_backend *b, const fh_dispatch *d, uint32_t first, co
   };
   RaggedAttention problem{};
   // q [heads, 1, D] per member -> [lanes, heads, D]; k_new / v_new [1, Hkv, D] -> [lanes, Hkv, D].
-  fh_status status = make_view(b, q0, false, &problem.q);
-  if (status != FH_OK) return status;
+  if ((status = make_view(b, q0, false, &problem.q)) != FH_OK) return status;
   problem.q.shape[0] = lanes;
   problem.q.shape[1] = heads;
   problem.q.stride[0] = (uint64_t)run.delta[0];
   problem.q.stride[1] = q0.stride[0];
   View *appended[2] = {&problem.k_new, &problem.v_new};
+  const fh_tensor *appended_from[2] = {&head.k_new, &head.v_new};
   for (uint32_t i = 0; i < 2; ++i) {
-    status = make_view(b, d0.inputs[1 + i], false, appended[i]);
-    if (status != FH_OK) return status;
+    if ((status = make_view(b, *appended_from[i], false, appended[i])) != FH_OK) return status;
     appended[i]->shape[0] = lanes;
     appended[i]->stride[0] = (uint64_t)run.delta[1 + i];
   }
-  if ((status = make_view(b, d0.inputs[4], false, &problem.generations)) != FH_OK) return status;
+  if ((status = make_view(b, head.generations, false, &problem.generations)) != FH_OK) return status;
   if ((status = make_view(b, kp, true, &problem.key_pool)) != FH_OK) return status;
   if ((status = make_view(b, vp, true, &problem.value_pool)) != FH_OK) return status;
   problem.tables = device_view((char *)tables, FH_U32, {lanes, table_pages, 2});
@@ -1415,33 +1511,32 @@ fh_status run_lane_group(fh_backend *b, const fh_dispatch *d, uint32_t first, co
   problem.kv_heads = kp.shape[2];
   problem.width = q0.shape[2];
   problem.value_width = vp.shape[3];
-  problem.page_tokens = d0.page_tokens;
+  problem.page_tokens = head.page_tokens;
   problem.physical_pages = kp.shape[0];
   problem.table_pages = table_pages;
-  problem.scale = d0.scale;
-  problem.metadata_buffers[4] = d0.inputs[4].buffer;  // the rest is watched through the gather
-  problem.error_stride = run.step;
-  // The last query row of a member sits at q_start; serial execution refuses a start at the
-  // sentinel before anything runs, and validation has done the same here.
+  problem.scale = head.scale;
+  problem.metadata_buffers[4] = head.generations.buffer;  // the rest is watched through the gather
+  problem.error_stride = head.dispatches;
+  problem.attention_error_offset = head.attention_at;
   if (!run_ragged_attention(b, problem, errors)) return FH_ALLOCATION_FAILED;
 
   for (uint32_t base = 0; base < lanes; base += kLaneChunk) {
     uint32_t chunk = std::min<uint32_t>(kLaneChunk, lanes - base);
     LaneRows targets{};
     for (uint32_t local = 0; local < chunk; ++local) {
-      uint32_t at = first + (base + local) * run.step;
+      const LaneMember &m = run.members[base + local];
       View row;
-      if ((status = make_view(b, d[at].outputs[0], true, &row)) != FH_OK) return status;
+      if ((status = make_view(b, m.out, true, &row)) != FH_OK) return status;
       targets.first[local] = row.base + row.offset * dtype_size(row.dtype);
-      if (run.step == 2) {
-        if ((status = make_view(b, d[at + 1].outputs[0], true, &row)) != FH_OK) return status;
+      if (m.has_copy) {
+        if ((status = make_view(b, m.copy_target, true, &row)) != FH_OK) return status;
         targets.second[local] = row.base + row.offset * dtype_size(row.dtype);
       }
     }
     launch_scatter_lane_rows(b->stream, targets, rows, base, chunk, (uint32_t)row_bytes);
   }
   b->fused_runs += 1;
-  b->fused_dispatches += (uint64_t)run.items * run.step;
+  b->fused_dispatches += run.dispatches;
   return FH_OK;
 }
 
@@ -1844,12 +1939,13 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   for (uint32_t i = 0; i < count && status == FH_OK;) {
     uint32_t consumed = 1;
     LaneRun run;
-    bool fused = b->lane_fusion && dispatches[i].op == FH_OP_PAGED_SDPA_APPEND &&
+    const uint32_t op = dispatches[i].op;
+    bool fused = b->lane_fusion && (op == FH_OP_PAGED_SDPA_APPEND || op == FH_OP_PAGED_COPY) &&
                  i >= no_run_before && find_lane_run(dispatches, count, i, &run);
     if (fused)
-      consumed = run.items * run.step;
-    else if (run.items > 1)
-      no_run_before = i + run.items * run.step;
+      consumed = run.dispatches;
+    else if (run.members.size() > 1)
+      no_run_before = i + run.dispatches;
     for (uint32_t member = 0; member < consumed; ++member) s->ops[i + member] = dispatches[i + member].op;
     hipEvent_t t0 = nullptr, t1 = nullptr;
     if (b->profiling >= 2) {
@@ -1858,13 +1954,13 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
       (void)hipEventRecord(t0, b->stream);
     }
     if (fused)
-      status = run_lane_group(b, dispatches, i, run, &s->device_errors[i]);
+      status = run_lane_group(b, run, &s->device_errors[i]);
     else
       status = process(b, dispatches[i], &s->device_errors[i], true);
     for (uint32_t member = 0; member < consumed; ++member) note_outputs(dispatches[i + member]);
     if (b->profiling >= 2) {
       (void)hipEventRecord(t1, b->stream);
-      b->timed.push_back({t0, t1, kernel_class_of(dispatches[i].op)});
+      b->timed.push_back({t0, t1, fused ? (uint32_t)FH_KC_ATTENTION : kernel_class_of(dispatches[i].op)});
     }
     i += consumed;
   }

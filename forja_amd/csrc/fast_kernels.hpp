@@ -101,6 +101,9 @@ struct RaggedAttention {
   // A failure of query token t is recorded in error[t * error_stride]: 0 for one dispatch, the
   // distance between the member dispatches' records when a run of per-lane dispatches is fused.
   uint32_t error_stride;
+  // ... and failures of the attention proper (as opposed to the append) that many records further
+  // on: the position of the attention dispatch within a fused member.
+  uint32_t attention_error_offset;
 };
 // Always handles the problem (specialised kernel when the layout allows, generic otherwise);
 // false only when workspace allocation fails.

@@ -1065,8 +1065,9 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   return true;
 }
 
-bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSlot *error) {
+bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSlot *append_error) {
   hipStream_t stream = backend_stream(backend);
+  ErrorSlot *error = append_error ? append_error + p.attention_error_offset : nullptr;
   const bool fast = fast_ragged_eligible(p);
   FastRagged f{};
   if (fast) {
@@ -1117,9 +1118,10 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
       (uint64_t)p.tokens * (p.kv_heads * p.width + p.kv_heads * p.value_width);
   if (append_by_pieces(p))
     ragged_append_pieces_kernel<<<dim3((unsigned)((append_work / 8 + 255) / 256)), 256, 0, stream>>>(
-        p, error);
+        p, append_error);
   else
-    ragged_append_kernel<<<dim3((unsigned)((append_work + 255) / 256)), 256, 0, stream>>>(p, error);
+    ragged_append_kernel<<<dim3((unsigned)((append_work + 255) / 256)), 256, 0, stream>>>(
+        p, append_error);
   if (fast) {
     launch_fast(backend, stream, f, error);
     return true;

@@ -235,8 +235,10 @@ FH_API fh_status fh_profile_read(fh_backend *backend, uint32_t kernel_class, uin
                           uint64_t *launches);
 
 /* Fusion of per-lane attention dispatches.  The engines record a decode batch as one
- * Op::PagedSdpaAppend per lane and layer, each followed by the Op::Copy of its output row into the
- * packed activation (engines/qwen3-coder/src/lib.rs:917-935).  fh_submit recognises such a run and
+ * Op::PagedSdpaAppend per lane and layer (engines/qwen3-coder/src/lib.rs:917-935), or as two
+ * Op::PagedCopy{IntoPages} plus one Op::PagedSdpa over a single query row
+ * (engines/qwen38/src/attention/batch.rs:37-53), each followed by the Op::Copy of the lane's
+ * output row into the packed activation.  fh_submit recognises such a run and
  * executes it as one ragged attention launch with the result serial execution gives; a run it
  * cannot prove independent is executed dispatch by dispatch.  On by default.  The Backend trait
  * has no switch for this (the Metal backend fuses in its encoder,

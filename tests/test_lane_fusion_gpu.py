@@ -9,7 +9,7 @@ import math
 import numpy as np
 import pytest
 
-from forja_amd.core import BackendError, CommandList, DType, Op, Status
+from forja_amd.core import BackendError, CommandList, DType, Op, Status, INTO_PAGES
 from oracle import cpu_backend as orc
 from tests.helpers import assert_close, normal_bf16, to_f32, upload
 
@@ -60,8 +60,10 @@ class LaneBatch:
         self.dtype = dtype
         self.lanes = lanes
 
-    def record_layer(self, commands, layer, starts=None, copy_rows=True, lanes=None):
-        """Appends the per-lane dispatches of one layer; returns (packed attended, lane rows)."""
+    def record_layer(self, commands, layer, starts=None, copy_rows=True, lanes=None, idiom="append"):
+        """Appends the per-lane dispatches of one layer; returns (packed attended, lane rows).
+        idiom "append": Op::PagedSdpaAppend per lane; "copies": two Op::PagedCopy{IntoPages} and
+        one Op::PagedSdpa per lane (engines/qwen38/src/attention/batch.rs:37-53)."""
         backend, hq = self.backend, self.hq
         starts = self.contexts if starts is None else starts
         scale = 1.0 / math.sqrt(WIDTH)
@@ -74,8 +76,18 @@ class LaneBatch:
                       self.v.narrow(0, lane, 1), self.tables[lane], self.generations]
             if self.activity is not None:
                 inputs.append(self.activity.narrow(0, lane, 1))
-            commands.dispatch_many(Op.paged_sdpa_append(scale, starts[lane], self.pt), inputs,
-                                   [row.permute([1, 0, 2]), keys, values])
+            if idiom == "append":
+                commands.dispatch_many(Op.paged_sdpa_append(scale, starts[lane], self.pt), inputs,
+                                       [row.permute([1, 0, 2]), keys, values])
+            else:
+                physical, elements = keys.shape[0], self.hkv * WIDTH
+                paging = inputs[3:]
+                for new_row, pool in ((inputs[1], keys), (inputs[2], values)):
+                    commands.dispatch(Op.paged_copy(INTO_PAGES, starts[lane], self.pt),
+                                      [new_row.reshape((1, elements)), *paging],
+                                      pool.reshape((physical, self.pt, elements)))
+                commands.dispatch(Op.paged_sdpa(scale, True, starts[lane], starts[lane] + 1, self.pt),
+                                  [inputs[0], keys, values, *paging], row.permute([1, 0, 2]))
             if copy_rows:
                 commands.dispatch(Op.copy(), [row.reshape((1, hq * WIDTH))], attended.narrow(0, lane, 1))
             rows.append(row)
@@ -99,8 +111,9 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("idiom", ["append", "copies"])
 @pytest.mark.parametrize("contexts,hq,hkv,pt", CASES)
-def test_lane_by_lane_batch_equals_serial_execution(cpu, hip, contexts, hq, hkv, pt):
+def test_lane_by_lane_batch_equals_serial_execution(cpu, hip, contexts, hq, hkv, pt, idiom):
     """Two layers on the same lanes (the second reuses the gathered metadata), fused on the
     device, serial on the oracle; pools bit for bit, attention rows to the float bar; then the
     library's own serial execution of the same list."""
@@ -113,13 +126,13 @@ def test_lane_by_lane_batch_equals_serial_execution(cpu, hip, contexts, hq, hkv,
         commands = CommandList()
         kept = []
         for layer in range(2):
-            attended, rows = batch.record_layer(commands, layer)
+            attended, rows = batch.record_layer(commands, layer, idiom=idiom)
             kept += [attended, rows[0], rows[-1], *batch.pools[layer]]
         run(backend, commands)
         outputs[name] = (backend, kept)
         runs, dispatches = (after - start for after, start in zip(hip.fusion_stats(), before))
         if name == "fused":
-            assert (runs, dispatches) == (2, 2 * 2 * len(contexts))
+            assert (runs, dispatches) == (2, 2 * (2 if idiom == "append" else 4) * len(contexts))
         else:
             assert (runs, dispatches) == (0, 0)
     hip.fusion_enable(True)
@@ -167,19 +180,24 @@ def test_gathered_metadata_follows_a_table_rewritten_between_layers(cpu, hip):
     check(cpu, hip, results[0], results[1], exact=(3, 4, 5, 6))
 
 
-def test_a_stale_page_is_reported_for_the_lane_that_holds_it(hip):
+@pytest.mark.parametrize("idiom,corrupt,expected", [
+    ("append", (2, 1), (4, 1)),      # stale history page: lane 2's attention dispatch, page 1
+    ("copies", (2, 1), (10, 1)),     # ... which is the third of its four dispatches
+    ("copies", (1, 4), (4, 4)),      # stale page under the appended row: lane 1's first copy
+])
+def test_a_stale_page_is_reported_for_the_dispatch_that_meets_it(hip, idiom, corrupt, expected):
     indices = []
     for fused in (True, False):
         hip.fusion_enable(fused)
-        batch = LaneBatch(hip, [33, 70, 50, 5], 8, 4, 16, seed=74, corrupt=(2, 1))
+        batch = LaneBatch(hip, [33, 70, 50, 5], 8, 4, 16, seed=74, corrupt=corrupt)
         commands = CommandList()
-        attended, rows = batch.record_layer(commands, 0)
+        attended, rows = batch.record_layer(commands, 0, idiom=idiom)
         with pytest.raises(BackendError) as info:
             run(hip, commands)
         assert info.value.status == Status.DEVICE_ERROR_FLAG
         indices.append((info.value.dispatch, info.value.index))
     hip.fusion_enable(True)
-    assert indices[0] == indices[1] == (4, 1)      # lane 2's attention dispatch, logical page 1
+    assert indices[0] == indices[1] == expected
 
 
 def test_runs_that_cannot_be_proved_independent_are_executed_serially(cpu, hip):

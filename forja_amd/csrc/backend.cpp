@@ -1398,6 +1398,14 @@ bool find_lane_run(const fh_dispatch *d, uint32_t count, uint32_t first, LaneRun
   }
   for (const Span &span : written)
     if (read.count(span.buffer)) return false;
+  // Two members on one table would append to the same slot: order matters, so no fusion.
+  {
+    std::vector<std::pair<uint64_t, uint64_t>> tables;
+    tables.reserve(run->members.size());
+    for (const LaneMember &m : run->members) tables.push_back({m.table.buffer, m.table.offset});
+    std::sort(tables.begin(), tables.end());
+    if (std::adjacent_find(tables.begin(), tables.end()) != tables.end()) return false;
+  }
   std::sort(written.begin(), written.end(), [](const Span &a, const Span &b) {
     return a.buffer != b.buffer ? a.buffer < b.buffer : a.lo < b.lo;
   });

@@ -223,3 +223,87 @@ def test_runs_that_cannot_be_proved_independent_are_executed_serially(cpu, hip):
         if backend is hip:
             assert hip.fusion_stats() == before
     check(cpu, hip, results[0], results[1], exact=(1, 2))
+
+
+def _random_scenario(rng):
+    """A decode batch recorded with random deviations from the regular pattern; every list is
+    valid dispatch by dispatch, only some of it can be fused."""
+    lanes = int(rng.integers(2, 10))
+    return dict(
+        contexts=[int(c) for c in rng.integers(0, 200, lanes)],
+        hq=int(rng.choice([4, 8, 16])), hkv=int(rng.choice([2, 4])),
+        idiom=str(rng.choice(["append", "copies"])),
+        copy_rows=bool(rng.integers(0, 2)),
+        activity=[int(a) for a in (rng.random(lanes) > 0.2)] if rng.integers(0, 2) else None,
+        order=[int(l) for l in (rng.permutation(lanes) if rng.integers(0, 3) == 0 else np.arange(lanes))],
+        repeat=bool(rng.integers(0, 4) == 0),          # one lane recorded twice in a row
+        shared_row=bool(rng.integers(0, 4) == 0),      # two lanes write the same output row
+        f32_rows=bool(rng.integers(0, 4) == 0),        # outputs in another dtype than q
+        interloper=bool(rng.integers(0, 3) == 0))      # an unrelated dispatch in the middle
+
+
+def _record_scenario(backend, scenario, seed):
+    batch = LaneBatch(backend, scenario["contexts"], scenario["hq"], scenario["hkv"], 16, seed,
+                      activity=scenario["activity"])
+    hq, scale = scenario["hq"], 1.0 / math.sqrt(WIDTH)
+    row_dtype = DType.F32 if scenario["f32_rows"] else DType.BF16
+    attended = backend.alloc(row_dtype, (batch.lanes, hq * WIDTH))
+    other = backend.alloc(DType.BF16, (4, 4))
+    keys, values = batch.pools[0]
+    commands = CommandList()
+    rows = {}
+    order = list(scenario["order"])
+    if scenario["repeat"]:
+        order.insert(1, order[0])
+    for position, lane in enumerate(order):
+        if scenario["shared_row"] and position == 1 and 0 in rows:
+            row = rows[0]
+        else:
+            row = backend.alloc(row_dtype, (1, hq, WIDTH))
+        rows[position] = row
+        start = scenario["contexts"][lane]
+        inputs = [batch.q.narrow(0, lane, 1).permute([1, 0, 2]), batch.k.narrow(0, lane, 1),
+                  batch.v.narrow(0, lane, 1), batch.tables[lane], batch.generations]
+        if batch.activity is not None:
+            inputs.append(batch.activity.narrow(0, lane, 1))
+        if scenario["idiom"] == "append":
+            commands.dispatch_many(Op.paged_sdpa_append(scale, start, 16), inputs,
+                                   [row.permute([1, 0, 2]), keys, values])
+        else:
+            physical, elements = keys.shape[0], scenario["hkv"] * WIDTH
+            for new_row, pool in ((inputs[1], keys), (inputs[2], values)):
+                commands.dispatch(Op.paged_copy(INTO_PAGES, start, 16),
+                                  [new_row.reshape((1, elements)), *inputs[3:]],
+                                  pool.reshape((physical, 16, elements)))
+            commands.dispatch(Op.paged_sdpa(scale, True, start, start + 1, 16),
+                              [inputs[0], keys, values, *inputs[3:]], row.permute([1, 0, 2]))
+        if scenario["copy_rows"]:
+            commands.dispatch(Op.copy(), [row.reshape((1, hq * WIDTH))], attended.narrow(0, lane, 1))
+        if scenario["interloper"] and position == len(order) // 2:
+            commands.dispatch(Op.copy(), [other], backend.alloc(DType.BF16, (4, 4)))
+    return commands, [attended, keys, values] + [rows[p] for p in sorted(rows)]
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_recordings_give_the_same_result_fused_and_dispatch_by_dispatch(cpu, hip, seed):
+    """Random lane orders, repeated lanes, shared output rows, other output dtypes and foreign
+    dispatches in the middle: whatever part of the list the library fuses, pools are bit for bit
+    what its own serial execution leaves and rows agree to the float bar; the first eight seeds
+    are also held to the oracle."""
+    scenario = _random_scenario(np.random.default_rng(1000 + seed))
+    results = {}
+    for name, backend in (("fused", hip), ("serial", hip)) + ((("cpu", cpu),) if seed < 8 else ()):
+        if backend is hip:
+            hip.fusion_enable(name == "fused")
+        commands, tensors = _record_scenario(backend, scenario, 200 + seed)
+        before = hip.fusion_stats()[0]
+        run(backend, commands)
+        results[name] = tensors
+        regular = scenario["order"] == sorted(scenario["order"]) and not scenario["repeat"] \
+            and not scenario["shared_row"]
+        if name == "fused" and regular:
+            assert hip.fusion_stats()[0] > before
+    hip.fusion_enable(True)
+    check(hip, hip, results["serial"], results["fused"], exact=(1, 2))
+    if "cpu" in results:
+        check(cpu, hip, results["cpu"], results["fused"], exact=(1, 2))

@@ -58,7 +58,8 @@ PARAMETERS = [
 
 
 @pytest.mark.parametrize("rows,width,kind", [(5, 7, "plain"), (3, 1025, "ties"), (4, 4097, "specials"),
-                                              (8, 151936, "plain"), (2, 151936, "ties")])
+                                              (8, 151936, "plain"), (2, 151936, "ties"),
+                                              (300, 333, "ties")])    # more rows than workgroups
 def test_sampled_indices_equal_the_oracle(cpu, hip, rows, width, kind):
     values = logits_case(rows, width, 101, kind)
     for number, (temperature, top_k, top_p) in enumerate(PARAMETERS):

@@ -779,7 +779,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_
   const uint32_t first_page = begin / pt, last_page = (end - 1) / pt;
   for (uint32_t page0 = first_page; page0 <= last_page; page0 += 64) {
     // Authenticate up to 64 table entries at once (every wave for itself: same entries, same
-    // verdict); nothing is dereferenced through a bad one.
+    // result); nothing is dereferenced through a bad one.
     uint32_t my_page = page0 + lane, physical = 0;
     bool mine = my_page <= last_page, ok = true;
     if (mine) {

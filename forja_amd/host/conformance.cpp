@@ -131,6 +131,47 @@ void top_k_normalises(HipBackend &backend) {
         "top-k normalised weights");
 }
 
+// sample_refuses_invalid_live_parameters, crates/forja-cpu/src/lib.rs:2664-2686 (a NaN temperature
+// read when the dispatch runs is InvalidInput), the greedy rule of sample_allowed (:1605-1614:
+// temperature 0 takes the largest value, the largest index among equals), and
+// top_k_and_top_p_keep_only_the_exact_allowed_set (:2536-2547): with top_k 3 over
+// [10,9,8,1,0,-1,-2] every draw is one of the first three.
+void sampling_known_answers(HipBackend &backend) {
+  Tensor logits = upload<float>(backend, DType::F32, {7}, {10.0f, 9.0f, 8.0f, 1.0f, 0.0f, -1.0f, -2.0f});
+  Tensor out = backend.alloc(DType::U32, {1}).value;
+  auto bits = [](float value) {
+    uint32_t word;
+    std::memcpy(&word, &value, 4);
+    return word;
+  };
+  auto draw = [&](const std::vector<uint32_t> &words, uint32_t position, uint32_t *index) {
+    Tensor params = upload<uint32_t>(backend, DType::U32, {5}, words);
+    CommandList commands;
+    commands.dispatch(Op::sample(position), {logits, params}, {out});
+    BackendError error = run(backend, commands);
+    Result<std::vector<uint8_t>> bytes = backend.read(out);
+    std::memcpy(index, bytes.value.data(), 4);
+    return error;
+  };
+  uint32_t index = 99;
+  check(draw({bits(NAN), 0, bits(1.0f), 0, 0}, 0, &index).code == FH_INVALID_INPUT,
+        "NaN temperature is refused when the dispatch runs");
+  check(draw({bits(0.0f), 0, bits(1.0f), 0, 0}, 0, &index).ok() && index == 0, "greedy sample");
+  Tensor ties = upload<float>(backend, DType::F32, {5}, {1.0f, 9.0f, 2.0f, 9.0f, 3.0f});
+  Tensor params = upload<uint32_t>(backend, DType::U32, {5}, {bits(0.0f), 0, bits(1.0f), 0, 0});
+  CommandList commands;
+  commands.dispatch(Op::sample(0), {ties, params}, {out});
+  check(run(backend, commands).ok(), "greedy sample over ties runs");
+  std::memcpy(&index, backend.read(out).value.data(), 4);
+  check(index == 3, "greedy sample picks the last of equal maxima");
+  bool inside = true;
+  for (uint32_t position = 0; position < 64; ++position) {
+    check(draw({bits(1.0f), 3, bits(1.0f), 11, 0}, position, &index).ok(), "top-k sample runs");
+    inside = inside && index <= 2;
+  }
+  check(inside, "top_k 3 keeps the draws inside the three largest");
+}
+
 // paged_append_stores_both_planes_before_attention, crates/forja-cpu/src/lib.rs:1926-1970: all-ones
 // V gives output exactly 1.0; the first 2048 bytes of the f16 value pool are f16(1.0), the rest 0.
 void paged_append_stores_both_planes(HipBackend &backend) {
@@ -219,6 +260,7 @@ int main() {
   quant_matmul_known_answers(backend);
   argmax_prefers_last(backend);
   top_k_normalises(backend);
+  sampling_known_answers(backend);
   paged_append_stores_both_planes(backend);
   paged_attention_hand_checked(backend);
   write_and_release_contract(backend);

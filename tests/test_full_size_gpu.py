@@ -208,3 +208,24 @@ def test_config1_packed_batch_attention(hip):
 def test_config4_prefill_attention_largest_prompt(hip):
     """The 3072-token prompt of the config 4 chunk plus decode rows, 40 query / 8 kv heads."""
     attention_both_ways(hip, [0, 1500, 4000], [3072, 1, 1], 40, 8)
+
+
+def test_config3_step_recorded_lane_by_lane_equals_the_packed_recording(hip):
+    """Two layers of the config 3 model on 128 lanes with contexts log-uniform over 256..32768:
+    the step recorded the way the engines record it (per lane one PagedSdpaAppend and one Copy per
+    layer) goes through the library's run fusion and must give the packed recording's tokens and
+    logits bit for bit over several steps, with every layer's run fused."""
+    from forja_amd.model import QWEN3_CODER_30B_A3B, DecodeSession, Model
+    rng = np.random.default_rng(9)
+    contexts = np.exp(rng.uniform(math.log(256), math.log(32768), 128)).astype(int).tolist()
+    packed, by_lane = (DecodeSession(Model(hip, QWEN3_CODER_30B_A3B, seed=21, layers=2), contexts, seed=21)
+                       for _ in range(2))
+    by_lane.record_lane_by_lane()
+    before = hip.fusion_stats()
+    for _ in range(3):
+        expected = packed.step()
+        actual = by_lane.step(lane_by_lane=True)
+        assert expected.tolist() == actual.tolist()
+    assert hip.read(packed.buffers.logits) == hip.read(by_lane.buffers.logits)
+    runs, replaced = (after - start for after, start in zip(hip.fusion_stats(), before))
+    assert (runs, replaced) == (3 * 2, 3 * 2 * 2 * 128)

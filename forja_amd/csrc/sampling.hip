@@ -14,7 +14,7 @@
 //     their own value as score.
 //
 // One workgroup of 1024 threads per row.  Ordering work is only done when the cut needs it: no
-// ordering for "all candidates, top_p = 1"; up to 64 candidates are extracted largest first by
+// ordering for "all candidates, top_p = 1"; up to 256 candidates are extracted largest first by
 // repeated block-wide maxima; more than that takes a stable LSD radix sort of (value key, index)
 // pairs in global scratch, after which one lane walks the sums through LDS-staged weights.
 // exp and ln are evaluated in f64 and rounded to f32, i.e. the correctly rounded f32 functions up
@@ -29,7 +29,7 @@ namespace {
 
 constexpr uint32_t kSampleThreads = 1024;
 constexpr uint32_t kSampleWaves = kSampleThreads / 64;
-constexpr uint32_t kSmallCandidates = 64;
+constexpr uint32_t kSmallCandidates = 256;
 constexpr uint32_t kStage = 4096;
 
 struct SampleArgs {
@@ -120,27 +120,52 @@ struct Row {
   __device__ bool allowed(uint32_t index) const {
     return a.allow == nullptr || ((a.allow[index >> 5] >> (index & 31)) & 1u) != 0;
   }
-  // visit(index, value) for every allowed column, each exactly once, in no particular order
+  // The columns of the row are dealt to the 1024 threads in fixed hands (eight adjacent columns
+  // at a time where the row can be read in 16-byte pieces).  visit(index, value) for every
+  // allowed column of thread `owner`'s hand, taking pieces first, first + step, ...
   template <typename Visit>
-  __device__ void for_each_allowed(Visit visit) const {
+  __device__ void for_hand(uint32_t owner, uint32_t first, uint32_t step, Visit visit) const {
     uint32_t done = 0;
     if (vector) {
       const uint16_t *x = (const uint16_t *)a.logits.base + base;
       done = a.width & ~7u;
-      for (uint32_t c = threadIdx.x * 8; c < done; c += kSampleThreads * 8) {
+#pragma unroll 4
+      for (uint64_t c = owner * 8 + (uint64_t)first * kSampleThreads * 8; c < done;
+           c += (uint64_t)step * kSampleThreads * 8) {
         const uint4 v = *(const uint4 *)(x + c);
         const uint32_t words[4] = {v.x, v.y, v.z, v.w};
         const uint32_t permitted = a.allow ? (a.allow[c >> 5] >> (c & 31)) & 0xffu : 0xffu;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          if ((permitted >> (2 * i)) & 1u) visit(c + 2 * i, __uint_as_float(words[i] << 16));
+          if ((permitted >> (2 * i)) & 1u)
+            visit((uint32_t)c + 2 * i, __uint_as_float(words[i] << 16));
           if ((permitted >> (2 * i + 1)) & 1u)
-            visit(c + 2 * i + 1, __uint_as_float(words[i] & 0xffff0000u));
+            visit((uint32_t)c + 2 * i + 1, __uint_as_float(words[i] & 0xffff0000u));
         }
       }
     }
-    for (uint32_t index = done + threadIdx.x; index < a.width; index += kSampleThreads)
-      if (allowed(index)) visit(index, value(index));
+    for (uint64_t index = done + owner + (uint64_t)first * kSampleThreads; index < a.width;
+         index += (uint64_t)step * kSampleThreads)
+      if (allowed((uint32_t)index)) visit((uint32_t)index, value((uint32_t)index));
+  }
+  // visit(index, value) for every allowed column, each exactly once over the workgroup
+  template <typename Visit>
+  __device__ void for_each_allowed(Visit visit) const {
+    for_hand(threadIdx.x, 0, 1, visit);
+  }
+  // Largest candidate below `below` in the hand of thread `owner`, found by the calling wave
+  // together (one piece per lane at a time); every lane of the wave gets the result.
+  __device__ uint64_t best_of_hand_below(uint32_t owner, uint64_t below) const {
+    uint64_t next = 0;
+    for_hand(owner, threadIdx.x & 63, 64, [&](uint32_t index, float value) {
+      const uint64_t mine = candidate(value, index);
+      if (mine < below && mine > next) next = mine;
+    });
+    for (int offset = 32; offset > 0; offset >>= 1) {
+      const uint64_t other = __shfl_xor(next, offset, 64);
+      next = other > next ? other : next;
+    }
+    return next;
   }
 };
 
@@ -300,19 +325,27 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a, Er
       }
     }
     if (limit <= kSmallCandidates) {
-      // ---- the `limit` largest, extracted one by one in descending order
-      uint64_t below = ~0ull;
+      // ---- the `limit` largest, extracted one by one in descending order.  Every thread keeps
+      // the best of its own columns that is still below the last extracted candidate; a round is
+      // one block-wide maximum, after which the winner's wave looks through the winner's columns
+      // again, one piece per lane.
+      uint64_t local = 0;
+      row.for_each_allowed([&](uint32_t index, float value) {
+        const uint64_t mine = candidate(value, index);
+        local = mine > local ? mine : local;
+      });
       uint32_t count = 0;
       for (; count < limit; ++count) {
-        uint64_t best = 0;
-        row.for_each_allowed([&](uint32_t index, float value) {
-          const uint64_t mine = candidate(value, index);
-          if (mine < below && mine > best) best = mine;
-        });
-        best = block_max(best, s);
+        const uint64_t best = block_max(local, s);
         if (best == 0) break;
         if (threadIdx.x == 0) s.small[count] = best - 1;
-        below = best;
+        const unsigned long long owners = __ballot(local == best);   // one lane of one wave
+        if (owners != 0) {
+          const uint32_t owner_lane = (uint32_t)__ffsll((long long)owners) - 1;
+          const uint64_t next =
+              row.best_of_hand_below((threadIdx.x & ~63u) + owner_lane, best);
+          if ((threadIdx.x & 63) == owner_lane) local = next;
+        }
       }
       __syncthreads();
       if (top_p < 1.0f) {

@@ -49,8 +49,9 @@ PARAMETERS = [
     (1.3, 1, 0.4),        # greedy by top_k
     (0.7, 0, 1.0),        # every column competes
     (1.0, 20, 0.8),       # the usual serving setting: few candidates, nucleus cut
-    (1.0, 64, 1.0),       # the largest extracted set
-    (0.9, 65, 0.95),      # just past it: ordered through the radix passes
+    (1.0, 64, 1.0),
+    (0.9, 256, 0.95),     # the largest extracted set
+    (0.9, 257, 0.95),     # just past it: ordered through the radix passes
     (0.8, 1000, 0.9),
     (1.0, 0, 0.9),        # nucleus cut over the whole row
     (2.0, 5000, 1.0),     # top_k beyond the row for the narrow cases

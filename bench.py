@@ -565,7 +565,7 @@ def main():
             trace = backend.alloc(DType.U32, (workload.model.n_layers, args.lanes, config.top_k))
             traced = CommandList()
             record_step(workload.model, session.cache, session.buffers, traced, feed_back=True,
-                        route_trace=trace)
+                        route_trace=trace, one_row_per_lane=True)
             session.prepare_step()
             backend.submit(traced).wait()
             session.contexts += 1

@@ -406,8 +406,11 @@ class Op:
                   key_length=key_length, page_tokens=page_tokens)
 
     @staticmethod
-    def paged_attention_ragged(scale, page_tokens):
-        return Op(OpKind.PAGED_ATTENTION_RAGGED, scale=scale, page_tokens=page_tokens)
+    def paged_attention_ragged(scale, page_tokens, one_row_per_lane=False):
+        """`one_row_per_lane`: the recorder's promise that no lane brings more than one query row
+        (a decode batch); checked when the dispatch runs."""
+        return Op(OpKind.PAGED_ATTENTION_RAGGED, scale=scale, page_tokens=page_tokens,
+                  k=1 if one_row_per_lane else 0)
 
     @staticmethod
     def route_pack(tile_rows): return Op(OpKind.ROUTE_PACK, k=tile_rows)

@@ -1038,7 +1038,7 @@ fh_status plan_ragged(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
   FH_REQUIRE(lanes != 0 && shape_is(cu, {lanes + 1}) && shape_is(starts, {lanes}));
   if (d.n_inputs == 8) FH_REQUIRE(shape_is(d.inputs[7], {lanes}));
   FH_REQUIRE(shape_is(gens, {kp.shape[0]}));
-  FH_REQUIRE(std::isfinite(d.scale) && d.page_tokens != 0);
+  FH_REQUIRE(std::isfinite(d.scale) && d.page_tokens != 0 && d.k <= 1);
   FH_REQUIRE(kp.shape[1] == d.page_tokens && vp.shape[1] == d.page_tokens);
   FH_REQUIRE(vp.shape[0] == kp.shape[0] && vp.shape[2] == kp.shape[2]);
   FH_REQUIRE(kp.shape[2] != 0 && q.shape[1] % kp.shape[2] == 0 && q.shape[1] != 0);
@@ -1075,6 +1075,7 @@ fh_status plan_ragged(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
   problem.metadata_buffers[2] = d.n_inputs == 8 ? d.inputs[7].buffer : 0;
   problem.metadata_buffers[3] = d.inputs[3].buffer;
   problem.metadata_buffers[4] = d.inputs[4].buffer;
+  problem.one_row_per_lane = d.k == 1;
   if (!run_ragged_attention(b, problem, error)) return FH_ALLOCATION_FAILED;
   return FH_OK;
 }
@@ -1526,6 +1527,7 @@ fh_status run_lane_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors) {
   problem.metadata_buffers[4] = head.generations.buffer;  // the rest is watched through the gather
   problem.error_stride = head.dispatches;
   problem.attention_error_offset = head.attention_at;
+  problem.one_row_per_lane = 1;   // by construction: every member is one query row of its own lane
   if (!run_ragged_attention(b, problem, errors)) return FH_ALLOCATION_FAILED;
 
   for (uint32_t base = 0; base < lanes; base += kLaneChunk) {

@@ -34,7 +34,7 @@ char *backend_route_plan(fh_backend *backend, const RoutePlanKey &key, uint64_t 
 // per-token failure flags kept with the plan come from them) and every scalar it depends on.
 struct AttentionPlanKey {
   uint64_t buffers[5], address[5];
-  uint32_t params[10];
+  uint32_t params[12];
 };
 // Like backend_route_plan, for the work plan the attention dispatches of one submission share:
 // every layer of a step attends with the same lanes, starts and tables.
@@ -104,6 +104,10 @@ struct RaggedAttention {
   // ... and failures of the attention proper (as opposed to the append) that many records further
   // on: the position of the attention dispatch within a fused member.
   uint32_t attention_error_offset;
+  // The caller vouches that no lane brings more than one query row (checked on the device when
+  // the work plan is built; a violation is reported).  The attention kernel can then store a
+  // lane's new key and value row itself, because no other row's attention reads them.
+  uint32_t one_row_per_lane;
 };
 // Always handles the problem (specialised kernel when the layout allows, generic otherwise);
 // false only when workspace allocation fails.

@@ -58,6 +58,10 @@ __global__ void ragged_append_kernel(RaggedAttention p, ErrorSlot *error) {
   const uint32_t *cu = (const uint32_t *)p.cu_seqlens.base + p.cu_seqlens.offset;
   if (token < cu[0] || token >= cu[p.lanes]) return;
   uint32_t lane = find_lane(cu, p.lanes, token);
+  if (p.one_row_per_lane && token != cu[lane]) {   // a second row of a lane: the promise is broken
+    if (element == 0) report_error(error + (uint64_t)token * p.error_stride, token);
+    return;
+  }
   if (p.activity.base && ((const uint32_t *)p.activity.base)[p.activity.offset + lane] == 0) return;
   uint64_t position =
       (uint64_t)((const uint32_t *)p.q_starts.base)[p.q_starts.offset + lane] + (token - cu[lane]);
@@ -99,6 +103,10 @@ __global__ __launch_bounds__(256) void ragged_append_pieces_kernel(RaggedAttenti
   const uint32_t *cu = (const uint32_t *)p.cu_seqlens.base + p.cu_seqlens.offset;
   if (token < cu[0] || token >= cu[p.lanes]) return;
   const uint32_t lane = find_lane(cu, p.lanes, token);
+  if (p.one_row_per_lane && token != cu[lane]) {   // a second row of a lane: the promise is broken
+    if (piece == 0) report_error(error + (uint64_t)token * p.error_stride, token);
+    return;
+  }
   if (p.activity.base && ((const uint32_t *)p.activity.base)[p.activity.offset + lane] == 0) return;
   const uint64_t position =
       (uint64_t)((const uint32_t *)p.q_starts.base)[p.q_starts.offset + lane] + (token - cu[lane]);
@@ -278,6 +286,14 @@ struct FastRagged {
   // limit (every row attends exactly that many keys).
   uint32_t one_start, fixed_attended;
   uint32_t error_stride;  // failures of token t go to error[t * error_stride]
+  // In-kernel append (decode batches with one query row per lane): the workgroup of a lane's last
+  // split stores the lane's new key and value row before it attends.  k_new / v_new are
+  // [T, Hkv, 128] with unit innermost stride; append failures are recorded `append_error_back`
+  // records before the attention's.
+  const uint16_t *k_new, *v_new;
+  uint64_t kn_stride_t, kn_stride_h, vn_stride_t, vn_stride_h;
+  uint32_t append_in_kernel, append_error_back;
+  uint32_t promised;   // one query row per lane, vouched for by the caller: verified by the plan
 };
 
 // Work decomposition of one token.  Tokens of a lane are grouped `group_tokens` at a time; a
@@ -299,6 +315,10 @@ __device__ inline TokenPlan plan_token(const FastRagged &p, uint32_t token, uint
     first_of_lane = p.cu[plan.lane];
     lane_tokens = p.cu[plan.lane + 1] - first_of_lane;
     start = p.starts[plan.lane];
+    if (p.promised && lane_tokens > 1) {   // the caller's promise does not hold
+      plan.lane = 0xfffffffeu;
+      return plan;
+    }
   }
   const uint64_t index = token - first_of_lane;
   const uint64_t leader = index - index % p.group_tokens;
@@ -361,6 +381,10 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
     uint32_t bad = 0;
     if (plan.lane == 0xffffffffu) {
       report_error(error + (uint64_t)token * p.error_stride, p.table_pages);
+      bad = 1;
+      plan.lane = 0;
+    } else if (plan.lane == 0xfffffffeu) {
+      report_error(error + (uint64_t)token * p.error_stride, token);
       bad = 1;
       plan.lane = 0;
     }
@@ -541,6 +565,27 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
   const uint32_t end = min(longest, begin + plan.chunk);
   const uint32_t pt = p.page_tokens;
   const uint32_t *table = p.tables + (uint64_t)plan.lane * p.table_pages * 2;
+  if (NT == 1 && p.append_in_kernel && split + 1 == plan.splits) {
+    // This wave's kv head of the lane's new row goes into the pool before anything is read: the
+    // row sits at the last attended position, which only this workgroup's range contains.
+    const uint32_t position = plan.attended - 1, logical = position / pt;
+    uint32_t physical;
+    if (entry_ok(table, p.generations, logical, p.table_pages, p.physical_pages, &physical)) {
+      const uint64_t pool_row = (uint64_t)physical * pt + position % pt;
+      const uint64_t at = (pool_row * p.kv_heads + kv_head) * 128;
+      const uint32_t *k_from =
+          (const uint32_t *)(p.k_new + (uint64_t)leader * p.kn_stride_t + (uint64_t)kv_head * p.kn_stride_h);
+      const uint32_t *v_from =
+          (const uint32_t *)(p.v_new + (uint64_t)leader * p.vn_stride_t + (uint64_t)kv_head * p.vn_stride_h);
+      ((uint32_t *)(const_cast<uint16_t *>(p.key_pool) + at))[lane] = k_from[lane];
+      ((uint32_t *)(const_cast<uint16_t *>(p.value_pool) + at))[lane] = v_from[lane];
+      // the loads below come from the same wave, after the stores have completed
+      __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+    } else if (lane == 0) {
+      // not written; the page walk below meets the same entry and ends the workgroup
+      report_error(error - p.append_error_back + (uint64_t)leader * p.error_stride, logical);
+    }
+  }
   LaneConst lc;
   lc.row_elems = p.kv_heads * 128;
   lc.k_offset = (hl * p.kv_heads + kv_head) * 128 + 8 * g;
@@ -1097,10 +1142,12 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     key.address[2] = (uint64_t)f.activity;
     key.address[3] = (uint64_t)f.tables;
     key.address[4] = (uint64_t)f.generations;
-    const uint32_t params[10] = {f.tokens, f.lanes, f.group_tokens, f.page_tokens, f.physical_pages,
+    f.promised = p.one_row_per_lane;
+    f.append_in_kernel = p.one_row_per_lane && append_by_pieces(p);
+    const uint32_t params[12] = {f.tokens, f.lanes, f.group_tokens, f.page_tokens, f.physical_pages,
                                  f.table_pages, f.max_splits, forced_split_tokens(), f.kv_heads,
-                                 f.query_heads};
-    for (int i = 0; i < 10; ++i) key.params[i] = params[i];
+                                 f.query_heads, f.append_in_kernel, f.promised};
+    for (int i = 0; i < 12; ++i) key.params[i] = params[i];
     bool reuse = false;
     char *plan_storage = backend_attention_plan(backend, key, plan_storage_bytes(f), &reuse);
     if (!plan_storage || !carve_partials(backend, &f, plan_storage)) return false;
@@ -1112,7 +1159,18 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     f.q_stride_h = p.q.stride[1];
     f.out_stride_t = p.out.stride[0];
     f.out_stride_h = p.out.stride[1];
+    f.k_new = (const uint16_t *)p.k_new.base + p.k_new.offset;
+    f.v_new = (const uint16_t *)p.v_new.base + p.v_new.offset;
+    f.kn_stride_t = p.k_new.stride[0];
+    f.kn_stride_h = p.k_new.stride[1];
+    f.vn_stride_t = p.v_new.stride[0];
+    f.vn_stride_h = p.v_new.stride[1];
+    f.append_error_back = p.attention_error_offset;
     if (!reuse) launch_plan(stream, f, error);
+  }
+  if (fast && f.append_in_kernel) {
+    launch_fast(backend, stream, f, error);
+    return true;
   }
   uint64_t append_work =
       (uint64_t)p.tokens * (p.kv_heads * p.width + p.kv_heads * p.value_width);

@@ -215,10 +215,12 @@ struct Op {
     op.record.page_tokens = page_tokens;
     return op;
   }
-  static Op paged_attention_ragged(float scale, uint32_t page_tokens) {
+  // one_row_per_lane: the recorder's promise of a decode batch, checked when the dispatch runs
+  static Op paged_attention_ragged(float scale, uint32_t page_tokens, bool one_row_per_lane = false) {
     Op op = of(FH_OP_PAGED_ATTENTION_RAGGED);
     op.record.scale = scale;
     op.record.page_tokens = page_tokens;
+    op.record.k = one_row_per_lane ? 1 : 0;
     return op;
   }
 };

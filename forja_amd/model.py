@@ -260,7 +260,8 @@ class StepBuffers:
 
 def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: CommandList,
                 feed_back: bool = False, route_trace: Optional[Tensor] = None,
-                head: bool = True, lane_starts=None, lane_sites: Optional[list] = None) -> None:
+                head: bool = True, lane_starts=None, lane_sites: Optional[list] = None,
+                one_row_per_lane: bool = False) -> None:
     """Appends one forward step over the packed batch to `commands`.  With `feed_back` the greedy
     tokens are copied into the id buffer for the next step (device to device).  `route_trace`
     (u32 [layers, tokens, top_k]) receives a copy of every layer's expert choices, for
@@ -271,7 +272,8 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
     per lane one Op::PagedSdpaAppend on the lane's rows of q/k/v with the lane's table and a row of
     its own for the result, followed by the Op::Copy of that row into the packed activation.  The
     start is an attribute of the op; `lane_sites` receives (dispatch index, lane) of every such
-    dispatch so that a replay can patch it."""
+    dispatch so that a replay can patch it.  `one_row_per_lane` passes the packed op the promise
+    that the batch is a decode batch (every lane at most one row)."""
     c, b = model.config, buffers
     tokens = b.tokens
     heads = c.q_heads + c.kv_heads
@@ -306,7 +308,7 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
              qk_weight.narrow(2, half, half), positions],
             [b.qk.narrow(2, 0, half), b.qk.narrow(2, half, half)])
         if lane_starts is None:
-            commands.dispatch_many(Op.paged_attention_ragged(scale, c.page_tokens),
+            commands.dispatch_many(Op.paged_attention_ragged(scale, c.page_tokens, one_row_per_lane),
                                    [q, k_new, v_new, *attention_inputs_tail],
                                    [b.attended, cache.keys[index], cache.values[index]])
         else:
@@ -396,7 +398,7 @@ class DecodeSession:
         first_ids = rng.integers(0, c.vocab, lanes).astype(np.uint32)
         backend.write(b.ids, first_ids.tobytes())
         commands = CommandList()
-        record_step(model, self.cache, b, commands, feed_back=True)
+        record_step(model, self.cache, b, commands, feed_back=True, one_row_per_lane=True)
         self.commands = commands
         self.encoded = backend.encode(commands) if hasattr(backend, "encode") else commands
         self.dispatches = len(commands)

@@ -89,7 +89,10 @@ typedef enum fh_op_kind {
    *            generations u32 [P], cu_seqlens u32 [L+1], q_starts u32 [L], activity u32 [L]
    *   outputs: out [T,Hq,Dv], key pool [P,pt,Hkv,D], value pool [P,pt,Hkv,Dv]
    * Lanes must address pairwise distinct (page,slot) destinations; inactive lanes produce zeros
-   * and leave the pools untouched. */
+   * and leave the pools untouched.  `k` = 1 is the recorder's promise that no lane brings more
+   * than one query row (a decode batch): the library then stores the new rows from inside the
+   * attention kernel.  The promise is checked on the device; a lane that breaks it is reported
+   * as FH_DEVICE_ERROR_FLAG with the first offending token as value.  `k` = 0: no promise. */
   FH_OP_PAGED_ATTENTION_RAGGED = 32,
   /* GPU-side token->expert packing on its own, for inspection: input indices u32 [R,k];
    * outputs counts u32 [E], offsets u32 [E+1], sorted_routes u32 [R*k], blocks u32 [B,3]

@@ -664,6 +664,69 @@ def test_ragged_attention_layers_share_metadata_until_it_is_rewritten(cpu, hip, 
     assert cpu.read(cpu_out[3]) == hip.read(hip_out[3]) and cpu.read(cpu_out[4]) == hip.read(hip_out[4])
 
 
+@pytest.mark.parametrize("contexts,hq,hkv,pt", [
+    ([17, 64, 130, 511], 16, 8, 16), ([300, 1, 2047, 700, 15, 16, 0], 32, 4, 16), ([100, 257], 32, 4, 64),
+    ([0], 8, 2, 16), (list(range(0, 520, 13)), 32, 4, 16)])
+def test_decode_batch_with_the_one_row_promise_stores_the_new_rows_itself(cpu, hip, contexts, hq, hkv, pt):
+    """With the recorder's promise of one query row per lane the attention kernel stores the new
+    key/value rows itself: pools still match the oracle bit for bit (lanes at context 0 attend
+    nothing but the row just stored), and so does a second layer that reuses the work plan."""
+    scale = 1.0 / math.sqrt(128)
+
+    def build(backend):
+        t, inputs = ragged_case(backend, contexts, [1] * len(contexts), hq, hkv, pt, seed=66)
+        physical = t["keys"].shape[0]
+        other_k = upload(backend, normal_bf16(66, 8, (physical, pt, hkv, 128)), DType.BF16)
+        other_v = upload(backend, normal_bf16(66, 9, (physical, pt, hkv, 128)), DType.BF16)
+        out2 = backend.alloc(DType.BF16, t["out"].shape)
+        op = Op.paged_attention_ragged(scale, pt, one_row_per_lane=True)
+        commands = CommandList()
+        commands.dispatch_many(op, inputs, [t["out"], t["keys"], t["values"]])
+        commands.dispatch_many(op, inputs, [out2, other_k, other_v])
+        return commands, [t["out"], out2, t["keys"], t["values"], other_k, other_v]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
+    for index in (2, 3, 4, 5):
+        assert cpu.read(cpu_out[index]) == hip.read(hip_out[index])
+
+
+def test_a_broken_one_row_promise_is_reported(cpu, hip):
+    def build(backend):
+        t, inputs = ragged_case(backend, [40, 0, 100], [1, 2, 1], 8, 2, 16, seed=67)
+        commands = CommandList()
+        commands.dispatch_many(Op.paged_attention_ragged(0.09, 16, one_row_per_lane=True), inputs,
+                               [t["out"], t["keys"], t["values"]])
+        return commands, []
+    for backend in (cpu, hip):
+        commands, _ = build(backend)
+        with pytest.raises(BackendError) as info:
+            run(backend, commands)
+        assert info.value.status == Status.DEVICE_ERROR_FLAG and info.value.index == 1
+
+
+def test_the_one_row_promise_keeps_inactive_lanes_and_stale_pages_unwritten(cpu, hip):
+    def build(backend, corrupt):
+        t, inputs = ragged_case(backend, [33, 70, 5], [1, 1, 1], 8, 4, 16, seed=68,
+                                activity=[1, 0, 1], corrupt=corrupt)
+        commands = CommandList()
+        commands.dispatch_many(Op.paged_attention_ragged(0.09, 16, one_row_per_lane=True), inputs,
+                               [t["out"], t["keys"], t["values"]])
+        return commands, [t["out"], t["keys"], t["values"]]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, lambda backend: build(backend, None))
+    assert cpu.read(cpu_out[1]) == hip.read(hip_out[1]) and cpu.read(cpu_out[2]) == hip.read(hip_out[2])
+    # lane 0 appends at position 33 = logical page 2: stale there, nothing of lane 0 is written
+    commands, tensors = build(hip, (0, 2))
+    before = hip.read(tensors[1])
+    with pytest.raises(BackendError) as info:
+        run(hip, commands)
+    assert info.value.status == Status.DEVICE_ERROR_FLAG and info.value.index == 2
+    # exactly one token row of the key pool changed: lane 2's (lane 1 is inactive, lane 0 refused)
+    token_row = 4 * 128 * 2
+    changed = np.frombuffer(hip.read(tensors[1]), np.uint8).reshape(-1, token_row) != \
+        np.frombuffer(before, np.uint8).reshape(-1, token_row)
+    assert changed.any(axis=1).sum() == 1
+    assert not to_f32(hip.read(tensors[0]), DType.BF16).reshape(3, -1)[0].any()
+
+
 def test_ragged_attention_skips_inactive_lanes(cpu, hip):
     def build(backend):
         t, inputs = ragged_case(backend, [33, 70, 5], [1, 1, 1], 8, 4, 16, seed=62, activity=[1, 0, 1])

@@ -54,6 +54,9 @@ struct QmmArgs {
   const uint32_t *run_if_set;   // when not null: do nothing unless this device word is non-zero
   const uint16_t *residual;     // optional bf16 rows added to the result before it is rounded
   uint64_t residual_row_stride;
+  // routed whole-K tile kernel: K is split inside the workgroup when tiles x column blocks is at
+  // most this (0: never)
+  uint32_t split_below;
 };
 
 __device__ inline uint32_t pack2(float lo, float hi) {
@@ -299,154 +302,229 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // memory round trip, one barrier) and then every wave streams the packed weights of its own 32
 // output columns (both projections for the gate/up pair) with no further synchronisation, a quad
 // of groups (one 128-byte line per weight row) at a time, two quads ahead.
-template <bool kPair>
-__global__ __launch_bounds__(512) void qmm_routed_tile_kernel(QmmArgs a) {
+// One (tile, column block) unit of qmm_routed_tile_kernel; kSplit: the column block is 4 x 32
+// columns and K is split over the workgroup's two wave quartets.  The two forms are separate
+// instantiations so that the common one keeps constant wave-to-column and K-range arithmetic.
+template <bool kPair, bool kSplit>
+__device__ __forceinline__ void routed_tile_unit_body(const QmmArgs &a, uint32_t tile, uint32_t column_block) {
   constexpr int kTileWaves = 8, kTileThreads = 64 * kTileWaves, kRows = 32;
   constexpr int kP = kPair ? 2 : 1;
+  constexpr uint32_t waves_across = kSplit ? kTileWaves / 2 : kTileWaves;
   extern __shared__ __attribute__((aligned(16))) unsigned char tile_lds[];
-  const uint32_t pitch = 2 * a.inner + 16;  // bytes per staged row
+  const uint32_t row_pitch = 2 * a.inner + 16;  // bytes per staged row
   unsigned char *xs = tile_lds;
-  float *xsum = (float *)(tile_lds + kRows * pitch);      // [K/64][32]
+  float *xsum = (float *)(tile_lds + kRows * row_pitch);      // [K/64][32]
   uint32_t *row_ids = (uint32_t *)(xsum + (a.inner / kGroup) * kRows);
-
   const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const uint32_t nl = lane & 31, h = lane >> 5;
-  const uint32_t column = (blockIdx.x * kTileWaves + wave) * kColsPerWave + nl;
-  const uint32_t column_c = min(column, a.columns - 1);
-  if (blockIdx.y >= a.n_blocks[0]) return;
-  const uint32_t expert = a.blocks[3 * blockIdx.y];
-  if (expert == kNoBlock) return;
-  const uint32_t first = a.blocks[3 * blockIdx.y + 1], count = a.blocks[3 * blockIdx.y + 2];
-  if (tid < kRows) row_ids[tid] = tid < count ? a.sorted_routes[first + tid] : 0;
-
+  uint32_t nl = lane & 31, h = lane >> 5;
+  asm volatile("" : "+v"(nl), "+v"(h));   // per unit: see pieces_per_row below
+  const uint32_t all_quads = a.inner / (4 * kGroup);
+  const uint32_t k_half = kSplit ? wave / waves_across : 0;
+  const uint32_t total_quads = kSplit ? all_quads / 2 : all_quads;   // this wave's share of K
+  const uint32_t quad0 = k_half * total_quads;
   const uint32_t words_per_row = a.inner / 8, groups_per_row = a.inner / kGroup;
-  const uint32_t total_quads = a.inner / (4 * kGroup);
-  const uint32_t *w_row[kP];
-  const uint16_t *s_row[kP], *b_row[kP];
-  for (int pj = 0; pj < kP; ++pj) {
-    w_row[pj] = a.packed[pj] + expert * a.expert_words + (uint64_t)column_c * words_per_row + 4 * h;
-    s_row[pj] = a.scales[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
-    b_row[pj] = a.biases[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
-  }
-  uint4 wq[kP][2][4];
-  uint2 scale_q[kP][2], bias_q[kP][2];
-  auto load_quad = [&](int slot, uint32_t quad) {
-    const uint32_t qd = min(quad, total_quads - 1);  // unconditional: the tail reloads the last quad
-    for (int pj = 0; pj < kP; ++pj) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        wq[pj][slot][i] = *(const uint4 *)(w_row[pj] + (uint64_t)(4 * qd + i) * 8);
-      scale_q[pj][slot] = *(const uint2 *)(s_row[pj] + 4 * qd);
-      bias_q[pj][slot] = *(const uint2 *)(b_row[pj] + 4 * qd);
-    }
-  };
-  load_quad(0, 0);   // cold memory: request before anything else
-  load_quad(1, 1);
-  __syncthreads();   // row_ids visible
-  // ---- stage the tile: permuted inside each 8, with per-group row sums
-  const uint32_t pieces_per_row = a.inner / 8, pieces = kRows * pieces_per_row;
-  for (uint32_t base = 0; base < pieces; base += 8 * kTileThreads) {
-    uint4 x_regs[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t piece = base + tid + i * kTileThreads;
-      const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
-      x_regs[i] = make_uint4(0, 0, 0, 0);
-      if (piece < pieces && row < count)
-        x_regs[i] = *(const uint4 *)(a.x + (uint64_t)(row_ids[row] / a.route_div) * a.x_row_stride + 8 * pc);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t piece = base + tid + i * kTileThreads;
-      const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
-      const uint4 v = x_regs[i];
-      float sum = bf16_bits_to_f32(v.x & 0xffffu) + bf16_bits_to_f32(v.x >> 16) +
-                  bf16_bits_to_f32(v.y & 0xffffu) + bf16_bits_to_f32(v.y >> 16) +
-                  bf16_bits_to_f32(v.z & 0xffffu) + bf16_bits_to_f32(v.z >> 16) +
-                  bf16_bits_to_f32(v.w & 0xffffu) + bf16_bits_to_f32(v.w >> 16);
-      sum += __shfl_xor(sum, 1, 64);   // eight consecutive pieces (= lanes) make one group
-      sum += __shfl_xor(sum, 2, 64);
-      sum += __shfl_xor(sum, 4, 64);
-      if (piece < pieces) {
-        uint4 permuted;
-        permuted.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
-        permuted.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
-        permuted.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
-        permuted.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
-        *(uint4 *)(xs + row * pitch + pc * 16) = permuted;
-        if ((pc & 7) == 0) xsum[(pc >> 3) * kRows + row] = sum;
-      }
-    }
-  }
-  __syncthreads();
+  {
+    __syncthreads();   // the previous unit is done with row_ids and the staged tile
+    const uint32_t expert = a.blocks[3 * tile];
+    if (expert == kNoBlock) return;
+    const uint32_t first = a.blocks[3 * tile + 1], count = a.blocks[3 * tile + 2];
+    if (tid < kRows) row_ids[tid] = tid < count ? a.sorted_routes[first + tid] : 0;
+    const uint32_t column = (column_block * waves_across + wave % waves_across) * kColsPerWave + nl;
+    const uint32_t column_c = min(column, a.columns - 1);
 
-  f32x16 acc[kP];
-  for (int pj = 0; pj < kP; ++pj)
-    for (int j = 0; j < 16; ++j) acc[pj][j] = 0.0f;
-  const unsigned char *my_row = xs + nl * pitch + 64 * h;
-  // Two consecutive groups (members i0, i0+1 of ring slot `slot`): independent accumulation
-  // chains per group and projection, scales applied per group, bias term as one f32 MFMA over
-  // the two groups (lane half h supplies group + h of both operands).
-  auto consume_pair = [&](int slot, int i0, uint32_t group) {
-    f32x16 part[2][kP];
+    const uint32_t *w_row[kP];
+    const uint16_t *s_row[kP], *b_row[kP];
+    for (int pj = 0; pj < kP; ++pj) {
+      w_row[pj] = a.packed[pj] + expert * a.expert_words + (uint64_t)column_c * words_per_row + 4 * h;
+      s_row[pj] = a.scales[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
+      b_row[pj] = a.biases[pj] + expert * a.expert_groups + (uint64_t)column_c * groups_per_row;
+    }
+    uint4 wq[kP][2][4];
+    uint2 scale_q[kP][2], bias_q[kP][2];
+    auto load_quad = [&](int slot, uint32_t quad) {
+      // unconditional: the tail reloads the last quad
+      const uint32_t qd = quad0 + min(quad, total_quads - 1);
+      for (int pj = 0; pj < kP; ++pj) {
 #pragma unroll
-    for (int q = 0; q < 2; ++q)
-      for (int pj = 0; pj < kP; ++pj)
-        for (int j = 0; j < 16; ++j) part[q][pj][j] = 0.0f;
+        for (int i = 0; i < 4; ++i)
+          wq[pj][slot][i] = *(const uint4 *)(w_row[pj] + (uint64_t)(4 * qd + i) * 8);
+        scale_q[pj][slot] = *(const uint2 *)(s_row[pj] + 4 * qd);
+        bias_q[pj][slot] = *(const uint2 *)(b_row[pj] + 4 * qd);
+      }
+    };
+    load_quad(0, 0);   // cold memory: request before anything else
+    load_quad(1, 1);
+    __syncthreads();   // row_ids visible
+    // ---- stage the tile: permuted inside each 8, with per-group row sums
+    // (a fresh value per unit: with a loop-invariant divisor the compiler computes every piece's
+    // row and column once, before the loop over units, and carries some forty registers of them
+    // through the matrix loop)
+    uint32_t pieces_per_row = a.inner / 8, pitch = row_pitch;
+    asm volatile("" : "+s"(pieces_per_row), "+s"(pitch));
+    const uint32_t pieces = kRows * pieces_per_row;
+    for (uint32_t base = 0; base < pieces; base += 8 * kTileThreads) {
+      uint4 x_regs[8];
 #pragma unroll
-    for (int step = 0; step < 4; ++step)
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t piece = base + tid + i * kTileThreads;
+        const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
+        x_regs[i] = make_uint4(0, 0, 0, 0);
+        if (piece < pieces && row < count)
+          x_regs[i] = *(const uint4 *)(a.x + (uint64_t)(row_ids[row] / a.route_div) * a.x_row_stride + 8 * pc);
+      }
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        const uint4 a_raw = *(const uint4 *)(my_row + (group + q) * (2 * kGroup) + 16 * step);
-        const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
-#pragma unroll
-        for (int pj = 0; pj < kP; ++pj) {
-          const uint4 w = wq[pj][slot][i0 + q];
-          const bf16x8 b_op =
-              unpack_word(step == 0 ? w.x : (step == 1 ? w.y : (step == 2 ? w.z : w.w)));
-          part[q][pj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op, part[q][pj], 0, 0, 0);
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t piece = base + tid + i * kTileThreads;
+        const uint32_t row = piece / pieces_per_row, pc = piece % pieces_per_row;
+        const uint4 v = x_regs[i];
+        float sum = bf16_bits_to_f32(v.x & 0xffffu) + bf16_bits_to_f32(v.x >> 16) +
+                    bf16_bits_to_f32(v.y & 0xffffu) + bf16_bits_to_f32(v.y >> 16) +
+                    bf16_bits_to_f32(v.z & 0xffffu) + bf16_bits_to_f32(v.z >> 16) +
+                    bf16_bits_to_f32(v.w & 0xffffu) + bf16_bits_to_f32(v.w >> 16);
+        sum += __shfl_xor(sum, 1, 64);   // eight consecutive pieces (= lanes) make one group
+        sum += __shfl_xor(sum, 2, 64);
+        sum += __shfl_xor(sum, 4, 64);
+        if (piece < pieces) {
+          uint4 permuted;
+          permuted.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
+          permuted.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
+          permuted.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+          permuted.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+          *(uint4 *)(xs + row * pitch + pc * 16) = permuted;
+          if ((pc & 7) == 0) xsum[(pc >> 3) * kRows + row] = sum;
         }
       }
-#pragma unroll
-    for (int pj = 0; pj < kP; ++pj) {
-      const uint32_t scale_bits = i0 == 0 ? scale_q[pj][slot].x : scale_q[pj][slot].y;
-      const uint32_t bias_bits = i0 == 0 ? bias_q[pj][slot].x : bias_q[pj][slot].y;
-      const float scale0 = bf16_bits_to_f32(scale_bits & 0xffffu);
-      const float scale1 = bf16_bits_to_f32(scale_bits >> 16);
-      const float shift0 = bf16_bits_to_f32(bias_bits & 0xffffu) - 16.0f * scale0;
-      const float shift1 = bf16_bits_to_f32(bias_bits >> 16) - 16.0f * scale1;
-#pragma unroll
-      for (int j = 0; j < 16; ++j)
-        acc[pj][j] = __builtin_fmaf(scale1, part[1][pj][j], __builtin_fmaf(scale0, part[0][pj][j], acc[pj][j]));
-      acc[pj] = __builtin_amdgcn_mfma_f32_32x32x2f32(xsum[(group + h) * kRows + nl],
-                                                     h ? shift1 : shift0, acc[pj], 0, 0, 0);
     }
-  };
-  for (uint32_t q0 = 0; q0 < total_quads; q0 += 2) {
+    __syncthreads();
+
+    f32x16 acc[kP];
+    for (int pj = 0; pj < kP; ++pj)
+      for (int j = 0; j < 16; ++j) acc[pj][j] = 0.0f;
+    const unsigned char *my_row = xs + nl * pitch + 64 * h;
+    // Two consecutive groups (members i0, i0+1 of ring slot `slot`): independent accumulation
+    // chains per group and projection, scales applied per group, bias term as one f32 MFMA over
+    // the two groups (lane half h supplies group + h of both operands).
+    auto consume_pair = [&](int slot, int i0, uint32_t group) {
+      f32x16 part[2][kP];
 #pragma unroll
-    for (int uq = 0; uq < 2; ++uq) {
-      const uint32_t quad = q0 + uq;
-      if (quad >= total_quads) break;
-      consume_pair(uq, 0, 4 * quad);
-      consume_pair(uq, 2, 4 * quad + 2);
-      load_quad(uq, quad + 2);
+      for (int q = 0; q < 2; ++q)
+        for (int pj = 0; pj < kP; ++pj)
+          for (int j = 0; j < 16; ++j) part[q][pj][j] = 0.0f;
+#pragma unroll
+      for (int step = 0; step < 4; ++step)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const uint4 a_raw = *(const uint4 *)(my_row + (group + q) * (2 * kGroup) + 16 * step);
+          const bf16x8 a_op = __builtin_bit_cast(bf16x8, a_raw);
+#pragma unroll
+          for (int pj = 0; pj < kP; ++pj) {
+            const uint4 w = wq[pj][slot][i0 + q];
+            const bf16x8 b_op =
+                unpack_word(step == 0 ? w.x : (step == 1 ? w.y : (step == 2 ? w.z : w.w)));
+            part[q][pj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op, part[q][pj], 0, 0, 0);
+          }
+        }
+#pragma unroll
+      for (int pj = 0; pj < kP; ++pj) {
+        const uint32_t scale_bits = i0 == 0 ? scale_q[pj][slot].x : scale_q[pj][slot].y;
+        const uint32_t bias_bits = i0 == 0 ? bias_q[pj][slot].x : bias_q[pj][slot].y;
+        const float scale0 = bf16_bits_to_f32(scale_bits & 0xffffu);
+        const float scale1 = bf16_bits_to_f32(scale_bits >> 16);
+        const float shift0 = bf16_bits_to_f32(bias_bits & 0xffffu) - 16.0f * scale0;
+        const float shift1 = bf16_bits_to_f32(bias_bits >> 16) - 16.0f * scale1;
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          acc[pj][j] = __builtin_fmaf(scale1, part[1][pj][j], __builtin_fmaf(scale0, part[0][pj][j], acc[pj][j]));
+        acc[pj] = __builtin_amdgcn_mfma_f32_32x32x2f32(xsum[(group + h) * kRows + nl],
+                                                       h ? shift1 : shift0, acc[pj], 0, 0, 0);
+      }
+    };
+    for (uint32_t q0 = 0; q0 < total_quads; q0 += 2) {
+#pragma unroll
+      for (int uq = 0; uq < 2; ++uq) {
+        const uint32_t quad = q0 + uq;
+        if (quad >= total_quads) break;
+        consume_pair(uq, 0, 4 * (quad0 + quad));
+        consume_pair(uq, 2, 4 * (quad0 + quad) + 2);
+        load_quad(uq, quad + 2);
+      }
+    }
+    if (kSplit) {
+      // the upper K half hands its sums to the quartet that owns the same columns; the staged
+      // activations are no longer needed, their LDS carries the hand-over
+      float *handed = (float *)tile_lds;   // [4 column groups][kP][16][64]
+      const uint32_t group_of_wave = wave % waves_across;
+      __syncthreads();
+      if (k_half == 1)
+        for (int pj = 0; pj < kP; ++pj)
+          for (int j = 0; j < 16; ++j) handed[((group_of_wave * kP + pj) * 16 + j) * 64 + lane] = acc[pj][j];
+      __syncthreads();
+      if (k_half == 0)
+        for (int pj = 0; pj < kP; ++pj)
+          for (int j = 0; j < 16; ++j) acc[pj][j] += handed[((group_of_wave * kP + pj) * 16 + j) * 64 + lane];
+    }
+    // ---- epilogue and store; lane (column nl, half h) holds rows 8*(j/4) + 4h + j%4
+    if (k_half != 0 || column >= a.columns) return;
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t row = 8 * (j / 4) + 4 * h + (j % 4);
+      if (row >= count) continue;
+      float value = acc[0][j];
+      if (kPair) {
+        const float gate = value, up = acc[kP - 1][j];
+        value = gate * (1.0f / (1.0f + __expf(-gate))) * up;
+      }
+      const uint64_t at = (uint64_t)row_ids[row] * a.out_row_stride + column;
+      if (a.out_f32)
+        ((float *)a.out)[at] = value;
+      else
+        ((uint16_t *)a.out)[at] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
     }
   }
-  // ---- epilogue and store; lane (column nl, half h) holds rows 8*(j/4) + 4h + j%4
-  if (column >= a.columns) return;
-  for (int j = 0; j < 16; ++j) {
-    const uint32_t row = 8 * (j / 4) + 4 * h + (j % 4);
-    if (row >= count) continue;
-    float value = acc[0][j];
-    if (kPair) {
-      const float gate = value, up = acc[kP - 1][j];
-      value = gate * (1.0f / (1.0f + __expf(-gate))) * up;
-    }
-    const uint64_t at = (uint64_t)row_ids[row] * a.out_row_stride + column;
-    if (a.out_f32)
-      ((float *)a.out)[at] = value;
+}
+
+template <bool kPair>
+__device__ __forceinline__ void routed_tile_unit(const QmmArgs &a, uint32_t tile, uint32_t column_block) {
+  routed_tile_unit_body<kPair, false>(a, tile, column_block);
+}
+template <bool kPair>
+__device__ __forceinline__ void routed_tile_unit_split(const QmmArgs &a, uint32_t tile,
+                                                       uint32_t column_block) {
+  routed_tile_unit_body<kPair, true>(a, tile, column_block);
+}
+
+template <bool kPair>
+__global__ __launch_bounds__(512) void qmm_routed_tile_kernel(QmmArgs a) {
+  constexpr int kTileWaves = 8;
+  // Work units are (tile, column block) pairs; the launch has as many workgroups as are resident
+  // at once (the staged tile fills most of a CU's LDS) and every workgroup walks the units
+  // unit, unit + gridDim.x, ...: the number of tiles is only known on the device, and a grid
+  // sized for the worst case would spend its time retiring workgroups that have nothing to do.
+  // Usually a column block is the 8 x 32 columns of the eight waves.  When the routes fall on
+  // few tiles (few experts hit, many rows each) that would leave most of the device idle behind
+  // long per-wave chains; a column block is then 4 x 32 columns and K is split over the two
+  // wave quartets, whose sums meet in LDS.
+  const uint32_t tiles = a.n_blocks[0];
+  const uint32_t wide_blocks = (a.columns + kTileWaves * kColsPerWave - 1) / (kTileWaves * kColsPerWave);
+  const uint32_t all_quads = a.inner / (4 * kGroup);
+  // (only the gate/up pair: its launches are the ones with few column blocks)
+  const bool split_k = kPair && (uint64_t)tiles * wide_blocks <= a.split_below && all_quads % 2 == 0;
+  const uint32_t waves_across = split_k ? kTileWaves / 2 : kTileWaves;
+  const uint32_t column_blocks =
+      (a.columns + waves_across * kColsPerWave - 1) / (waves_across * kColsPerWave);
+  // unit -> (tile, column block) without a division per step
+  const uint32_t tile_step = gridDim.x / column_blocks, block_step = gridDim.x % column_blocks;
+  uint32_t tile = blockIdx.x / column_blocks, column_block = blockIdx.x % column_blocks;
+  while (tile < tiles) {
+    if (kPair && split_k)
+      routed_tile_unit_split<true>(a, tile, column_block);
     else
-      ((uint16_t *)a.out)[at] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+      routed_tile_unit<kPair>(a, tile, column_block);
+    tile += tile_step;
+    column_block += block_step;
+    if (column_block >= column_blocks) {
+      column_block -= column_blocks;
+      ++tile;
+    }
   }
 }
 
@@ -1111,7 +1189,7 @@ bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, Er
 // Routed product over the packed tiles: whole-K tile kernel when the tile fits LDS, else the
 // multi-pass kernel.
 template <bool kPair>
-void launch_routed(hipStream_t stream, const QmmArgs &a, uint32_t max_blocks) {
+void launch_routed(hipStream_t stream, const QmmArgs &a, uint32_t max_blocks, uint32_t resident /* CUs */) {
   if (a.inner <= kTileMaxInner) {
     static bool configured = false;   // raise the dynamic LDS limit once per process
     if (!configured) {
@@ -1120,8 +1198,12 @@ void launch_routed(hipStream_t stream, const QmmArgs &a, uint32_t max_blocks) {
                                 (int)routed_tile_lds_bytes(kTileMaxInner));
       configured = true;
     }
-    dim3 grid((a.columns + 8 * kColsPerWave - 1) / (8 * kColsPerWave), max_blocks);
-    qmm_routed_tile_kernel<kPair><<<grid, 512, routed_tile_lds_bytes(a.inner), stream>>>(a);
+    // as many workgroups as are resident at once (LDS and the 2048 threads of a CU decide how
+    // many per compute unit) walk the (tile, column block) units
+    const uint64_t most_units = (uint64_t)max_blocks * 2 * ((a.columns + 8 * kColsPerWave - 1) / (8 * kColsPerWave));
+    const uint32_t per_unit = std::max<uint32_t>(1, std::min<uint32_t>(4, (160u * 1024u) / routed_tile_lds_bytes(a.inner)));
+    const uint32_t grid = (uint32_t)std::min<uint64_t>(most_units, (uint64_t)resident * per_unit);
+    qmm_routed_tile_kernel<kPair><<<dim3(grid), 512, routed_tile_lds_bytes(a.inner), stream>>>(a);
     return;
   }
   launch_qmm<kPair, true>(stream, a, max_blocks, 1);
@@ -1181,11 +1263,12 @@ bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int
   a.blocks = plan.blocks;
   a.n_blocks = plan.n_blocks;
   a.route_div = p.k;
+  a.split_below = backend_compute_units(backend) / 2;
   KernelTimer timer(backend, FH_KC_MOE_KERNEL);
   if (projections == 2)
-    launch_routed<true>(stream, a, plan.max_blocks);
+    launch_routed<true>(stream, a, plan.max_blocks, backend_compute_units(backend));
   else
-    launch_routed<false>(stream, a, plan.max_blocks);
+    launch_routed<false>(stream, a, plan.max_blocks, backend_compute_units(backend));
   return true;
 }
 
@@ -1219,9 +1302,10 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
   a.blocks = plan.blocks;
   a.n_blocks = plan.n_blocks;
   a.route_div = 1;
+  a.split_below = backend_compute_units(backend) / 2;
   {
     KernelTimer timer(backend, FH_KC_MOE_KERNEL);
-    launch_routed<false>(stream, a, plan.max_blocks);
+    launch_routed<false>(stream, a, plan.max_blocks, backend_compute_units(backend));
   }
   uint64_t work = (uint64_t)p.rows * p.columns;
   auto row_view = [&](const View &v) {   // bf16 [rows, columns], 8-byte aligned row pieces

@@ -92,8 +92,8 @@ __global__ void ragged_append_kernel(RaggedAttention p, ErrorSlot *error) {
   }
 }
 
-// The same append for bf16 rows and pools whose head rows are 16-byte aligned: a thread moves
-// eight elements.
+// The same append for rows and pools of one 2-byte dtype whose head rows are 16-byte aligned: a
+// thread moves eight elements.
 __global__ __launch_bounds__(256) void ragged_append_pieces_kernel(RaggedAttention p, ErrorSlot *error) {
   const uint32_t key_pieces = p.kv_heads * p.width / 8, value_pieces = p.kv_heads * p.value_width / 8;
   const uint32_t per_token = key_pieces + value_pieces;
@@ -136,11 +136,13 @@ __global__ __launch_bounds__(256) void ragged_append_pieces_kernel(RaggedAttenti
 }
 
 bool append_by_pieces(const RaggedAttention &p) {
+  const uint32_t dtype = p.key_pool.dtype;
+  if (dtype != FH_BF16 && dtype != FH_F16) return false;
   for (const View *v : {&p.k_new, &p.v_new})
-    if (v->dtype != FH_BF16 || v->stride[2] != 1 || v->stride[0] % 8 || v->stride[1] % 8 || v->offset % 8)
+    if (v->dtype != dtype || v->stride[2] != 1 || v->stride[0] % 8 || v->stride[1] % 8 || v->offset % 8)
       return false;
   for (const View *v : {&p.key_pool, &p.value_pool})
-    if (v->dtype != FH_BF16 || v->offset % 8) return false;
+    if (v->dtype != dtype || v->offset % 8) return false;
   return p.width % 8 == 0 && p.value_width % 8 == 0;
 }
 
@@ -227,7 +229,12 @@ __global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *er
 }
 
 
-// ---------------------------------------------------------------- bf16, D = Dv = 128 fast path
+// ------------------------------------------------- 2-byte pools (bf16 or f16), D = Dv = 128
+//
+// The pools' dtype is the matrix cores' operand type (kHalf: f16, else bf16).  Queries are of that
+// dtype, or f32 against f16 pools (rounded to f16 once, as they enter the operand registers: an
+// 11-bit significand on one factor of a 128-term dot product moves a score by ~1e-4); outputs are
+// written in any float dtype.
 //
 // Split-KV decode-style attention on the matrix cores, registers only.  One wave owns
 // (token, split, kv head): it streams its span of the lane's K/V pages once, 32 tokens per step.
@@ -248,6 +255,8 @@ __global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *er
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr uint32_t kMinSplitTokens = 128, kMaxSplitTokens = 1024;  // split length bounds
@@ -263,8 +272,11 @@ struct TokenPlan {
 };
 
 struct FastRagged {
-  const uint16_t *q, *key_pool, *value_pool;
-  uint16_t *out;
+  const void *q;       // q_dtype elements
+  const uint16_t *key_pool, *value_pool;
+  void *out;           // out_dtype elements
+  uint32_t q_dtype, out_dtype;   // strides below count elements of these
+  uint32_t pool_half;            // pools are f16 (else bf16)
   const uint32_t *tables, *generations, *cu, *starts, *activity;
   float *partial_o;    // [T, S, Hq, 128]
   float2 *partial_ml;  // [T, S, Hq]
@@ -290,7 +302,7 @@ struct FastRagged {
   // split stores the lane's new key and value row before it attends.  k_new / v_new are
   // [T, Hkv, 128] with unit innermost stride; append failures are recorded `append_error_back`
   // records before the attention's.
-  const uint16_t *k_new, *v_new;
+  const void *k_new, *v_new;   // q_dtype elements
   uint64_t kn_stride_t, kn_stride_h, vn_stride_t, vn_stride_h;
   uint32_t append_in_kernel, append_error_back;
   uint32_t promised;   // one query row per lane, vouched for by the caller: verified by the plan
@@ -419,18 +431,76 @@ __device__ inline uint32_t pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
+__device__ inline uint32_t pack_f16(float lo, float hi) {
+  f16x2 v = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Two values as a pair of matrix-core operand elements.
+template <bool kHalf>
+__device__ inline uint32_t pack_operand(float lo, float hi) {
+  return kHalf ? pack_f16(lo, hi) : pack_bf16(lo, hi);
+}
+
+template <bool kHalf>
+__device__ inline f32x4 mfma_16x16x32(const uint4 &a, const uint4 &b, const f32x4 &c) {
+  if constexpr (kHalf)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// Eight query elements from `element` as operand words.  An f32 query beyond the f16 range is
+// held at the largest finite f16 (a NaN stays a NaN): the scores stay finite, as the reference's.
+template <bool kHalf, bool kMixed>
+__device__ inline uint4 load_query(const FastRagged &p, uint64_t element) {
+  if (!kMixed || p.q_dtype != FH_F32) return *(const uint4 *)((const uint16_t *)p.q + element);
+  const float4 lo = *(const float4 *)((const float *)p.q + element);
+  const float4 hi = *(const float4 *)((const float *)p.q + element + 4);
+  auto held = [](float v) { return fabsf(v) > 65504.0f ? copysignf(65504.0f, v) : v; };
+  return make_uint4(pack_operand<kHalf>(held(lo.x), held(lo.y)), pack_operand<kHalf>(held(lo.z), held(lo.w)),
+                    pack_operand<kHalf>(held(hi.x), held(hi.y)), pack_operand<kHalf>(held(hi.z), held(hi.w)));
+}
+
+// Four consecutive output elements from `element` (a multiple of 4 on a row whose strides are).
+// kMixed false: queries and outputs are of the pools' dtype, known when the kernel is compiled
+// (the attention kernels have no registers to spare for the choice).
+template <bool kHalf, bool kMixed>
+__device__ inline void store_out4(const FastRagged &p, uint64_t element, float a, float b, float c,
+                                  float d) {
+  if (!kMixed) {
+    *(uint2 *)((uint16_t *)p.out + element) =
+        make_uint2(pack_operand<kHalf>(a, b), pack_operand<kHalf>(c, d));
+    return;
+  }
+  if (p.out_dtype == FH_F32)
+    *(float4 *)((float *)p.out + element) = make_float4(a, b, c, d);
+  else if (p.out_dtype == FH_F16)
+    *(uint2 *)((uint16_t *)p.out + element) = make_uint2(pack_f16(a, b), pack_f16(c, d));
+  else
+    *(uint2 *)((uint16_t *)p.out + element) = make_uint2(pack_bf16(a, b), pack_bf16(c, d));
+}
+
 __device__ inline uint32_t dword_of(const uint4 &v, int index) {
   return index == 0 ? v.x : (index == 1 ? v.y : (index == 2 ? v.z : v.w));
 }
 
 // Zero output rows of `count` tokens from `first` for the query heads of one kv head (a wave's
 // duty when it refuses a page and no merge will follow: the token has a single split).
+template <bool kMixed>
 __device__ inline void zero_head_rows(const FastRagged &p, uint32_t first, uint32_t count,
                                       uint32_t kv_head, uint32_t lane) {
   for (uint32_t member = 0; member < count; ++member)
-    for (uint32_t head = kv_head * p.group; head < (kv_head + 1) * p.group; ++head)
-      *(uint32_t *)(p.out + (uint64_t)(first + member) * p.out_stride_t + (uint64_t)head * p.out_stride_h +
-                    2 * lane) = 0;
+    for (uint32_t head = kv_head * p.group; head < (kv_head + 1) * p.group; ++head) {
+      const uint64_t element =
+          (uint64_t)(first + member) * p.out_stride_t + (uint64_t)head * p.out_stride_h + 2 * lane;
+      if (kMixed && p.out_dtype == FH_F32)
+        *(uint2 *)((float *)p.out + element) = make_uint2(0, 0);
+      else
+        *(uint32_t *)((uint16_t *)p.out + element) = 0;
+    }
 }
 
 struct TileRegs {
@@ -485,7 +555,7 @@ struct Softmax {
 // (16 query rows each: this lane holds row hl of every tile).  `limit[nt]` is the first key the
 // lane's row of tile nt may NOT attend (0 for an unused row); with kMasked false every key of
 // the tile is below every limit.
-template <int NT, bool kMasked>
+template <int NT, bool kMasked, bool kHalf>
 __device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[NT][4],
                                     f32x4 (&o)[NT][8], Softmax (&sm)[NT], uint32_t tile0,
                                     const uint32_t (&limit)[NT], float scale_log2, uint32_t g) {
@@ -496,9 +566,7 @@ __device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[NT
     for (int sub = 0; sub < 2; ++sub) {
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
       for (int step = 0; step < 4; ++step)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, cur.k[sub][step]),
-                                                      __builtin_bit_cast(bf16x8, q_reg[nt][step]),
-                                                      acc, 0, 0, 0);
+        acc = mfma_16x16x32<kHalf>(cur.k[sub][step], q_reg[nt][step], acc);
       for (int j = 0; j < 4; ++j) {
         s_val[4 * sub + j] = acc[j] * scale_log2;
         if (kMasked && tile0 + 16 * sub + 4 * g + j >= limit[nt]) s_val[4 * sub + j] = -__builtin_inff();
@@ -525,8 +593,8 @@ __device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[NT
       sm[nt].m = m_new;
     }
     sm[nt].l += p_sum;
-    p_reg[nt] = make_uint4(pack_bf16(p_val[0], p_val[1]), pack_bf16(p_val[2], p_val[3]),
-                           pack_bf16(p_val[4], p_val[5]), pack_bf16(p_val[6], p_val[7]));
+    p_reg[nt] = make_uint4(pack_operand<kHalf>(p_val[0], p_val[1]), pack_operand<kHalf>(p_val[2], p_val[3]),
+                           pack_operand<kHalf>(p_val[4], p_val[5]), pack_operand<kHalf>(p_val[6], p_val[7]));
   }
   // O^T += V^T . P^T.  Tile mt takes element mt of each of the lane's 8 token pieces; the
   // transposed value operand serves all NT query tiles.
@@ -539,15 +607,13 @@ __device__ inline void consume_tile(const TileRegs &cur, const uint4 (&q_reg)[NT
     const uint4 a_reg = make_uint4(a_words[0], a_words[1], a_words[2], a_words[3]);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
-      o[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_reg),
-                                                         __builtin_bit_cast(bf16x8, p_reg[nt]),
-                                                         o[nt][mt], 0, 0, 0);
+      o[nt][mt] = mfma_16x16x32<kHalf>(a_reg, p_reg[nt], o[nt][mt]);
   }
 }
 
 // NT query tiles of 16 rows per wave: row hl of tile nt is (query token nt * per_tile + hl / group
 // of the item's group, head hl % group of the kv head), per_tile = 16 / group.
-template <int NT>
+template <int NT, bool kHalf, bool kMixed>
 __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *error) {
   // a workgroup is one work item; its waves take one kv head each, so the slices of a K/V page
   // (one 256-byte piece of every token row per kv head) are requested close together in time
@@ -573,12 +639,23 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
     if (entry_ok(table, p.generations, logical, p.table_pages, p.physical_pages, &physical)) {
       const uint64_t pool_row = (uint64_t)physical * pt + position % pt;
       const uint64_t at = (pool_row * p.kv_heads + kv_head) * 128;
-      const uint32_t *k_from =
-          (const uint32_t *)(p.k_new + (uint64_t)leader * p.kn_stride_t + (uint64_t)kv_head * p.kn_stride_h);
-      const uint32_t *v_from =
-          (const uint32_t *)(p.v_new + (uint64_t)leader * p.vn_stride_t + (uint64_t)kv_head * p.vn_stride_h);
-      ((uint32_t *)(const_cast<uint16_t *>(p.key_pool) + at))[lane] = k_from[lane];
-      ((uint32_t *)(const_cast<uint16_t *>(p.value_pool) + at))[lane] = v_from[lane];
+      const uint64_t k_at = (uint64_t)leader * p.kn_stride_t + (uint64_t)kv_head * p.kn_stride_h;
+      const uint64_t v_at = (uint64_t)leader * p.vn_stride_t + (uint64_t)kv_head * p.vn_stride_h;
+      uint32_t k_pair, v_pair;   // this lane's two elements of the row, in the pools' dtype
+      if (kMixed && p.q_dtype == FH_F32) {
+        // rounded exactly as a store into the pool rounds (nearest even, NaN kept quiet)
+        const float2 k_two = ((const float2 *)((const float *)p.k_new + k_at))[lane];
+        const float2 v_two = ((const float2 *)((const float *)p.v_new + v_at))[lane];
+        k_pair = kHalf ? f32_to_f16(k_two.x) | (uint32_t)f32_to_f16(k_two.y) << 16
+                       : f32_to_bf16(k_two.x) | (uint32_t)f32_to_bf16(k_two.y) << 16;
+        v_pair = kHalf ? f32_to_f16(v_two.x) | (uint32_t)f32_to_f16(v_two.y) << 16
+                       : f32_to_bf16(v_two.x) | (uint32_t)f32_to_bf16(v_two.y) << 16;
+      } else {
+        k_pair = ((const uint32_t *)((const uint16_t *)p.k_new + k_at))[lane];
+        v_pair = ((const uint32_t *)((const uint16_t *)p.v_new + v_at))[lane];
+      }
+      ((uint32_t *)(const_cast<uint16_t *>(p.key_pool) + at))[lane] = k_pair;
+      ((uint32_t *)(const_cast<uint16_t *>(p.value_pool) + at))[lane] = v_pair;
       // the loads below come from the same wave, after the stores have completed
       __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
     } else if (lane == 0) {
@@ -605,11 +682,11 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
                         : (!used ? 0
                                  : min(end, p.fixed_attended ? plan.attended
                                                              : plan.attended + member_of[nt]));
-    const uint16_t *q_row = p.q + (uint64_t)(leader + member_of[nt]) * p.q_stride_t +
-                            (uint64_t)head * p.q_stride_h;
+    const uint64_t q_row = (uint64_t)(leader + member_of[nt]) * p.q_stride_t +
+                           (uint64_t)head * p.q_stride_h;
     for (int step = 0; step < 4; ++step) {  // same head-dim slice per (step, g) as the K operand
       q_reg[nt][step] = make_uint4(0, 0, 0, 0);
-      if (used) q_reg[nt][step] = *(const uint4 *)(q_row + 32 * step + 8 * g);
+      if (used) q_reg[nt][step] = load_query<kHalf, kMixed>(p, q_row + 32 * step + 8 * g);
     }
     if (NT > 1 && !used) member_of[nt] = 0xffffffffu;
   }
@@ -639,7 +716,7 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
         report_error(error + (uint64_t)leader * p.error_stride, my_page);
         for (uint32_t member = 0; member < members; ++member) p.bad[leader + member] = 1;
       }
-      if (plan.splits == 1) zero_head_rows(p, leader, members, kv_head, lane);
+      if (plan.splits == 1) zero_head_rows<kMixed>(p, leader, members, kv_head, lane);
       return;
     }
     const uint32_t tok_lo = max(begin, page0 * pt);
@@ -663,11 +740,11 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
           load_tile<false>(p, nxt, next0, end, page0, physical, lc, hl, g);
         else if (next0 < tok_hi)
           load_tile<true>(p, nxt, next0, end, page0, physical, lc, hl, g);
-        consume_tile<NT, false>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+        consume_tile<NT, false, kHalf>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
         if (next0 < tok_hi) cur = nxt;
       }
       if (full_hi < tok_hi)
-        consume_tile<NT, true>(cur, q_reg, o, sm, full_hi, limit, p.scale_log2, g);
+        consume_tile<NT, true, kHalf>(cur, q_reg, o, sm, full_hi, limit, p.scale_log2, g);
     } else {
       for (uint32_t tile0 = tok_lo; tile0 < tok_hi; tile0 += kTile) {
         TileRegs nxt;
@@ -677,9 +754,9 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
         else if (next0 < tok_hi)
           load_tile<true>(p, nxt, next0, end, page0, physical, lc, hl, g);
         if (tile0 < full_hi)
-          consume_tile<NT, false>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+          consume_tile<NT, false, kHalf>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
         else
-          consume_tile<NT, true>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+          consume_tile<NT, true, kHalf>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
         if (next0 < tok_hi) cur = nxt;
       }
     }
@@ -694,14 +771,12 @@ __device__ inline void ragged_attention_body(const FastRagged &p, ErrorSlot *err
     const uint32_t token = leader + member_of[nt];
     if (plan.splits == 1) {
       float inv = 1.0f / l_run;
-      uint16_t *out_row = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
+      const uint64_t out_row = (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
       for (int j = 0; j < 4; ++j) {
-        uint2 lo = make_uint2(pack_bf16(o[nt][0][j] * inv, o[nt][1][j] * inv),
-                              pack_bf16(o[nt][2][j] * inv, o[nt][3][j] * inv));
-        uint2 hi = make_uint2(pack_bf16(o[nt][4][j] * inv, o[nt][5][j] * inv),
-                              pack_bf16(o[nt][6][j] * inv, o[nt][7][j] * inv));
-        *(uint2 *)(out_row + 32 * g + 8 * j) = lo;
-        *(uint2 *)(out_row + 32 * g + 8 * j + 4) = hi;
+        store_out4<kHalf, kMixed>(p, out_row + 32 * g + 8 * j, o[nt][0][j] * inv, o[nt][1][j] * inv,
+                   o[nt][2][j] * inv, o[nt][3][j] * inv);
+        store_out4<kHalf, kMixed>(p, out_row + 32 * g + 8 * j + 4, o[nt][4][j] * inv, o[nt][5][j] * inv,
+                   o[nt][6][j] * inv, o[nt][7][j] * inv);
       }
       continue;
     }
@@ -772,6 +847,7 @@ __device__ inline void read_tile(const SharedTiles &lds, uint32_t buffer, TileRe
   }
 }
 
+template <bool kHalf, bool kMixed>
 __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_eu(3, 3))) void ragged_attention_prefill_kernel(
     FastRagged p, ErrorSlot *error) {
   constexpr int NT = kSharedTiles;
@@ -803,11 +879,11 @@ __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_
     member_of[nt] = first + nt * per_tile + hl / p.group;
     const bool used = hl < per_tile * p.group && member_of[nt] < plan.members;
     limit[nt] = !used ? 0 : min(end, p.fixed_attended ? plan.attended : plan.attended + member_of[nt]);
-    const uint16_t *q_row = p.q + (uint64_t)(leader + (used ? member_of[nt] : 0)) * p.q_stride_t +
-                            (uint64_t)head * p.q_stride_h;
+    const uint64_t q_row = (uint64_t)(leader + (used ? member_of[nt] : 0)) * p.q_stride_t +
+                           (uint64_t)head * p.q_stride_h;
     for (int step = 0; step < 4; ++step) {
       q_reg[nt][step] = make_uint4(0, 0, 0, 0);
-      if (used) q_reg[nt][step] = *(const uint4 *)(q_row + 32 * step + 8 * g);
+      if (used) q_reg[nt][step] = load_query<kHalf, kMixed>(p, q_row + 32 * step + 8 * g);
     }
     if (!used) member_of[nt] = 0xffffffffu;
   }
@@ -838,7 +914,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_
         report_error(error + (uint64_t)leader * p.error_stride, my_page);
         for (uint32_t member = 0; member < plan.members; ++member) p.bad[leader + member] = 1;
       }
-      if (plan.splits == 1) zero_head_rows(p, leader + first, members, kv_head, lane);
+      if (plan.splits == 1) zero_head_rows<kMixed>(p, leader + first, members, kv_head, lane);
       return;
     }
     const uint32_t tok_lo = max(begin, page0 * pt);
@@ -854,9 +930,9 @@ __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_
         TileRegs cur;
         read_tile(lds, buffer, cur, hl, g);
         if (tile0 + kTile <= unmasked_end)
-          consume_tile<NT, false>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+          consume_tile<NT, false, kHalf>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
         else
-          consume_tile<NT, true>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
+          consume_tile<NT, true, kHalf>(cur, q_reg, o, sm, tile0, limit, p.scale_log2, g);
       }
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -871,14 +947,12 @@ __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_
     const uint32_t token = leader + member_of[nt];
     if (plan.splits == 1) {
       float inv = 1.0f / l_run;
-      uint16_t *out_row = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
+      const uint64_t out_row = (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h;
       for (int j = 0; j < 4; ++j) {
-        uint2 lo = make_uint2(pack_bf16(o[nt][0][j] * inv, o[nt][1][j] * inv),
-                              pack_bf16(o[nt][2][j] * inv, o[nt][3][j] * inv));
-        uint2 hi = make_uint2(pack_bf16(o[nt][4][j] * inv, o[nt][5][j] * inv),
-                              pack_bf16(o[nt][6][j] * inv, o[nt][7][j] * inv));
-        *(uint2 *)(out_row + 32 * g + 8 * j) = lo;
-        *(uint2 *)(out_row + 32 * g + 8 * j + 4) = hi;
+        store_out4<kHalf, kMixed>(p, out_row + 32 * g + 8 * j, o[nt][0][j] * inv, o[nt][1][j] * inv,
+                   o[nt][2][j] * inv, o[nt][3][j] * inv);
+        store_out4<kHalf, kMixed>(p, out_row + 32 * g + 8 * j + 4, o[nt][4][j] * inv, o[nt][5][j] * inv,
+                   o[nt][6][j] * inv, o[nt][7][j] * inv);
       }
       continue;
     }
@@ -893,9 +967,10 @@ __global__ __launch_bounds__(64 * kSharedWaves) __attribute__((amdgpu_waves_per_
 }
 
 // Decode batches: one query token per wave, two waves per SIMD to hide the K/V stream's latency.
+template <bool kHalf, bool kMixed>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void ragged_attention_mfma_kernel(
     FastRagged p, ErrorSlot *error) {
-  ragged_attention_body<1>(p, error);
+  ragged_attention_body<1, kHalf, kMixed>(p, error);
 }
 
 // Merges the per-split partials of one (token, head): out = sum_s O_s 2^(m_s-M) / sum_s l_s
@@ -914,9 +989,9 @@ __global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
     const uint32_t token = p.merge_tokens[entry];
     const TokenPlan plan = p.plans[token];
     const bool zero = plan.splits == 0 || p.bad[token] != 0;
-    uint16_t *dst = p.out + (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
+    const uint64_t dst = (uint64_t)token * p.out_stride_t + (uint64_t)head * p.out_stride_h + column;
     if (zero) {
-      if (threadIdx.x < 32) *(uint2 *)dst = make_uint2(0, 0);
+      if (threadIdx.x < 32) store_out4<false, true>(p, dst, 0.0f, 0.0f, 0.0f, 0.0f);
       continue;
     }
     const uint64_t base = (uint64_t)token * p.max_splits * p.query_heads + head;
@@ -955,16 +1030,32 @@ __global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
         acc.w += part.w;
       }
       const float inv = 1.0f / l_all;
-      *(uint2 *)dst = make_uint2(pack_bf16(acc.x * inv, acc.y * inv), pack_bf16(acc.z * inv, acc.w * inv));
+      store_out4<false, true>(p, dst, acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
     }
   }
 }
 
+// Pools of one 2-byte dtype; queries of the same dtype, or f32 against f16 pools; any float output.
+bool fast_dtypes(const View &q, const View &out, const View &key_pool, const View &value_pool) {
+  const uint32_t pool = key_pool.dtype;
+  if ((pool != FH_BF16 && pool != FH_F16) || value_pool.dtype != pool) return false;
+  if (q.dtype != pool && !(pool == FH_F16 && q.dtype == FH_F32)) return false;
+  return out.dtype == FH_F32 || out.dtype == FH_F16 || out.dtype == FH_BF16;
+}
+
+// The decode kernel stores a lane's new row itself when the rows are of the queries' dtype (the
+// pools' own, or f32 converted on the way), a lane's two elements are one aligned load, and the
+// pool rows are word aligned.
+bool append_in_kernel_possible(const RaggedAttention &p) {
+  for (const View *v : {&p.k_new, &p.v_new})
+    if (v->dtype != p.q.dtype || v->stride[2] != 1 || v->stride[0] % 2 || v->stride[1] % 2 || v->offset % 2)
+      return false;
+  return p.key_pool.offset % 2 == 0 && p.value_pool.offset % 2 == 0;
+}
+
 bool fast_ragged_eligible(const RaggedAttention &p) {
-  auto bf16 = [](const View &v) { return v.dtype == FH_BF16; };
-  if (!bf16(p.q) || !bf16(p.k_new) || !bf16(p.v_new) || !bf16(p.out) || !bf16(p.key_pool) ||
-      !bf16(p.value_pool))
-    return false;
+  if (!fast_dtypes(p.q, p.out, p.key_pool, p.value_pool)) return false;
+  if (p.k_new.dtype != p.q.dtype || p.v_new.dtype != p.q.dtype) return false;
   if (p.width != 128 || p.value_width != 128 || p.page_tokens % 16 != 0) return false;
   uint32_t group = p.query_heads / p.kv_heads;
   if (group > 16) return false;
@@ -1046,16 +1137,27 @@ void launch_plan(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
 void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
   uint64_t groups = f.group_tokens > 1 ? f.tokens / f.group_tokens + f.lanes : f.tokens;
   uint64_t blocks = groups * f.max_splits;
+  // queries or outputs of another dtype than the pools': the kernels choose at run time
+  const uint32_t pool_dtype = f.pool_half ? FH_F16 : FH_BF16;
+  const bool mixed = f.q_dtype != pool_dtype || f.out_dtype != pool_dtype;
   {
     KernelTimer timer(backend, FH_KC_ATTENTION_KERNEL);
     // one workgroup per work item, up to 8 (decode) or 4 (prefill) kv heads of it per workgroup
     if (f.group_tokens > 1) {
-      ragged_attention_prefill_kernel<<<dim3((unsigned)blocks, f.kv_heads), 64 * kSharedWaves, 0,
-                                        stream>>>(f, error);
+      const dim3 grid((unsigned)blocks, f.kv_heads);
+      auto *kernel = f.pool_half ? (mixed ? ragged_attention_prefill_kernel<true, true>
+                                          : ragged_attention_prefill_kernel<true, false>)
+                                 : (mixed ? ragged_attention_prefill_kernel<false, true>
+                                          : ragged_attention_prefill_kernel<false, false>);
+      kernel<<<grid, 64 * kSharedWaves, 0, stream>>>(f, error);
     } else {
       const uint32_t waves = f.kv_heads < 8 ? f.kv_heads : 8;
-      ragged_attention_mfma_kernel<<<dim3((unsigned)blocks, (f.kv_heads + waves - 1) / waves),
-                                     64 * waves, 0, stream>>>(f, error);
+      const dim3 grid((unsigned)blocks, (f.kv_heads + waves - 1) / waves);
+      auto *kernel = f.pool_half ? (mixed ? ragged_attention_mfma_kernel<true, true>
+                                          : ragged_attention_mfma_kernel<true, false>)
+                                 : (mixed ? ragged_attention_mfma_kernel<false, true>
+                                          : ragged_attention_mfma_kernel<false, false>);
+      kernel<<<grid, 64 * waves, 0, stream>>>(f, error);
     }
   }
   ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens < 1024 ? f.tokens : 1024), 256, 0, stream>>>(f);
@@ -1064,9 +1166,7 @@ void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, E
 }  // namespace
 
 bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, ErrorSlot *error) {
-  auto bf16 = [](const View &v) { return v.dtype == FH_BF16; };
-  if (!bf16(lane.q) || !bf16(lane.out) || !bf16(lane.key_pool) || !bf16(lane.value_pool))
-    return false;
+  if (!fast_dtypes(lane.q, lane.out, lane.key_pool, lane.value_pool)) return false;
   if (lane.width != 128 || lane.value_width != 128 || lane.page_tokens % 16 != 0) return false;
   uint32_t group = lane.query_heads / lane.kv_heads;
   if (group > 16 || lane.query_length == 0) return false;
@@ -1089,8 +1189,11 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   f.one_start = lane.query_start;
   f.fixed_attended = lane.causal ? 0 : lane.key_length;
   if (!carve_partials(backend, &f, nullptr)) return false;
-  f.q = (const uint16_t *)lane.q.base + lane.q.offset;
-  f.out = (uint16_t *)lane.out.base + lane.out.offset;
+  f.q = (const char *)lane.q.base + lane.q.offset * dtype_size(lane.q.dtype);
+  f.out = (char *)lane.out.base + lane.out.offset * dtype_size(lane.out.dtype);
+  f.q_dtype = lane.q.dtype;
+  f.out_dtype = lane.out.dtype;
+  f.pool_half = lane.key_pool.dtype == FH_F16;
   f.key_pool = (const uint16_t *)lane.key_pool.base + lane.key_pool.offset;
   f.value_pool = (const uint16_t *)lane.value_pool.base + lane.value_pool.offset;
   f.tables = (const uint32_t *)lane.table.base + lane.table.offset;
@@ -1143,7 +1246,7 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     key.address[3] = (uint64_t)f.tables;
     key.address[4] = (uint64_t)f.generations;
     f.promised = p.one_row_per_lane;
-    f.append_in_kernel = p.one_row_per_lane && append_by_pieces(p);
+    f.append_in_kernel = p.one_row_per_lane && append_in_kernel_possible(p);
     const uint32_t params[12] = {f.tokens, f.lanes, f.group_tokens, f.page_tokens, f.physical_pages,
                                  f.table_pages, f.max_splits, forced_split_tokens(), f.kv_heads,
                                  f.query_heads, f.append_in_kernel, f.promised};
@@ -1151,16 +1254,19 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     bool reuse = false;
     char *plan_storage = backend_attention_plan(backend, key, plan_storage_bytes(f), &reuse);
     if (!plan_storage || !carve_partials(backend, &f, plan_storage)) return false;
-    f.q = (const uint16_t *)p.q.base + p.q.offset;
-    f.out = (uint16_t *)p.out.base + p.out.offset;
+    f.q = (const char *)p.q.base + p.q.offset * dtype_size(p.q.dtype);
+    f.out = (char *)p.out.base + p.out.offset * dtype_size(p.out.dtype);
+    f.q_dtype = p.q.dtype;
+    f.out_dtype = p.out.dtype;
+    f.pool_half = p.key_pool.dtype == FH_F16;
     f.key_pool = (const uint16_t *)p.key_pool.base + p.key_pool.offset;
     f.value_pool = (const uint16_t *)p.value_pool.base + p.value_pool.offset;
     f.q_stride_t = p.q.stride[0];
     f.q_stride_h = p.q.stride[1];
     f.out_stride_t = p.out.stride[0];
     f.out_stride_h = p.out.stride[1];
-    f.k_new = (const uint16_t *)p.k_new.base + p.k_new.offset;
-    f.v_new = (const uint16_t *)p.v_new.base + p.v_new.offset;
+    f.k_new = (const char *)p.k_new.base + p.k_new.offset * dtype_size(p.k_new.dtype);
+    f.v_new = (const char *)p.v_new.base + p.v_new.offset * dtype_size(p.v_new.dtype);
     f.kn_stride_t = p.k_new.stride[0];
     f.kn_stride_h = p.k_new.stride[1];
     f.vn_stride_t = p.v_new.stride[0];

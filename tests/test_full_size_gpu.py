@@ -197,6 +197,39 @@ def test_config3_decode_attention_full_batch(hip):
     attention_both_ways(hip, contexts, [1] * 128, 32, 4)
 
 
+def test_config3_decode_attention_with_the_engine_dtypes(hip):
+    """The same batch with the qwen3-coder engine's dtypes: f32 rows against an f16 KV cache.  The
+    specialised kernels against the strided ones, which an output view with unaligned rows selects;
+    both round the new rows into the pools identically."""
+    rng = np.random.default_rng(7)
+    contexts = np.exp(rng.uniform(math.log(256), math.log(32768), 128)).astype(int).tolist()
+    hq, hkv, pt, scale = 32, 4, 16, 1.0 / math.sqrt(128)
+    t = ragged_batch(hip, contexts, [1] * 128, hq, hkv, pt, seed=302)
+    rows = [seeded(hip, DType.F32, t[name].shape, 302, 6 + index) for index, name in enumerate(("q", "k_new", "v_new"))]
+    pools = [seeded(hip, DType.F16, t["keys"].shape, 302, 9 + index) for index in range(2)]
+    tail = [t["tables"], t["generations"], t["cu"], t["starts"], t["activity"]]
+    fast = hip.alloc(DType.F32, (128, hq, 128))
+    commands = CommandList()
+    commands.dispatch_many(Op.paged_attention_ragged(scale, pt, one_row_per_lane=True), [*rows, *tail],
+                           [fast, *pools])
+    run(hip, commands)
+    keys_after, values_after = hip.read(pools[0]), hip.read(pools[1])
+    padded = hip.alloc(DType.F32, (128, hq, 129))
+    commands = CommandList()
+    commands.dispatch_many(Op.paged_attention_ragged(scale, pt), [*rows, *tail],
+                           [padded.narrow(2, 0, 128), *pools])
+    run(hip, commands)
+    assert hip.read(pools[0]) == keys_after and hip.read(pools[1]) == values_after
+    generic = to_f32(hip.read(padded), DType.F32).reshape(128, hq, 129)[:, :, :128]
+    assert_close(to_f32(hip.read(fast), DType.F32), generic, DType.F16)
+    # the stored rows are the f32 rows rounded to f16, at the positions the tables name
+    new_rows = to_f32(hip.read(rows[1]), DType.F32).reshape(128, hkv * 128).astype(np.float16)
+    pool = np.frombuffer(keys_after, np.float16).reshape(-1, pt, hkv * 128)
+    for lane in (0, 17, 127):
+        page = int(t["table_array"][lane, contexts[lane] // pt, 0])
+        assert np.array_equal(pool[page, contexts[lane] % pt], new_rows[lane])
+
+
 def test_config1_packed_batch_attention(hip):
     """48 decode lanes (contexts uniform 128..4096) and prefill chunks of 256, 384, 512 and 848
     tokens packed into 2048 tokens, 16 query / 8 kv heads."""

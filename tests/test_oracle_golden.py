@@ -386,7 +386,7 @@ def test_paged_attention_matches_a_hand_checked_case(cpu):
     np.testing.assert_allclose(to_f32(cpu.read(out), DType.F32), [expected, 1 - expected], atol=1e-6)
 
 
-def paged_case(backend, hq, hkv, sq, key_length, pt, q_start, pool_dtype=DType.BF16, seed=3):
+def paged_case(backend, hq, hkv, sq, key_length, pt, q_start, pool_dtype=DType.BF16, seed=3, q_dtype=None):
     """Deterministic paged K/V in the style of crates/forja-metal/tests/paged.rs:645-659 with a
     shuffled table, generations 11+page, NaN in unused slots and a poisoned table tail."""
     width = 128
@@ -407,13 +407,14 @@ def paged_case(backend, hq, hkv, sq, key_length, pt, q_start, pool_dtype=DType.B
     table[logical:] = [0, 0xffffffff]
     index = np.arange(hq * sq * width)
     query = ((index * 17) % 89) / 88.0 - 0.5
+    q_dtype = pool_dtype if q_dtype is None else q_dtype      # the dtype of the query and of the output
     tensors = dict(
-        q=upload(backend, query.reshape(hq, sq, width), pool_dtype),
+        q=upload(backend, query.reshape(hq, sq, width), q_dtype),
         keys=upload(backend, keys.reshape(physical, pt, hkv, width), pool_dtype),
         values=upload(backend, vals.reshape(physical, pt, hkv, width), pool_dtype),
         table=upload(backend, table, DType.U32),
         generations=upload(backend, 11 + np.arange(physical), DType.U32),
-        out=backend.alloc(pool_dtype, (hq, sq, width)))
+        out=backend.alloc(q_dtype, (hq, sq, width)))
     host = dict(q=query.reshape(hq, sq, width), keys=keys, vals=vals, rows=rows, pt=pt)
     return tensors, host
 

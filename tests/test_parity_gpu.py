@@ -23,13 +23,20 @@ def run(backend, commands):
     backend.submit(commands).wait()
 
 
-def compare(cpu, hip, cpu_tensor, hip_tensor, **kw):
+def coarser(*dtypes):
+    """The dtype whose tolerance judges an attention output: the reference holds f32 outputs
+    computed from f16 or bf16 pools to the pools' tolerance (crates/forja-metal/tests/paged.rs:982-988)."""
+    return max(dtypes, key=[DType.F32, DType.F16, DType.BF16].index)
+
+
+def compare(cpu, hip, cpu_tensor, hip_tensor, bar=None, **kw):
+    """`bar`: the dtype whose tolerance applies to float outputs (their own when not given)."""
     dtype = cpu_tensor.dtype
     a, b = cpu.read(cpu_tensor), hip.read(hip_tensor)
     if dtype in (DType.U32, DType.I32):
         assert a == b
     else:
-        assert_close(to_f32(b, dtype), to_f32(a, dtype), dtype, **kw)
+        assert_close(to_f32(b, dtype), to_f32(a, dtype), coarser(dtype, bar or dtype), **kw)
 
 
 def differential(cpu, hip, build, expect_error=None, **kw):
@@ -501,6 +508,31 @@ def test_paged_sdpa(cpu, hip, hq, hkv, sq, key_length, q_start, causal, dtype, p
     differential(cpu, hip, build)
 
 
+@pytest.mark.parametrize("sq,key_length,q_start", [(1, 300, 299), (77, 177, 100)])
+@pytest.mark.parametrize("q_dtype", [DType.F32, DType.F16])
+def test_paged_sdpa_and_append_with_f16_pools(cpu, hip, q_dtype, sq, key_length, q_start):
+    """The qwen3-coder engine's dtypes: f32 activations against an f16 KV cache
+    (engines/qwen3-coder/src/lib.rs: the pools are allocated as F16, the rows arrive as F32)."""
+    hq, hkv, pt = 32, 4, 64
+    scale = 1.0 / math.sqrt(128)
+    k_new = normal_bf16(52, 1, (sq, hkv, 128)) * 1.001      # not representable in f16 as they stand
+    v_new = normal_bf16(52, 2, (sq, hkv, 128)) * 1.001
+
+    def build(backend):
+        t, _ = paged_case(backend, hq, hkv, sq, key_length, pt, q_start, pool_dtype=DType.F16, q_dtype=q_dtype)
+        appended = backend.alloc(q_dtype, (hq, sq, 128))
+        commands = CommandList()
+        commands.dispatch(Op.paged_sdpa(scale, True, q_start, key_length, pt),
+                          [t["q"], t["keys"], t["values"], t["table"], t["generations"]], t["out"])
+        if sq == 1:       # the appending form takes a single query row (check_paged_append, ops.rs:2266)
+            commands.dispatch_many(Op.paged_sdpa_append(scale, q_start, pt),
+                                   [t["q"], upload(backend, k_new, q_dtype), upload(backend, v_new, q_dtype),
+                                    t["table"], t["generations"]], [appended, t["keys"], t["values"]])
+        return commands, [t["out"], appended, t["keys"], t["values"]]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build, bar=DType.F16)
+    assert cpu.read(cpu_out[2]) == hip.read(hip_out[2]) and cpu.read(cpu_out[3]) == hip.read(hip_out[3])
+
+
 def test_paged_sdpa_through_a_permuted_query_view(cpu, hip):
     """Engines pass q as a permuted [Hq,Sq,D] view of [Sq,Hq,D] storage and read the output the
     same way (crates/forja-host/src/lib.rs:6223-6333)."""
@@ -570,10 +602,13 @@ def test_stale_generation_is_reported_and_never_dereferenced(hip):
 # ------------------------------------------------------------------ ragged batch
 
 def ragged_case(backend, contexts, counts, hq, hkv, pt, seed, activity=None, dtype=DType.BF16,
-                corrupt=None):
+                corrupt=None, pool_dtype=None, out_dtype=None):
     """Lanes with `contexts[l]` tokens already cached and `counts[l]` new queries each.  Shuffled
-    physical pages shared by all lanes, generations 11+page, poisoned table tails."""
+    physical pages shared by all lanes, generations 11+page, poisoned table tails.  `dtype` is
+    that of the query and of the new rows; pools and output follow it unless named."""
     width = 128
+    pool_dtype = dtype if pool_dtype is None else pool_dtype
+    out_dtype = dtype if out_dtype is None else out_dtype
     lanes = len(contexts)
     pages_needed = [(c + n + pt - 1) // pt for c, n in zip(contexts, counts)]
     table_pages = max(pages_needed) + 2
@@ -601,9 +636,9 @@ def ragged_case(backend, contexts, counts, hq, hkv, pt, seed, activity=None, dty
         generations=upload(backend, 11 + np.arange(physical), DType.U32),
         cu=upload(backend, cu, DType.U32),
         starts=upload(backend, np.array(contexts), DType.U32),
-        out=backend.alloc(dtype, (total, hq, width)),
-        keys=upload(backend, pool_k.reshape(physical, pt, hkv, width), dtype),
-        values=upload(backend, pool_v.reshape(physical, pt, hkv, width), dtype))
+        out=backend.alloc(out_dtype, (total, hq, width)),
+        keys=upload(backend, pool_k.reshape(physical, pt, hkv, width), pool_dtype),
+        values=upload(backend, pool_v.reshape(physical, pt, hkv, width), pool_dtype))
     inputs = [tensors[n] for n in ("q", "k_new", "v_new", "tables", "generations", "cu", "starts")]
     if activity is not None:
         inputs.append(upload(backend, np.array(activity), DType.U32))
@@ -635,6 +670,67 @@ def test_ragged_attention_equals_the_per_lane_sequence(cpu, hip, contexts, count
     (cpu_out, _), (hip_out, _) = differential(cpu, hip, build)
     # block-table gather and append placement are pure addressing: pools must match bit for bit
     assert cpu.read(cpu_out[1]) == hip.read(hip_out[1]) and cpu.read(cpu_out[2]) == hip.read(hip_out[2])
+
+
+DTYPE_MIXES = [
+    # query and new rows, pools, output
+    (DType.F32, DType.F16, DType.F32),      # the qwen3-coder engine
+    (DType.F16, DType.F16, DType.F16),
+    (DType.F16, DType.F16, DType.BF16),
+    (DType.BF16, DType.BF16, DType.F32),
+]
+
+
+@pytest.mark.parametrize("dtype,pool_dtype,out_dtype", DTYPE_MIXES)
+@pytest.mark.parametrize("contexts,counts,hq,hkv,pt,promise", [
+    ([300, 1, 2047, 700, 15, 16, 0], [1] * 7, 32, 4, 16, True),
+    ([300, 1, 2047, 700, 15, 16, 0], [1] * 7, 32, 4, 64, False),
+    ([0, 130, 33, 900], [70, 1, 45, 1], 40, 8, 16, False),
+    (list(range(0, 520, 13)), [1] * 40, 16, 8, 16, True)])
+def test_ragged_attention_across_activation_and_pool_dtypes(cpu, hip, dtype, pool_dtype, out_dtype, contexts,
+                                                            counts, hq, hkv, pt, promise):
+    """f16 or bf16 pools fed by rows of their own dtype or (f16) by f32 rows, any float output: the
+    stored rows are rounded once, exactly as the oracle rounds them, so the pools match bit for
+    bit; a second layer reuses the work plan on other pools."""
+    scale = 1.0 / math.sqrt(128)
+
+    def build(backend):
+        t, inputs = ragged_case(backend, contexts, counts, hq, hkv, pt, seed=69, dtype=dtype,
+                                pool_dtype=pool_dtype, out_dtype=out_dtype)
+        # new rows with more significand bits than the pools hold
+        rows = sum(counts)
+        inputs[1] = upload(backend, normal_bf16(69, 6, (rows, hkv, 128)) * 1.001, dtype)
+        inputs[2] = upload(backend, normal_bf16(69, 7, (rows, hkv, 128)) * 1.001, dtype)
+        physical = t["keys"].shape[0]
+        other_k = upload(backend, normal_bf16(69, 8, (physical, pt, hkv, 128)), pool_dtype)
+        other_v = upload(backend, normal_bf16(69, 9, (physical, pt, hkv, 128)), pool_dtype)
+        out2 = backend.alloc(out_dtype, t["out"].shape)
+        op = Op.paged_attention_ragged(scale, pt, one_row_per_lane=promise)
+        commands = CommandList()
+        commands.dispatch_many(op, inputs, [t["out"], t["keys"], t["values"]])
+        commands.dispatch_many(op, inputs, [out2, other_k, other_v])
+        return commands, [t["out"], out2, t["keys"], t["values"], other_k, other_v]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build, bar=pool_dtype)
+    for index in (2, 3, 4, 5):
+        assert cpu.read(cpu_out[index]) == hip.read(hip_out[index])
+
+
+def test_f32_queries_beyond_the_f16_range_stay_finite(cpu, hip):
+    """An f32 query element no f16 holds: the oracle's scores are huge but finite, and so are the
+    device's (the element is held at the largest finite f16); the winner of such a softmax is
+    one key on both sides."""
+    def build(backend):
+        t, inputs = ragged_case(backend, [40, 7], [1, 1], 8, 2, 16, seed=70, dtype=DType.F32,
+                                pool_dtype=DType.F16)
+        values = normal_bf16(70, 3, (2, 8, 128)).astype(np.float32)
+        values[0, 3, 5] = 3.0e6
+        values[1, 0, 100] = -1.0e9
+        inputs[0] = upload(backend, values, DType.F32)
+        commands = CommandList()
+        commands.dispatch_many(Op.paged_attention_ragged(0.09, 16), inputs, [t["out"], t["keys"], t["values"]])
+        return commands, [t["out"]]
+    (cpu_out, _), (hip_out, _) = differential(cpu, hip, build, bar=DType.F16)
+    assert np.isfinite(to_f32(hip.read(hip_out[0]), DType.F32)).all()
 
 
 @pytest.mark.parametrize("contexts,counts,hq,hkv", [([300, 40, 2047, 700], [1, 1, 1, 1], 32, 4),

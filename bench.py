@@ -426,6 +426,63 @@ def prefill_attention_c4(backend, seed=93, repeats=3):
             "tflops": flops / (op_ns / repeats * 1e-9) / 1e12}
 
 
+def decode_attention_f16_cache(backend, config, seed=99, repeats=5):
+    """One layer's decode attention of the timed workload's shape (128 lanes, contexts log-uniform
+    256..32768) with the dtypes the qwen3-coder engine records: f32 query and new rows, an f16 KV
+    cache, f32 output; one row per lane promised, so the kernel stores the new rows itself."""
+    rng = np.random.default_rng(seed)
+    lanes, pt = 128, config.page_tokens
+    contexts = log_uniform(rng, 256, 32768, lanes)
+    pages_of = [(int(ctx) + 1 + pt - 1) // pt for ctx in contexts]
+    table_pages, physical = max(pages_of), sum(pages_of) + 7
+    order = rng.permutation(physical)
+    tables = np.zeros((lanes, table_pages, 2), np.uint32)
+    tables[:, :, 1] = 0xffffffff
+    cursor = 0
+    for lane, n_pages in enumerate(pages_of):
+        pages = order[cursor:cursor + n_pages]
+        cursor += n_pages
+        tables[lane, :n_pages, 0] = pages
+        tables[lane, :n_pages, 1] = 11 + pages
+
+    def up(array, shape):
+        tensor = backend.alloc(DType.U32, shape)
+        backend.write(tensor, np.ascontiguousarray(array, dtype=np.uint32).tobytes())
+        return tensor
+    metadata = [up(tables, tables.shape), up(11 + np.arange(physical), (physical,)),
+                up(np.arange(lanes + 1), (lanes + 1,)), up(np.array(contexts), (lanes,))]
+    q = backend.alloc(DType.F32, (lanes, config.q_heads, config.head_dim))
+    k_new = backend.alloc(DType.F32, (lanes, config.kv_heads, config.head_dim))
+    v_new = backend.alloc(DType.F32, (lanes, config.kv_heads, config.head_dim))
+    out = backend.alloc(DType.F32, (lanes, config.q_heads, config.head_dim))
+    keys = backend.alloc(DType.F16, (physical, pt, config.kv_heads, config.head_dim))
+    values = backend.alloc(DType.F16, (physical, pt, config.kv_heads, config.head_dim))
+    fill = CommandList()
+    for stream, tensor in enumerate((q, k_new, v_new, keys, values)):
+        fill.dispatch(Op.fill_seeded(2, seed, 30 + stream), [], tensor)
+    backend.submit(fill).wait()
+    commands = CommandList()
+    commands.dispatch_many(Op.paged_attention_ragged(1.0 / math.sqrt(config.head_dim), pt, one_row_per_lane=True),
+                           [q, k_new, v_new, *metadata], [out, keys, values])
+    encoded = backend.encode(commands)
+    backend.submit(encoded).wait()
+    backend.profile_enable(2)
+    backend.profile_reset()
+    for _ in range(repeats):
+        backend.submit(encoded).wait()
+    op_ns, _ = backend.profile_read(KC_ATTENTION)
+    kernel_ns, _ = backend.profile_read(KC_ATTENTION_KERNEL)
+    backend.profile_enable(0)
+    for tensor in (*metadata, q, k_new, v_new, out, keys, values):
+        backend.release(tensor)
+    kv_bytes = sum(int(ctx) + 1 for ctx in contexts) * config.kv_heads * config.head_dim * 2 * 2
+    gbps = kv_bytes / (kernel_ns / repeats)
+    return {"workload": "one layer's decode attention, 128 lanes, contexts log-uniform 256-32768, f32 rows, "
+                        "f16 KV cache, f32 output",
+            "us_op": op_ns / repeats / 1e3, "us_kernel": kernel_ns / repeats / 1e3,
+            "algorithmic_bytes": kv_bytes, "achieved_gbps": gbps, "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS}
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -619,7 +676,8 @@ def main():
         result["secondary_workloads"] = {"prefill_gemm_c4": gemm,
                                          "prefill_attention_c4": prefill_attention_c4(backend),
                                          "prefill_layer_c4": prefill_layer_c4(backend),
-                                         "packed_step_c1": packed_step_c1(backend)}
+                                         "packed_step_c1": packed_step_c1(backend),
+                                         "decode_attention_f16_cache": decode_attention_f16_cache(backend, config)}
         if config.moe:
             result["secondary_workloads"]["moe_block_c2"] = moe_block_c2(backend, workload.model)
     step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction

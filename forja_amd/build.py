@@ -9,7 +9,7 @@ LIB = os.path.join(HERE, "libforja_hip.so")
 PROBES = os.path.join(HERE, "libforja_probes.so")
 CONFORMANCE = os.path.join(HERE, "host", "conformance")
 
-SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "qmm_gemm.hip", "programs_fast.hip", "lane_fusion.hip", "sampling.hip"]
+SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "qmm_gemm.hip", "programs_fast.hip", "lane_fusion.hip", "sampling.hip", "qmm_valu.hip"]
 
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -17,7 +17,8 @@ COMMON = [
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
 ]
 # The generic kernels follow the reference's mul-then-add order; no fused contraction there.
-PER_FILE = {"generic_ops.hip": ["-ffp-contract=off"], "sampling.hip": ["-ffp-contract=off"]}
+PER_FILE = {"generic_ops.hip": ["-ffp-contract=off"], "sampling.hip": ["-ffp-contract=off"],
+            "qmm_valu.hip": ["-ffp-contract=off"]}
 
 
 def build(verbose=False, jobs=8):

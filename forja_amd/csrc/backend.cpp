@@ -574,7 +574,7 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
   if (!d.epilogue) {
     QmmProblem problem{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows, inner, columns,
                        d.bits, d.group_size};
-    if (try_fast_quant_matmul(b, problem)) return FH_OK;
+    if (try_fast_quant_matmul(b, problem) || try_valu_quant_matmul(b, problem)) return FH_OK;
     launch_quant_matmul_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows,
                                 inner, columns, d.bits, d.group_size);
     return FH_OK;
@@ -587,7 +587,7 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
       shape_is(d.inputs[primitive], {rows, columns})) {
     QmmProblem fused{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows, inner, columns,
                      d.bits, d.group_size, &pl.in[primitive]};
-    if (try_fast_quant_matmul(b, fused)) return FH_OK;
+    if (try_fast_quant_matmul(b, fused) || try_valu_quant_matmul(b, fused)) return FH_OK;
   }
   // The accumulators live apart from the workspace, which the product kernels use themselves.
   uint64_t elements = (uint64_t)rows * columns;
@@ -596,7 +596,7 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
   View acc_view = contiguous_view(acc, FH_F32, out);
   QmmProblem problem{pl.in[0], pl.in[1], pl.in[2], pl.in[3], acc_view, rows, inner, columns,
                      d.bits, d.group_size};
-  if (!try_fast_quant_matmul(b, problem))
+  if (!try_fast_quant_matmul(b, problem) && !try_valu_quant_matmul(b, problem))
     launch_quant_matmul_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], acc_view, rows,
                                 inner, columns, d.bits, d.group_size);
   return run_epilogue(b, pl, primitive, acc, 1);
@@ -644,6 +644,9 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
     if (!d.epilogue) {
       problem.out = pl.out[0];
       if (try_fast_gather_weighted(b, problem, nullptr, error)) return FH_OK;
+      if (try_valu_gather(b, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4], &pl.in[5], pl.out[0], rows,
+                          routes, inner, experts, columns, d.bits, d.group_size, error))
+        return FH_OK;
       launch_gather_weighted_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4],
                                      pl.in[5], pl.out[0], rows, routes, inner, experts, columns,
                                      d.bits, d.group_size, error);
@@ -664,9 +667,11 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
     char *acc = b->ensure_workspace(elements * 4);
     if (!acc) return FH_ALLOCATION_FAILED;
     View acc_view = contiguous_view(acc, FH_F32, out);
-    launch_gather_weighted_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4],
-                                   pl.in[5], acc_view, rows, routes, inner, experts, columns,
-                                   d.bits, d.group_size, error);
+    if (!try_valu_gather(b, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4], &pl.in[5], acc_view, rows,
+                         routes, inner, experts, columns, d.bits, d.group_size, error))
+      launch_gather_weighted_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4],
+                                     pl.in[5], acc_view, rows, routes, inner, experts, columns,
+                                     d.bits, d.group_size, error);
     return run_epilogue(b, pl, primitive, acc, 1);
   }
   // check_gather_quant_projection (ops.rs:1933-1992), once or twice.
@@ -710,6 +715,9 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
   problem.group = d.group_size;
   if (!d.epilogue) {
     if (try_fast_gather_projection(b, problem, 1, false, error)) return FH_OK;
+    if (try_valu_gather(b, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[primitive - 1], nullptr, pl.out[0],
+                        rows, k, inner, experts, columns, d.bits, d.group_size, error))
+      return FH_OK;
     launch_gather_projection_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3],
                                      pl.in[primitive - 1], pl.out[0], rows, inner, experts,
                                      columns, k, d.bits, d.group_size, error);
@@ -727,14 +735,18 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
   char *acc = b->ensure_workspace(elements * 4 * accumulators);
   if (!acc) return FH_ALLOCATION_FAILED;
   View acc0 = contiguous_view(acc, FH_F32, out);
-  launch_gather_projection_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3],
-                                   pl.in[primitive - 1], acc0, rows, inner, experts, columns, k,
-                                   d.bits, d.group_size, error);
+  if (!try_valu_gather(b, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[primitive - 1], nullptr, acc0, rows,
+                       k, inner, experts, columns, d.bits, d.group_size, error))
+    launch_gather_projection_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3],
+                                     pl.in[primitive - 1], acc0, rows, inner, experts, columns, k,
+                                     d.bits, d.group_size, error);
   if (primitive == 8) {
     View acc1 = contiguous_view(acc + elements * 4, FH_F32, out);
-    launch_gather_projection_generic(b->stream, pl.in[0], pl.in[4], pl.in[5], pl.in[6], pl.in[7],
-                                     acc1, rows, inner, experts, columns, k, d.bits, d.group_size,
-                                     error);
+    if (!try_valu_gather(b, pl.in[0], pl.in[4], pl.in[5], pl.in[6], pl.in[7], nullptr, acc1, rows, k, inner,
+                         experts, columns, d.bits, d.group_size, error))
+      launch_gather_projection_generic(b->stream, pl.in[0], pl.in[4], pl.in[5], pl.in[6], pl.in[7],
+                                       acc1, rows, inner, experts, columns, k, d.bits, d.group_size,
+                                       error);
   }
   return run_epilogue(b, pl, primitive, acc, accumulators);
 }

@@ -59,6 +59,17 @@ struct QmmProblem {
   const View *residual = nullptr;
 };
 bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &problem);
+// The f32 vector-ALU kernel for what the matrix-core kernels do not take: any float activation and
+// output dtype, 4- or 8-bit weights, groups of 32/64/128, f16 or bf16 scales, contiguous rows
+// (`residual` of any float dtype).  False when the operands do not fit it either.
+bool try_valu_quant_matmul(fh_backend *backend, const QmmProblem &problem);
+// Its routed forms: the projection out[r,s,:] = x[r,:] . W[indices[r,s]]^T (`weights` null) and
+// the weighted sum out[r,:] = sum_s weights[r,s] * (x[r,s,:] . W[indices[r,s]]^T); `out` may be an
+// f32 accumulator view.  Same operand conditions; false when they do not hold.
+bool try_valu_gather(fh_backend *backend, const View &x, const View &packed, const View &scales,
+                     const View &biases, const View &indices, const View *weights, const View &out,
+                     uint32_t rows, uint32_t k, uint32_t inner, uint32_t experts, uint32_t columns,
+                     uint32_t bits, uint32_t group, ErrorSlot *error);
 // Dequantise-once tiled GEMM for many rows; operands as checked by try_fast_quant_matmul.  False
 // when the launch could not be configured.  On success `*refused` points at a device word the
 // launched kernels leave non-zero when some scale or bias is outside their fp16 scheme; they

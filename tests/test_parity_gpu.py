@@ -164,6 +164,14 @@ QMM_CASES = [
     (257, 300, 512, 4, 64, DType.BF16),     # GEMM with row and column tails
     (1000, 96, 256, 4, 64, DType.BF16),     # GEMM, a single column tile, four row tiles
     (512, 1024, 2048, 4, 64, DType.BF16),   # GEMM, whole tiles
+    # f32 / f16 activations and 8-bit weights: the f32 vector-ALU kernel
+    (8, 5120, 2048, 4, 64, DType.F32),      # the qwen3-coder engine's decode batch: stacked qkv
+    (8, 128, 2048, 8, 64, DType.F32),       # its 8-bit router
+    (128, 2048, 4096, 4, 64, DType.F32),    # o_proj on a full decode batch
+    (19, 130, 1056, 4, 32, DType.F16),      # row, column and wave tails; 33 pieces over 8 waves
+    (70, 200, 384, 8, 128, DType.F16),
+    (3, 70, 32, 4, 32, DType.F32),          # a single piece: one wave
+    (300, 96, 256, 8, 32, DType.BF16),      # prefill rows with 8-bit weights
 ]
 
 
@@ -179,6 +187,32 @@ def test_quant_matmul(cpu, hip, rows, n, k, bits, group, dtype):
         commands = CommandList()
         commands.dispatch(Op.quant_matmul(bits, group), [x, packed, scales, biases], out)
         return commands, [out]
+    differential(cpu, hip, build)
+
+
+@pytest.mark.parametrize("dtype,bits,group", [(DType.F32, 4, 64), (DType.F16, 8, 32), (DType.BF16, 4, 128)])
+def test_quant_matmul_with_f16_scales_and_a_residual_in_other_dtypes(cpu, hip, dtype, bits, group):
+    """f16 affine parameters (the reference allows f16 or bf16, quantized.rs:78-121) and the
+    residual-add epilogue on activations that are not bf16, plus an unrecognised epilogue."""
+    rows, n, k = 40, 200, 768
+    weights = Quantised(24, n + k, (n, k), bits=bits, group=group)
+    x_values = normal_bf16(24, 1, (rows, k))
+    extra_values = normal_bf16(24, 2, (rows, n))
+
+    def build(backend):
+        x = upload(backend, x_values, dtype)
+        extra = upload(backend, extra_values, dtype)
+        plain, added, scaled = (backend.alloc(dtype, (rows, n)) for _ in range(3))
+        triple = weights.upload(backend, scale_dtype=DType.F16)
+        b = ProgramBuilder(ProgramKind.MAP)
+        b.output(0, b.mul(b.input(0), b.input(1)))
+        commands = CommandList()
+        commands.dispatch(Op.quant_matmul(bits, group), [x, *triple], plain)
+        commands.dispatch_epilogue(Op.quant_matmul(bits, group), [x, *triple], added,
+                                   backend.prepare_epilogue(programs.add_elements()), [extra])
+        commands.dispatch_epilogue(Op.quant_matmul(bits, group), [x, *triple], scaled,
+                                   backend.prepare_epilogue(b.finish()), [extra])
+        return commands, [plain, added, scaled]
     differential(cpu, hip, build)
 
 
@@ -312,6 +346,68 @@ def test_gather_projection_pair_and_weighted_sum(cpu, hip, rows, k, experts, n, 
         commands.dispatch(Op.gather_quant_matmul(4, 64), [activated, *d, idx, weights], summed)
         return commands, [plain, activated, combined, summed]
     differential(cpu, hip, build)
+
+
+@pytest.mark.parametrize("dtype,bits,group,scale_dtype", [
+    (DType.F32, 4, 64, DType.BF16),      # the qwen3-coder engine: f32 activations
+    (DType.F16, 8, 32, DType.F16),
+    (DType.BF16, 4, 128, DType.BF16),    # a group size the matrix-core kernels do not take
+])
+@pytest.mark.parametrize("rows,k,experts,n,inner", [(8, 8, 128, 768, 2048), (37, 3, 5, 96, 256)])
+def test_gather_in_other_dtypes_bits_and_groups(cpu, hip, rows, k, experts, n, inner, dtype, bits, group,
+                                                scale_dtype):
+    """The routed forms through the f32 vector-ALU kernels, with two bad routes: the valid routes
+    agree with the oracle, the lowest bad expert is reported, bad projection rows read zero and bad
+    routes are left out of the weighted sum."""
+    gate = Quantised(35, 1, (n, inner), bits=bits, group=group, experts=experts)
+    up = Quantised(35, 11, (n, inner), bits=bits, group=group, experts=experts)
+    down = Quantised(35, 21, (inner, n), bits=bits, group=group if n % group == 0 else 32, experts=experts)
+    down_group = down.group
+    indices = routed_case(35, rows, k, experts, n, inner, bad=[(1, 2, experts + 9), (rows - 1, 0, experts)])
+    x_values = normal_bf16(35, 40, (rows, inner))
+    logits = orc.fill_normal_f32(35, 41, rows * k).reshape(rows, k)
+    w_values = np.exp(logits) / np.exp(logits).sum(axis=1, keepdims=True)
+    residual_values = normal_bf16(35, 42, (rows, inner))
+
+    def build(backend, good_only):
+        x = upload(backend, x_values, dtype)
+        idx = upload(backend, indices if not good_only else indices % experts, DType.U32)
+        g, u, d = (w.upload(backend, scale_dtype=scale_dtype) for w in (gate, up, down))
+        plain, activated = (backend.alloc(dtype, (rows, k, n)) for _ in range(2))
+        combined, summed = (backend.alloc(dtype, (rows, inner)) for _ in range(2))
+        weights = upload(backend, w_values, dtype)
+        residual = upload(backend, residual_values, dtype)
+        swiglu = backend.prepare_epilogue(programs.silu_mul_elements())
+        add = backend.prepare_epilogue(programs.add_elements())
+        first, second = CommandList(), CommandList()
+        first.dispatch(Op.gather_quant_matmul(bits, group), [x, *g, idx], plain)
+        second.dispatch_epilogue(Op.gather_quant_matmul(bits, group), [x, *g, *u, idx], activated, swiglu, [])
+        second.dispatch_epilogue(Op.gather_quant_matmul(bits, down_group), [activated, *d, idx, weights],
+                                 combined, add, [residual])
+        second.dispatch(Op.gather_quant_matmul(bits, down_group), [activated, *d, idx, weights], summed)
+        return (first, second), [plain, activated, combined, summed]
+
+    # without bad routes: every output against the oracle
+    outputs = []
+    for backend in (cpu, hip):
+        lists, tensors = build(backend, True)
+        for commands in lists:
+            run(backend, commands)
+        outputs.append(tensors)
+    for a, b in zip(*outputs):
+        compare(cpu, hip, a, b)
+    # with them: the lowest bad expert is reported by both, the projection's bad rows are zero
+    for backend in (cpu, hip):
+        lists, tensors = build(backend, False)
+        with pytest.raises(BackendError) as info:
+            run(backend, lists[0])
+        assert info.value.index == experts
+        if backend is hip:
+            values = to_f32(hip.read(tensors[0]), dtype).reshape(rows, k, n)
+            assert not values[1, 2].any() and not values[rows - 1, 0].any() and values[0, 0].any()
+            with pytest.raises(BackendError) as info:
+                run(backend, lists[1])
+            assert info.value.index == experts
 
 
 def test_gather_reports_lowest_bad_expert_and_zeroes_its_rows(cpu, hip):

@@ -644,6 +644,7 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
     if (!d.epilogue) {
       problem.out = pl.out[0];
       if (try_fast_gather_weighted(b, problem, nullptr, error)) return FH_OK;
+      if (try_valu_gather_grouped(b, problem, 0, pl.out[0], true, nullptr, error)) return FH_OK;
       if (try_valu_gather(b, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[4], &pl.in[5], pl.out[0], rows,
                           routes, inner, experts, columns, d.bits, d.group_size, error))
         return FH_OK;
@@ -662,6 +663,7 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
       FH_REQUIRE(shape_is(residual, {rows, columns}) && is_float(residual.dtype));
       problem.out = pl.out[0];
       if (try_fast_gather_weighted(b, problem, &pl.in[primitive], error)) return FH_OK;
+      if (try_valu_gather_grouped(b, problem, 0, pl.out[0], true, &pl.in[primitive], error)) return FH_OK;
     }
     uint64_t elements = (uint64_t)rows * columns;
     char *acc = b->ensure_workspace(elements * 4);
@@ -715,6 +717,7 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
   problem.group = d.group_size;
   if (!d.epilogue) {
     if (try_fast_gather_projection(b, problem, 1, false, error)) return FH_OK;
+    if (try_valu_gather_grouped(b, problem, 0, pl.out[0], false, nullptr, error)) return FH_OK;
     if (try_valu_gather(b, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[primitive - 1], nullptr, pl.out[0],
                         rows, k, inner, experts, columns, d.bits, d.group_size, error))
       return FH_OK;
@@ -735,14 +738,16 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
   char *acc = b->ensure_workspace(elements * 4 * accumulators);
   if (!acc) return FH_ALLOCATION_FAILED;
   View acc0 = contiguous_view(acc, FH_F32, out);
-  if (!try_valu_gather(b, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[primitive - 1], nullptr, acc0, rows,
+  if (!try_valu_gather_grouped(b, problem, 0, acc0, false, nullptr, error) &&
+      !try_valu_gather(b, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.in[primitive - 1], nullptr, acc0, rows,
                        k, inner, experts, columns, d.bits, d.group_size, error))
     launch_gather_projection_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3],
                                      pl.in[primitive - 1], acc0, rows, inner, experts, columns, k,
                                      d.bits, d.group_size, error);
   if (primitive == 8) {
     View acc1 = contiguous_view(acc + elements * 4, FH_F32, out);
-    if (!try_valu_gather(b, pl.in[0], pl.in[4], pl.in[5], pl.in[6], pl.in[7], nullptr, acc1, rows, k, inner,
+    if (!try_valu_gather_grouped(b, problem, 1, acc1, false, nullptr, error) &&
+        !try_valu_gather(b, pl.in[0], pl.in[4], pl.in[5], pl.in[6], pl.in[7], nullptr, acc1, rows, k, inner,
                          experts, columns, d.bits, d.group_size, error))
       launch_gather_projection_generic(b->stream, pl.in[0], pl.in[4], pl.in[5], pl.in[6], pl.in[7],
                                        acc1, rows, inner, experts, columns, k, d.bits, d.group_size,

@@ -63,6 +63,7 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &problem);
 // output dtype, 4- or 8-bit weights, groups of 32/64/128, f16 or bf16 scales, contiguous rows
 // (`residual` of any float dtype).  False when the operands do not fit it either.
 bool try_valu_quant_matmul(fh_backend *backend, const QmmProblem &problem);
+
 // Its routed forms: the projection out[r,s,:] = x[r,:] . W[indices[r,s]]^T (`weights` null) and
 // the weighted sum out[r,:] = sum_s weights[r,s] * (x[r,s,:] . W[indices[r,s]]^T); `out` may be an
 // f32 accumulator view.  Same operand conditions; false when they do not hold.
@@ -85,6 +86,26 @@ struct GatherProblem {
   View out;         // projection: [R,k,N]; weighted sum: [R,N]
   uint32_t rows, k, inner, experts, columns, bits, group;
 };
+
+// The routes of a gather problem packed by expert on the device (or the plan the previous routed
+// dispatch packed from the same indices): `blocks` holds (expert, first, count <= tile) triples over
+// `sorted_routes`, `n_blocks[0]` how many; bad routes are left out and reported.  `rest` is `extra`
+// bytes of workspace.
+struct PackedRoutes {
+  const uint32_t *sorted_routes, *blocks, *n_blocks;
+  uint32_t max_blocks, tile;
+  char *rest;
+};
+bool pack_routes(fh_backend *backend, const GatherProblem &problem, uint64_t extra, ErrorSlot *error,
+                 PackedRoutes *packed);
+// out[r,:] = residual? + sum_s weights[r,s] * partial[r*k+s,:] over the valid routes, ascending s.
+void launch_combine_routes(hipStream_t stream, const float *partial, const GatherProblem &problem,
+                           const View *residual);
+// Routed products grouped by expert on the f32 vector ALUs, for batches with several routes per
+// expert: `weighted` false computes out[r,s,:] (a dense [R,k,N] view, zero rows for bad routes),
+// true the weighted sum with an optional residual.  False when the operands do not fit.
+bool try_valu_gather_grouped(fh_backend *backend, const GatherProblem &problem, int projection,
+                             const View &out, bool weighted, const View *residual, ErrorSlot *error);
 // projections = 1 (plain) or 2 (gate/up pair); swiglu = fuse silu(acc0)*acc1.
 bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &problem, int projections,
                                 bool swiglu, ErrorSlot *error);

@@ -1220,6 +1220,30 @@ bool gather_eligible(const GatherProblem &p, int projections) {
 
 }  // namespace
 
+bool pack_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, ErrorSlot *error,
+                 PackedRoutes *packed) {
+  if ((uint64_t)p.rows * p.k > (1u << 24) || p.experts > 512) return false;
+  RoutePlan plan;
+  if (!plan_routes(backend, p, extra, error, &plan)) return false;
+  packed->sorted_routes = plan.sorted_routes;
+  packed->blocks = plan.blocks;
+  packed->n_blocks = plan.n_blocks;
+  packed->max_blocks = plan.max_blocks;
+  packed->tile = kRouteTile;
+  packed->rest = plan.rest;
+  return true;
+}
+
+void launch_combine_routes(hipStream_t stream, const float *partial, const GatherProblem &p,
+                           const View *residual) {
+  View none{};
+  none.base = nullptr;
+  const uint64_t work = (uint64_t)p.rows * p.columns;
+  combine_routes_kernel<<<dim3((unsigned)((work + 255) / 256)), 256, 0, stream>>>(
+      partial, p.indices, p.weights, residual ? *residual : none, residual ? 1 : 0, p.out, p.rows,
+      p.k, p.columns, p.experts);
+}
+
 bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int projections,
                                 bool swiglu, ErrorSlot *error) {
   if (!gather_eligible(p, projections)) return false;

@@ -14,6 +14,7 @@
 // weights, and multiplies them into its 16 row sums; the activations of a step are the same for
 // all lanes, so they arrive through scalar loads and cost no vector registers or LDS.
 #include "fast_kernels.hpp"
+#include "kernels.hpp"
 
 namespace fh {
 
@@ -253,6 +254,112 @@ void launch_gather_valu(hipStream_t stream, const GatherValuArgs &a, dim3 grid, 
     gather_valu_kernel<kBits, FH_BF16><<<grid, 256, 0, stream>>>(a, error);
 }
 
+// ---- routed products grouped by expert ------------------------------------------------------
+//
+// With several routes per expert the weights are formed once per tile of routes: a workgroup owns
+// 64 columns of half a packed tile (an expert and up to 16 of its routes), its four waves a
+// quarter of K each.  Route r of the tile reads the activation row `route / route_div` and
+// writes row `route` of a dense [routes, N] output (the [R,k,N] result, or f32 partial sums the
+// weighted form folds afterwards).
+struct GroupedValuArgs {
+  const void *x;
+  uint64_t x_row_stride;
+  const uint32_t *packed;
+  const uint16_t *scales, *biases;
+  uint32_t params_f16;
+  void *out;
+  uint32_t out_dtype;
+  const uint32_t *sorted_routes, *blocks, *n_blocks;
+  uint32_t route_div, inner, columns, group_shift;
+};
+
+template <int kBits, uint32_t kX>
+__global__ __launch_bounds__(256) void gather_grouped_valu_kernel(GroupedValuArgs a) {
+  constexpr int kValues = 128 / kBits, kAhead = 4, kRows = 16;
+  __shared__ float handed[3][kRows][64];
+  // blockIdx.y is (tile, half): 16 of the tile's routes per workgroup.  (A loop over the halves
+  // would put the first half's stores before the second half's loads, and the compiler then
+  // reads the activations through vector loads instead of scalar ones.)
+  const uint32_t tile = blockIdx.y >> 1, pass = (blockIdx.y & 1) * kRows;
+  if (tile >= a.n_blocks[0]) return;
+  const uint32_t expert = a.blocks[3 * tile], tile_first = a.blocks[3 * tile + 1], tile_count = a.blocks[3 * tile + 2];
+  if (pass >= tile_count) return;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t column = blockIdx.x * 64 + lane, column_in = min(column, a.columns - 1);
+  const uint32_t pieces_per_row = a.inner / kValues, groups_per_row = a.inner >> a.group_shift;
+  const uint32_t per_wave = (pieces_per_row + 3) / 4;
+  const uint32_t first = min(wave * per_wave, pieces_per_row), last = min(first + per_wave, pieces_per_row);
+  const uint64_t weight_row = (uint64_t)expert * a.columns + column_in;
+  const uint4 *w_row = (const uint4 *)a.packed + weight_row * pieces_per_row;
+  const uint16_t *s_row = a.scales + weight_row * groups_per_row;
+  const uint16_t *b_row = a.biases + weight_row * groups_per_row;
+  {
+    const uint32_t live = min((uint32_t)kRows, tile_count - pass);
+    uint32_t route[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r)
+      route[r] = a.sorted_routes[tile_first + pass + min((uint32_t)r, live - 1)];
+    float acc[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) acc[r] = 0.0f;
+    for (uint32_t step = first; step < last; step += kAhead) {
+      uint4 piece[kAhead];
+      uint16_t scale_bits[kAhead], bias_bits[kAhead];
+#pragma unroll
+      for (int i = 0; i < kAhead; ++i) {
+        const uint32_t at = min(step + i, last - 1);
+        piece[i] = w_row[at];
+        scale_bits[i] = s_row[(at * kValues) >> a.group_shift];
+        bias_bits[i] = b_row[(at * kValues) >> a.group_shift];
+      }
+#pragma unroll
+      for (int i = 0; i < kAhead; ++i) {
+        if (step + i >= last) continue;   // the same for every lane
+        const float scale = a.params_f16 ? f16_to_f32(scale_bits[i]) : bf16_to_f32(scale_bits[i]);
+        const float bias = a.params_f16 ? f16_to_f32(bias_bits[i]) : bf16_to_f32(bias_bits[i]);
+        float w[kValues];
+        form_weights<kBits>(piece[i], scale, bias, w);
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+          if ((uint32_t)r >= live) continue;
+          const uint64_t at = (uint64_t)(route[r] / a.route_div) * a.x_row_stride + (uint64_t)(step + i) * kValues;
+          acc[r] = row_product<kX, kValues>(a.x, at, w, acc[r]);
+        }
+      }
+    }
+    if (wave != 0) {
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) handed[wave - 1][r][lane] = acc[r];
+    }
+    __syncthreads();
+    if (wave == 0 && column < a.columns) {
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        if ((uint32_t)r >= live) continue;
+        const float value = ((acc[r] + handed[0][r][lane]) + handed[1][r][lane]) + handed[2][r][lane];
+        const uint64_t at = (uint64_t)route[r] * a.columns + column;
+        if (a.out_dtype == FH_F32)
+          ((float *)a.out)[at] = value;
+        else if (a.out_dtype == FH_F16)
+          ((uint16_t *)a.out)[at] = f32_to_f16(value);
+        else
+          ((uint16_t *)a.out)[at] = f32_to_bf16(value);
+      }
+    }
+  }
+}
+
+template <int kBits>
+void launch_grouped_valu(hipStream_t stream, const GroupedValuArgs &a, dim3 grid, uint32_t x_dtype) {
+  if (x_dtype == FH_F32)
+    gather_grouped_valu_kernel<kBits, FH_F32><<<grid, 256, 0, stream>>>(a);
+  else if (x_dtype == FH_F16)
+    gather_grouped_valu_kernel<kBits, FH_F16><<<grid, 256, 0, stream>>>(a);
+  else
+    gather_grouped_valu_kernel<kBits, FH_BF16><<<grid, 256, 0, stream>>>(a);
+}
+
 bool is_float_dtype(uint32_t dtype) { return dtype == FH_F32 || dtype == FH_F16 || dtype == FH_BF16; }
 
 char *element_address(const View &v) { return v.base + v.offset * dtype_size(v.dtype); }
@@ -356,6 +463,81 @@ bool try_valu_gather(fh_backend *backend, const View &x, const View &packed, con
     launch_gather_valu<4>(backend_stream(backend), a, grid, x.dtype, error);
   else
     launch_gather_valu<8>(backend_stream(backend), a, grid, x.dtype, error);
+  return true;
+}
+
+bool try_valu_gather_grouped(fh_backend *backend, const GatherProblem &p, int projection, const View &out,
+                             bool weighted, const View *residual, ErrorSlot *error) {
+  // worth the packing launch only when the weights formed for a tile serve several routes
+  if ((uint64_t)p.rows * p.k < 4ull * p.experts) return false;
+  const View &packed = p.packed[projection], &scales = p.scales[projection], &biases = p.biases[projection];
+  if (p.bits != 4 && p.bits != 8) return false;
+  if (p.group != 32 && p.group != 64 && p.group != 128) return false;
+  if (p.inner == 0 || p.inner % p.group != 0 || p.columns == 0) return false;
+  if (!is_float_dtype(p.x.dtype) || !is_float_dtype(out.dtype)) return false;
+  if ((scales.dtype != FH_BF16 && scales.dtype != FH_F16) || biases.dtype != scales.dtype) return false;
+  const uint64_t words_per_row = (uint64_t)p.inner * p.bits / 32, groups_per_row = p.inner / p.group;
+  if (packed.stride[2] != 1 || packed.stride[1] != words_per_row ||
+      packed.stride[0] != words_per_row * p.columns || packed.offset % 4 != 0)
+    return false;
+  for (const View *v : {&scales, &biases})
+    if (v->stride[2] != 1 || v->stride[1] != groups_per_row || v->stride[0] != groups_per_row * p.columns)
+      return false;
+  // activation rows: [R,K] rows, or [R,k,K] dense over its first two axes so that route r*k+s is row r*k+s
+  uint64_t x_row_stride;
+  if (weighted) {
+    if (p.x.stride[2] != 1 || p.x.stride[0] != (uint64_t)p.k * p.x.stride[1]) return false;
+    x_row_stride = p.x.stride[1];
+  } else {
+    if (p.x.stride[1] != 1) return false;
+    x_row_stride = p.x.stride[0];
+  }
+  if (p.x.dtype != FH_F32 && (x_row_stride % 2 != 0 || p.x.offset % 2 != 0)) return false;
+  const uint64_t routes = (uint64_t)p.rows * p.k;
+  if (!weighted && (out.stride[2] != 1 || out.stride[1] != p.columns || out.stride[0] != (uint64_t)p.k * p.columns))
+    return false;
+  if (!weighted && dtype_size(out.dtype) == 2 && ((routes * p.columns) % 2 != 0 || out.offset % 2 != 0))
+    return false;
+  PackedRoutes plan;
+  if (!pack_routes(backend, p, weighted ? routes * p.columns * sizeof(float) : 0, error, &plan)) return false;
+  if (plan.tile != 32 || 2 * plan.max_blocks > 65535) return false;   // two halves of 16 routes per tile
+  hipStream_t stream = backend_stream(backend);
+  GroupedValuArgs a{};
+  a.x = element_address(p.x);
+  a.x_row_stride = x_row_stride;
+  a.packed = (const uint32_t *)element_address(packed);
+  a.scales = (const uint16_t *)element_address(scales);
+  a.biases = (const uint16_t *)element_address(biases);
+  a.params_f16 = scales.dtype == FH_F16;
+  a.sorted_routes = plan.sorted_routes;
+  a.blocks = plan.blocks;
+  a.n_blocks = plan.n_blocks;
+  a.route_div = weighted ? 1 : p.k;
+  a.inner = p.inner;
+  a.columns = p.columns;
+  a.group_shift = p.group == 32 ? 5 : (p.group == 64 ? 6 : 7);
+  if (weighted) {
+    a.out = plan.rest;       // f32 partial sums per route; rows of bad routes are never read
+    a.out_dtype = FH_F32;
+  } else {
+    a.out = element_address(out);
+    a.out_dtype = out.dtype;
+    // rows of bad routes, which are never packed, read zero
+    launch_fill_u32(stream, (uint32_t *)a.out, routes * p.columns * dtype_size(out.dtype) / 4, 0);
+  }
+  const dim3 grid((p.columns + 63) / 64, 2 * plan.max_blocks);
+  {
+    KernelTimer timer(backend, FH_KC_MOE_KERNEL);
+    if (p.bits == 4)
+      launch_grouped_valu<4>(stream, a, grid, p.x.dtype);
+    else
+      launch_grouped_valu<8>(stream, a, grid, p.x.dtype);
+  }
+  if (weighted) {
+    GatherProblem folded = p;
+    folded.out = out;
+    launch_combine_routes(stream, (const float *)plan.rest, folded, residual);
+  }
   return true;
 }
 

@@ -353,10 +353,12 @@ def test_gather_projection_pair_and_weighted_sum(cpu, hip, rows, k, experts, n, 
     (DType.F16, 8, 32, DType.F16),
     (DType.BF16, 4, 128, DType.BF16),    # a group size the matrix-core kernels do not take
 ])
-@pytest.mark.parametrize("rows,k,experts,n,inner", [(8, 8, 128, 768, 2048), (37, 3, 5, 96, 256)])
+@pytest.mark.parametrize("rows,k,experts,n,inner", [(8, 8, 128, 768, 2048), (37, 3, 5, 96, 256),
+                                                   (70, 8, 16, 192, 512)])   # ≈35 routes per expert: two tiles
 def test_gather_in_other_dtypes_bits_and_groups(cpu, hip, rows, k, experts, n, inner, dtype, bits, group,
                                                 scale_dtype):
-    """The routed forms through the f32 vector-ALU kernels, with two bad routes: the valid routes
+    """The routed forms through the f32 vector-ALU kernels (route by route for the first case, grouped
+    by expert for the others), with two bad routes: the valid routes
     agree with the oracle, the lowest bad expert is reported, bad projection rows read zero and bad
     routes are left out of the weighted sum."""
     gate = Quantised(35, 1, (n, inner), bits=bits, group=group, experts=experts)

@@ -322,6 +322,44 @@ def lane_by_lane_step(workload, backend, steps=8, warmup=2):
             "unfused_ms_per_step": serial_wall_ms, "unfused_device_ms_per_step": serial_device_ms}
 
 
+class _FixedLanes:
+    """A decode session without churn, in the shape lane_by_lane_step drives."""
+
+    def __init__(self, session):
+        self.session = session
+
+    def churn_lanes(self):
+        pass
+
+
+def engine_dtype_step(backend, workload, seed, ctx_lo, ctx_hi, lanes=8):
+    """The qwen3-coder engine's own regime: decode batches of at most 8 lanes recorded lane by lane,
+    f32 activations, an f16 KV cache and an 8-bit router (engines/qwen3-coder/src/lib.rs:296-437),
+    on a second full-depth model of the timed config; beside it the same 8 lanes in the bench's
+    bf16 dtypes on the timed model.  The f32 products run on the vector ALUs, attention on the
+    matrix cores in f16."""
+    from dataclasses import replace
+    config = workload.model.config
+    rng = np.random.default_rng(seed + 5)
+    contexts = log_uniform(rng, ctx_lo, ctx_hi, lanes)
+    pt = config.page_tokens
+    pages = int(contexts.sum() * 1.1) // pt + 8 * lanes
+    table_pages = (ctx_hi + 4096 + pt) // pt
+    results = {}
+    for name, model in (("bf16", workload.model), ("f32_activations_f16_cache_q8_router", None)):
+        if model is None:
+            mixed = replace(config, activation_dtype=DType.F32, kv_dtype=DType.F16, router_bits=8)
+            model = Model(backend, mixed, seed=seed + 6, layers=workload.model.n_layers)
+        session = DecodeSession(model, contexts, seed=seed + 7, physical_pages=pages, table_pages=table_pages)
+        timing = lane_by_lane_step(_FixedLanes(session), backend, steps=6, warmup=2)
+        results[name] = {key: timing[key] for key in ("dispatches_per_step", "fused_runs_per_step", "ms_per_step",
+                                                      "device_ms_per_step", "decode_tokens_per_s",
+                                                      "unfused_device_ms_per_step")}
+    results["workload"] = ("%d decode lanes, contexts log-uniform %d-%d, full depth, recorded lane by lane"
+                           % (lanes, ctx_lo, ctx_hi))
+    return results
+
+
 def stream_read_rate(backend, rows=4096, width=1 << 20, repeats=3):
     """What a plain read-only stream sustains on this device: a row-wise argmax over 8 GiB of
     bf16 (16-byte loads, one workgroup per row).  The practical ceiling the HBM-bound kernels are
@@ -680,6 +718,8 @@ def main():
                                          "decode_attention_f16_cache": decode_attention_f16_cache(backend, config)}
         if config.moe:
             result["secondary_workloads"]["moe_block_c2"] = moe_block_c2(backend, workload.model)
+            result["secondary_workloads"]["engine_dtype_step"] = engine_dtype_step(
+                backend, workload, args.seed, ctx_lo, ctx_hi)
     step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction
     result["step_algorithmic_gb"] = step_bytes / 1e9
     result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS

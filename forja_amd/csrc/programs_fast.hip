@@ -2,7 +2,8 @@
 // (crates/forja-sdk/src/nn/blocks.rs:380-443): the row programs rms_norm_rows, residual_norm_rows
 // and qk_norm_rope_rows, and the element-wise silu_mul_elements and add_elements.  A program is recognised by its canonical expression (commutative operands
 // sorted, constants captured), never by name, so any instruction order the SDK emits matches;
-// everything else runs on the generic interpreter.  bf16 rows, innermost axis contiguous.
+// everything else runs on the generic interpreter.  bf16 rows (the row programs: f32 rows too),
+// innermost axis contiguous.
 #include "fast_kernels.hpp"
 
 #include <algorithm>
@@ -33,9 +34,34 @@ __device__ inline float block_sum(float v, float *scratch) {
   return total;
 }
 
+// Eight consecutive elements of bf16 (kWide false) or f32 rows.
+template <bool kWide>
+__device__ inline void load8(const void *base, uint64_t element, float (&v)[8]) {
+  if constexpr (kWide) {
+    const float4 a = *(const float4 *)((const float *)base + element);
+    const float4 b = *(const float4 *)((const float *)base + element + 4);
+    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+  } else {
+    const uint4 w = *(const uint4 *)((const uint16_t *)base + element);
+    v[0] = lo_f32(w.x), v[1] = hi_f32(w.x), v[2] = lo_f32(w.y), v[3] = hi_f32(w.y);
+    v[4] = lo_f32(w.z), v[5] = hi_f32(w.z), v[6] = lo_f32(w.w), v[7] = hi_f32(w.w);
+  }
+}
+
+template <bool kWide>
+__device__ inline void store8(void *base, uint64_t element, const float (&v)[8]) {
+  if constexpr (kWide) {
+    *(float4 *)((float *)base + element) = make_float4(v[0], v[1], v[2], v[3]);
+    *(float4 *)((float *)base + element + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  } else {
+    *(uint4 *)((uint16_t *)base + element) =
+        make_uint4(pack2(v[0], v[1]), pack2(v[2], v[3]), pack2(v[4], v[5]), pack2(v[6], v[7]));
+  }
+}
+
 struct RowArgs {
-  const uint16_t *x, *update, *weight;
-  uint16_t *out0, *out1;
+  const void *x, *update, *weight;   // bf16 or f32 rows, strides in elements
+  void *out0, *out1;
   uint64_t x_stride, update_stride, weight_stride, out0_stride, out1_stride;
   uint32_t width;
   float eps;
@@ -43,61 +69,45 @@ struct RowArgs {
 
 // out = x * rsqrt(mean(x^2) + eps) * w            (kResidual = false)
 // value = x + update; out0 = value; out1 = value * rsqrt(mean(value^2) + eps) * w
-template <bool kResidual>
+template <bool kResidual, bool kWide>
 __global__ __launch_bounds__(256) void norm_rows_kernel(RowArgs a) {
   __shared__ float scratch[4];
   const uint64_t row = blockIdx.x;
-  const uint16_t *x = a.x + row * a.x_stride;
-  const uint16_t *u = kResidual ? a.update + row * a.update_stride : nullptr;
-  const uint16_t *w = a.weight + row * a.weight_stride;
+  const uint64_t x_at = row * a.x_stride, u_at = row * a.update_stride, w_at = row * a.weight_stride;
   float acc = 0.0f;
   for (uint32_t c = threadIdx.x * 8; c < a.width; c += 256 * 8) {
-    uint4 v = *(const uint4 *)(x + c);
-    uint32_t words[4] = {v.x, v.y, v.z, v.w};
-    uint4 uv = make_uint4(0, 0, 0, 0);
-    if (kResidual) uv = *(const uint4 *)(u + c);
-    uint32_t uwords[4] = {uv.x, uv.y, uv.z, uv.w};
-    for (int i = 0; i < 4; ++i) {
-      float lo = lo_f32(words[i]), hi = hi_f32(words[i]);
-      if (kResidual) {
-        lo += lo_f32(uwords[i]);
-        hi += hi_f32(uwords[i]);
-      }
-      acc += lo * lo;
-      acc += hi * hi;
+    float v[8], u[8];
+    load8<kWide>(a.x, x_at + c, v);
+    if (kResidual) load8<kWide>(a.update, u_at + c, u);
+    for (int i = 0; i < 8; ++i) {
+      const float value = kResidual ? v[i] + u[i] : v[i];
+      acc += value * value;
     }
   }
   const float total = block_sum(acc, scratch);
   const float inverse = 1.0f / sqrtf(total / (float)a.width + a.eps);
-  uint16_t *out_norm = (kResidual ? a.out1 + row * a.out1_stride : a.out0 + row * a.out0_stride);
   for (uint32_t c = threadIdx.x * 8; c < a.width; c += 256 * 8) {
-    uint4 v = *(const uint4 *)(x + c);
-    uint4 wv = *(const uint4 *)(w + c);
-    uint32_t words[4] = {v.x, v.y, v.z, v.w}, wwords[4] = {wv.x, wv.y, wv.z, wv.w};
-    uint4 uv = make_uint4(0, 0, 0, 0);
-    if (kResidual) uv = *(const uint4 *)(u + c);
-    uint32_t uwords[4] = {uv.x, uv.y, uv.z, uv.w};
-    uint32_t value_words[4], norm_words[4];
-    for (int i = 0; i < 4; ++i) {
-      float lo = lo_f32(words[i]), hi = hi_f32(words[i]);
-      if (kResidual) {
-        lo += lo_f32(uwords[i]);
-        hi += hi_f32(uwords[i]);
-      }
-      value_words[i] = pack2(lo, hi);
-      norm_words[i] = pack2(lo * inverse * lo_f32(wwords[i]), hi * inverse * hi_f32(wwords[i]));
+    float v[8], u[8], w[8], normed[8];
+    load8<kWide>(a.x, x_at + c, v);
+    load8<kWide>(a.weight, w_at + c, w);
+    if (kResidual) load8<kWide>(a.update, u_at + c, u);
+    for (int i = 0; i < 8; ++i) {
+      if (kResidual) v[i] += u[i];
+      normed[i] = v[i] * inverse * w[i];
     }
-    if (kResidual)
-      *(uint4 *)(a.out0 + row * a.out0_stride + c) =
-          make_uint4(value_words[0], value_words[1], value_words[2], value_words[3]);
-    *(uint4 *)(out_norm + c) = make_uint4(norm_words[0], norm_words[1], norm_words[2], norm_words[3]);
+    if (kResidual) {
+      store8<kWide>(a.out0, row * a.out0_stride + c, v);
+      store8<kWide>(a.out1, row * a.out1_stride + c, normed);
+    } else {
+      store8<kWide>(a.out0, row * a.out0_stride + c, normed);
+    }
   }
 }
 
 struct QkArgs {
-  const uint16_t *lo, *hi, *w_lo, *w_hi;
+  const void *lo, *hi, *w_lo, *w_hi;   // bf16 or f32, strides in elements
   const float *positions;
-  uint16_t *out_lo, *out_hi;
+  void *out_lo, *out_hi;
   uint64_t lo_s[2], hi_s[2], wlo_s[2], whi_s[2], pos_s[3], olo_s[2], ohi_s[2];
   uint32_t rows, heads, width;
   float head_dim, eps, theta, exponent_scale;
@@ -108,6 +118,21 @@ struct QkArgs {
 // rotate the (lo, hi) pair by angle = position * theta^(i * exponent_scale).  The rotation is the
 // same for every head of a row when the positions do not vary along the head axis (the usual
 // broadcast view), and is then computed once per wave.
+template <bool kWide>
+__device__ inline float load1(const void *base, uint64_t element) {
+  if constexpr (kWide) return ((const float *)base)[element];
+  return __uint_as_float((uint32_t)((const uint16_t *)base)[element] << 16);
+}
+
+template <bool kWide>
+__device__ inline void store1(void *base, uint64_t element, float value) {
+  if constexpr (kWide)
+    ((float *)base)[element] = value;
+  else
+    ((uint16_t *)base)[element] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+}
+
+template <bool kWide>
 __global__ __launch_bounds__(256) void qk_norm_rope_kernel(QkArgs a) {
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t row = blockIdx.x;
@@ -123,15 +148,15 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(QkArgs a) {
   for (uint32_t head = blockIdx.y * 4 + wave; head < a.heads; head += 4 * gridDim.y) {
     float lo = 0.0f, hi = 0.0f;
     if (live) {
-      lo = __uint_as_float((uint32_t)a.lo[row * a.lo_s[0] + head * a.lo_s[1] + lane] << 16);
-      hi = __uint_as_float((uint32_t)a.hi[row * a.hi_s[0] + head * a.hi_s[1] + lane] << 16);
+      lo = load1<kWide>(a.lo, row * a.lo_s[0] + head * a.lo_s[1] + lane);
+      hi = load1<kWide>(a.hi, row * a.hi_s[0] + head * a.hi_s[1] + lane);
     }
     float square_sum = lo * lo + hi * hi;
     for (int offset = 32; offset > 0; offset >>= 1) square_sum += __shfl_xor(square_sum, offset, 64);
     if (!live) continue;
     const float inverse = 1.0f / sqrtf(square_sum / a.head_dim + a.eps);
-    const float w_lo = __uint_as_float((uint32_t)a.w_lo[row * a.wlo_s[0] + head * a.wlo_s[1] + lane] << 16);
-    const float w_hi = __uint_as_float((uint32_t)a.w_hi[row * a.whi_s[0] + head * a.whi_s[1] + lane] << 16);
+    const float w_lo = load1<kWide>(a.w_lo, row * a.wlo_s[0] + head * a.wlo_s[1] + lane);
+    const float w_hi = load1<kWide>(a.w_hi, row * a.whi_s[0] + head * a.whi_s[1] + lane);
     const float n_lo = lo * inverse * w_lo, n_hi = hi * inverse * w_hi;
     if (!shared_angle) {
       const float angle = a.positions[row * a.pos_s[0] + head * a.pos_s[1] + lane * a.pos_s[2]] * frequency;
@@ -139,8 +164,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(QkArgs a) {
       s = sinf(angle);
     }
     const float r_lo = n_lo * c - n_hi * s, r_hi = n_hi * c + n_lo * s;
-    a.out_lo[row * a.olo_s[0] + head * a.olo_s[1] + lane] = (uint16_t)(pack2(r_lo, 0.0f) & 0xffffu);
-    a.out_hi[row * a.ohi_s[0] + head * a.ohi_s[1] + lane] = (uint16_t)(pack2(r_hi, 0.0f) & 0xffffu);
+    store1<kWide>(a.out_lo, row * a.olo_s[0] + head * a.olo_s[1] + lane, r_lo);
+    store1<kWide>(a.out_hi, row * a.ohi_s[0] + head * a.ohi_s[1] + lane, r_hi);
   }
 }
 
@@ -221,6 +246,11 @@ const std::string kConst = "c([0-9a-f]{8})";
 
 bool bf16_rows(const View &v, uint32_t rank) {
   return v.dtype == FH_BF16 && v.rank == rank && v.stride[rank - 1] == 1;
+}
+
+// Rows of `dtype` (bf16 or f32) with a contiguous innermost axis.
+bool typed_rows(const View &v, uint32_t rank, uint32_t dtype) {
+  return v.dtype == dtype && v.rank == rank && v.stride[rank - 1] == 1;
 }
 
 }  // namespace
@@ -338,10 +368,14 @@ bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const Program
     const bool residual = cls.kind == kProgramResidualNorm;
     if (rank != 2 || p.n_inputs != (residual ? 3u : 2u)) return false;
     const uint32_t n_out = residual ? 2 : 1;
+    const uint32_t dtype = p.inputs[0].dtype;
+    if (dtype != FH_BF16 && dtype != FH_F32) return false;
+    const bool wide = dtype == FH_F32;
+    auto ptr = [](const View &v) { return (void *)(v.base + v.offset * dtype_size(v.dtype)); };
     for (uint32_t i = 0; i < p.n_inputs; ++i)
-      if (!bf16_rows(p.inputs[i], 2) || !aligned(p.inputs[i])) return false;
+      if (!typed_rows(p.inputs[i], 2, dtype) || !aligned(p.inputs[i])) return false;
     for (uint32_t i = 0; i < n_out; ++i)
-      if (!bf16_rows(p.outputs[i], 2) || !aligned(p.outputs[i])) return false;
+      if (!typed_rows(p.outputs[i], 2, dtype) || !aligned(p.outputs[i])) return false;
     const uint32_t width = p.shape[1];
     if (width % 8 != 0) return false;
     RowArgs a{};
@@ -363,19 +397,21 @@ bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const Program
     }
     a.width = width;
     a.eps = cls.c[0];
-    if (residual)
-      norm_rows_kernel<true><<<dim3(p.shape[0]), 256, 0, stream>>>(a);
-    else
-      norm_rows_kernel<false><<<dim3(p.shape[0]), 256, 0, stream>>>(a);
+    auto *kernel = residual ? (wide ? norm_rows_kernel<true, true> : norm_rows_kernel<true, false>)
+                            : (wide ? norm_rows_kernel<false, true> : norm_rows_kernel<false, false>);
+    kernel<<<dim3(p.shape[0]), 256, 0, stream>>>(a);
     return true;
   }
   if (cls.kind == kProgramQkNormRope) {
     if (rank != 3 || p.n_inputs != 5 || p.shape[2] > 64) return false;
+    const uint32_t dtype = p.inputs[0].dtype;
+    if (dtype != FH_BF16 && dtype != FH_F32) return false;
+    auto ptr = [](const View &v) { return (void *)(v.base + v.offset * dtype_size(v.dtype)); };
     for (uint32_t i = 0; i < 4; ++i)
-      if (!bf16_rows(p.inputs[i], 3)) return false;
+      if (!typed_rows(p.inputs[i], 3, dtype)) return false;
     if (p.inputs[4].dtype != FH_F32 || p.inputs[4].rank != 3) return false;
     for (uint32_t i = 0; i < 2; ++i)
-      if (!bf16_rows(p.outputs[i], 3)) return false;
+      if (!typed_rows(p.outputs[i], 3, dtype)) return false;
     QkArgs a{};
     auto set = [](uint64_t (&dst)[2], const View &v) {
       dst[0] = v.stride[0];
@@ -406,7 +442,10 @@ bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const Program
     const uint32_t head_blocks = (a.heads + 3) / 4;
     uint32_t per_row = 4096 / a.rows;
     per_row = per_row < 1 ? 1 : (per_row > head_blocks ? head_blocks : per_row);
-    qk_norm_rope_kernel<<<dim3(a.rows, per_row), 256, 0, stream>>>(a);
+    if (dtype == FH_F32)
+      qk_norm_rope_kernel<true><<<dim3(a.rows, per_row), 256, 0, stream>>>(a);
+    else
+      qk_norm_rope_kernel<false><<<dim3(a.rows, per_row), 256, 0, stream>>>(a);
     return true;
   }
   return false;

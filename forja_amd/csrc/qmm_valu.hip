@@ -104,20 +104,33 @@ __global__ __launch_bounds__(64 * kValuWaves) void qmm_valu_kernel(ValuArgs a) {
   for (int r = 0; r < kValuRows; ++r) acc[r] = 0.0f;
   const uint32_t first = wave * a.steps_per_wave;
   const uint32_t last = min(first + a.steps_per_wave, pieces_per_row);
-  for (uint32_t step = first; step < last; ++step) {
-    const uint32_t k0 = step * kValues;
-    const uint4 piece = w_row[step];
-    const uint32_t group = k0 >> a.group_shift;
-    const float scale = a.params_f16 ? f16_to_f32(s_row[group]) : bf16_to_f32(s_row[group]);
-    const float bias = a.params_f16 ? f16_to_f32(b_row[group]) : bf16_to_f32(b_row[group]);
-    float w[kValues];
-    form_weights<kBits>(piece, scale, bias, w);
+  // 64 bytes of the weight row are requested at a time: with few rows a wave is a chain of
+  // dependent loads, and this makes it four times shorter
+  constexpr int kAhead = 4;
+  for (uint32_t step = first; step < last; step += kAhead) {
+    uint4 piece[kAhead];
+    uint16_t scale_bits[kAhead], bias_bits[kAhead];
 #pragma unroll
-    for (int r = 0; r < kValuRows; ++r) {
-      if ((uint32_t)r >= live_rows) continue;   // the same for every lane
-      const uint64_t at = (uint64_t)(row0 + r) * a.x_row_stride + k0;
-      const float sum = row_product<kX, kValues>(a.x, at, w, acc[r]);
-      acc[r] = sum;
+    for (int i = 0; i < kAhead; ++i) {
+      const uint32_t at = min(step + i, last - 1);
+      piece[i] = w_row[at];
+      scale_bits[i] = s_row[(at * kValues) >> a.group_shift];
+      bias_bits[i] = b_row[(at * kValues) >> a.group_shift];
+    }
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      if (step + i >= last) continue;   // the same for every lane
+      const uint32_t k0 = (step + i) * kValues;
+      const float scale = a.params_f16 ? f16_to_f32(scale_bits[i]) : bf16_to_f32(scale_bits[i]);
+      const float bias = a.params_f16 ? f16_to_f32(bias_bits[i]) : bf16_to_f32(bias_bits[i]);
+      float w[kValues];
+      form_weights<kBits>(piece[i], scale, bias, w);
+#pragma unroll
+      for (int r = 0; r < kValuRows; ++r) {
+        if ((uint32_t)r >= live_rows) continue;   // the same for every lane
+        const uint64_t at = (uint64_t)(row0 + r) * a.x_row_stride + k0;
+        acc[r] = row_product<kX, kValues>(a.x, at, w, acc[r]);
+      }
     }
   }
   if (wave != 0) {

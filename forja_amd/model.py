@@ -39,6 +39,11 @@ class ModelConfig:
     rms_eps: float = 1e-6
     rope_theta: float = 1e6
     page_tokens: int = 16
+    # The qwen38 engine records bf16 activations over a bf16 cache, the qwen3-coder engine f32
+    # activations over an f16 cache with an 8-bit router (engines/qwen3-coder/src/lib.rs:296-437).
+    activation_dtype: DType = DType.BF16
+    kv_dtype: DType = DType.BF16
+    router_bits: int = 4
 
     @property
     def moe(self) -> bool:
@@ -46,7 +51,7 @@ class ModelConfig:
 
     @property
     def kv_bytes_per_token(self) -> int:
-        return self.layers * 2 * self.kv_heads * self.head_dim * 2
+        return self.layers * 2 * self.kv_heads * self.head_dim * self.kv_dtype.byte_size
 
 
 QWEN3_0_6B = ModelConfig("qwen3-0.6b-shaped", hidden=1024, layers=28, q_heads=16, kv_heads=8,
@@ -61,10 +66,10 @@ DENSE_27B = ModelConfig("dense-27b-shaped", hidden=5120, layers=64, q_heads=40, 
 class QuantLinear:
     """packed u32 [N, K/8] (or [E, N, K/8]), bf16 scales/biases [.., N, K/64]."""
 
-    def __init__(self, backend, n: int, k: int, experts: int = 0):
+    def __init__(self, backend, n: int, k: int, experts: int = 0, bits: int = BITS):
         lead = (experts,) if experts else ()
-        self.n, self.k, self.experts = n, k, experts
-        self.packed = backend.alloc(DType.U32, lead + (n, k * BITS // 32))
+        self.n, self.k, self.experts, self.bits = n, k, experts, bits
+        self.packed = backend.alloc(DType.U32, lead + (n, k * bits // 32))
         self.scales = backend.alloc(DType.BF16, lead + (n, k // GROUP))
         self.biases = backend.alloc(DType.BF16, lead + (n, k // GROUP))
 
@@ -80,7 +85,7 @@ class QuantLinear:
     @property
     def weight_bytes(self) -> int:
         count = (self.experts or 1) * self.n
-        return count * (self.k // 2 + 2 * (self.k // GROUP) * 2)
+        return count * (self.k * self.bits // 8 + 2 * (self.k // GROUP) * 2)
 
 
 @dataclass
@@ -121,7 +126,7 @@ class Model:
                 o_proj=self._linear(fill, c.hidden, c.q_heads * c.head_dim),
                 post_norm=self._norm(fill, (c.hidden,)))
             if c.moe:
-                lw.router = self._linear(fill, c.experts, c.hidden)
+                lw.router = self._linear(fill, c.experts, c.hidden, bits=c.router_bits)
                 lw.gate = self._linear(fill, c.expert_intermediate, c.hidden, c.experts)
                 lw.up = self._linear(fill, c.expert_intermediate, c.hidden, c.experts)
                 lw.down = self._linear(fill, c.hidden, c.expert_intermediate, c.experts)
@@ -146,15 +151,20 @@ class Model:
         self._stream += count
         return first
 
-    def _linear(self, fill, n, k, experts=0) -> QuantLinear:
-        linear = QuantLinear(self.backend, n, k, experts)
+    def _linear(self, fill, n, k, experts=0, bits=BITS) -> QuantLinear:
+        linear = QuantLinear(self.backend, n, k, experts, bits)
         linear.fill(fill, self.seed, self._next_stream(3))
         return linear
 
     def _norm(self, fill, shape) -> Tensor:
         tensor = self.backend.alloc(DType.BF16, shape)
         fill.dispatch(Op.fill_seeded(1, self.seed, self._next_stream(1), lo=0.9, hi=1.1), [], tensor)
-        return tensor
+        if self.config.activation_dtype == DType.BF16:
+            return tensor
+        # the seeded uniform fill is defined for bf16: widen its values into the activations' dtype
+        wide = self.backend.alloc(self.config.activation_dtype, shape)
+        fill.dispatch(Op.copy(), [tensor], wide)
+        return wide
 
     def weight_bytes_per_step(self, rows: int) -> dict:
         """Algorithmic weight bytes one decode step reads (packed + scales + biases), by class."""
@@ -182,8 +192,8 @@ class KvCache:
         self.backend, self.config = backend, config
         self.lanes, self.physical_pages, self.table_pages = lanes, physical_pages, table_pages
         shape = (physical_pages, c.page_tokens, c.kv_heads, c.head_dim)
-        self.keys = [backend.alloc(DType.BF16, shape) for _ in range(layers)]
-        self.values = [backend.alloc(DType.BF16, shape) for _ in range(layers)]
+        self.keys = [backend.alloc(c.kv_dtype, shape) for _ in range(layers)]
+        self.values = [backend.alloc(c.kv_dtype, shape) for _ in range(layers)]
         if fill_pools:
             fill = CommandList()
             for layer in range(layers):
@@ -233,7 +243,7 @@ class StepBuffers:
     def __init__(self, backend, config: ModelConfig, tokens: int, lanes: int, head: bool = True):
         c = config
         qkv_width = (c.q_heads + 2 * c.kv_heads) * c.head_dim
-        a = lambda *shape: backend.alloc(DType.BF16, shape)
+        a = lambda *shape: backend.alloc(c.activation_dtype, shape)
         self.tokens, self.lanes = tokens, lanes
         self.ids = backend.alloc(DType.U32, (tokens,))
         self.positions = backend.alloc(DType.F32, (tokens,))     # rope positions, one per row
@@ -334,7 +344,8 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
         hidden, other = other, hidden
         normalized, normalized_next = normalized_next, normalized
         if c.moe:
-            commands.dispatch(q4, [normalized, *layer.router.triple], b.router_logits)
+            commands.dispatch(Op.quant_matmul(c.router_bits, GROUP), [normalized, *layer.router.triple],
+                              b.router_logits)
             commands.dispatch_many(Op.top_k(c.top_k, True), [b.router_logits],
                                    [b.route_weights, b.route_indices])
             if route_trace is not None:
@@ -411,7 +422,7 @@ class DecodeSession:
         if self.lane_encoded is not None:
             return
         c, b, backend = self.model.config, self.buffers, self.model.backend
-        b.lane_rows = backend.alloc(DType.BF16, (len(self.contexts), c.q_heads, c.head_dim))
+        b.lane_rows = backend.alloc(c.activation_dtype, (len(self.contexts), c.q_heads, c.head_dim))
         self.lane_sites = []
         self.lane_commands = CommandList()
         record_step(self.model, self.cache, b, self.lane_commands, feed_back=True,

@@ -61,6 +61,24 @@ def test_greedy_tokens_identical_over_32_steps_moe(cpu, hip):
     assert_close(b, a, DType.BF16, abs_=3e-2)
 
 
+def test_greedy_tokens_identical_over_32_steps_with_the_qwen3_coder_dtypes(cpu, hip):
+    """f32 activations, an f16 KV cache and an 8-bit router, recorded lane by lane as that engine
+    records its decode batches (engines/qwen3-coder/src/lib.rs:296-437): the f32 vector-ALU
+    products, the f16 attention kernels and the run fusion together."""
+    from dataclasses import replace
+    config = replace(TINY_MOE, activation_dtype=DType.F32, kv_dtype=DType.F16, router_bits=8)
+    ref, dev = sessions(cpu, hip, config, 2, [5, 40, 300, 77, 16, 15], seed=14)
+    dev.record_lane_by_lane()
+    before = hip.fusion_stats()[0]
+    ref_tokens = np.stack([ref.step() for _ in range(32)])
+    dev_tokens = np.stack([dev.step(lane_by_lane=True) for _ in range(32)])
+    assert hip.fusion_stats()[0] - before == 2 * 32          # every layer's lanes ran as one launch
+    assert ref_tokens.tolist() == dev_tokens.tolist()
+    a = to_f32(cpu.read(ref.buffers.logits), DType.F32)
+    b = to_f32(hip.read(dev.buffers.logits), DType.F32)
+    assert_close(b, a, DType.F16)
+
+
 SMALL_DENSE = ModelConfig("small-dense", hidden=512, layers=2, q_heads=8, kv_heads=4, head_dim=128,
                           vocab=2000, intermediate=1024)
 

@@ -718,8 +718,9 @@ def main():
                                          "decode_attention_f16_cache": decode_attention_f16_cache(backend, config)}
         if config.moe:
             result["secondary_workloads"]["moe_block_c2"] = moe_block_c2(backend, workload.model)
-            result["secondary_workloads"]["engine_dtype_step"] = engine_dtype_step(
-                backend, workload, args.seed, ctx_lo, ctx_hi)
+            if not args.no_lane_by_lane:
+                result["secondary_workloads"]["engine_dtype_step"] = engine_dtype_step(
+                    backend, workload, args.seed, ctx_lo, ctx_hi)
     step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction
     result["step_algorithmic_gb"] = step_bytes / 1e9
     result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS

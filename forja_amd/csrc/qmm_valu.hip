@@ -157,6 +157,66 @@ __global__ __launch_bounds__(64 * kValuWaves) void qmm_valu_kernel(ValuArgs a) {
   }
 }
 
+// Few rows and not many columns (a decode batch of at most 8 rows against a layer's projections):
+// 64 columns per workgroup would leave most of the device idle, so here a wave owns one column
+// and its lanes split K in 16-byte pieces, every lane reading its own slice of each activation
+// row; the lanes' sums meet in a butterfly.
+constexpr int kFewRows = 8;
+
+template <int kBits, uint32_t kX>
+__global__ __launch_bounds__(256) void qmm_valu_few_rows_kernel(ValuArgs a) {
+  constexpr int kValues = 128 / kBits;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t column = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (column >= a.columns) return;
+  const uint32_t pieces_per_row = a.inner / kValues, groups_per_row = a.inner >> a.group_shift;
+  const uint4 *w_row = (const uint4 *)a.packed + (uint64_t)column * pieces_per_row;
+  const uint16_t *s_row = a.scales + (uint64_t)column * groups_per_row;
+  const uint16_t *b_row = a.biases + (uint64_t)column * groups_per_row;
+  float acc[kFewRows];
+#pragma unroll
+  for (int r = 0; r < kFewRows; ++r) acc[r] = 0.0f;
+  for (uint32_t piece = lane; piece < pieces_per_row; piece += 64) {
+    const uint32_t k0 = piece * kValues, group = k0 >> a.group_shift;
+    const float scale = a.params_f16 ? f16_to_f32(s_row[group]) : bf16_to_f32(s_row[group]);
+    const float bias = a.params_f16 ? f16_to_f32(b_row[group]) : bf16_to_f32(b_row[group]);
+    float w[kValues];
+    form_weights<kBits>(w_row[piece], scale, bias, w);
+#pragma unroll
+    for (int r = 0; r < kFewRows; ++r) {
+      if ((uint32_t)r >= a.rows) continue;
+      acc[r] = row_product<kX, kValues>(a.x, (uint64_t)r * a.x_row_stride + k0, w, acc[r]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < kFewRows; ++r) {
+    if ((uint32_t)r >= a.rows) continue;
+    float value = acc[r];
+    for (int offset = 32; offset > 0; offset >>= 1) value += __shfl_xor(value, offset, 64);
+    if (lane != 0) continue;
+    if (a.residual)
+      value += typed_load(a.residual, a.residual_dtype, (uint64_t)r * a.residual_row_stride + column);
+    const uint64_t at = (uint64_t)r * a.out_row_stride + column;
+    if (a.out_dtype == FH_F32)
+      ((float *)a.out)[at] = value;
+    else if (a.out_dtype == FH_F16)
+      ((uint16_t *)a.out)[at] = f32_to_f16(value);
+    else
+      ((uint16_t *)a.out)[at] = f32_to_bf16(value);
+  }
+}
+
+template <int kBits>
+void launch_valu_few_rows(hipStream_t stream, const ValuArgs &a, uint32_t x_dtype) {
+  const dim3 grid((a.columns + 3) / 4);
+  if (x_dtype == FH_F32)
+    qmm_valu_few_rows_kernel<kBits, FH_F32><<<grid, 256, 0, stream>>>(a);
+  else if (x_dtype == FH_F16)
+    qmm_valu_few_rows_kernel<kBits, FH_F16><<<grid, 256, 0, stream>>>(a);
+  else
+    qmm_valu_few_rows_kernel<kBits, FH_BF16><<<grid, 256, 0, stream>>>(a);
+}
+
 template <int kBits>
 void launch_valu(hipStream_t stream, const ValuArgs &a, dim3 grid, uint32_t threads, uint32_t x_dtype) {
   if (x_dtype == FH_F32)
@@ -421,6 +481,15 @@ bool try_valu_quant_matmul(fh_backend *backend, const QmmProblem &p) {
   if (row_blocks > 65535) return false;
   const dim3 grid((p.columns + 63) / 64, (unsigned)row_blocks);
   KernelTimer timer(backend, FH_KC_QMM_KERNEL);
+  // (each wave of the few-rows kernel reads the activation rows for itself, through L1: beyond a
+  // couple of thousand columns that traffic costs more than the idle compute units did)
+  if (p.rows <= (uint32_t)kFewRows && p.columns <= 2048) {
+    if (p.bits == 4)
+      launch_valu_few_rows<4>(backend_stream(backend), a, p.x.dtype);
+    else
+      launch_valu_few_rows<8>(backend_stream(backend), a, p.x.dtype);
+    return true;
+  }
   if (p.bits == 4)
     launch_valu<4>(backend_stream(backend), a, grid, 64 * waves, p.x.dtype);
   else

@@ -49,7 +49,9 @@ __device__ inline bool entry_ok(const uint32_t *table, const uint32_t *generatio
 
 // Stores every lane's new K and V rows (thread per (token, element)).  A row whose page entry is
 // not authentic is skipped and reported; it is never written.
-__global__ void ragged_append_kernel(RaggedAttention p, ErrorSlot *error) {
+__global__ void ragged_append_kernel(RaggedAttention p, ErrorSlot *error,
+                                     const uint32_t *malformed) {
+  if (malformed[0]) return;   // cu_seqlens refused: nothing is stored
   uint32_t key_row = p.kv_heads * p.width, value_row = p.kv_heads * p.value_width;
   uint32_t per_token = key_row + value_row;
   uint64_t flat = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -94,7 +96,9 @@ __global__ void ragged_append_kernel(RaggedAttention p, ErrorSlot *error) {
 
 // The same append for rows and pools of one 2-byte dtype whose head rows are 16-byte aligned: a
 // thread moves eight elements.
-__global__ __launch_bounds__(256) void ragged_append_pieces_kernel(RaggedAttention p, ErrorSlot *error) {
+__global__ __launch_bounds__(256) void ragged_append_pieces_kernel(RaggedAttention p, ErrorSlot *error,
+                                                                   const uint32_t *malformed) {
+  if (malformed[0]) return;   // cu_seqlens refused: nothing is stored
   const uint32_t key_pieces = p.kv_heads * p.width / 8, value_pieces = p.kv_heads * p.value_width / 8;
   const uint32_t per_token = key_pieces + value_pieces;
   const uint64_t flat = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -148,14 +152,15 @@ bool append_by_pieces(const RaggedAttention &p) {
 
 // Any dtype / width: one wave per (token, query head); per-lane online softmax merged at the end.
 template <int kMaxDv>
-__global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *error) {
+__global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *error,
+                                                const uint32_t *malformed) {
   __shared__ float q_row[512];
   __shared__ int bad;
   uint32_t token = blockIdx.x / p.query_heads, head = blockIdx.x % p.query_heads;
   uint32_t lane_id = threadIdx.x;
   const uint32_t *cu = (const uint32_t *)p.cu_seqlens.base + p.cu_seqlens.offset;
   uint64_t out_base = p.out.offset + token * p.out.stride[0] + head * p.out.stride[1];
-  bool covered = token >= cu[0] && token < cu[p.lanes];
+  bool covered = !malformed[0] && token >= cu[0] && token < cu[p.lanes];
   uint32_t lane = covered ? find_lane(cu, p.lanes, token) : 0;
   bool active = covered && !(p.activity.base &&
                              ((const uint32_t *)p.activity.base)[p.activity.offset + lane] == 0);
@@ -283,7 +288,8 @@ struct FastRagged {
   uint32_t *bad;       // [T]
   TokenPlan *plans;    // [T]
   uint2 *items;        // [T * S] (group leader token, split) of every live split, compacted
-  uint32_t *item_count;   // [0] work items, [1] tokens the merge kernel has work for
+  uint32_t *item_count;   // [0] work items, [1] tokens the merge kernel has work for,
+                          // [2] non-zero: cu_seqlens was refused
   uint32_t *merge_tokens; // [T] those tokens (several splits, or a zero row to write)
   uint64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h;
   uint32_t tokens, lanes, query_heads, kv_heads, group, page_tokens, physical_pages, table_pages,
@@ -359,16 +365,67 @@ __device__ inline TokenPlan plan_token(const FastRagged &p, uint32_t token, uint
 // hardware, which starts workgroups in list order, ends the launch on its shortest items.
 constexpr uint32_t kSizeClasses = 65;   // split length / 32, clamped
 
+// Lowest lane whose token range breaks the cu_seqlens contract (non-decreasing, ending inside
+// the packed batch), over the lanes this thread looks at; 0xffffffff when they all keep it.
+__device__ inline uint32_t first_malformed_lane(const uint32_t *cu, uint32_t lanes, uint32_t tokens,
+                                                uint32_t first, uint32_t step) {
+  for (uint32_t lane = first; lane < lanes; lane += step)
+    if (cu[lane + 1] < cu[lane] || cu[lane + 1] > tokens) return lane;
+  return 0xffffffffu;
+}
+
+// For the kernels that do not go through a work plan: raises `flag[0]` and reports the lane when
+// cu_seqlens is refused.
+__global__ __launch_bounds__(256) void ragged_validate_kernel(const uint32_t *cu, uint32_t lanes,
+                                                              uint32_t tokens, uint32_t *flag,
+                                                              ErrorSlot *error) {
+  __shared__ uint32_t lowest;
+  if (threadIdx.x == 0) lowest = 0xffffffffu;
+  __syncthreads();
+  const uint32_t mine = first_malformed_lane(cu, lanes, tokens, threadIdx.x, 256);
+  if (mine != 0xffffffffu) atomicMin(&lowest, mine);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    flag[0] = lowest != 0xffffffffu;
+    if (lowest != 0xffffffffu) report_error(error, lowest);
+  }
+}
+
 __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlot *error) {
   __shared__ uint32_t class_items[kSizeClasses];   // items per class, then the class's cursor
   __shared__ unsigned long long total_attended;
-  __shared__ uint32_t merge_count;
+  __shared__ uint32_t merge_count, malformed_lane;
   for (uint32_t c = threadIdx.x; c < kSizeClasses; c += 256) class_items[c] = 0;
   if (threadIdx.x == 0) {
     total_attended = 0;
     merge_count = 0;
+    malformed_lane = 0xffffffffu;
   }
   __syncthreads();
+  // cu_seqlens is device data nobody has looked at: token ranges that run backwards or past the
+  // packed batch would send the grouped kernels beyond q, out and the plan itself.  A refused
+  // cu_seqlens fails the whole dispatch: every row reads zero, nothing is appended, and the
+  // lowest offending lane is reported.
+  if (p.cu != nullptr) {
+    const uint32_t mine = first_malformed_lane(p.cu, p.lanes, p.tokens, threadIdx.x, 256);
+    if (mine != 0xffffffffu) atomicMin(&malformed_lane, mine);
+    __syncthreads();
+    if (malformed_lane != 0xffffffffu) {
+      for (uint32_t token = threadIdx.x; token < p.tokens; token += 256) {
+        p.bad[token] = 1;
+        p.plans[token] = TokenPlan{0, 0, 0, 0, token, 1};
+        p.merge_tokens[token] = token;
+      }
+      if (threadIdx.x == 0) {
+        report_error(error, malformed_lane);
+        p.item_count[0] = 0;
+        p.item_count[1] = p.tokens;
+        p.item_count[2] = 1;
+      }
+      return;
+    }
+  }
+  if (threadIdx.x == 0) p.item_count[2] = 0;
   // Split length: long enough that a wave's fixed start-up cost (plan, table, query) is small
   // against its stream, short enough that the batch still yields ~kTargetItems work items.
   uint32_t split_tokens = p.split_tokens;
@@ -1278,25 +1335,35 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     launch_fast(backend, stream, f, error);
     return true;
   }
+  // Whether cu_seqlens was refused: the work plan records it; without a plan a kernel of its own
+  // finds out.
+  const uint32_t *malformed = fast ? f.item_count + 2 : nullptr;
+  if (!fast) {
+    uint32_t *flag = (uint32_t *)backend_workspace(backend, 256);
+    if (!flag) return false;
+    ragged_validate_kernel<<<dim3(1), 256, 0, stream>>>(
+        (const uint32_t *)p.cu_seqlens.base + p.cu_seqlens.offset, p.lanes, p.tokens, flag, error);
+    malformed = flag;
+  }
   uint64_t append_work =
       (uint64_t)p.tokens * (p.kv_heads * p.width + p.kv_heads * p.value_width);
   if (append_by_pieces(p))
     ragged_append_pieces_kernel<<<dim3((unsigned)((append_work / 8 + 255) / 256)), 256, 0, stream>>>(
-        p, append_error);
+        p, append_error, malformed);
   else
     ragged_append_kernel<<<dim3((unsigned)((append_work + 255) / 256)), 256, 0, stream>>>(
-        p, append_error);
+        p, append_error, malformed);
   if (fast) {
     launch_fast(backend, stream, f, error);
     return true;
   }
   uint32_t blocks = p.tokens * p.query_heads;
   if (p.value_width <= 64)
-    ragged_attention_generic_kernel<64><<<dim3(blocks), 64, 0, stream>>>(p, error);
+    ragged_attention_generic_kernel<64><<<dim3(blocks), 64, 0, stream>>>(p, error, malformed);
   else if (p.value_width <= 128)
-    ragged_attention_generic_kernel<128><<<dim3(blocks), 64, 0, stream>>>(p, error);
+    ragged_attention_generic_kernel<128><<<dim3(blocks), 64, 0, stream>>>(p, error, malformed);
   else
-    ragged_attention_generic_kernel<256><<<dim3(blocks), 64, 0, stream>>>(p, error);
+    ragged_attention_generic_kernel<256><<<dim3(blocks), 64, 0, stream>>>(p, error, malformed);
   return true;
 }
 

@@ -640,6 +640,13 @@ class CpuBackend:
         out, key_pool, value_pool = d.outputs
         cu_values, start_values = self._u32(cu), self._u32(starts)
         lanes = tables.shape[0]
+        # cu_seqlens is data: token ranges must be non-decreasing and end inside the packed batch,
+        # else the dispatch is refused whole (zero rows, pools untouched, lowest offending lane).
+        ends = cu_values.astype(np.int64)
+        malformed = (ends[1:] < ends[:-1]) | (ends[1:] > q.shape[0])
+        if malformed.any():
+            self._write_output(out, np.zeros(out.layout.element_count, dtype=np.float32))
+            raise BackendError(Status.DEVICE_ERROR_FLAG, index=int(np.argmax(malformed)))
         if d.op.k == 1:     # the recorder promised at most one query row per lane
             counts = np.diff(cu_values.astype(np.int64))
             if (counts > 1).any():

@@ -921,6 +921,43 @@ def test_the_one_row_promise_keeps_inactive_lanes_and_stale_pages_unwritten(cpu,
     assert not to_f32(hip.read(tensors[0]), DType.BF16).reshape(3, -1)[0].any()
 
 
+@pytest.mark.parametrize("hq,hkv,pt,counts,cu", [
+    (8, 4, 16, [1, 1, 1, 1], [0, 100, 4, 4, 4]),      # decode batch: lane 0 claims 100 rows of 4
+    (8, 4, 16, [20, 30, 14], [0, 20, 10, 64]),        # prefill groups: lane 1 runs backwards
+    (8, 4, 16, [20, 30, 14], [0, 20, 50, 4000]),      # the last lane runs past the packed batch
+    (6, 2, 8, [3, 2, 1], [0, 3, 70, 6])])             # a page size only the generic kernels take
+def test_ragged_attention_refuses_malformed_cu_seqlens(cpu, hip, hq, hkv, pt, counts, cu):
+    """cu_seqlens is read on the device: ranges that run backwards or beyond the packed batch fail
+    the dispatch (lowest offending lane reported), every output row reads zero, and neither the
+    pools nor the allocations around q and out are touched.  Every kernel exits normally."""
+    contexts = [40 + 3 * lane for lane in range(len(counts))]
+    bad_lane = next(l for l in range(len(counts)) if cu[l + 1] < cu[l] or cu[l + 1] > sum(counts))
+    for promise in (False, True) if max(counts) == 1 else (False,):
+        for backend in (cpu, hip):
+            guard_before = upload(backend, normal_bf16(72, 1, (4096,)), DType.BF16)
+            t, inputs = ragged_case(backend, contexts, counts, hq, hkv, pt, seed=71)
+            guard_after = upload(backend, normal_bf16(72, 2, (4096,)), DType.BF16)
+            inputs[5] = upload(backend, np.array(cu), DType.U32)
+            backend.write(t["out"], np.full(sum(counts) * hq * 128, 0x3f80, np.uint16).tobytes())
+            pools = backend.read(t["keys"]), backend.read(t["values"])
+            guards = backend.read(guard_before), backend.read(guard_after)
+            commands = CommandList()
+            commands.dispatch_many(Op.paged_attention_ragged(0.09, pt, one_row_per_lane=promise), inputs,
+                                   [t["out"], t["keys"], t["values"]])
+            with pytest.raises(BackendError) as info:
+                run(backend, commands)
+            assert info.value.status == Status.DEVICE_ERROR_FLAG and info.value.index == bad_lane
+            assert not np.frombuffer(backend.read(t["out"]), np.uint16).any()
+            assert (backend.read(t["keys"]), backend.read(t["values"])) == pools
+            assert (backend.read(guard_before), backend.read(guard_after)) == guards
+            # and the backend keeps working: the same batch with its real cu_seqlens succeeds
+            inputs[5] = t["cu"]
+            commands = CommandList()
+            commands.dispatch_many(Op.paged_attention_ragged(0.09, pt), inputs, [t["out"], t["keys"], t["values"]])
+            run(backend, commands)
+            assert np.frombuffer(backend.read(t["out"]), np.uint16).any()
+
+
 def test_ragged_attention_skips_inactive_lanes(cpu, hip):
     def build(backend):
         t, inputs = ragged_case(backend, [33, 70, 5], [1, 1, 1], 8, 4, 16, seed=62, activity=[1, 0, 1])

@@ -33,6 +33,8 @@ struct Program {
   std::vector<fh_inst> insts;
   std::vector<uint32_t> pairs;  // (slot, value)
   ProgramClass fast{};          // recognised fused form, if any
+  bool add_epilogue = false;    // `accumulator + extra`, recognised when the program is prepared
+  bool swiglu_epilogue = false; // `silu(accumulator 0) * accumulator 1`
   uint32_t n_inputs = 0;
   uint32_t n_outputs = 0;
   uint32_t n_reduce = 0;
@@ -73,6 +75,61 @@ bool shape_is(const fh_tensor &t, std::initializer_list<uint32_t> shape) {
 }  // namespace fh
 
 using namespace fh;
+
+// ---------------------------------------------------------------- fixed scratch (fh_submit_static)
+//
+// Device memory for callers that cannot allocate.  Every GPU the library runs on holds its own
+// copy of this array, at its own address, until the process ends; host code never uses the
+// array's name as an address (it is a host-side stand-in) but the pointer hipGetSymbolAddress
+// gives for the current device, looked up once per device in fh_create.  The array is cut into
+// fixed regions, one per kind of scratch the kernels of fh_submit use.
+constexpr uint64_t kStaticErrorBytes = 64ull << 10;       // 8192 dispatch error records
+constexpr uint64_t kStaticProgramBytes = 960ull << 10;    // typed instructions of a call's programs
+constexpr uint64_t kStaticRoutePlanBytes = 1ull << 20;
+constexpr uint64_t kStaticAttentionPlanBytes = 2ull << 20;
+constexpr uint64_t kStaticAccumulatorBytes = 8ull << 20;
+constexpr uint64_t kStaticWorkspaceBytes = 36ull << 20;
+constexpr uint64_t kStaticScratchBytes = kStaticErrorBytes + kStaticProgramBytes +
+                                         kStaticRoutePlanBytes + kStaticAttentionPlanBytes +
+                                         kStaticAccumulatorBytes + kStaticWorkspaceBytes;
+static_assert(kStaticScratchBytes == FH_STATIC_SCRATCH_BYTES, "the header states the size");
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+char *g_scratch_of_device[kMaxDevices] = {};   // the array's address on each device seen so far
+
+// The array's device address on `device`, which must be the current device.
+char *static_scratch_address(int device) {
+  if (device < 0 || device >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_of_device[device]) {
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return nullptr;
+    g_scratch_of_device[device] = (char *)ptr;
+  }
+  return g_scratch_of_device[device];
+}
+
+// Up to 64 typed instructions by value (1 KB of kernel arguments) into device memory.
+struct InstructionChunk {
+  DInst v[64];
+};
+__global__ void upload_instructions_kernel(InstructionChunk chunk, DInst *target, uint32_t count) {
+  if (threadIdx.x < count) target[threadIdx.x] = chunk.v[threadIdx.x];
+}
+void upload_instructions(hipStream_t stream, const DInst *insts, uint32_t count, DInst *target) {
+  for (uint32_t first = 0; first < count; first += 64) {
+    InstructionChunk chunk{};
+    const uint32_t n = std::min<uint32_t>(64, count - first);
+    for (uint32_t i = 0; i < n; ++i) chunk.v[i] = insts[first + i];
+    upload_instructions_kernel<<<dim3(1), 64, 0, stream>>>(chunk, target + first, n);
+  }
+}
+
+}  // namespace
 
 struct fh_submission {
   fh_backend *backend = nullptr;
@@ -144,20 +201,40 @@ struct fh_backend {
   std::vector<uint64_t> lane_metadata_key;          // what the gathered metadata was built from
   std::unordered_set<uint64_t> lane_metadata_watch; // allocations whose writes invalidate it
   uint64_t fused_runs = 0, fused_dispatches = 0;
-  char *ensure_lane_scratch(uint64_t bytes) {
-    if (bytes <= lane_scratch_bytes) return lane_scratch;
+  // Scratch taken from the library's fixed device array instead of the heap while
+  // fh_submit_static runs: nothing may then be allocated or freed, and a need beyond a region's
+  // size fails the dispatch (static_overflow tells that failure from an out-of-memory one).
+  bool static_mode = false;
+  bool static_overflow = false;
+  char *static_scratch = nullptr;        // this device's copy of the array
+  ErrorSlot *static_host_errors = nullptr;  // pinned mirror of its error records
+  char *static_programs = nullptr;       // typed instructions of the call's programs (bump)
+  uint64_t static_programs_used = 0;
+
+  // Makes `ptr` hold at least `bytes` (at least `floor` when it has to be allocated anew).
+  bool grow(char *&ptr, uint64_t &have, uint64_t bytes, uint64_t floor) {
+    if (bytes <= have) return true;
+    if (static_mode) {
+      static_overflow = true;
+      return false;
+    }
     (void)hipStreamSynchronize(stream);
-    if (lane_scratch) (void)hipFree(lane_scratch);
-    lane_scratch = nullptr;
-    lane_scratch_bytes = 0;
-    lane_metadata_valid = false;
-    attention_plan_valid = false;
-    uint64_t want = std::max<uint64_t>(bytes, 4ull << 20);
-    void *ptr = nullptr;
-    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
-    lane_scratch = (char *)ptr;
-    lane_scratch_bytes = want;
-    return lane_scratch;
+    if (ptr) (void)hipFree(ptr);
+    ptr = nullptr;
+    have = 0;
+    uint64_t want = std::max<uint64_t>(bytes, floor);
+    void *fresh = nullptr;
+    if (hipMalloc(&fresh, want) != hipSuccess) return false;
+    ptr = (char *)fresh;
+    have = want;
+    return true;
+  }
+  char *ensure_lane_scratch(uint64_t bytes) {
+    if (bytes > lane_scratch_bytes) {
+      lane_metadata_valid = false;
+      attention_plan_valid = false;
+    }
+    return grow(lane_scratch, lane_scratch_bytes, bytes, 4ull << 20) ? lane_scratch : nullptr;
   }
 
   // f32 accumulators handed to an epilogue program; separate from `workspace` because the kernel
@@ -165,30 +242,10 @@ struct fh_backend {
   char *accumulators = nullptr;
   uint64_t accumulator_bytes = 0;
   char *ensure_accumulators(uint64_t bytes) {
-    if (bytes <= accumulator_bytes) return accumulators;
-    (void)hipStreamSynchronize(stream);
-    if (accumulators) (void)hipFree(accumulators);
-    accumulators = nullptr;
-    accumulator_bytes = 0;
-    uint64_t want = std::max<uint64_t>(bytes, 16ull << 20);
-    void *ptr = nullptr;
-    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
-    accumulators = (char *)ptr;
-    accumulator_bytes = want;
-    return accumulators;
+    return grow(accumulators, accumulator_bytes, bytes, 16ull << 20) ? accumulators : nullptr;
   }
   char *ensure_workspace(uint64_t bytes) {
-    if (bytes <= workspace_bytes) return workspace;
-    (void)hipStreamSynchronize(stream);
-    if (workspace) (void)hipFree(workspace);
-    workspace = nullptr;
-    workspace_bytes = 0;
-    uint64_t want = std::max<uint64_t>(bytes, 64ull << 20);
-    void *ptr = nullptr;
-    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
-    workspace = (char *)ptr;
-    workspace_bytes = want;
-    return workspace;
+    return grow(workspace, workspace_bytes, bytes, 64ull << 20) ? workspace : nullptr;
   }
 };
 
@@ -309,10 +366,12 @@ View null_view() {
 // (crates/forja-core/src/program.rs): SSA order, typed operands, reductions only in row
 // programs and at most four, f32 outputs.  `u32_mask` bit i = input slot i is bound to a u32
 // tensor.  Produces the typed device instructions.
+constexpr uint32_t kMaxProgramInsts = 256;   // crates/forja-core/src/program.rs:25-31
+
 fh_status type_program(const Program &p, uint32_t u32_mask, uint32_t rank,
-                       std::vector<DInst> *out) {
-  std::vector<uint8_t> types(p.insts.size());
-  out->resize(p.insts.size());
+                       DInst *out /* [p.insts.size()] */) {
+  FH_REQUIRE(p.insts.size() <= kMaxProgramInsts);
+  uint8_t types[kMaxProgramInsts];
   uint32_t reductions = 0;
   for (size_t i = 0; i < p.insts.size(); ++i) {
     const fh_inst &in = p.insts[i];
@@ -365,7 +424,7 @@ fh_status type_program(const Program &p, uint32_t u32_mask, uint32_t rank,
     default: return FH_INVALID_INPUT;
     }
     if (in.kind == 4) d.ty = 0;
-    (*out)[i] = d;
+    out[i] = d;
   }
   for (size_t pair = 0; pair + 1 < p.pairs.size(); pair += 2) {
     FH_REQUIRE(p.pairs[pair] < p.n_outputs && p.pairs[pair + 1] < p.insts.size());
@@ -395,19 +454,35 @@ fh_status bind_program(fh_backend *b, Program &p, const fh_tensor *inputs, uint3
   }
   auto cached = p.typed.find(mask | (rank << 16));
   DInst *device = nullptr;
-  if (cached == p.typed.end()) {
-    std::vector<DInst> typed;
-    fh_status status = type_program(p, mask, rank, &typed);
-    if (status != FH_OK) return status;
-    void *ptr = nullptr;
-    if (hipMalloc(&ptr, typed.size() * sizeof(DInst)) != hipSuccess) return FH_ALLOCATION_FAILED;
-    if (hipMemcpy(ptr, typed.data(), typed.size() * sizeof(DInst), hipMemcpyHostToDevice) !=
-        hipSuccess)
-      return FH_DEVICE_EXECUTION_FAILED;
-    device = (DInst *)ptr;
-    p.typed[mask | (rank << 16)] = device;
-  } else {
+  if (cached != p.typed.end()) {
     device = cached->second;
+  } else {
+    DInst typed[kMaxProgramInsts];
+    fh_status status = type_program(p, mask, rank, typed);
+    if (status != FH_OK) return status;
+    const uint64_t bytes = p.insts.size() * sizeof(DInst);
+    if (b->static_mode) {
+      // Nothing may be allocated: the instructions travel as kernel arguments into the call's
+      // share of the fixed scratch array and are not kept.  (During validation, before the
+      // regions are set up, only the typing is checked.)
+      if (b->static_programs) {
+        const uint64_t need = (bytes + 255) / 256 * 256;
+        if (b->static_programs_used + need > kStaticProgramBytes) {
+          b->static_overflow = true;
+          return FH_ALLOCATION_FAILED;
+        }
+        device = (DInst *)(b->static_programs + b->static_programs_used);
+        b->static_programs_used += need;
+        upload_instructions(b->stream, typed, (uint32_t)p.insts.size(), device);
+      }
+    } else {
+      void *ptr = nullptr;
+      if (hipMalloc(&ptr, bytes) != hipSuccess) return FH_ALLOCATION_FAILED;
+      if (hipMemcpy(ptr, typed, bytes, hipMemcpyHostToDevice) != hipSuccess)
+        return FH_DEVICE_EXECUTION_FAILED;
+      device = (DInst *)ptr;
+      p.typed[mask | (rank << 16)] = device;
+    }
   }
   memset(args, 0, sizeof(*args));
   args->insts = device;
@@ -583,8 +658,7 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
   auto prog = b->programs.find(d.epilogue);
   FH_REQUIRE(prog != b->programs.end());
   if (d.accumulator_count == 1 && d.n_extras == 1 &&
-      is_add_epilogue(prog->second.insts, prog->second.pairs) &&
-      shape_is(d.inputs[primitive], {rows, columns})) {
+      prog->second.add_epilogue && shape_is(d.inputs[primitive], {rows, columns})) {
     QmmProblem fused{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows, inner, columns,
                      d.bits, d.group_size, &pl.in[primitive]};
     if (try_fast_quant_matmul(b, fused) || try_valu_quant_matmul(b, fused)) return FH_OK;
@@ -656,8 +730,7 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
     // Recognised epilogue: out = accumulator + extra (the MoE residual add).
     auto prog = b->programs.find(d.epilogue);
     FH_REQUIRE(prog != b->programs.end());
-    fuse_residual = d.accumulator_count == 1 && extras == 1 && is_add_epilogue(prog->second.insts,
-                                                                               prog->second.pairs);
+    fuse_residual = d.accumulator_count == 1 && extras == 1 && prog->second.add_epilogue;
     if (fuse_residual) {
       const fh_tensor &residual = d.inputs[primitive];
       FH_REQUIRE(shape_is(residual, {rows, columns}) && is_float(residual.dtype));
@@ -728,8 +801,7 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
   }
   auto prog = b->programs.find(d.epilogue);
   FH_REQUIRE(prog != b->programs.end());
-  if (primitive == 8 && extras == 0 &&
-      is_swiglu_epilogue(prog->second.insts, prog->second.pairs) &&
+  if (primitive == 8 && extras == 0 && prog->second.swiglu_epilogue &&
       try_fast_gather_projection(b, problem, 2, true, error))
     return FH_OK;
   uint32_t accumulators = primitive == 8 ? 2 : 1;
@@ -1567,6 +1639,24 @@ fh_status run_lane_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors) {
   return FH_OK;
 }
 
+// The BackendError a raised error record of dispatch `index` (operation `op`) stands for.
+fh_status failure_of(uint32_t op, uint32_t index, uint64_t serial, const ErrorSlot &record,
+                     fh_error *error) {
+  const bool index_error = op == FH_OP_GATHER_QUANT_MATMUL || op == FH_OP_QUANT_EMBED ||
+                           op == FH_OP_ROUTE_PACK;
+  // Sampling refuses its live parameters or mask as InvalidInput (lib.rs:1560-1567, 1639-1652).
+  const bool refused_input = op == FH_OP_SAMPLE || op == FH_OP_SAMPLE_MASKED;
+  const fh_status result = refused_input ? FH_INVALID_INPUT
+                                         : (index_error ? FH_INDEX_OUT_OF_RANGE : FH_DEVICE_ERROR_FLAG);
+  error->code = result;
+  error->dispatch = index;
+  error->submission = serial;
+  error->operation = op;
+  error->flag = record.flag;
+  error->value = record.value;
+  return result;
+}
+
 hipEvent_t take_event(fh_backend *b) {
   if (!b->event_pool.empty()) {
     hipEvent_t e = b->event_pool.back();
@@ -1624,6 +1714,17 @@ fh_status fh_create(int device, fh_backend **out) {
     delete b;
     return FH_DEVICE_EXECUTION_FAILED;
   }
+  // fh_submit_static may allocate nothing, so what it needs is set up here: this device's address
+  // of the fixed scratch array and a pinned mirror of its error records.
+  b->static_scratch = static_scratch_address(device);
+  void *mirror = nullptr;
+  if (!b->static_scratch ||
+      hipHostMalloc(&mirror, kStaticErrorBytes, hipHostMallocDefault) != hipSuccess) {
+    (void)hipStreamDestroy(b->stream);
+    delete b;
+    return FH_DEVICE_EXECUTION_FAILED;
+  }
+  b->static_host_errors = (ErrorSlot *)mirror;
   {
     std::lock_guard<std::mutex> lock(g_live_mutex);
     g_live_backends.insert(b);
@@ -1664,6 +1765,7 @@ void fh_destroy(fh_backend *b) {
       (void)hipHostFree(e.host);
     }
     if (b->ring) (void)hipHostFree(b->ring);
+    if (b->static_host_errors) (void)hipHostFree(b->static_host_errors);
     for (auto &open : b->open_timers)
       for (auto e : open) (void)hipEventDestroy(e);
     for (auto &t : b->timed) {
@@ -1870,8 +1972,8 @@ fh_status fh_prepare_program(fh_backend *b, uint32_t kind, const fh_inst *insts,
     }
   }
   // Typing check with every input assumed f32; u32 bindings are re-typed at dispatch.
-  std::vector<DInst> typed;
-  fh_status status = type_program(p, 0, FH_MAX_RANK, &typed);
+  DInst typed[kMaxProgramInsts];
+  fh_status status = type_program(p, 0, FH_MAX_RANK, typed);
   if (status != FH_OK) {
     // A program whose integer inputs make the all-f32 typing fail is still legal; defer.
     bool uses_index_math = false;
@@ -1880,6 +1982,8 @@ fh_status fh_prepare_program(fh_backend *b, uint32_t kind, const fh_inst *insts,
     if (!uses_index_math) return status;
   }
   p.fast = classify_program(kind, p.insts.data(), n_insts, p.pairs.data(), n_pairs);
+  p.add_epilogue = kind == 0 && is_add_epilogue(p.insts, p.pairs);
+  p.swiglu_epilogue = kind == 0 && is_swiglu_epilogue(p.insts, p.pairs);
   std::lock_guard<std::mutex> lock(b->mutex);
   uint64_t id = b->next_id++;
   b->programs[id] = std::move(p);
@@ -2012,6 +2116,110 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   return FH_OK;
 }
 
+fh_status fh_submit_static(fh_backend *b, const fh_dispatch *dispatches, uint32_t count,
+                           fh_error *error) {
+  if (!b || (!dispatches && count)) return FH_INVALID_INPUT;
+  if (error) memset(error, 0, sizeof(*error));
+  auto fail = [&](fh_status status, uint32_t index) {
+    if (error) {
+      error->code = status;
+      error->dispatch = index;
+    }
+    return status;
+  };
+  if ((uint64_t)count * sizeof(ErrorSlot) > kStaticErrorBytes) return fail(FH_QUOTA_EXCEEDED, count);
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  // From here on no allocator may run: scratch needs beyond the fixed regions fail instead.
+  struct Regions {
+    char *workspace, *accumulators, *route_plan, *attention_plan;
+    uint64_t workspace_bytes, accumulator_bytes, route_plan_bytes, attention_plan_bytes;
+    int profiling;
+  } saved{b->workspace, b->accumulators, b->route_plan, b->attention_plan, b->workspace_bytes,
+          b->accumulator_bytes, b->route_plan_bytes, b->attention_plan_bytes, b->profiling};
+  b->static_mode = true;
+  b->static_overflow = false;
+  b->static_programs = nullptr;
+  b->static_programs_used = 0;
+  b->profiling = 0;   // the timers take events from a pool that grows by allocation
+  auto leave = [&] {
+    b->workspace = saved.workspace;
+    b->accumulators = saved.accumulators;
+    b->route_plan = saved.route_plan;
+    b->attention_plan = saved.attention_plan;
+    b->workspace_bytes = saved.workspace_bytes;
+    b->accumulator_bytes = saved.accumulator_bytes;
+    b->route_plan_bytes = saved.route_plan_bytes;
+    b->attention_plan_bytes = saved.attention_plan_bytes;
+    b->profiling = saved.profiling;
+    b->static_mode = false;
+    b->static_programs = nullptr;
+    b->route_plan_valid = false;   // the plans lived in the fixed array
+    b->attention_plan_valid = false;
+    b->lane_metadata_valid = false;
+  };
+  // Validate the whole list before anything is enqueued, as fh_submit does.
+  for (uint32_t i = 0; i < count; ++i) {
+    fh_status status = process(b, dispatches[i], nullptr, false);
+    if (status != FH_OK) {
+      leave();
+      return fail(status, i);
+    }
+  }
+  char *at = b->static_scratch;
+  ErrorSlot *records = (ErrorSlot *)at;
+  at += kStaticErrorBytes;
+  b->static_programs = at;
+  at += kStaticProgramBytes;
+  b->route_plan = at;
+  b->route_plan_bytes = kStaticRoutePlanBytes;
+  at += kStaticRoutePlanBytes;
+  b->attention_plan = at;
+  b->attention_plan_bytes = kStaticAttentionPlanBytes;
+  at += kStaticAttentionPlanBytes;
+  b->accumulators = at;
+  b->accumulator_bytes = kStaticAccumulatorBytes;
+  at += kStaticAccumulatorBytes;
+  b->workspace = at;
+  b->workspace_bytes = kStaticWorkspaceBytes;
+  b->route_plan_valid = false;
+  b->attention_plan_valid = false;
+  b->lane_metadata_valid = false;
+  const uint32_t slots = count == 0 ? 1 : count;
+  // The array keeps the previous call's contents: the error records must start clear (a fill
+  // kernel, so that a caller may capture this call into a graph); every other region is written
+  // by the kernels that read it.
+  launch_init_errors(b->stream, records, slots);
+  fh_status status = FH_OK;
+  uint32_t index = 0;
+  for (; index < count; ++index) {
+    const fh_dispatch &d = dispatches[index];
+    status = process(b, d, &records[index], true);
+    if (status != FH_OK) break;
+    for (uint32_t o = 0; o < d.n_outputs && o < FH_MAX_OUTPUTS; ++o) {
+      const uint64_t written = d.outputs[o].buffer;
+      if (b->route_plan_valid && written == b->route_plan_key.buffer) b->route_plan_valid = false;
+      if (b->attention_plan_valid)
+        for (uint64_t watched : b->attention_plan_key.buffers)
+          if (watched != 0 && written == watched) b->attention_plan_valid = false;
+    }
+  }
+  const bool overflow = b->static_overflow;
+  leave();
+  if (status != FH_OK)   // a need beyond the fixed array is a quota, not an out-of-memory
+    return fail(status == FH_ALLOCATION_FAILED && overflow ? FH_QUOTA_EXCEEDED : status, index);
+  if (hipGetLastError() != hipSuccess) return fail(FH_DEVICE_EXECUTION_FAILED, 0);
+  if (!error) return FH_OK;   // enqueued; the caller does not want to wait
+  if (hipMemcpyAsync(b->static_host_errors, records, slots * sizeof(ErrorSlot),
+                     hipMemcpyDeviceToHost, b->stream) != hipSuccess ||
+      hipStreamSynchronize(b->stream) != hipSuccess)
+    return fail(FH_DEVICE_EXECUTION_FAILED, 0);
+  for (uint32_t i = 0; i < count; ++i)
+    if (b->static_host_errors[i].flag)
+      return failure_of(dispatches[i].op, i, 0, b->static_host_errors[i], error);
+  return FH_OK;
+}
+
 fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
   if (!s) return FH_INVALID_INPUT;
   fh_backend *b = s->backend;
@@ -2063,19 +2271,7 @@ fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
         s->gpu_ns = (uint64_t)((double)ms * 1e6);
       for (uint32_t i = 0; i < s->count; ++i) {
         if (!s->host_errors[i].flag) continue;
-        uint32_t op = s->ops[i];
-        bool index_error = op == FH_OP_GATHER_QUANT_MATMUL || op == FH_OP_QUANT_EMBED ||
-                           op == FH_OP_ROUTE_PACK;
-        // Sampling refuses its live parameters or mask as InvalidInput (lib.rs:1560-1567, 1639-1652).
-        bool refused_input = op == FH_OP_SAMPLE || op == FH_OP_SAMPLE_MASKED;
-        s->result = refused_input ? FH_INVALID_INPUT
-                                  : (index_error ? FH_INDEX_OUT_OF_RANGE : FH_DEVICE_ERROR_FLAG);
-        s->error.code = s->result;
-        s->error.dispatch = i;
-        s->error.submission = s->serial;
-        s->error.operation = op;
-        s->error.flag = s->host_errors[i].flag;
-        s->error.value = s->host_errors[i].value;
+        s->result = failure_of(s->ops[i], i, s->serial, s->host_errors[i], &s->error);
         break;
       }
     }
@@ -2201,6 +2397,9 @@ fh_status fh_profile_read(fh_backend *b, uint32_t kernel_class, uint64_t *nanose
 
 namespace fh {
 char *backend_workspace(fh_backend *backend, uint64_t bytes) { return backend->ensure_workspace(bytes); }
+uint64_t backend_workspace_limit(fh_backend *backend) {
+  return backend->static_mode ? backend->workspace_bytes : ~0ull;
+}
 char *backend_route_plan(fh_backend *b, const RoutePlanKey &key, uint64_t bytes, bool *reuse) {
   const RoutePlanKey &have = b->route_plan_key;
   *reuse = b->route_plan_valid && bytes <= b->route_plan_bytes && have.buffer == key.buffer &&
@@ -2209,17 +2408,7 @@ char *backend_route_plan(fh_backend *b, const RoutePlanKey &key, uint64_t bytes,
            have.tile == key.tile;
   if (*reuse) return b->route_plan;
   b->route_plan_valid = false;
-  if (bytes > b->route_plan_bytes) {
-    (void)hipStreamSynchronize(b->stream);
-    if (b->route_plan) (void)hipFree(b->route_plan);
-    b->route_plan = nullptr;
-    b->route_plan_bytes = 0;
-    uint64_t want = std::max<uint64_t>(bytes, 1ull << 20);
-    void *ptr = nullptr;
-    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
-    b->route_plan = (char *)ptr;
-    b->route_plan_bytes = want;
-  }
+  if (!b->grow(b->route_plan, b->route_plan_bytes, bytes, 1ull << 20)) return nullptr;
   b->route_plan_key = key;
   b->route_plan_valid = true;
   return b->route_plan;
@@ -2230,17 +2419,7 @@ char *backend_attention_plan(fh_backend *b, const AttentionPlanKey &key, uint64_
            memcmp(&b->attention_plan_key, &key, sizeof(key)) == 0;
   if (*reuse) return b->attention_plan;
   b->attention_plan_valid = false;
-  if (bytes > b->attention_plan_bytes) {
-    (void)hipStreamSynchronize(b->stream);
-    if (b->attention_plan) (void)hipFree(b->attention_plan);
-    b->attention_plan = nullptr;
-    b->attention_plan_bytes = 0;
-    uint64_t want = std::max<uint64_t>(bytes, 1ull << 20);
-    void *ptr = nullptr;
-    if (hipMalloc(&ptr, want) != hipSuccess) return nullptr;
-    b->attention_plan = (char *)ptr;
-    b->attention_plan_bytes = want;
-  }
+  if (!b->grow(b->attention_plan, b->attention_plan_bytes, bytes, 1ull << 20)) return nullptr;
   b->attention_plan_key = key;
   b->attention_plan_valid = true;
   return b->attention_plan;

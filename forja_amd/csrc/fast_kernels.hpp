@@ -13,6 +13,9 @@ namespace fh {
 
 // Implemented in backend.cpp.
 char *backend_workspace(fh_backend *backend, uint64_t bytes);
+// The most backend_workspace can hand out: unbounded, except while the backend takes its scratch
+// from the library's fixed array.
+uint64_t backend_workspace_limit(fh_backend *backend);
 hipStream_t backend_stream(fh_backend *backend);
 uint32_t backend_compute_units(fh_backend *backend);
 void backend_profile_begin(fh_backend *backend, uint32_t kernel_class);

@@ -1187,6 +1187,19 @@ bool carve_partials(fh_backend *backend, FastRagged *f, char *plan_storage) {
   return true;
 }
 
+// Shortens the split count until the partials (and the plan, when it lives in the workspace too)
+// fit what the workspace can hand out.
+void fit_splits(fh_backend *backend, FastRagged *f, bool plan_in_workspace) {
+  const uint64_t limit = backend_workspace_limit(backend);
+  auto need = [&] {
+    const uint64_t slots = (uint64_t)f->tokens * f->max_splits;
+    return (plan_in_workspace ? plan_storage_bytes(*f) : 0) +
+           round_256(slots * f->query_heads * sizeof(float2)) +
+           slots * f->query_heads * 128 * sizeof(float);
+  };
+  while (f->max_splits > 1 && need() > limit) --f->max_splits;
+}
+
 void launch_plan(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
   ragged_plan_kernel<<<dim3(1), 256, 0, stream>>>(f, error);
 }
@@ -1241,6 +1254,7 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   f.physical_pages = lane.physical_pages;
   f.table_pages = lane.logical_pages;
   f.max_splits = splits_for(f.tokens);
+  fit_splits(backend, &f, true);
   f.group_tokens = f.tokens > 1 ? kSharedWaves * kSharedTiles * (16 / group) : 1;
   f.scale_log2 = lane.scale * 1.4426950408889634f;
   f.one_start = lane.query_start;
@@ -1286,6 +1300,7 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     f.physical_pages = p.physical_pages;
     f.table_pages = p.table_pages;
     f.max_splits = splits_for(p.tokens);
+    fit_splits(backend, &f, false);
     f.error_stride = p.error_stride;
     f.scale_log2 = p.scale * 1.4426950408889634f;
     f.tables = (const uint32_t *)p.tables.base + p.tables.offset;

@@ -58,7 +58,7 @@ class FhDeviceInfo(C.Structure):
 
 EXPORTS = [
     "fh_create", "fh_destroy", "fh_alloc", "fh_release", "fh_import", "fh_write", "fh_read",
-    "fh_read_tensor", "fh_prepare_program", "fh_release_program", "fh_submit", "fh_wait",
+    "fh_read_tensor", "fh_prepare_program", "fh_release_program", "fh_submit", "fh_submit_static", "fh_wait",
     "fh_gpu_time_ns", "fh_submission_free", "fh_device_info_get", "fh_memory_usage",
     "fh_synchronize", "fh_profile_enable", "fh_profile_select", "fh_profile_reset", "fh_profile_read",
     "fh_fusion_enable", "fh_fusion_stats", "fh_version",
@@ -90,6 +90,7 @@ def load_library():
                                        C.POINTER(u64)]
     lib.fh_release_program.argtypes = [vp, u64]
     lib.fh_submit.argtypes = [vp, C.POINTER(FhDispatch), u32, C.POINTER(vp)]
+    lib.fh_submit_static.argtypes = [vp, C.POINTER(FhDispatch), u32, C.POINTER(FhError)]
     lib.fh_wait.argtypes = [vp, u64, C.POINTER(FhError)]
     lib.fh_gpu_time_ns.argtypes = [vp]
     lib.fh_gpu_time_ns.restype = u64
@@ -307,6 +308,17 @@ class HipBackend:
         handle = C.c_void_p()
         _check(self._lib.fh_submit(self._handle, encoded.array, encoded.count, C.byref(handle)))
         return HipSubmission(self, handle)
+
+    def submit_static(self, commands, wait: bool = True) -> None:
+        """fh_submit_static: the same dispatches executed without any allocation, all device
+        scratch taken from the library's fixed array.  `wait` false only enqueues."""
+        encoded = commands if isinstance(commands, EncodedCommands) else self.encode(commands)
+        error = FhError()
+        status = self._lib.fh_submit_static(self._handle, encoded.array, encoded.count,
+                                            C.byref(error) if wait else None)
+        if status != 0:
+            raise BackendError(Status(status), index=error.value, dispatch=error.dispatch,
+                               operation=error.operation, flag=error.flag)
 
     def synchronize(self):
         _check(self._lib.fh_synchronize(self._handle))

@@ -53,8 +53,8 @@ typedef enum fh_status {
 /* wit/compute.wit:4-10 */
 typedef enum fh_dtype { FH_F32 = 0, FH_F16 = 1, FH_BF16 = 2, FH_I32 = 3, FH_U32 = 4 } fh_dtype;
 
-/* `Op` (crates/forja-core/src/ops.rs:163-302).  State ops, dense gather-matmul, contiguous sdpa
- * and sampling are outside this backend's path and answer FH_UNSUPPORTED_OPERATION. */
+/* `Op` (crates/forja-core/src/ops.rs:163-302).  State ops, dense gather-matmul and contiguous
+ * sdpa are outside this backend's path and answer FH_UNSUPPORTED_OPERATION. */
 typedef enum fh_op_kind {
   FH_OP_PROGRAM = 1,             /* Op::Program: validated map/row scalar program */
   FH_OP_COPY = 2,                /* Op::Copy */
@@ -199,6 +199,28 @@ FH_API fh_status fh_release_program(fh_backend *backend, fh_program program);
  * dispatches in order on the backend's stream.  Returns without waiting. */
 FH_API fh_status fh_submit(fh_backend *backend, const fh_dispatch *dispatches, uint32_t count,
                     fh_submission **out);
+/* fh_submit for callers that cannot allocate.  It has no counterpart in the reference: it exists
+ * for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  It
+ * validates and enqueues the dispatches exactly as fh_submit does, in order, one by one (runs of
+ * per-lane attention dispatches are not fused: record FH_OP_PAGED_ATTENTION_RAGGED), but takes all
+ * device scratch - error records, typed program instructions, route plans, attention plans,
+ * epilogue accumulators, kernel workspace - from a fixed array of FH_STATIC_SCRATCH_BYTES inside
+ * the library's device image (one copy per GPU, held until the process ends) and calls no
+ * hipMalloc, hipFree, hipHostMalloc or event creation.  Inputs and outputs are the caller's
+ * tensors as always.  Limits: at most 8192 dispatches; 36 MiB of kernel workspace, 8 MiB of
+ * epilogue accumulators, 1 MiB of route plan, 2 MiB of attention plan, 960 KiB of program
+ * instructions per call.  Split-KV attention shortens its split count to fit the workspace; any
+ * other need beyond a region fails the call with FH_QUOTA_EXCEEDED, `error->dispatch` naming the
+ * dispatch that did not fit (earlier dispatches have run, as when fh_submit stops at a failing
+ * dispatch).  `error` not null: the call waits for the work and reports data-dependent failures
+ * as fh_wait does.  `error` null: the call returns once the work is enqueued and synchronises
+ * nothing.  All calls on one GPU share that GPU's array, which keeps the previous call's
+ * contents (what must start clear is cleared by a kernel): calls that overlap on one GPU - two
+ * backends on it, or a call whose kernels still run when the next call's kernels start on another
+ * stream - race. */
+#define FH_STATIC_SCRATCH_BYTES (48ull << 20)
+FH_API fh_status fh_submit_static(fh_backend *backend, const fh_dispatch *dispatches, uint32_t count,
+                           fh_error *error);
 /* Submission::wait / wait_timeout (backend.rs:609-647).  timeout_ns 0 = no deadline. */
 FH_API fh_status fh_wait(fh_submission *submission, uint64_t timeout_ns, fh_error *error);
 /* Submission::gpu_time: device time between the first and last kernel, in ns (0 before wait). */

@@ -7,6 +7,12 @@ It owns no compute: every tensor operation is a dispatch executed by the backend
 `PagedSdpaAppend` dispatches are replaced by the one packed ragged-attention dispatch.
 Weights are synthetic (seeded on the device with FILL_SEEDED): MLX-4bit packed words uniform over
 u32, bf16 scale ~ U(0.001, 0.02), bf16 bias ~ U(-0.1, 0.1); norm weights ~ U(0.9, 1.1).
+
+A second weight law, "zero_mean", exists for tests only: bias = -7.5 * scale + U(-0.02, 0.02) (-127.5 * scale
+for 8-bit weights), so that a dequantised weight scale * (q - 7.5) + noise has no common sign.  Under the prescribed law
+every weight has a positive mean about as large as its spread, one direction swamps the hidden
+state and every lane emits the same token at every step; under the zero-mean law tokens depend on
+the lane's context, its attention and its routing.
 """
 from __future__ import annotations
 
@@ -73,10 +79,16 @@ class QuantLinear:
         self.scales = backend.alloc(DType.BF16, lead + (n, k // GROUP))
         self.biases = backend.alloc(DType.BF16, lead + (n, k // GROUP))
 
-    def fill(self, commands: CommandList, seed: int, stream: int):
+    def fill(self, commands: CommandList, seed: int, stream: int, center=None, noise=None):
+        """`center`: the prepared program bias = noise - 7.5 * scale of the zero-mean law, with
+        `noise` a scratch tensor of the biases' shape."""
         commands.dispatch(Op.fill_seeded(0, seed, stream), [], self.packed)
         commands.dispatch(Op.fill_seeded(1, seed, stream + 1, lo=0.001, hi=0.02), [], self.scales)
-        commands.dispatch(Op.fill_seeded(1, seed, stream + 2, lo=-0.1, hi=0.1), [], self.biases)
+        if center is None:
+            commands.dispatch(Op.fill_seeded(1, seed, stream + 2, lo=-0.1, hi=0.1), [], self.biases)
+            return
+        commands.dispatch(Op.fill_seeded(1, seed, stream + 2, lo=-0.02, hi=0.02), [], noise)
+        commands.dispatch_kernel(center, [self.scales, noise], [self.biases])
 
     @property
     def triple(self):
@@ -109,14 +121,19 @@ def strided(tensor: Tensor, offset: int, shape, strides) -> Tensor:
 
 
 class Model:
-    def __init__(self, backend, config: ModelConfig, seed: int = 1234, layers: Optional[int] = None):
+    def __init__(self, backend, config: ModelConfig, seed: int = 1234, layers: Optional[int] = None,
+                 weight_law: str = "baseline"):
+        """`weight_law`: "baseline" (the prescribed synthetic law) or "zero_mean" (tests only)."""
+        assert weight_law in ("baseline", "zero_mean")
         self.backend, self.config, self.seed = backend, config, seed
         c = config
         self.n_layers = c.layers if layers is None else layers
         self._stream = 0
+        self._center = {bits: backend.prepare_program(programs.centered_bias_elements(bits))
+                        for bits in {BITS, c.router_bits}} if weight_law == "zero_mean" else None
+        self._noise: List[Tensor] = []
         fill = CommandList()
-        self.embed = QuantLinear(backend, c.vocab, c.hidden)
-        self.embed.fill(fill, seed, self._next_stream(3))
+        self.embed = self._linear(fill, c.vocab, c.hidden)
         self.layers: List[LayerWeights] = []
         for _ in range(self.n_layers):
             lw = LayerWeights(
@@ -137,6 +154,9 @@ class Model:
         self.final_norm = self._norm(fill, (c.hidden,))
         self.lm_head = self._linear(fill, c.vocab, c.hidden)
         backend.submit(fill).wait()
+        for noise in self._noise:
+            backend.release(noise)
+        self._noise = []
         self.rms_norm = backend.prepare_program(programs.rms_norm_rows(c.rms_eps))
         self.residual_norm = backend.prepare_program(programs.residual_norm_rows(c.rms_eps))
         self.qk_norm_rope = backend.prepare_program(
@@ -153,7 +173,12 @@ class Model:
 
     def _linear(self, fill, n, k, experts=0, bits=BITS) -> QuantLinear:
         linear = QuantLinear(self.backend, n, k, experts, bits)
-        linear.fill(fill, self.seed, self._next_stream(3))
+        noise = None
+        if self._center is not None:
+            noise = self.backend.alloc(DType.BF16, linear.biases.shape)
+            self._noise.append(noise)
+        linear.fill(fill, self.seed, self._next_stream(3),
+                    self._center[bits] if self._center is not None else None, noise)
         return linear
 
     def _norm(self, fill, shape) -> Tensor:

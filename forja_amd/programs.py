@@ -63,3 +63,13 @@ def add_elements():
     b = ProgramBuilder(ProgramKind.MAP)
     b.output(0, b.add(b.input(0), b.input(1)))
     return b.finish()
+
+
+def centered_bias_elements(bits: int = 4):
+    """bias = noise - ((2^bits - 1) / 2) * scale: the affine bias that centres the quantised values
+    0..2^bits-1 on zero (the zero-mean weight law of the model-level tests; not a reference
+    program)."""
+    b = ProgramBuilder(ProgramKind.MAP)
+    scale, noise = b.input(0), b.input(1)
+    b.output(0, b.add(b.mul(scale, b.const(-((1 << bits) - 1) / 2.0)), noise))
+    return b.finish()

@@ -28,7 +28,7 @@ def test_config0_single_layer_decode_step(cpu, hip):
     for name in ("attended", "projected", "logits"):
         a = to_f32(cpu.read(getattr(ref.buffers, name)), DType.BF16)
         b = to_f32(hip.read(getattr(dev.buffers, name)), DType.BF16)
-        assert_close(b, a, DType.BF16, abs_=2e-2)
+        assert_close(b, a, DType.BF16)
     # The appended K/V rows land at identical (page, slot) positions (block-table addressing is
     # exact); their values are computed activations and agree to the bf16 bar.
     for pools in ("keys", "values"):
@@ -40,8 +40,81 @@ def test_config0_single_layer_decode_step(cpu, hip):
             page = ref.cache.lane_pages[lane][context // 16]
             expected_rows.add(page * 16 + context % 16)
         assert set(rows_a.tolist()) <= expected_rows
-        assert_close(b, a, DType.BF16, abs_=2e-2)
+        assert_close(b, a, DType.BF16)
     assert ref_tokens.tolist() == dev_tokens.tolist()
+
+
+def teacher_forced_parity(cpu, hip, ref, dev, steps, dtype, lane_by_lane=False):
+    """The reference's own model-level protocol for reduced precision (docs/engines.md:65-68,
+    support/golden-fixtures/src/comparison.rs:4-8): the oracle decodes `steps` greedy steps on its
+    own tokens, the device decodes the same steps fed the oracle's tokens ("reference-token
+    teacher forcing"), and over all steps and lanes the mean KL divergence of the logit
+    distributions is at most 1e-2, the greedy tokens agree on at least 95 % of the draws and the
+    normwise error of the hidden state is at most 5e-2.  Free-running greedy decoding is only
+    informative there: one bf16 rounding that differs flips a near-tie (under the zero-mean law
+    13 % of the oracle's draws have a top-2 margin below two bf16 steps) or, in a routed model,
+    swaps the last chosen expert, and every later token differs.  Returns the oracle's tokens."""
+    lanes = len(ref.contexts)
+    tokens, agree, divergence = [], [], []
+    error_squared = norm_squared = 0.0
+
+    def log_softmax(x):
+        x = x - x.max(axis=1, keepdims=True)
+        return x - np.log(np.exp(x).sum(axis=1, keepdims=True))
+    for step in range(steps):
+        if step:
+            hip.write(dev.buffers.ids, tokens[-1].astype(np.uint32).tobytes())
+        ref_tokens, dev_tokens = ref.step(), dev.step(lane_by_lane)
+        a = to_f32(cpu.read(ref.buffers.logits), dtype).reshape(lanes, -1).astype(np.float64)
+        b = to_f32(hip.read(dev.buffers.logits), dtype).reshape(lanes, -1).astype(np.float64)
+        assert np.isfinite(b).all(), step
+        la, lb = log_softmax(a), log_softmax(b)
+        divergence.append((np.exp(la) * (la - lb)).sum(axis=1))
+        agree.append(ref_tokens == dev_tokens)
+        for index in range(2):      # the residual stream after the last layer and before it
+            ha = to_f32(cpu.read(ref.buffers.hidden[index]), dtype).astype(np.float64)
+            hb = to_f32(hip.read(dev.buffers.hidden[index]), dtype).astype(np.float64)
+            error_squared += float(((ha - hb) ** 2).sum())
+            norm_squared += float((ha ** 2).sum())
+        tokens.append(ref_tokens)
+    assert np.mean(divergence) <= 1e-2, np.mean(divergence)
+    assert np.mean(agree) >= 0.95, np.mean(agree)
+    assert np.sqrt(error_squared / norm_squared) <= 5e-2, np.sqrt(error_squared / norm_squared)
+    return np.stack(tokens)
+
+
+def assert_tokens_depend_on_lane_and_step(tokens):
+    """The check the prescribed weight law cannot give: many distinct tokens, lanes that differ."""
+    assert len(np.unique(tokens)) >= 16, np.unique(tokens)
+    assert all(len(set(row.tolist())) > 1 for row in tokens), tokens
+    assert all(len(set(column.tolist())) > 1 for column in tokens.T), tokens
+
+
+def test_zero_mean_weights_32_steps_dense(cpu, hip):
+    """Dense model under the zero-mean test law: tokens vary by lane and step, so a wrong lane
+    mapping, a cache mix-up or a stale page would move the logits compared at every step."""
+    ref, dev = (DecodeSession(Model(backend, QWEN3_0_6B, seed=31, layers=2, weight_law="zero_mean"),
+                              [17, 64, 130, 511], seed=31) for backend in (cpu, hip))
+    assert_tokens_depend_on_lane_and_step(teacher_forced_parity(cpu, hip, ref, dev, 32, DType.BF16))
+
+
+def test_zero_mean_weights_32_steps_moe(cpu, hip):
+    ref, dev = (DecodeSession(Model(backend, TINY_MOE, seed=32, layers=2, weight_law="zero_mean"),
+                              [5, 40, 300, 77, 16, 15], seed=32) for backend in (cpu, hip))
+    assert_tokens_depend_on_lane_and_step(teacher_forced_parity(cpu, hip, ref, dev, 32, DType.BF16))
+
+
+def test_zero_mean_weights_32_steps_with_the_qwen3_coder_dtypes(cpu, hip):
+    """f32 activations, f16 cache, 8-bit router, recorded lane by lane (the fused runs)."""
+    from dataclasses import replace
+    config = replace(TINY_MOE, activation_dtype=DType.F32, kv_dtype=DType.F16, router_bits=8)
+    ref, dev = (DecodeSession(Model(backend, config, seed=33, layers=2, weight_law="zero_mean"),
+                              [5, 40, 300, 77, 16, 15], seed=33) for backend in (cpu, hip))
+    dev.record_lane_by_lane()
+    before = hip.fusion_stats()[0]
+    tokens = teacher_forced_parity(cpu, hip, ref, dev, 32, DType.F32, lane_by_lane=True)
+    assert hip.fusion_stats()[0] - before == 2 * 32
+    assert_tokens_depend_on_lane_and_step(tokens)
 
 
 def test_greedy_tokens_identical_over_32_steps_dense(cpu, hip):
@@ -58,7 +131,7 @@ def test_greedy_tokens_identical_over_32_steps_moe(cpu, hip):
     assert ref_tokens.tolist() == dev_tokens.tolist()
     a = to_f32(cpu.read(ref.buffers.logits), DType.BF16)
     b = to_f32(hip.read(dev.buffers.logits), DType.BF16)
-    assert_close(b, a, DType.BF16, abs_=3e-2)
+    assert_close(b, a, DType.BF16)
 
 
 def test_greedy_tokens_identical_over_32_steps_with_the_qwen3_coder_dtypes(cpu, hip):
@@ -125,7 +198,7 @@ def test_packed_prefill_and_decode_step_matches_the_oracle(cpu, hip, config, con
     for name in ("attended", "projected", "logits"):
         a = to_f32(cpu.read(getattr(ref.buffers, name)), DType.BF16)
         b = to_f32(hip.read(getattr(dev.buffers, name)), DType.BF16)
-        assert_close(b, a, DType.BF16, abs_=2e-2)
+        assert_close(b, a, DType.BF16)
     last_rows = np.cumsum(counts) - 1
     a = np.frombuffer(cpu.read(ref.buffers.next_tokens), np.uint32)[last_rows]
     b = np.frombuffer(hip.read(dev.buffers.next_tokens), np.uint32)[last_rows]

@@ -9,7 +9,7 @@ LIB = os.path.join(HERE, "libforja_hip.so")
 PROBES = os.path.join(HERE, "libforja_probes.so")
 CONFORMANCE = os.path.join(HERE, "host", "conformance")
 
-SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "qmm_gemm.hip", "programs_fast.hip", "lane_fusion.hip", "sampling.hip", "qmm_valu.hip"]
+SOURCES = ["backend.cpp", "generic_ops.hip", "moe.hip", "paged_attention.hip", "qmm_fast.hip", "qmm_gemm.hip", "programs_fast.hip", "lane_fusion.hip", "sampling.hip", "qmm_valu.hip", "qmm_ksplit.hip"]
 
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

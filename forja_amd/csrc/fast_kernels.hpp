@@ -80,6 +80,42 @@ bool try_valu_gather(fh_backend *backend, const View &x, const View &packed, con
 // have then written nothing and the caller must run a kernel conditioned on that word.
 bool launch_quant_gemm(fh_backend *backend, const QmmProblem &problem, const uint32_t **refused);
 
+// ---- qmm_ksplit.hip: products over at most 32 activation rows per weight (decode GEMV, routed
+// MoE tiles), K split over the waves of a workgroup with the rows stationary in registers.
+// Operands as try_fast_quant_matmul checks them: bf16 rows, 4-bit weights in groups of 64 with
+// bf16 scales and biases, aligned contiguous rows.
+// Whether K has an instantiation (dense: at most 16 rows for the longest rows; routed: tiles of
+// 16 or 32 rows) and the output columns are whole batches of the kernel (32 or 64 columns; 16 or
+// 32 per projection of a pair).
+bool ksplit_supports(uint32_t inner, uint32_t columns, bool pair, bool routed);
+struct KsplitDense {
+  const uint16_t *x;
+  uint64_t x_row_stride;
+  const uint32_t *packed;
+  const uint16_t *scales, *biases;
+  void *out;
+  uint64_t out_row_stride;
+  uint32_t out_f32;
+  const uint16_t *residual;
+  uint64_t residual_row_stride;
+  uint32_t rows, inner, columns;
+};
+// False when K has no instantiation or the rows are more than 32: nothing was launched.
+bool launch_ksplit_dense(fh_backend *backend, const KsplitDense &problem);
+struct KsplitRouted {
+  const uint16_t *x;
+  uint64_t x_row_stride;
+  const uint32_t *packed[2];
+  const uint16_t *scales[2], *biases[2];
+  bool pair;                // gate/up pair with SwiGLU (bf16 out), else one projection
+  void *out;                // [routes, columns] dense rows, bf16 or f32
+  uint32_t out_f32;
+  uint32_t inner, columns;
+  const uint32_t *sorted_routes, *blocks, *n_blocks;
+  uint32_t max_blocks, tile_rows, route_div;
+};
+bool launch_ksplit_routed(fh_backend *backend, const KsplitRouted &problem);
+
 struct GatherProblem {
   View x;           // projection: [R,K]; weighted sum: [R,k,K]
   View packed[2], scales[2], biases[2];

@@ -1113,6 +1113,12 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
     residual = u16_ptr(r);
     residual_row_stride = r.stride[0];
   }
+  // At most 32 rows: the wave-reduced GEMV, K split over the waves of a workgroup.
+  if (p.rows <= 32 && ksplit_supports(p.inner, p.columns, false, false)) {
+    KsplitDense d{a.x, a.x_row_stride, a.packed[0], a.scales[0], a.biases[0], a.out, a.out_row_stride,
+                  a.out_f32, residual, residual_row_stride, p.rows, p.inner, p.columns};
+    if (launch_ksplit_dense(backend, d)) return true;
+  }
   // Decode rows.  When one workgroup per compute unit covers the output, the single-kernel tile
   // product; wider outputs go through the K slabs.
   if (p.rows <= 128 &&
@@ -1153,14 +1159,15 @@ struct RoutePlan {
 // Packs the routes on the device (or reuses the plan the previous routed projection packed from
 // the same indices); `extra` bytes of ordinary workspace are returned in plan->rest.
 bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, ErrorSlot *error,
-                 RoutePlan *plan, uint32_t *zero_rows = nullptr, uint32_t zero_row_words = 0) {
+                 RoutePlan *plan, uint32_t *zero_rows = nullptr, uint32_t zero_row_words = 0,
+                 uint32_t tile = kRouteTile) {
   uint64_t routes = (uint64_t)p.rows * p.k;
-  plan->max_blocks = p.experts + (uint32_t)(routes / kRouteTile) + 1;
+  plan->max_blocks = p.experts + (uint32_t)(routes / tile) + 1;
   auto round = [](uint64_t bytes) { return (bytes + 255) / 256 * 256; };
   uint64_t counts_b = round(p.experts * 4ull), offsets_b = round((p.experts + 1) * 4ull),
            sorted_b = round(routes * 4), blocks_b = round(plan->max_blocks * 12ull), nb_b = 256;
   RoutePlanKey key{p.indices_buffer, p.indices.offset, p.indices.stride[0], p.indices.stride[1],
-                   p.rows, p.k, p.experts, kRouteTile};
+                   p.rows, p.k, p.experts, tile};
   bool reuse = false;
   char *ws = backend_route_plan(backend, key, counts_b + offsets_b + sorted_b + blocks_b + nb_b, &reuse);
   if (!ws) return false;
@@ -1180,7 +1187,7 @@ bool plan_routes(fh_backend *backend, const GatherProblem &p, uint64_t extra, Er
   plan->n_blocks = (uint32_t *)ws;
   plan->reused = reuse;
   if (!reuse)
-    launch_route_pack(backend_stream(backend), p.indices, p.rows, p.k, p.experts, kRouteTile,
+    launch_route_pack(backend_stream(backend), p.indices, p.rows, p.k, p.experts, tile,
                       plan->counts, plan->offsets, plan->sorted_routes, plan->blocks,
                       plan->max_blocks, plan->n_blocks, error, zero_rows, zero_row_words);
   return true;
@@ -1207,6 +1214,37 @@ void launch_routed(hipStream_t stream, const QmmArgs &a, uint32_t max_blocks, ui
     return;
   }
   launch_qmm<kPair, true>(stream, a, max_blocks, 1);
+}
+
+// Route tile of the K-split kernels: 16 rows while an expert sees few routes on average (an
+// expert with more gets a second tile and its weights are read again), else 32; 0 when the
+// kernels do not take this K.
+uint32_t ksplit_route_tile(const GatherProblem &p, bool pair) {
+  if (!ksplit_supports(p.inner, p.columns, pair, true)) return 0;
+  return (uint64_t)p.rows * p.k <= 10ull * p.experts ? 16 : 32;
+}
+
+bool launch_routed_ksplit(fh_backend *backend, const QmmArgs &a, bool pair, uint32_t max_blocks, uint32_t tile) {
+  KsplitRouted r{};
+  r.x = a.x;
+  r.x_row_stride = a.x_row_stride;
+  for (int pj = 0; pj < (pair ? 2 : 1); ++pj) {
+    r.packed[pj] = a.packed[pj];
+    r.scales[pj] = a.scales[pj];
+    r.biases[pj] = a.biases[pj];
+  }
+  r.pair = pair;
+  r.out = a.out;
+  r.out_f32 = a.out_f32;
+  r.inner = a.inner;
+  r.columns = a.columns;
+  r.sorted_routes = a.sorted_routes;
+  r.blocks = a.blocks;
+  r.n_blocks = a.n_blocks;
+  r.max_blocks = max_blocks;
+  r.tile_rows = tile;
+  r.route_div = a.route_div;
+  return launch_ksplit_routed(backend, r);
 }
 
 bool gather_eligible(const GatherProblem &p, int projections) {
@@ -1259,9 +1297,10 @@ bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int
   // packs, and the whole output is cleared first.
   RoutePlan plan;
   const bool row_words = p.columns % 2 == 0 && p.out.offset % 2 == 0;
+  const uint32_t ksplit_tile = ksplit_route_tile(p, projections == 2);
   if (!plan_routes(backend, p, 0, error, &plan,
                    row_words ? (uint32_t *)((uint16_t *)p.out.base + p.out.offset) : nullptr,
-                   p.columns / 2))
+                   p.columns / 2, ksplit_tile ? ksplit_tile : kRouteTile))
     return false;
   hipStream_t stream = backend_stream(backend);
   if (plan.reused || !row_words)
@@ -1289,6 +1328,7 @@ bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int
   a.route_div = p.k;
   a.split_below = backend_compute_units(backend) / 2;
   KernelTimer timer(backend, FH_KC_MOE_KERNEL);
+  if (ksplit_tile && launch_routed_ksplit(backend, a, projections == 2, plan.max_blocks, ksplit_tile)) return true;
   if (projections == 2)
     launch_routed<true>(stream, a, plan.max_blocks, backend_compute_units(backend));
   else
@@ -1305,7 +1345,9 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
     return false;
   uint64_t partial_bytes = (uint64_t)p.rows * p.k * p.columns * sizeof(float);
   RoutePlan plan;
-  if (!plan_routes(backend, p, partial_bytes, error, &plan)) return false;
+  const uint32_t ksplit_tile = ksplit_route_tile(p, false);
+  if (!plan_routes(backend, p, partial_bytes, error, &plan, nullptr, 0, ksplit_tile ? ksplit_tile : kRouteTile))
+    return false;
   hipStream_t stream = backend_stream(backend);
   float *partial = (float *)plan.rest;
   QmmArgs a{};
@@ -1329,7 +1371,8 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
   a.split_below = backend_compute_units(backend) / 2;
   {
     KernelTimer timer(backend, FH_KC_MOE_KERNEL);
-    launch_routed<false>(stream, a, plan.max_blocks, backend_compute_units(backend));
+    if (!(ksplit_tile && launch_routed_ksplit(backend, a, false, plan.max_blocks, ksplit_tile)))
+      launch_routed<false>(stream, a, plan.max_blocks, backend_compute_units(backend));
   }
   uint64_t work = (uint64_t)p.rows * p.columns;
   auto row_view = [&](const View &v) {   // bf16 [rows, columns], 8-byte aligned row pieces

@@ -1,0 +1,619 @@
+// MLX-4bit affine quantised products over few activation rows: the wave-reduced GEMV of decode
+// batches (dense, at most 32 rows) and the routed products of a decode-sized MoE block (route
+// tiles of at most 32 rows per expert).  Same arithmetic as qmm_fast.hip:
+//   y[m,n] = sum_k x[m,k] * (scale[n,k/64] * q[n,k] + bias[n,k/64])      (affine_quant_dot,
+//   crates/forja-cpu/src/lib.rs:1277-1310), q = nibble k%8 of word k/8, low nibble first;
+// a nibble becomes the bf16 value 16+q, a 64-value group is contracted exactly in f32 on the
+// matrix cores, and scale and (bias - 16 scale) * sum(x) are applied per group.
+//
+// The work is HBM-bound on the packed weights and every weight is used for one 16- or 32-row
+// tile only, so the activations are the stationary operand: the waves of a workgroup split K
+// between them, each wave keeps ITS K slice of the tile's rows in registers (64 values per group
+// and row as two v_mfma_f32_16x16x32_bf16 A operands), loaded straight from memory in operand
+// layout, and streams the matching K slice of every weight row the workgroup owns.  Lane (column
+// n, quarter g) reads 16 bytes (half of one group, a quarter of a pair of groups) at a time, so a
+// wave's load covers 64 contiguous bytes of 16 weight rows: the narrowest access that still
+// reaches the read rate of a plain stream on this device (8-byte pieces stay 20 % below it).  Two
+// half-wave swaps (v_permlane32_swap) then sort the words by group.  Nothing is staged through
+// LDS and no barrier separates loading from computing; the waves' partial sums of a batch of
+// columns meet in LDS once per batch (one barrier, double buffered) and the waves share the
+// epilogue.
+//
+// What the instruction stream must not do, because it empties the ring of weight batches in
+// flight (each was measured): wait on a vector load that is younger than the ring (table words
+// are read as scalars; row ids are claimed where they are loaded), issue ring loads under a
+// branch, or leave the loop body through an exit that rejoins it -- the wait-count pass then
+// assumes the path with the fewest loads in flight and waits for all of them.
+//
+// Work units are (tile, batch of columns); a launch has as many workgroups as stay resident and
+// workgroup w takes the contiguous units [w U / W, (w+1) U / W): every workgroup streams the same
+// number of weight bytes to within one batch, whatever the number of tiles turns out to be on the
+// device.
+#include "fast_kernels.hpp"
+
+namespace fh {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kGroup = 64;
+constexpr uint32_t kNoBlock = 0xffffffffu;
+
+struct KsplitArgs {
+  const uint16_t *x;        // bf16 activations, innermost axis contiguous
+  uint64_t x_row_stride;    // elements between input rows
+  const uint32_t *packed[2];
+  const uint16_t *scales[2], *biases[2];
+  uint64_t expert_words;    // u32 words per expert matrix (N*K/8); 0 for dense
+  uint64_t expert_groups;   // scale entries per expert matrix (N*K/64)
+  void *out;                // bf16 or f32
+  uint64_t out_row_stride;  // elements
+  uint32_t out_f32;
+  const uint16_t *residual; // dense only: optional bf16 rows added before the result is rounded
+  uint64_t residual_row_stride;
+  uint32_t rows, inner, columns;
+  // routed form: tiles (expert, first, count) over sorted_routes; input row = route / route_div
+  const uint32_t *sorted_routes, *blocks, *n_blocks;
+  uint32_t route_div;
+  uint32_t batches_per_tile;
+};
+
+// A word the whole wave reads from a table no kernel writes while this one runs (the route plan):
+// read through the constant address space it becomes a scalar load, which is waited for on its own
+// counter.  As a vector load it would have to be waited for with vmcnt(0), i.e. together with every
+// batch of weights still in flight.
+__device__ inline uint32_t table_word(const uint32_t *table, uint32_t index) {
+  typedef const __attribute__((address_space(4))) uint32_t *constant_words;
+  return ((constant_words)(uintptr_t)table)[index];
+}
+
+__device__ inline uint32_t pack_bf16_pair(float lo, float hi) {
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ inline float bf16_bits(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+// (x & mask) | magic in one instruction (mask in a scalar register, magic in a vector register).
+__device__ inline uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
+  return r;
+}
+
+// Eight nibbles of `w` as bf16 (16+q) in slot order (0,4)(1,5)(2,6)(3,7).
+__device__ inline bf16x8 unpack_word(uint32_t w) {
+  const uint32_t mask = 0x00780078u, magic = 0x41804180u;
+  uint4 r;
+  r.x = and_or(w << 3, mask, magic);
+  r.y = and_or(w >> 1, mask, magic);
+  r.z = and_or(w >> 5, mask, magic);
+  r.w = and_or(w >> 9, mask, magic);
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+// The same slot order for eight consecutive activations.
+__device__ inline uint4 permute_slots(const uint4 &v) {
+  uint4 p;
+  p.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (x0, x4)
+  p.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (x1, x5)
+  p.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+  p.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+  return p;
+}
+
+__device__ inline float sum8(const uint4 &v) {
+  return bf16_bits(v.x & 0xffffu) + bf16_bits(v.x >> 16) + bf16_bits(v.y & 0xffffu) +
+         bf16_bits(v.y >> 16) + bf16_bits(v.z & 0xffffu) + bf16_bits(v.z >> 16) +
+         bf16_bits(v.w & 0xffffu) + bf16_bits(v.w >> 16);
+}
+
+// Element `index` (a per-lane value, 0..2*kWords-1) of bf16 values packed two to a word, as f32;
+// 0 beyond the words.
+template <int kWords>
+__device__ inline float packed_bf16_at(const uint32_t (&words)[kWords], uint32_t index) {
+  uint32_t word = 0;
+#pragma unroll
+  for (int i = 0; i < kWords; ++i)
+    if ((index >> 1) == (uint32_t)i) word = words[i];
+  return __uint_as_float((index & 1u) ? (word & 0xffff0000u) : (word << 16));
+}
+
+// WAVES waves split K; G = quantisation groups per wave (K = 64 * G * WAVES, G even);
+// RT = 16-row tiles of activations (the rows a weight is used for: 16 or 32).
+// 16-column tiles per batch and projection: a batch is 4 KiB of weights per wave (two
+// tile-projections of a four-group K slice, four of a two-group one), so that two batches fit
+// the registers beside the stationary rows.
+constexpr int batch_tiles(bool pair, int groups) { return (groups <= 2 ? 2 : 1) * (pair ? 1 : 2); }
+
+// Batches of weights a wave keeps requested ahead of its arithmetic: two, and three where the
+// stationary rows of a 32-row routed tile of a four-group K slice leave room for a single
+// workgroup per compute unit, whose eight waves alone must keep that unit's share of HBM busy.
+constexpr int ring_slots(int row_tiles, int groups, bool routed) { return row_tiles == 2 && groups > 2 && routed ? 3 : 2; }
+
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+
+// Waves per SIMD the registers must leave room for: two workgroups per compute unit where the
+// stationary rows are few (one contracts while the other waits at its exchange barrier).
+constexpr int resident_waves(int waves, int row_tiles, int groups, bool routed) {
+  const bool two = row_tiles == 1 ? groups <= 4 : groups <= 2 && waves <= 6 && routed;
+  return two ? (2 * waves + 3) / 4 : (waves + 3) / 4;
+}
+
+template <int WAVES, int G, int RT, bool kPair, bool kRouted>
+__global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) void qmm_ksplit_kernel(KsplitArgs a) {
+  constexpr int P = kPair ? 2 : 1;
+  constexpr int NS = ring_slots(RT, G, kRouted);
+  constexpr int CT = batch_tiles(kPair, G);
+  constexpr int kBatchCols = 16 * CT;
+  constexpr int Q = (G + 3) / 4;             // f32 matrix steps of the bias term (4 groups each)
+  constexpr int W2 = G / 2;                  // words of a lane's scales (or biases) of a column
+  constexpr int kSlots = P * CT * RT;        // 16 x 16 accumulator blocks of a wave and batch
+  constexpr int kQuads = CT * RT;            // blocks of results of a batch (both projections of a pair)
+  constexpr int QPW = (kQuads + WAVES - 1) / WAVES;     // blocks a wave finishes per batch
+  // With fewer blocks than waves the epilogue is dealt row by row instead (four times as many
+  // pieces), so that every wave takes part in it.
+  constexpr bool kWide = kQuads >= WAVES / 2;
+  constexpr int kTriples = kQuads * 4;       // (column tile, row tile, row) triples of a batch
+  constexpr int TPW = (kTriples + WAVES - 1) / WAVES;
+  constexpr int kShare = kWide ? QPW * 4 : TPW;         // results per lane this wave finishes per batch
+  extern __shared__ __attribute__((aligned(16))) float exchange[];   // f32x4 [2][WAVES][kSlots][64]
+  const uint32_t lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t words_per_row = a.inner / 8, groups_per_row = a.inner / kGroup;
+  const uint32_t tiles = kRouted ? table_word(a.n_blocks, 0) : 1;
+  const uint32_t units = tiles * a.batches_per_tile;
+  const uint32_t first_unit = (uint32_t)((uint64_t)blockIdx.x * units / gridDim.x);
+  const uint32_t last_unit = (uint32_t)((uint64_t)(blockIdx.x + 1) * units / gridDim.x);
+
+  // ---- the stationary operand: this wave's K slice of the current tile's rows.
+  // A lane reads 16 weight bytes (half a group) at a time, so that a wave's load covers 64
+  // contiguous bytes of each of 16 weight rows; two half-wave swaps then leave the lane quarters
+  // g = 0..3 holding words (0,4,2,6) and (1,5,3,7) of ONE group, and the activations are laid out
+  // to match: quarter g holds the group's values [16 g', 16 g' + 16), g' = (0,2,1,3)[g].
+  uint4 xa[RT][G][2];      // A operands: [row tile][group][half of the lane's 16 values]
+  float xs[RT][Q];         // sum of the row's activations over group 4q + g (bias term operand)
+  uint32_t out_rows[RT][4]; // output row of accumulator (row tile, i): tile row 16 rt + 4 g + i
+  uint32_t tile_first = 0, tile_count = 0, current_tile = kNoBlock;
+  const uint32_t g_perm = 2 * (g & 1) + (g >> 1);
+  auto load_tile = [&](uint32_t tile) {
+    current_tile = tile;
+    if (kRouted) {
+      const uint32_t expert = table_word(a.blocks, 3 * tile);
+      tile_first = expert == kNoBlock ? 0 : table_word(a.blocks, 3 * tile + 1);
+      tile_count = expert == kNoBlock ? 0 : table_word(a.blocks, 3 * tile + 2);
+    } else {
+      tile_count = a.rows;
+    }
+    // the rows this lane's accumulators belong to: fetched with the tile, not when a batch ends.
+    // Rows past the tile's count read the tile's first row (or row 0): their products are
+    // computed and never stored, which keeps this code free of branches.
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t row = 16 * rt + 4 * g + i;
+        out_rows[rt][i] = kRouted ? a.sorted_routes[tile_first + (row < tile_count ? row : 0)] : row;
+      }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const uint32_t row = 16 * rt + n;
+      const uint32_t safe = row < tile_count ? row : 0;
+      const uint64_t in_row = kRouted ? a.sorted_routes[tile_first + safe] / a.route_div : safe;
+      const uint16_t *xp = a.x + in_row * a.x_row_stride + (uint64_t)wave * (G * kGroup) + 16 * g_perm;
+      float sums[G];
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const uint4 lo = *(const uint4 *)(xp + kGroup * j), hi = *(const uint4 *)(xp + kGroup * j + 8);
+        float s = sum8(lo) + sum8(hi);
+        s += __shfl_xor(s, 16, 64);      // the four quarters of the group
+        s += __shfl_xor(s, 32, 64);
+        sums[j] = s;
+        xa[rt][j][0] = permute_slots(lo);
+        xa[rt][j][1] = permute_slots(hi);
+      }
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        float mine = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (4 * q + i < G && g == (uint32_t)i) mine = sums[4 * q + i];
+        xs[rt][q] = mine;
+      }
+      __builtin_amdgcn_sched_barrier(0);   // one row tile's loads in flight at a time (registers)
+    }
+    // The row ids are used when a batch ends; claim them here, so that the wait for them stands in
+    // this (rare) path and not, as a wait for everything in flight, at the end of every batch.
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(out_rows[rt][i]));
+  };
+
+  // ---- the streamed operand: one batch of columns, this wave's K slice.  Every load is issued
+  // unconditionally (addresses are clamped instead) so that the hardware counter a wave waits on
+  // before it touches a batch counts exactly the younger batches still in flight.
+  struct Batch {
+    uint4 w[P][CT][W2];         // the lane's 32 nibbles of each pair of groups
+    uint32_t s[P][CT][W2], b[P][CT][W2];   // the column's G scales and biases, two to a word
+    uint32_t residual[kShare];  // dense only: the values added to this wave's share of the results
+  };
+  // Where a stream of units stands: the loads run a ring ahead of the arithmetic, each with its own
+  // cursor, advanced without divisions; the expert of a tile is read when the cursor enters it.
+  struct Cursor {
+    uint32_t unit, tile, batch, expert;
+  };
+  auto expert_of = [&](uint32_t tile) -> uint32_t {
+    if (!kRouted) return 0;
+    const uint32_t expert = table_word(a.blocks, 3 * tile);
+    return expert == kNoBlock ? 0 : expert;
+  };
+  auto advance = [&](Cursor &c) {
+    if (c.unit + 1 >= last_unit) return;     // the loads past the end repeat the last unit
+    ++c.unit;
+    if (++c.batch == a.batches_per_tile) {
+      c.batch = 0;
+      ++c.tile;
+      c.expert = expert_of(c.tile);
+    }
+  };
+  // Byte offsets of this lane inside a 16-column tile of one expert matrix: the rest of an address
+  // is the same for the whole wave and stays in scalar registers.
+  const uint32_t lane_weight_bytes = (n * words_per_row + wave * (G * 8) + 4 * g) * 4;
+  const uint32_t lane_group_bytes = (n * groups_per_row + wave * G) * 2;
+  auto load_batch = [&](Batch &r, const Cursor &c) {
+    const uint32_t batch = c.batch;
+#pragma unroll
+    for (int pj = 0; pj < P; ++pj)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const uint64_t tile_column = batch * kBatchCols + 16 * ct;   // a multiple of 16 below a.columns
+        const uint64_t words = c.expert * a.expert_words + tile_column * words_per_row;
+        const uint64_t groups = c.expert * a.expert_groups + tile_column * groups_per_row;
+        const char *wp = (const char *)(a.packed[pj] + words) + lane_weight_bytes;
+        const char *sp = (const char *)(a.scales[pj] + groups) + lane_group_bytes;
+        const char *bp = (const char *)(a.biases[pj] + groups) + lane_group_bytes;
+#pragma unroll
+        for (int k = 0; k < W2; ++k) r.w[pj][ct][k] = *(const uint4 *)(wp + 64 * k);
+#pragma unroll
+        for (int i = 0; i < W2; ++i) {
+          r.s[pj][ct][i] = *(const uint32_t *)(sp + 4 * i);
+          r.b[pj][ct][i] = *(const uint32_t *)(bp + 4 * i);
+        }
+      }
+    if (!kRouted) {
+      if constexpr (kWide) {
+#pragma unroll
+        for (int qq = 0; qq < QPW; ++qq) {
+          const uint32_t quad = wave + qq * WAVES;
+          if (quad >= (uint32_t)kQuads) break;     // uniform: waves that finish no block load nothing
+          const uint32_t ct = quad / RT, rt = quad % RT;
+          const uint32_t column = min(batch * kBatchCols + 16 * ct + n, a.columns - 1);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t row = min(16 * rt + 4 * g + i, a.rows - 1);
+            const uint16_t *rp = a.residual ? a.residual + (uint64_t)row * a.residual_row_stride + column : a.x;
+            r.residual[4 * qq + i] = *rp;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int tt = 0; tt < TPW; ++tt) {
+          const uint32_t t = min(wave + tt * WAVES, (uint32_t)kTriples - 1);
+          const uint32_t ct = t / (RT * 4), rt = (t / 4) % RT, i = t % 4;
+          const uint32_t row = min(16 * rt + 4 * g + i, a.rows - 1);
+          const uint32_t column = min(batch * kBatchCols + 16 * ct + n, a.columns - 1);
+          const uint16_t *rp = a.residual ? a.residual + (uint64_t)row * a.residual_row_stride + column : a.x;
+          r.residual[tt] = *rp;
+        }
+      }
+    }
+  };
+
+  // Contracts the batch against the stationary rows, hands the partial sums to LDS buffer `buf`,
+  // and takes this wave's share of the epilogue.
+  auto finish_batch = [&](const Batch &r, uint32_t batch, uint32_t buf) {
+    f32x4 acc[P * CT][RT];
+    // bias term sum_j (bias_j - 16 scale_j) * xsum_j[row] first: an f32 matrix step over four
+    // groups, lane quarter g supplying group 4q + g of both operands
+#pragma unroll
+    for (int tp = 0; tp < P * CT; ++tp) {
+      const int pj = tp / CT, ct = tp % CT;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) acc[tp][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        const float shift = packed_bf16_at<W2>(r.b[pj][ct], 4 * q + g) -
+                            16.0f * packed_bf16_at<W2>(r.s[pj][ct], 4 * q + g);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          acc[tp][rt] = __builtin_amdgcn_mfma_f32_16x16x4f32(xs[rt][q], shift, acc[tp][rt], 0, 0, 0);
+      }
+    }
+    // the groups: each group's exact f32 sum is scaled into the accumulators one group late, so
+    // that the matrix unit's result is not waited for
+    f32x4 late[RT];
+    float late_scale = 0.0f;
+    u32x2 first_words = {0, 0}, second_words = {0, 0};
+#pragma unroll
+    for (int s = 0; s < P * CT * G; ++s) {
+      const int tp = s / G, j = s % G, pj = tp / CT, ct = tp % CT;
+      if (j % 2 == 0) {
+        const uint4 w = r.w[pj][ct][j / 2];
+        first_words = __builtin_amdgcn_permlane32_swap(w.x, w.z, false, false);
+        second_words = __builtin_amdgcn_permlane32_swap(w.y, w.w, false, false);
+      }
+      const bf16x8 b0 = unpack_word(first_words[j % 2]), b1 = unpack_word(second_words[j % 2]);
+      const uint32_t word = r.s[pj][ct][j / 2];
+      const float scale = __uint_as_float((j & 1) ? (word & 0xffff0000u) : (word << 16));
+      f32x4 part[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        part[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        part[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[rt][j][0]), b0, part[rt], 0, 0, 0);
+        part[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[rt][j][1]), b1, part[rt], 0, 0, 0);
+      }
+      if (s > 0) {
+        const int before = (s - 1) / G;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[before][rt][i] = __builtin_fmaf(late_scale, late[rt][i], acc[before][rt][i]);
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) late[rt] = part[rt];
+      late_scale = scale;
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc[P * CT - 1][rt][i] = __builtin_fmaf(late_scale, late[rt][i], acc[P * CT - 1][rt][i]);
+    // One result: activation of a pair, residual of a dense product, rounding, store.
+    auto store_result = [&](float value, float up, uint32_t out_row, uint32_t column, uint32_t residual_bits) {
+      if (kPair) value = value * (1.0f / (1.0f + __expf(-value))) * up;
+      if (!kRouted && a.residual) value += bf16_bits(residual_bits & 0xffffu);
+      const uint64_t at = (uint64_t)out_row * a.out_row_stride + column;
+      if (a.out_f32)
+        ((float *)a.out)[at] = value;
+      else
+        ((uint16_t *)a.out)[at] = (uint16_t)(pack_bf16_pair(value, 0.0f) & 0xffffu);
+    };
+    if constexpr (kWide) {
+      f32x4 *mine = (f32x4 *)exchange + ((uint64_t)(buf * WAVES + wave) * kSlots) * 64 + lane;
+#pragma unroll
+      for (int tp = 0; tp < P * CT; ++tp)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) mine[(tp * RT + rt) * 64] = acc[tp][rt];
+      __syncthreads();
+      // (column tile, row tile) blocks of 16 x 16 results are dealt round-robin to the waves; the
+      // owner adds the waves' sums in wave order (fixed: results do not depend on scheduling), four
+      // rows of a column to a lane
+#pragma unroll
+      for (int qq = 0; qq < QPW; ++qq) {
+        const int quad = (int)wave + qq * WAVES;
+        if (quad >= kQuads) break;
+        const int ct = quad / RT, rt = quad % RT;
+        f32x4 total[P];
+#pragma unroll
+        for (int pj = 0; pj < P; ++pj) {
+          const f32x4 *from = (const f32x4 *)exchange + ((uint64_t)(buf * WAVES) * kSlots + ((pj * CT + ct) * RT + rt)) * 64 + lane;
+          total[pj] = from[0];
+#pragma unroll
+          for (int v = 1; v < WAVES; ++v) total[pj] += from[(uint64_t)v * kSlots * 64];
+        }
+        const uint32_t column = batch * kBatchCols + 16 * ct + n;
+        if (column >= a.columns) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (16 * rt + 4 * g + i >= tile_count) continue;
+          uint32_t out_row = out_rows[0][i];
+#pragma unroll
+          for (int r2 = 1; r2 < RT; ++r2)
+            if (r2 == rt) out_row = out_rows[r2][i];
+          store_result(total[0][i], total[P - 1][i], out_row, column, kRouted ? 0 : r.residual[4 * qq + i]);
+        }
+      }
+    } else {
+      float *mine = exchange + ((uint64_t)(buf * WAVES + wave) * kSlots * 4) * 64 + lane;
+#pragma unroll
+      for (int tp = 0; tp < P * CT; ++tp)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mine[((tp * RT + rt) * 4 + i) * 64] = acc[tp][rt][i];
+      __syncthreads();
+      // (column tile, row tile, row) triples are dealt round-robin to the waves, one result to a lane
+#pragma unroll
+      for (int tt = 0; tt < TPW; ++tt) {
+        const int t = (int)wave + tt * WAVES;
+        if (t >= kTriples) break;
+        const int ct = t / (RT * 4), rt = (t / 4) % RT, i = t % 4;
+        float total[P];
+#pragma unroll
+        for (int pj = 0; pj < P; ++pj) {
+          const float *from = exchange + ((uint64_t)(buf * WAVES) * kSlots * 4 + (((pj * CT + ct) * RT + rt) * 4 + i)) * 64 + lane;
+          total[pj] = from[0];
+#pragma unroll
+          for (int v = 1; v < WAVES; ++v) total[pj] += from[(uint64_t)v * kSlots * 4 * 64];
+        }
+        const uint32_t row = 16 * rt + 4 * g + i, column = batch * kBatchCols + 16 * ct + n;
+        if (row >= tile_count || column >= a.columns) continue;
+        uint32_t out_row = 0;   // out_rows[rt][i], picked without indexing registers dynamically
+#pragma unroll
+        for (int r2 = 0; r2 < RT; ++r2)
+#pragma unroll
+          for (int i2 = 0; i2 < 4; ++i2)
+            if (r2 == rt && i2 == i) out_row = out_rows[r2][i2];
+        store_result(total[0], total[P - 1], out_row, column, kRouted ? 0 : r.residual[tt]);
+      }
+    }
+  };
+
+  if (first_unit >= last_unit) return;
+  Cursor loading{first_unit, first_unit / a.batches_per_tile, first_unit % a.batches_per_tile, 0};
+  loading.expert = expert_of(loading.tile);
+  Cursor computing = loading;
+  Batch ring[NS];
+#pragma unroll
+  for (int slot = 0; slot < NS; ++slot) {
+    load_batch(ring[slot], loading);
+    advance(loading);
+  }
+  if (!kRouted) load_tile(0);
+  // Whole rounds of the ring first, in a loop without exits in its body (an exit that rejoins the
+  // loop would make every wait assume the shortest path, i.e. drain the ring); the last, partial
+  // round is a copy of the body that requests nothing.
+  uint32_t base = first_unit, buf = 0;
+  for (; base + NS <= last_unit; base += NS) {
+#pragma unroll
+    for (int slot = 0; slot < NS; ++slot) {
+      if (kRouted && computing.tile != current_tile) load_tile(computing.tile);
+      finish_batch(ring[slot], computing.batch, buf);
+      buf ^= 1u;
+      load_batch(ring[slot], loading);
+      advance(loading);
+      advance(computing);
+    }
+  }
+#pragma unroll
+  for (int slot = 0; slot < NS - 1; ++slot) {
+    if (base + slot >= last_unit) break;
+    if (kRouted && computing.tile != current_tile) load_tile(computing.tile);
+    finish_batch(ring[slot], computing.batch, buf);
+    buf ^= 1u;
+    advance(computing);
+  }
+}
+
+// How K is split: waves and groups per wave; false when this K has no instantiation.
+bool ksplit_shape(uint32_t inner, int *waves, int *groups) {
+  switch (inner) {
+  case 512: *waves = 4, *groups = 2; return true;
+  case 768: *waves = 6, *groups = 2; return true;
+  case 1024: *waves = 8, *groups = 2; return true;
+  case 1536: *waves = 6, *groups = 4; return true;
+  case 2048: *waves = 8, *groups = 4; return true;
+  case 3072: *waves = 8, *groups = 6; return true;
+  case 4096: *waves = 8, *groups = 8; return true;
+  default: return false;
+  }
+}
+
+// One launch: as many workgroups as stay resident at once (the runtime's own occupancy figure for
+// this instantiation), never more than there are units of work.
+template <int WAVES, int G, int RT, bool kPair, bool kRouted>
+void launch_one(fh_backend *backend, const KsplitArgs &a, uint64_t most_units) {
+  constexpr int P = kPair ? 2 : 1, CT = batch_tiles(kPair, G);
+  constexpr uint32_t lds = 2u * WAVES * (CT * P * RT * 4) * 64 * sizeof(float);
+  const void *kernel = reinterpret_cast<const void *>(&qmm_ksplit_kernel<WAVES, G, RT, kPair, kRouted>);
+  static int per_unit = 0;   // set once per process: the dynamic LDS limit and the occupancy
+  if (per_unit == 0) {
+    (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    int blocks = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, 64 * WAVES, lds) != hipSuccess || blocks < 1)
+      blocks = 1;
+    per_unit = blocks > 2 ? 2 : blocks;
+  }
+  const uint64_t resident = (uint64_t)backend_compute_units(backend) * (uint32_t)per_unit;
+  const uint32_t grid = (uint32_t)(most_units < resident ? most_units : resident);
+  qmm_ksplit_kernel<WAVES, G, RT, kPair, kRouted><<<dim3(grid), 64 * WAVES, lds, backend_stream(backend)>>>(a);
+}
+
+template <int RT, bool kPair, bool kRouted>
+bool launch_shape(fh_backend *backend, const KsplitArgs &a, uint64_t most_units) {
+  int waves = 0, groups = 0;
+  if (!ksplit_shape(a.inner, &waves, &groups)) return false;
+  switch (waves * 16 + groups) {
+  case 4 * 16 + 2: launch_one<4, 2, RT, kPair, kRouted>(backend, a, most_units); return true;
+  case 6 * 16 + 2: launch_one<6, 2, RT, kPair, kRouted>(backend, a, most_units); return true;
+  case 8 * 16 + 2: launch_one<8, 2, RT, kPair, kRouted>(backend, a, most_units); return true;
+  case 6 * 16 + 4: launch_one<6, 4, RT, kPair, kRouted>(backend, a, most_units); return true;
+  case 8 * 16 + 4: launch_one<8, 4, RT, kPair, kRouted>(backend, a, most_units); return true;
+  default: break;
+  }
+  if constexpr (RT == 1 && !kRouted) {   // the long rows of dense decode products
+    if (waves == 8 && groups == 6) {
+      launch_one<8, 6, 1, false, false>(backend, a, most_units);
+      return true;
+    }
+    if (waves == 8 && groups == 8) {
+      launch_one<8, 8, 1, false, false>(backend, a, most_units);
+      return true;
+    }
+  }
+  return false;
+}
+
+}  // namespace
+
+bool ksplit_supports(uint32_t inner, uint32_t columns, bool pair, bool routed) {
+  int waves, groups;
+  if (!ksplit_shape(inner, &waves, &groups) || (routed && groups > 4)) return false;
+  return columns % (16u * batch_tiles(pair, groups)) == 0;   // whole batches of columns only
+}
+
+bool launch_ksplit_dense(fh_backend *backend, const KsplitDense &d) {
+  int waves = 0, groups = 0;
+  if (d.rows == 0 || d.rows > 32 || !ksplit_shape(d.inner, &waves, &groups)) return false;
+  if (!ksplit_supports(d.inner, d.columns, false, false)) return false;
+  if (d.rows > 16 && groups > 4) return false;   // two row tiles of that many groups do not fit
+  KsplitArgs a{};
+  a.x = d.x;
+  a.x_row_stride = d.x_row_stride;
+  a.packed[0] = d.packed;
+  a.scales[0] = d.scales;
+  a.biases[0] = d.biases;
+  a.out = d.out;
+  a.out_row_stride = d.out_row_stride;
+  a.out_f32 = d.out_f32;
+  a.residual = d.residual;
+  a.residual_row_stride = d.residual_row_stride;
+  a.rows = d.rows;
+  a.inner = d.inner;
+  a.columns = d.columns;
+  const uint32_t batch_cols = 16 * batch_tiles(false, groups);
+  a.batches_per_tile = (d.columns + batch_cols - 1) / batch_cols;
+  KernelTimer timer(backend, FH_KC_QMM_KERNEL);
+  return d.rows <= 16 ? launch_shape<1, false, false>(backend, a, a.batches_per_tile)
+                      : launch_shape<2, false, false>(backend, a, a.batches_per_tile);
+}
+
+bool launch_ksplit_routed(fh_backend *backend, const KsplitRouted &r) {
+  int waves = 0, groups = 0;
+  if ((r.tile_rows != 16 && r.tile_rows != 32) || !ksplit_shape(r.inner, &waves, &groups)) return false;
+  if (!ksplit_supports(r.inner, r.columns, r.pair, true)) return false;
+  if (groups > 4) return false;
+  KsplitArgs a{};
+  a.x = r.x;
+  a.x_row_stride = r.x_row_stride;
+  for (int pj = 0; pj < (r.pair ? 2 : 1); ++pj) {
+    a.packed[pj] = r.packed[pj];
+    a.scales[pj] = r.scales[pj];
+    a.biases[pj] = r.biases[pj];
+  }
+  a.expert_words = (uint64_t)r.columns * r.inner / 8;
+  a.expert_groups = (uint64_t)r.columns * r.inner / kGroup;
+  a.out = r.out;
+  a.out_row_stride = r.columns;
+  a.out_f32 = r.out_f32;
+  a.inner = r.inner;
+  a.columns = r.columns;
+  a.sorted_routes = r.sorted_routes;
+  a.blocks = r.blocks;
+  a.n_blocks = r.n_blocks;
+  a.route_div = r.route_div;
+  const uint32_t batch_cols = 16 * batch_tiles(r.pair, groups);
+  a.batches_per_tile = (r.columns + batch_cols - 1) / batch_cols;
+  const uint64_t most = (uint64_t)r.max_blocks * a.batches_per_tile;
+  if (r.pair)
+    return r.tile_rows == 16 ? launch_shape<1, true, true>(backend, a, most)
+                             : launch_shape<2, true, true>(backend, a, most);
+  return r.tile_rows == 16 ? launch_shape<1, false, true>(backend, a, most)
+                           : launch_shape<2, false, true>(backend, a, most);
+}
+
+}  // namespace fh

@@ -140,6 +140,7 @@ struct fh_submission {
   ErrorSlot *device_errors = nullptr;
   ErrorSlot *host_errors = nullptr;  // pinned
   hipEvent_t start = nullptr, end = nullptr;
+  hipEvent_t done = nullptr;   // recorded behind the copy of the error records: this submission's completion
   bool waited = false;
   fh_status result = FH_OK;
   fh_error error{};
@@ -1674,9 +1675,10 @@ void recycle_submission(fh_backend *b, fh_submission *s) {
     b->error_pool.push_back({s->device_errors, s->host_errors, s->error_capacity});
   if (s->start) b->event_pool.push_back(s->start);
   if (s->end) b->event_pool.push_back(s->end);
+  if (s->done) b->event_pool.push_back(s->done);
   s->device_errors = nullptr;
   s->host_errors = nullptr;
-  s->start = s->end = nullptr;
+  s->start = s->end = s->done = nullptr;
 }
 
 void drain_profile(fh_backend *b) {
@@ -1748,6 +1750,7 @@ void fh_destroy(fh_backend *b) {
       (void)hipHostFree(s->host_errors);
       (void)hipEventDestroy(s->start);
       (void)hipEventDestroy(s->end);
+      (void)hipEventDestroy(s->done);
       s->device_errors = nullptr;
       s->host_errors = nullptr;
     }
@@ -2048,6 +2051,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   }
   s->start = take_event(b);
   s->end = take_event(b);
+  s->done = take_event(b);
   b->route_plan_valid = false;  // host writes between submissions are not tracked
   b->attention_plan_valid = false;
   launch_init_errors(b->stream, s->device_errors, slots);
@@ -2098,6 +2102,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   (void)hipEventRecord(s->end, b->stream);
   (void)hipMemcpyAsync(s->host_errors, s->device_errors, slots * sizeof(ErrorSlot),
                        hipMemcpyDeviceToHost, b->stream);
+  (void)hipEventRecord(s->done, b->stream);
   if (status != FH_OK) {
     (void)hipStreamSynchronize(b->stream);
     recycle_submission(b, s);
@@ -2229,8 +2234,9 @@ fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
     s->result = FH_EXECUTION_FAILED;
   }
   if (!s->waited) {
-    // The trailing async copy of the error slots is the last work of the submission; a pinned
-    // target makes stream synchronisation the completion point.
+    // The event behind the trailing copy of the error records is this submission's completion
+    // (Submission::wait is per submission, crates/forja-core/src/backend.rs:609-647): work
+    // submitted later neither delays the wait nor counts against its deadline.
     if (timeout_ns != 0) {
       auto deadline = std::chrono::steady_clock::now() + std::chrono::nanoseconds(timeout_ns);
       for (;;) {
@@ -2238,7 +2244,7 @@ fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
         {
           std::lock_guard<std::mutex> lock(b->mutex);
           (void)hipSetDevice(b->device);
-          q = hipStreamQuery(b->stream);
+          q = hipEventQuery(s->done);
         }
         if (q == hipSuccess) break;
         if (q != hipErrorNotReady) {
@@ -2256,9 +2262,14 @@ fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
         std::this_thread::sleep_for(std::chrono::microseconds(50));
       }
     }
+    // Waiting happens outside the backend's mutex, so that other threads keep submitting.
+    {
+      std::lock_guard<std::mutex> lock(b->mutex);
+      (void)hipSetDevice(b->device);
+    }
+    hipError_t sync = hipEventSynchronize(s->done);
     std::lock_guard<std::mutex> lock(b->mutex);
     (void)hipSetDevice(b->device);
-    hipError_t sync = hipStreamSynchronize(b->stream);
     s->waited = true;
     if (sync != hipSuccess) {
       s->result = FH_DEVICE_EXECUTION_FAILED;
@@ -2275,7 +2286,10 @@ fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
         break;
       }
     }
-    if (b->profiling) drain_profile(b);
+    if (b->profiling) {   // the timers of later submissions must have run out before they are read
+      (void)hipStreamSynchronize(b->stream);
+      drain_profile(b);
+    }
   }
   if (error) {
     *error = s->error;
@@ -2299,7 +2313,7 @@ void fh_submission_free(fh_submission *s) {
   {
     std::lock_guard<std::mutex> lock(b->mutex);
     (void)hipSetDevice(b->device);
-    if (!s->waited) (void)hipStreamSynchronize(b->stream);
+    if (!s->waited) (void)hipEventSynchronize(s->done);
     b->submissions.erase(s);
     recycle_submission(b, s);
   }

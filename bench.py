@@ -23,17 +23,29 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+from forja_amd import cost as costs  # noqa: E402
 from forja_amd.core import CommandList, DType, Op  # noqa: E402
 from forja_amd.hip_backend import HipBackend  # noqa: E402
 from forja_amd.model import (QWEN3_CODER_30B_A3B, QWEN3_0_6B, DecodeSession, Model,  # noqa: E402
                              ModelConfig)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes moved by ragged_attention_mfma_kernel per algorithmic byte on this workload, from the
-# hardware counters: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over the same launches, each
-# scaled by what the counter reads for a 1 GiB copy (FETCH_SIZE counts half of it, WRITE_SIZE all
-# of it); figures and commands in profiles/c3_decode_step_hbm_traffic.txt.
-ATTENTION_TRAFFIC_RATIO = 1.019
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "c3_decode_step_hbm_traffic.txt")
+
+
+def measured_traffic_ratio():
+    """HBM bytes moved by ragged_attention_mfma_kernel per algorithmic byte on the timed workload,
+    as the hardware counters gave it (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over the same
+    launches, each scaled by what the counter reads for a 1 GiB copy): read from the tracked
+    summary of that measurement.  None when the summary is not there."""
+    import re
+    try:
+        match = re.search(r"ratio ([0-9.]+)", open(TRAFFIC_SUMMARY).read())
+    except OSError:
+        return None
+    return float(match.group(1)) if match else None
+
+
 KC_ATTENTION, KC_MOE, KC_QMM = 3, 2, 1
 KC_ATTENTION_KERNEL, KC_MOE_KERNEL, KC_QMM_KERNEL = 4, 5, 6
 
@@ -46,7 +58,7 @@ class Workload:
     """Config 3: 128 decode lanes, 8 retire + 8 admit per step."""
 
     def __init__(self, backend, config: ModelConfig, lanes, ctx_lo, ctx_hi, churn, seed, layers=None,
-                 capacity_factor=1.45):
+                 capacity_factor=1.45, router_noise_seed=None):
         self.rng = np.random.default_rng(seed)
         self.lanes, self.ctx_lo, self.ctx_hi, self.churn = lanes, ctx_lo, ctx_hi, churn
         contexts = log_uniform(self.rng, ctx_lo, ctx_hi, lanes)
@@ -57,7 +69,7 @@ class Workload:
         table_pages = (ctx_hi + 4096 + pt) // pt
         self.model = Model(backend, config, seed=seed, layers=layers)
         self.session = DecodeSession(self.model, contexts, seed=seed, physical_pages=self.capacity_pages,
-                                     table_pages=table_pages)
+                                     table_pages=table_pages, router_noise_seed=router_noise_seed)
         self.next_lane = 0
 
     def churn_lanes(self):
@@ -79,14 +91,37 @@ class Workload:
             s.cache.upload_tables([lane])
 
 
-def algorithmic_bytes(workload, contexts):
-    """Logical bytes of a step: every K/V row read once per kv head, weights with their scales and
-    biases (the accounting of crates/forja-core/src/cost/attention.rs:5-90 and cost.rs:111-153)."""
-    model = workload.model
-    c = model.config
-    kv = int((contexts + 1).sum()) * (model.n_layers * 2 * c.kv_heads * c.head_dim * 2)
-    weights = model.weight_bytes_per_step(len(contexts))
-    return kv, weights
+def attention_launch_cost(config, contexts):
+    """Logical work of one layer's decode attention over lanes at `contexts` (one new row each), by
+    the reference's accounting (crates/forja-core/src/cost/attention.rs:5-129): K/V rows once per
+    kv head, query and output rows, the appended rows, 12 bytes per page touched."""
+    width = config.head_dim
+    pool_bytes = config.kv_dtype.byte_size
+    return costs.ragged_attention_cost(config.q_heads, config.kv_heads, width, width, [1] * len(contexts),
+                                       [int(v) for v in contexts], config.page_tokens,
+                                       config.activation_dtype.byte_size, pool_bytes)
+
+
+def step_costs(model, buffers_session, distinct_experts=None):
+    """Logical traffic of the weights one decode step reads, dispatch by dispatch
+    (crates/forja-core/src/cost.rs:111-153, cost/routed.rs:19-91): dense products with scales and
+    biases; routed products at `distinct_experts` experts per layer when given, else at the
+    reference's bounds (minimum: top-k experts, maximum: min(experts, routes))."""
+    dense = routed_min = routed_max = routed_seen = 0
+    for dispatch in buffers_session.commands.dispatches:
+        cost = costs.of(dispatch)
+        if cost is None:
+            continue
+        if cost.maximum_weight_bytes:
+            routed_min += costs.traffic(cost, True)
+            routed_max += costs.traffic(cost, False)
+            if distinct_experts is not None:
+                seen = costs.distinct_expert_traffic(dispatch, int(round(distinct_experts)))
+                routed_seen += seen if seen is not None else costs.traffic(cost, False)
+        elif cost.weight_bytes:
+            dense += costs.traffic(cost, True)
+    return {"dense": dense, "routed_minimum": routed_min, "routed_maximum": routed_max,
+            "routed_seen": routed_seen if distinct_experts is not None else None}
 
 
 def cpu_baseline(config, seed, sample_lanes, ctx_lo, ctx_hi):
@@ -521,6 +556,63 @@ def decode_attention_f16_cache(backend, config, seed=99, repeats=5):
             "algorithmic_bytes": kv_bytes, "achieved_gbps": gbps, "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS}
 
 
+def decode_gemv(backend, model, row_counts=(1, 4, 8), seed=83):
+    """The quantised GEMV of small decode batches (the reference's own regime: at most 8 lanes),
+    product by product on cold weights: every layer's stacked qkv and o_proj in turn, and lm_head
+    over four copies of its weights (one copy fits the 256 MB of cache in front of HBM).  Times
+    are device time of back-to-back launches (one submission, no timers between them); bytes are
+    the reference's logical traffic of the dispatch (weights with scales and biases, rows in and
+    out)."""
+    from forja_amd.model import QuantLinear
+    c = model.config
+    heads = [model.lm_head]
+    fill = CommandList()
+    for copy in range(3):
+        extra = QuantLinear(backend, c.vocab, c.hidden)
+        extra.fill(fill, seed, 40 + 3 * copy)
+        heads.append(extra)
+    backend.submit(fill).wait()
+    groups = [("qkv", [layer.qkv for layer in model.layers]),
+              ("o_proj", [layer.o_proj for layer in model.layers]),
+              ("lm_head", heads)]
+    q4 = Op.quant_matmul(4, 64)
+    results = {}
+    for rows in row_counts:
+        per_product = {}
+        for name, linears in groups:
+            x = backend.alloc(DType.BF16, (rows, linears[0].k))
+            out = backend.alloc(DType.BF16, (rows, linears[0].n))
+            fill = CommandList()
+            fill.dispatch(Op.fill_seeded(2, seed, 60), [], x)
+            backend.submit(fill).wait()
+            commands = CommandList()
+            for linear in linears:
+                commands.dispatch(q4, [x, *linear.triple], out)
+            encoded = backend.encode(commands)
+            backend.submit(encoded).wait()
+            nanoseconds, repeats = 0, 3
+            for _ in range(repeats):
+                submission = backend.submit(encoded)
+                submission.wait()
+                nanoseconds += submission.gpu_time_ns()
+                submission.free()
+            per_launch = nanoseconds / repeats / len(linears)
+            logical = costs.traffic(costs.of(commands.dispatches[0]), True)
+            per_product[name] = {"n": linears[0].n, "k": linears[0].k, "us": per_launch / 1e3,
+                                 "logical_mb": logical / 1e6,
+                                 "achieved_gbps": logical / per_launch,
+                                 "frac_of_hbm_peak": logical / per_launch / HBM_PEAK_GBPS}
+            backend.release(x)
+            backend.release(out)
+        results["rows_%d" % rows] = per_product
+    for linear in heads[1:]:
+        for tensor in linear.triple:
+            backend.release(tensor)
+    results["workload"] = ("dense 4-bit products of a decode batch of 1, 4 and 8 rows at the timed model's "
+                           "shapes, cold weights, back-to-back launches")
+    return results
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -539,6 +631,12 @@ def main():
                         help="skip the HIP-event kernel timing inside the timed region")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only run the config 4 prefill projection measurement and exit")
+    parser.add_argument("--gemv-only", action="store_true",
+                        help="only run the small-batch GEMV measurement (on --layers layers, default 8) "
+                             "and exit")
+    parser.add_argument("--moe-only", action="store_true",
+                        help="only run the config 2 MoE block measurement (on --layers layers' "
+                             "experts, default 8) and exit")
     parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                         help="only run 8 plain copies of MIB mebibytes (a known-size kernel to "
                              "scale hardware traffic counters by) and exit")
@@ -554,6 +652,16 @@ def main():
             backend.submit(commands).wait()
         print(json.dumps({"copy_bytes_read": elements * 4, "copy_bytes_written": elements * 4,
                           "kernel": "copy_flat_kernel", "launches": 8}))
+        return
+    if args.gemv_only:
+        backend = HipBackend(0)
+        model = Model(backend, QWEN3_CODER_30B_A3B, seed=args.seed, layers=args.layers or 8)
+        print(json.dumps({"decode_gemv": decode_gemv(backend, model)}))
+        return
+    if args.moe_only:
+        backend = HipBackend(0)
+        model = Model(backend, QWEN3_CODER_30B_A3B, seed=args.seed, layers=args.layers or 8)
+        print(json.dumps({"moe_block_c2": moe_block_c2(backend, model)}))
         return
     if args.prefill_only:
         backend = HipBackend(0)
@@ -573,41 +681,68 @@ def main():
     default_workload = args.layers is None and args.lanes == 128 and args.seed == 20261
     backend = HipBackend(0)
     info = backend.device_info()
-    workload = Workload(backend, config, args.lanes, ctx_lo, ctx_hi, churn, args.seed, layers=args.layers)
+    # Config 3 routes "as in config 2": top-8 of the softmax of N(0,1) router logits, seeded per
+    # layer.  (Under the prescribed weight law alone every token picks the same few experts; that
+    # variant is reported beside the headline as `c3_weight_law_routing`.)
+    workload = Workload(backend, config, args.lanes, ctx_lo, ctx_hi, churn, args.seed, layers=args.layers,
+                        router_noise_seed=args.seed + 1)
     session = workload.session
+    n_layers = workload.model.n_layers
     backend.synchronize()
 
-    def run_step():
+    def run_step(encoded=None):
         contexts = session.contexts.copy()
-        submission = session.submit_step()
+        submission = session.submit_step(encoded)
         workload.churn_lanes()
         return submission, contexts
 
-    for _ in range(args.warmup):
-        submission, _ = run_step()
-        submission.wait()
-        submission.free()
-    backend.synchronize()
+    def timed_steps(count, encoded=None, on_step=None):
+        backend.synchronize()
+        started = time.perf_counter()
+        submissions = []
+        for _ in range(count):
+            submission, contexts = run_step(encoded)
+            if on_step:
+                on_step(contexts)
+            submissions.append(submission)
+        backend.synchronize()
+        elapsed = time.perf_counter() - started
+        device_ns = 0
+        for submission in submissions:
+            submission.wait()            # surfaces any device error flag
+            device_ns += submission.gpu_time_ns()
+            submission.free()
+        return elapsed, device_ns
+
+    def traced_distinct_experts(router_noise_seed):
+        """Distinct experts per layer on one more (untimed) step that copies out every layer's
+        choices: the routed kernels read the weights of the experts chosen, nothing else."""
+        from forja_amd.model import record_step
+        trace = backend.alloc(DType.U32, (n_layers, args.lanes, config.top_k))
+        traced = CommandList()
+        record_step(workload.model, session.cache, session.buffers, traced, feed_back=True,
+                    route_trace=trace, one_row_per_lane=True, router_noise_seed=router_noise_seed)
+        session.prepare_step()
+        backend.submit(traced).wait()
+        session.contexts += 1
+        chosen = np.frombuffer(backend.read(trace), np.uint32).reshape(n_layers, args.lanes * config.top_k)
+        backend.release(trace)
+        return np.array([len(np.unique(layer)) for layer in chosen])
+
+    timed_steps(args.warmup)
     if not args.no_profile:
         # inside the timed region only the dominant kernel is timed (two event records per launch)
         backend.profile_select(1 << KC_ATTENTION_KERNEL)
         backend.profile_enable(1)
         backend.profile_reset()
 
-    kv_bytes_total, submissions = 0, []
-    backend.synchronize()
-    started = time.perf_counter()
-    for _ in range(args.steps):
-        submission, contexts = run_step()
-        kv_bytes_total += algorithmic_bytes(workload, contexts)[0]
-        submissions.append(submission)
-    backend.synchronize()
-    elapsed = time.perf_counter() - started
-    device_ns = 0
-    for submission in submissions:
-        submission.wait()            # surfaces any device error flag
-        device_ns += submission.gpu_time_ns()
-        submission.free()
+    attention = {"bytes": 0, "kv_bytes": 0}
+
+    def account(contexts):
+        launch = attention_launch_cost(config, contexts)
+        attention["bytes"] += costs.traffic(launch, True) * n_layers
+        attention["kv_bytes"] += launch.kv_bytes * n_layers
+    elapsed, device_ns = timed_steps(args.steps, on_step=account)
 
     tokens = args.lanes * args.steps
     result = {
@@ -619,27 +754,29 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": ("BASELINE config 3: Qwen3-Coder-30B-A3B-shaped full model, "
-                         f"{workload.model.n_layers} layers, MLX-4bit random weights, {args.lanes} decode "
+                         f"{n_layers} layers, MLX-4bit random weights, {args.lanes} decode "
                          f"lanes, contexts log-uniform {ctx_lo}-{ctx_hi}, paged bf16 KV page 16, "
-                         f"non-contiguous block tables, {churn} retire+admit per step"),
-            "lanes": args.lanes, "layers": workload.model.n_layers, "page_tokens": config.page_tokens,
+                         f"non-contiguous block tables, {churn} retire+admit per step, MoE routed as "
+                         "in config 2 (top-8 of softmax of seeded N(0,1) router logits)"),
+            "lanes": args.lanes, "layers": n_layers, "page_tokens": config.page_tokens,
             "dispatches_per_step": session.dispatches, "device": info["family"],
         },
     }
-    weights = workload.model.weight_bytes_per_step(args.lanes)
-    kv_per_step = kv_bytes_total / args.steps
-    routed_fraction = 1.0
+    attention_per_step = attention["bytes"] / args.steps
+    distinct = None
     if not args.no_profile:
         ns, launches = backend.profile_read(KC_ATTENTION_KERNEL)
-        kernel_bytes = kv_bytes_total / max(launches, 1)          # per launch = per layer per step
+        kernel_bytes = attention["bytes"] / max(launches, 1)          # per launch = per layer per step
         average = ns / max(launches, 1) * 1e-9
         achieved = kernel_bytes / average / 1e9 if average > 0 else 0.0
+        ratio = measured_traffic_ratio() if default_workload else None
         result["roofline"] = {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": kernel_bytes * ATTENTION_TRAFFIC_RATIO if default_workload else None,
+            "traffic": kernel_bytes * ratio if ratio else None,
             "kernel": "ragged_attention_mfma_kernel", "launches": launches,
             "avg_launch_us": average * 1e6, "algorithmic_bytes_per_launch": kernel_bytes,
+            "kv_bytes_per_launch": attention["kv_bytes"] / max(launches, 1),
         }
         # Secondary kernels from a few extra steps with every kernel class timed, then a per-op
         # breakdown with every dispatch timed (neither is part of `value`).
@@ -654,34 +791,21 @@ def main():
         qmm_ns, qmm_launches = backend.profile_read(KC_QMM_KERNEL)
         secondary = {}
         if moe_launches:
-            # one more (untimed) step that also copies out every layer's expert choices: the
-            # routed kernels read the weights of the DISTINCT experts chosen, nothing else
-            from forja_amd.model import record_step
-            trace = backend.alloc(DType.U32, (workload.model.n_layers, args.lanes, config.top_k))
-            traced = CommandList()
-            record_step(workload.model, session.cache, session.buffers, traced, feed_back=True,
-                        route_trace=trace, one_row_per_lane=True)
-            session.prepare_step()
-            backend.submit(traced).wait()
-            session.contexts += 1
-            chosen = np.frombuffer(backend.read(trace), np.uint32).reshape(
-                workload.model.n_layers, args.lanes * config.top_k)
-            distinct = np.array([len(np.unique(layer)) for layer in chosen])
-            fraction = float(distinct.mean()) / config.experts
-            moe_bytes = weights["routed_all_experts"] * fraction * secondary_steps / moe_launches
-            secondary["routed_qmm_mfma_kernel"] = {
+            distinct = traced_distinct_experts(session.router_noise_seed)
+            weights = step_costs(workload.model, session, float(distinct.mean()))
+            moe_bytes = weights["routed_seen"] * secondary_steps / moe_launches
+            secondary["routed_qmm_kernel"] = {
                 "avg_launch_us": moe_ns / moe_launches / 1e3,
                 "achieved_gbps": moe_bytes / (moe_ns / moe_launches * 1e-9) / 1e9,
                 "frac": moe_bytes / (moe_ns / moe_launches * 1e-9) / 1e9 / HBM_PEAK_GBPS,
                 "distinct_experts_per_layer": {"mean": float(distinct.mean()),
                                                "min": int(distinct.min()), "max": int(distinct.max()),
                                                "of": config.experts},
-                "note": ("bytes = weights of the distinct experts the router chose (measured on "
-                         "one traced step), per projection launch")}
-            routed_fraction = fraction
+                "note": ("bytes = logical traffic of the routed products at the distinct experts the "
+                         "router chose (measured on one traced step), per projection launch")}
         if qmm_launches:
-            qmm_bytes = weights["dense"] * secondary_steps / qmm_launches
-            secondary["dense_qmm_mfma_kernel"] = {
+            qmm_bytes = step_costs(workload.model, session)["dense"] * secondary_steps / qmm_launches
+            secondary["dense_qmm_kernel"] = {
                 "avg_launch_us": qmm_ns / qmm_launches / 1e3,
                 "achieved_gbps": qmm_bytes / (qmm_ns / qmm_launches * 1e-9) / 1e9,
                 "frac": qmm_bytes / (qmm_ns / qmm_launches * 1e-9) / 1e9 / HBM_PEAK_GBPS}
@@ -700,6 +824,29 @@ def main():
             breakdown[name] = class_ns / 1e6 / extra
         result["gpu_ms_per_step_by_op"] = breakdown
         backend.profile_enable(0)
+    weights = step_costs(workload.model, session, float(distinct.mean()) if distinct is not None else None)
+    routed = weights["routed_seen"] if weights["routed_seen"] is not None else weights["routed_maximum"]
+    step_bytes = attention_per_step + weights["dense"] + routed
+    result["step_algorithmic_gb"] = step_bytes / 1e9
+    result["step_algorithmic_gb_by_part"] = {"attention": attention_per_step / 1e9, "dense_products": weights["dense"] / 1e9,
+                                            "routed_products": routed / 1e9,
+                                            "routed_products_reference_bounds": [weights["routed_minimum"] / 1e9,
+                                                                                 weights["routed_maximum"] / 1e9]}
+    result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS
+    if not args.no_profile:
+        if config.moe:
+            # The same step with the routing the prescribed weights give by themselves.
+            plain = session.encode_variant(None)
+            timed_steps(2, plain)
+            plain_elapsed, plain_device_ns = timed_steps(16, plain)
+            plain_distinct = traced_distinct_experts(None)
+            plain_weights = step_costs(workload.model, session, float(plain_distinct.mean()))
+            result["c3_weight_law_routing"] = {
+                "workload": "the timed step with the router logits the prescribed random weights produce",
+                "value": args.lanes * 16 / plain_elapsed, "unit": "tok/s",
+                "ms_per_step": plain_elapsed / 16 * 1e3, "device_ms_per_step": plain_device_ns / 16 / 1e6,
+                "distinct_experts_per_layer": float(plain_distinct.mean()),
+                "step_algorithmic_gb": (attention_per_step + plain_weights["dense"] + plain_weights["routed_seen"]) / 1e9}
         if not args.no_lane_by_lane:
             result["lane_by_lane_step"] = lane_by_lane_step(workload, backend)
         result["roofline"]["measured_stream_read_gbps"] = stream_read_rate(backend)
@@ -715,15 +862,13 @@ def main():
                                          "prefill_attention_c4": prefill_attention_c4(backend),
                                          "prefill_layer_c4": prefill_layer_c4(backend),
                                          "packed_step_c1": packed_step_c1(backend),
-                                         "decode_attention_f16_cache": decode_attention_f16_cache(backend, config)}
+                                         "decode_attention_f16_cache": decode_attention_f16_cache(backend, config),
+                                         "decode_gemv": decode_gemv(backend, workload.model)}
         if config.moe:
             result["secondary_workloads"]["moe_block_c2"] = moe_block_c2(backend, workload.model)
             if not args.no_lane_by_lane:
                 result["secondary_workloads"]["engine_dtype_step"] = engine_dtype_step(
                     backend, workload, args.seed, ctx_lo, ctx_hi)
-    step_bytes = kv_per_step + weights["dense"] + weights["routed_all_experts"] * routed_fraction
-    result["step_algorithmic_gb"] = step_bytes / 1e9
-    result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(config, args.seed, args.cpu_sample_lanes, ctx_lo, ctx_hi)
     print(json.dumps(result))

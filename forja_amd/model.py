@@ -296,7 +296,7 @@ class StepBuffers:
 def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: CommandList,
                 feed_back: bool = False, route_trace: Optional[Tensor] = None,
                 head: bool = True, lane_starts=None, lane_sites: Optional[list] = None,
-                one_row_per_lane: bool = False) -> None:
+                one_row_per_lane: bool = False, router_noise_seed: Optional[int] = None) -> None:
     """Appends one forward step over the packed batch to `commands`.  With `feed_back` the greedy
     tokens are copied into the id buffer for the next step (device to device).  `route_trace`
     (u32 [layers, tokens, top_k]) receives a copy of every layer's expert choices, for
@@ -308,7 +308,12 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
     its own for the result, followed by the Op::Copy of that row into the packed activation.  The
     start is an attribute of the op; `lane_sites` receives (dispatch index, lane) of every such
     dispatch so that a replay can patch it.  `one_row_per_lane` passes the packed op the promise
-    that the batch is a decode batch (every lane at most one row)."""
+    that the batch is a decode batch (every lane at most one row).
+
+    `router_noise_seed`: every layer's router logits are overwritten, after the router product has
+    run, with seeded N(0,1) values (a stream per layer): the routing law of the single-block
+    configuration ("top-8 of softmax of N(0,1) router logits"), under which nearly every expert is
+    touched; under the prescribed weight law alone all tokens choose the same few experts."""
     c, b = model.config, buffers
     tokens = b.tokens
     heads = c.q_heads + c.kv_heads
@@ -371,6 +376,8 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
         if c.moe:
             commands.dispatch(Op.quant_matmul(c.router_bits, GROUP), [normalized, *layer.router.triple],
                               b.router_logits)
+            if router_noise_seed is not None:
+                commands.dispatch(Op.fill_seeded(2, router_noise_seed, 7000 + index), [], b.router_logits)
             commands.dispatch_many(Op.top_k(c.top_k, True), [b.router_logits],
                                    [b.route_weights, b.route_indices])
             if route_trace is not None:
@@ -408,7 +415,8 @@ class DecodeSession:
 
     def __init__(self, model: Model, contexts, seed: int = 7, headroom_tokens: int = 64,
                  physical_pages: Optional[int] = None, table_pages: Optional[int] = None,
-                 fill_pools: bool = True, lane_by_lane: bool = False):
+                 fill_pools: bool = True, lane_by_lane: bool = False,
+                 router_noise_seed: Optional[int] = None):
         c = model.config
         backend = model.backend
         self.model = model
@@ -433,8 +441,10 @@ class DecodeSession:
         backend.write(b.activity, np.ones(lanes, dtype=np.uint32).tobytes())
         first_ids = rng.integers(0, c.vocab, lanes).astype(np.uint32)
         backend.write(b.ids, first_ids.tobytes())
+        self.router_noise_seed = router_noise_seed
         commands = CommandList()
-        record_step(model, self.cache, b, commands, feed_back=True, one_row_per_lane=True)
+        record_step(model, self.cache, b, commands, feed_back=True, one_row_per_lane=True,
+                    router_noise_seed=router_noise_seed)
         self.commands = commands
         self.encoded = backend.encode(commands) if hasattr(backend, "encode") else commands
         self.dispatches = len(commands)
@@ -451,7 +461,8 @@ class DecodeSession:
         self.lane_sites = []
         self.lane_commands = CommandList()
         record_step(self.model, self.cache, b, self.lane_commands, feed_back=True,
-                    lane_starts=self.contexts, lane_sites=self.lane_sites)
+                    lane_starts=self.contexts, lane_sites=self.lane_sites,
+                    router_noise_seed=self.router_noise_seed)
         self.lane_encoded = backend.encode(self.lane_commands) if hasattr(backend, "encode") \
             else self.lane_commands
         self._site_index = np.array([site for site, _ in self.lane_sites])
@@ -490,10 +501,18 @@ class DecodeSession:
             self.cache.upload_tables(grown)
         self.upload_positions()
 
-    def submit_step(self):
+    def encode_variant(self, router_noise_seed: Optional[int]):
+        """The same step on the same storage recorded with another routing law."""
+        commands = CommandList()
+        record_step(self.model, self.cache, self.buffers, commands, feed_back=True,
+                    one_row_per_lane=True, router_noise_seed=router_noise_seed)
+        backend = self.model.backend
+        return backend.encode(commands) if hasattr(backend, "encode") else commands
+
+    def submit_step(self, encoded=None):
         """Uploads this step's metadata and enqueues the step; returns the submission."""
         self.prepare_step()
-        submission = self.model.backend.submit(self.encoded)
+        submission = self.model.backend.submit(self.encoded if encoded is None else encoded)
         self.contexts += 1
         return submission
 

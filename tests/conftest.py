@@ -9,12 +9,6 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
-def pytest_addoption(parser):
-    parser.addoption("--parity-dry-run", action="store_true", default=False,
-                     help="developer aid: run the gpu-marked tests' plumbing against a second "
-                          "oracle instance instead of the HIP library (proves nothing about HIP)")
-
-
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X (runs the HIP library through the C ABI)")
 
@@ -26,11 +20,7 @@ def cpu():
 
 
 @pytest.fixture(scope="session")
-def hip(request):
-    if request.config.getoption("--parity-dry-run"):
-        from oracle.cpu_backend import CpuBackend
-        yield CpuBackend()
-        return
+def hip():
     # No fallback: a missing library or device is an error, not a skip.
     from forja_amd.hip_backend import HipBackend
     backend = HipBackend(0)

@@ -199,6 +199,8 @@ struct fh_backend {
   char *lane_scratch = nullptr;
   uint64_t lane_scratch_bytes = 0;
   bool lane_metadata_valid = false;
+  bool lane_conflict = false;     // verdict of the overlap check for the gathered metadata
+  uint32_t *host_flag = nullptr;  // pinned word the verdict is read through
   std::vector<uint64_t> lane_metadata_key;          // what the gathered metadata was built from
   std::unordered_set<uint64_t> lane_metadata_watch; // allocations whose writes invalidate it
   uint64_t fused_runs = 0, fused_dispatches = 0;
@@ -1507,14 +1509,17 @@ bool find_lane_run(const fh_dispatch *d, uint32_t count, uint32_t first, LaneRun
 
 // Executes the run found by find_lane_run.  `errors` is the record of the run's first dispatch;
 // member i's records start at errors[i * dispatches per member].
-fh_status run_lane_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors) {
+// `*executed` is false when the lanes' tables overlap in a way that makes the order of the
+// dispatches matter: nothing of the run has been executed then and the caller runs it one by one.
+fh_status run_lane_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors, bool *executed) {
+  *executed = true;
   const LaneMember &head = run.members[0];
   const fh_tensor &q0 = head.q, &out0 = head.out, &kp = head.key_pool, &vp = head.value_pool;
   const uint32_t lanes = (uint32_t)run.members.size(), heads = q0.shape[0];
   const uint32_t table_pages = head.table.shape[0], table_words = table_pages * 2;
   const uint64_t row_bytes = (uint64_t)heads * out0.shape[2] * dtype_size(out0.dtype);
   FH_REQUIRE(row_bytes < (1ull << 31));
-  const uint64_t metadata_words = (uint64_t)lanes * table_words + 3ull * lanes + 1;
+  const uint64_t metadata_words = (uint64_t)lanes * table_words + 3ull * lanes + 2;
   const uint64_t rows_at = (metadata_words * 4 + 255) / 256 * 256;
   char *scratch = b->ensure_lane_scratch(rows_at + lanes * row_bytes);
   if (!scratch) return FH_ALLOCATION_FAILED;
@@ -1560,8 +1565,24 @@ fh_status run_lane_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors) {
       launch_gather_lane_metadata(b->stream, sources, base, chunk, lanes, table_words, tables,
                                   activity, starts, cu);
     }
+    // The one thing the tensors cannot show: an append into a slot another lane attends.  Checked
+    // on the gathered tables, once per set of tables (not per layer); the verdict is needed here,
+    // so the stream is waited for.
+    uint32_t *flag = cu + lanes + 1;
+    b->lane_conflict = true;
+    if (launch_lane_conflict_check(b->stream, tables, activity, starts, lanes, table_pages,
+                                   head.page_tokens, flag)) {
+      if (hipMemcpyAsync(b->host_flag, flag, sizeof(uint32_t), hipMemcpyDeviceToHost, b->stream) != hipSuccess ||
+          hipStreamSynchronize(b->stream) != hipSuccess)
+        return FH_DEVICE_EXECUTION_FAILED;
+      b->lane_conflict = *b->host_flag != 0;
+    }
     b->lane_metadata_key = std::move(key);
     b->lane_metadata_valid = true;
+  }
+  if (b->lane_conflict) {
+    *executed = false;
+    return FH_OK;
   }
 
   auto device_view = [](char *base, uint32_t dtype, std::initializer_list<uint32_t> shape) {
@@ -1727,6 +1748,14 @@ fh_status fh_create(int device, fh_backend **out) {
     return FH_DEVICE_EXECUTION_FAILED;
   }
   b->static_host_errors = (ErrorSlot *)mirror;
+  void *word = nullptr;
+  if (hipHostMalloc(&word, 64, hipHostMallocDefault) != hipSuccess) {
+    (void)hipHostFree(mirror);
+    (void)hipStreamDestroy(b->stream);
+    delete b;
+    return FH_DEVICE_EXECUTION_FAILED;
+  }
+  b->host_flag = (uint32_t *)word;
   {
     std::lock_guard<std::mutex> lock(g_live_mutex);
     g_live_backends.insert(b);
@@ -1769,6 +1798,7 @@ void fh_destroy(fh_backend *b) {
     }
     if (b->ring) (void)hipHostFree(b->ring);
     if (b->static_host_errors) (void)hipHostFree(b->static_host_errors);
+    if (b->host_flag) (void)hipHostFree(b->host_flag);
     for (auto &open : b->open_timers)
       for (auto e : open) (void)hipEventDestroy(e);
     for (auto &t : b->timed) {
@@ -2088,10 +2118,19 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
       t1 = take_event(b);
       (void)hipEventRecord(t0, b->stream);
     }
-    if (fused)
-      status = run_lane_group(b, run, &s->device_errors[i]);
-    else
+    if (fused) {
+      bool executed = true;
+      status = run_lane_group(b, run, &s->device_errors[i], &executed);
+      if (!executed) {
+        fused = false;
+        for (uint32_t member = 0; member < consumed && status == FH_OK; ++member) {
+          status = process(b, dispatches[i + member], &s->device_errors[i + member], true);
+          note_outputs(dispatches[i + member]);
+        }
+      }
+    } else {
       status = process(b, dispatches[i], &s->device_errors[i], true);
+    }
     for (uint32_t member = 0; member < consumed; ++member) note_outputs(dispatches[i + member]);
     if (b->profiling >= 2) {
       (void)hipEventRecord(t1, b->stream);

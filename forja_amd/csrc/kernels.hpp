@@ -115,11 +115,18 @@ struct LaneRows {
   void *second[kLaneChunk];  // a second copy of it, or null
 };
 // Lanes [first, first + count) of `lanes`: tables [lanes, table_words], activity/starts [lanes],
-// cu [lanes + 1] (one query row per lane).
+// cu [lanes + 1] (one query row per lane) followed by one word, cleared here, that
+// launch_lane_conflict_check raises.
 void launch_gather_lane_metadata(hipStream_t s, const LaneSources &sources, uint32_t first,
                                  uint32_t count, uint32_t lanes, uint32_t table_words,
                                  uint32_t *tables, uint32_t *activity, uint32_t *starts,
                                  uint32_t *cu);
+// Sets *conflict to 1 when an active lane appends into a slot another active lane attends (the
+// gathered arrays of launch_gather_lane_metadata; tables as (page, generation) pairs).  False,
+// and nothing launched, when there are more lanes than the check holds in LDS.
+bool launch_lane_conflict_check(hipStream_t s, const uint32_t *tables, const uint32_t *activity,
+                                const uint32_t *starts, uint32_t lanes, uint32_t table_pages,
+                                uint32_t page_tokens, uint32_t *conflict);
 // rows: [lanes, row_bytes] contiguous.
 void launch_scatter_lane_rows(hipStream_t s, const LaneRows &targets, const void *rows,
                               uint32_t first, uint32_t count, uint32_t row_bytes);

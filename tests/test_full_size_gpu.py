@@ -1,11 +1,13 @@
 """The BASELINE configurations at their full sizes, where the CPU oracle is out of reach.
 
-Each case runs the operation twice on the device with the same seeded data: once through the
-specialised bf16 kernels and once through the strided generic kernels (reached by giving the
-activations as f32; those kernels follow the oracle's arithmetic order and are checked against it
-at small sizes in test_parity_gpu.py).  The two are independent implementations, and they must
-agree to the stated bf16 bar, |a - b| <= 1e-2 + 1e-2 |b|.  Paging is checked through its
-round-trip property: rows appended through block tables read back bit for bit."""
+Each case runs the operation twice on the device with the same seeded data, through two
+independent implementations that must agree to the stated bf16 bar, |a - b| <= 1e-2 + 1e-2 |b|:
+once through the specialised bf16 matrix-core kernels and once with the activations given as f32,
+which selects the f32 vector-ALU kernels for the quantised products (qmm_valu.hip) and the strided
+f32 kernel for attention; both follow the oracle's arithmetic order and are checked against it at
+small sizes in test_parity_gpu.py.  The cases named "strided" go further and hand over views with
+padded rows, which only the any-stride kernels of generic_ops.hip accept.  Paging is checked
+through its round-trip property: rows appended through block tables read back bit for bit."""
 import math
 
 import numpy as np
@@ -72,6 +74,48 @@ def test_quantised_projection_fast_and_generic_paths_agree(hip, rows, n, k, note
     run(hip, commands)
     assert_close(to_f32(hip.read(fast), DType.BF16), to_f32(hip.read(generic), DType.F32), DType.BF16)
     release(hip, x, x_wide, fast, generic, *weights)
+
+
+def test_config3_qkv_projection_through_the_strided_kernel(hip):
+    """Config 3 stacked qkv (128 x 5120 x 2048) against the any-stride kernel: its activations and
+    output are views into rows padded by one element, which no specialised kernel accepts."""
+    rows, n, k = 128, 5120, 2048
+    weights = quantised(hip, n, k, seed=121)
+    x = seeded(hip, DType.BF16, (rows, k), 121, 4)
+    padded_x = hip.alloc(DType.BF16, (rows, k + 1))
+    padded_out = hip.alloc(DType.BF16, (rows, n + 1))
+    fast = hip.alloc(DType.BF16, (rows, n))
+    commands = CommandList()
+    commands.dispatch(Op.copy(), [x], padded_x.narrow(1, 0, k))
+    commands.dispatch(Op.quant_matmul(4, 64), [x, *weights], fast)
+    commands.dispatch(Op.quant_matmul(4, 64), [padded_x.narrow(1, 0, k), *weights], padded_out.narrow(1, 0, n))
+    run(hip, commands)
+    strided = to_f32(hip.read(padded_out), DType.BF16).reshape(rows, n + 1)[:, :n]
+    assert_close(to_f32(hip.read(fast), DType.BF16).reshape(rows, n), strided, DType.BF16)
+    release(hip, x, padded_x, padded_out, fast, *weights)
+
+
+def test_config4_gate_up_projection_at_full_width(hip):
+    """Config 4's stacked gate/up projection at its real shape, 8256 rows x 34816 columns x 5120:
+    one product on the matrix cores over all rows, and the f32 kernels over three 64-row blocks of
+    the same rows (first, middle, last), every column."""
+    rows, n, k = 8256, 34816, 5120
+    weights = quantised(hip, n, k, seed=131)
+    x = seeded(hip, DType.BF16, (rows, k), 131, 4)
+    fast = hip.alloc(DType.BF16, (rows, n))
+    commands = CommandList()
+    commands.dispatch(Op.quant_matmul(4, 64), [x, *weights], fast)
+    run(hip, commands)
+    for first in (0, 4096, rows - 64):
+        block = as_f32(hip, x.narrow(0, first, 64))
+        generic = hip.alloc(DType.F32, (64, n))
+        commands = CommandList()
+        commands.dispatch(Op.quant_matmul(4, 64), [block, *weights], generic)
+        run(hip, commands)
+        assert_close(to_f32(hip.read(fast.narrow(0, first, 64)), DType.BF16),
+                     to_f32(hip.read(generic), DType.F32), DType.BF16)
+        release(hip, block, generic)
+    release(hip, x, fast, *weights)
 
 
 @pytest.mark.parametrize("rows,n,k,note", [
@@ -241,6 +285,59 @@ def test_config1_packed_batch_attention(hip):
 def test_config4_prefill_attention_largest_prompt(hip):
     """The 3072-token prompt of the config 4 chunk plus decode rows, 40 query / 8 kv heads."""
     attention_both_ways(hip, [0, 1500, 4000], [3072, 1, 1], 40, 8)
+
+
+def test_config4_prefill_chunk_full_batch(hip):
+    """The whole config 4 batch: an 8192-token prefill chunk packed from six prompts of 512 to 3072
+    tokens (two of them continuing an earlier chunk) plus 64 decode rows, 40 query / 8 kv heads."""
+    rng = np.random.default_rng(10)
+    prompts = [512, 768, 1024, 1280, 1536, 3072]
+    assert sum(prompts) == 8192
+    contexts = [0, 0, 2048, 0, 512, 0] + rng.integers(64, 8193, 64).tolist()
+    attention_both_ways(hip, contexts, prompts + [1] * 64, 40, 8)
+
+
+def test_config3_churn_lane_by_lane_equals_the_packed_recording(hip):
+    """Config 3's continuous batch under churn: 128 lanes, contexts log-uniform over 256..32768,
+    eight steps, and before every step eight sequences retire and eight are admitted into the freed
+    pages.  The lane-by-lane recording (fused by the library) and the packed recording run on
+    separate storage with the same seeds: tokens every step and the final logits must be equal bit
+    for bit, and the last layer's newly appended key rows must read back from the pool through the
+    block tables bit for bit."""
+    from forja_amd.model import QWEN3_CODER_30B_A3B, DecodeSession, Model
+    rng = np.random.default_rng(12)
+    lanes, pt = 128, 16
+    contexts = np.exp(rng.uniform(math.log(256), math.log(32768), lanes)).astype(int).tolist()
+    pages = int(sum((c + 64 + pt) // pt for c in contexts) * 1.4)
+    sessions = [DecodeSession(Model(hip, QWEN3_CODER_30B_A3B, seed=23, layers=2), contexts, seed=23,
+                              physical_pages=pages, table_pages=(32768 + 4096) // pt)
+                for _ in range(2)]
+    packed, by_lane = sessions
+    by_lane.record_lane_by_lane()
+    before = hip.fusion_stats()
+    retired = 0
+    for step in range(8):
+        for _ in range(8):
+            lane = retired % lanes
+            retired += 1
+            context = int(math.exp(rng.uniform(math.log(256), math.log(8192))))
+            for session in sessions:
+                session.replace_lane(lane, context)
+        expected = packed.step()
+        actual = by_lane.step(lane_by_lane=True)
+        assert expected.tolist() == actual.tolist(), step
+    assert hip.read(packed.buffers.logits) == hip.read(by_lane.buffers.logits)
+    runs, replaced = (after - start for after, start in zip(hip.fusion_stats(), before))
+    assert (runs, replaced) == (8 * 2, 8 * 2 * 2 * lanes)
+    # round trip: the key rows the last step appended in the last layer, through the tables
+    c = QWEN3_CODER_30B_A3B
+    for session in sessions:
+        qk = np.frombuffer(hip.read(session.buffers.qk), np.uint16).reshape(lanes, c.q_heads + c.kv_heads, c.head_dim)
+        pool = np.frombuffer(hip.read(session.cache.keys[-1]), np.uint16).reshape(-1, pt, c.kv_heads, c.head_dim)
+        for lane in range(lanes):
+            position = int(session.contexts[lane]) - 1          # the token this step appended
+            page = int(session.cache.table_values[lane, position // pt, 0])
+            assert np.array_equal(pool[page, position % pt], qk[lane, c.q_heads:]), lane
 
 
 def test_config3_step_recorded_lane_by_lane_equals_the_packed_recording(hip):

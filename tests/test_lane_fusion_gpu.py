@@ -252,6 +252,41 @@ def test_runs_that_cannot_be_proved_independent_are_executed_serially(cpu, hip):
     check(cpu, hip, results[0], results[1], exact=(1, 2))
 
 
+@pytest.mark.parametrize("idiom", ["append", "copies"])
+@pytest.mark.parametrize("case", ["reader_first", "writer_first", "same_slot"])
+def test_tables_that_share_a_tail_page_run_dispatch_by_dispatch(cpu, hip, case, idiom):
+    """Two lanes whose tables name the same physical tail page: the slot one lane appends lies in
+    the range the other attends (or is the very slot the other appends), so the order of the
+    dispatches decides what each lane sees.  Nothing in the tensors shows it; the library finds it
+    on the device, in the tables, and executes that run one dispatch at a time: the result is the
+    oracle's serial result, pools included, and a batch without the overlap is fused as before."""
+    pt = 16
+    contexts = {"reader_first": [25, 21, 40], "writer_first": [21, 25, 40], "same_slot": [21, 21, 40]}[case]
+    results = []
+    for backend in (cpu, hip):
+        batch = LaneBatch(backend, contexts, 8, 4, pt, seed=91)
+        # lane 1's tail (logical page 1) becomes the physical page that is lane 0's tail
+        table = batch.host_tables[1].copy()
+        table[1] = batch.host_tables[0][1]
+        backend.write(batch.tables[1], table.tobytes())
+        before = hip.fusion_stats()
+        commands = CommandList()
+        attended, rows = batch.record_layer(commands, 0, idiom=idiom)
+        run(backend, commands)
+        if backend is hip:
+            assert hip.fusion_stats() == before          # not fused
+        results.append([attended, *rows, *batch.pools[0]])
+    pools = (len(results[0]) - 2, len(results[0]) - 1)
+    check(cpu, hip, results[0], results[1], exact=pools)
+    # the same shapes without the shared page are fused
+    batch = LaneBatch(hip, contexts, 8, 4, pt, seed=91)
+    before = hip.fusion_stats()
+    commands = CommandList()
+    batch.record_layer(commands, 0, idiom=idiom)
+    run(hip, commands)
+    assert hip.fusion_stats()[0] == before[0] + 1
+
+
 def _random_scenario(rng):
     """A decode batch recorded with random deviations from the regular pattern; every list is
     valid dispatch by dispatch, only some of it can be fused."""

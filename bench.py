@@ -556,9 +556,10 @@ def decode_attention_f16_cache(backend, config, seed=99, repeats=5):
             "algorithmic_bytes": kv_bytes, "achieved_gbps": gbps, "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS}
 
 
-def decode_gemv(backend, model, row_counts=(1, 4, 8), seed=83):
-    """The quantised GEMV of small decode batches (the reference's own regime: at most 8 lanes),
-    product by product on cold weights: every layer's stacked qkv and o_proj in turn, and lm_head
+def decode_gemv(backend, model, row_counts=(1, 4, 8, 128), seed=83):
+    """The quantised GEMV of small decode batches (the reference's own regime: at most 8 lanes) and
+    the same products at the timed batch's 128 rows, product by product on cold weights: every
+    layer's stacked qkv, o_proj and (4-bit) router in turn, and lm_head
     over four copies of its weights (one copy fits the 256 MB of cache in front of HBM).  Times
     are device time of back-to-back launches (one submission, no timers between them); bytes are
     the reference's logical traffic of the dispatch (weights with scales and biases, rows in and
@@ -573,8 +574,10 @@ def decode_gemv(backend, model, row_counts=(1, 4, 8), seed=83):
         heads.append(extra)
     backend.submit(fill).wait()
     groups = [("qkv", [layer.qkv for layer in model.layers]),
-              ("o_proj", [layer.o_proj for layer in model.layers]),
-              ("lm_head", heads)]
+              ("o_proj", [layer.o_proj for layer in model.layers])]
+    if c.moe and model.layers[0].router.bits == 4:
+        groups.append(("router", [layer.router for layer in model.layers]))
+    groups.append(("lm_head", heads))
     q4 = Op.quant_matmul(4, 64)
     results = {}
     for rows in row_counts:
@@ -608,8 +611,8 @@ def decode_gemv(backend, model, row_counts=(1, 4, 8), seed=83):
     for linear in heads[1:]:
         for tensor in linear.triple:
             backend.release(tensor)
-    results["workload"] = ("dense 4-bit products of a decode batch of 1, 4 and 8 rows at the timed model's "
-                           "shapes, cold weights, back-to-back launches")
+    results["workload"] = ("dense 4-bit products of a decode batch of 1, 4, 8 and 128 rows at the timed "
+                           "model's shapes, cold weights, back-to-back launches")
     return results
 
 

@@ -100,7 +100,10 @@ struct KsplitDense {
   uint64_t residual_row_stride;
   uint32_t rows, inner, columns;
 };
-// False when K has no instantiation or the rows are more than 32: nothing was launched.
+// Whether launch_ksplit_dense takes a product of `rows` rows: at most 128, in row tiles of 16 or
+// 32, and more than one tile only for weights small enough to stay cached between the tiles.
+bool ksplit_dense_supports(uint32_t rows, uint32_t inner, uint32_t columns);
+// False when ksplit_dense_supports is: nothing was launched.
 bool launch_ksplit_dense(fh_backend *backend, const KsplitDense &problem);
 struct KsplitRouted {
   const uint16_t *x;

@@ -1113,8 +1113,9 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
     residual = u16_ptr(r);
     residual_row_stride = r.stride[0];
   }
-  // At most 32 rows: the wave-reduced GEMV, K split over the waves of a workgroup.
-  if (p.rows <= 32 && ksplit_supports(p.inner, p.columns, false, false)) {
+  // Decode rows whose weights stay cached between row tiles: K split over the waves of a
+  // workgroup, the rows stationary in registers.
+  if (ksplit_dense_supports(p.rows, p.inner, p.columns)) {
     KsplitDense d{a.x, a.x_row_stride, a.packed[0], a.scales[0], a.biases[0], a.out, a.out_row_stride,
                   a.out_f32, residual, residual_row_stride, p.rows, p.inner, p.columns};
     if (launch_ksplit_dense(backend, d)) return true;

@@ -164,7 +164,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   const uint32_t lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t words_per_row = a.inner / 8, groups_per_row = a.inner / kGroup;
-  const uint32_t tiles = kRouted ? table_word(a.n_blocks, 0) : 1;
+  const uint32_t tiles = kRouted ? table_word(a.n_blocks, 0) : (a.rows + 16 * RT - 1) / (16 * RT);
   const uint32_t units = tiles * a.batches_per_tile;
   const uint32_t first_unit = (uint32_t)((uint64_t)blockIdx.x * units / gridDim.x);
   const uint32_t last_unit = (uint32_t)((uint64_t)(blockIdx.x + 1) * units / gridDim.x);
@@ -185,8 +185,9 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
       const uint32_t expert = table_word(a.blocks, 3 * tile);
       tile_first = expert == kNoBlock ? 0 : table_word(a.blocks, 3 * tile + 1);
       tile_count = expert == kNoBlock ? 0 : table_word(a.blocks, 3 * tile + 2);
-    } else {
-      tile_count = a.rows;
+    } else {   // dense: row tile `tile` of the activation matrix
+      tile_first = tile * (16 * RT);
+      tile_count = min((uint32_t)(16 * RT), a.rows - tile_first);
     }
     // the rows this lane's accumulators belong to: fetched with the tile, not when a batch ends.
     // Rows past the tile's count read the tile's first row (or row 0): their products are
@@ -196,13 +197,14 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const uint32_t row = 16 * rt + 4 * g + i;
-        out_rows[rt][i] = kRouted ? a.sorted_routes[tile_first + (row < tile_count ? row : 0)] : row;
+        const uint32_t at = tile_first + (row < tile_count ? row : 0);
+        out_rows[rt][i] = kRouted ? a.sorted_routes[at] : at;
       }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const uint32_t row = 16 * rt + n;
       const uint32_t safe = row < tile_count ? row : 0;
-      const uint64_t in_row = kRouted ? a.sorted_routes[tile_first + safe] / a.route_div : safe;
+      const uint64_t in_row = kRouted ? a.sorted_routes[tile_first + safe] / a.route_div : tile_first + safe;
       const uint16_t *xp = a.x + in_row * a.x_row_stride + (uint64_t)wave * (G * kGroup) + 16 * g_perm;
       float sums[G];
 #pragma unroll
@@ -294,7 +296,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
           const uint32_t column = min(batch * kBatchCols + 16 * ct + n, a.columns - 1);
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const uint32_t row = min(16 * rt + 4 * g + i, a.rows - 1);
+            const uint32_t row = min(c.tile * (16 * RT) + 16 * rt + 4 * g + i, a.rows - 1);
             const uint16_t *rp = a.residual ? a.residual + (uint64_t)row * a.residual_row_stride + column : a.x;
             r.residual[4 * qq + i] = *rp;
           }
@@ -304,7 +306,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
         for (int tt = 0; tt < TPW; ++tt) {
           const uint32_t t = min(wave + tt * WAVES, (uint32_t)kTriples - 1);
           const uint32_t ct = t / (RT * 4), rt = (t / 4) % RT, i = t % 4;
-          const uint32_t row = min(16 * rt + 4 * g + i, a.rows - 1);
+          const uint32_t row = min(c.tile * (16 * RT) + 16 * rt + 4 * g + i, a.rows - 1);
           const uint32_t column = min(batch * kBatchCols + 16 * ct + n, a.columns - 1);
           const uint16_t *rp = a.residual ? a.residual + (uint64_t)row * a.residual_row_stride + column : a.x;
           r.residual[tt] = *rp;
@@ -463,7 +465,6 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
     load_batch(ring[slot], loading);
     advance(loading);
   }
-  if (!kRouted) load_tile(0);
   // Whole rounds of the ring first, in a loop without exits in its body (an exit that rejoins the
   // loop would make every wait assume the shortest path, i.e. drain the ring); the last, partial
   // round is a copy of the body that requests nothing.
@@ -471,7 +472,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   for (; base + NS <= last_unit; base += NS) {
 #pragma unroll
     for (int slot = 0; slot < NS; ++slot) {
-      if (kRouted && computing.tile != current_tile) load_tile(computing.tile);
+      if (computing.tile != current_tile) load_tile(computing.tile);
       finish_batch(ring[slot], computing.batch, buf);
       buf ^= 1u;
       load_batch(ring[slot], loading);
@@ -482,7 +483,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
 #pragma unroll
   for (int slot = 0; slot < NS - 1; ++slot) {
     if (base + slot >= last_unit) break;
-    if (kRouted && computing.tile != current_tile) load_tile(computing.tile);
+    if (computing.tile != current_tile) load_tile(computing.tile);
     finish_batch(ring[slot], computing.batch, buf);
     buf ^= 1u;
     advance(computing);
@@ -556,11 +557,24 @@ bool ksplit_supports(uint32_t inner, uint32_t columns, bool pair, bool routed) {
   return columns % (16u * batch_tiles(pair, groups)) == 0;   // whole batches of columns only
 }
 
+// Dense products of up to 128 rows: one row tile (16 rows, or 32 where the K slice of 32 rows fits
+// the registers) per pass over the weights.  More than one pass only where the passes after the
+// first find the weights in the caches in front of HBM.
+constexpr uint64_t kCachedWeightBytes = 32ull << 20;
+
+bool ksplit_dense_supports(uint32_t rows, uint32_t inner, uint32_t columns) {
+  int waves = 0, groups = 0;
+  if (rows == 0 || rows > 128 || !ksplit_shape(inner, &waves, &groups)) return false;
+  if (!ksplit_supports(inner, columns, false, false)) return false;
+  const uint32_t tile_rows = rows > 16 && groups <= 4 ? 32 : 16;
+  // (row tiles of 16, which the long K slices are held to, would take eight passes for 128 rows)
+  return rows <= tile_rows || (groups <= 4 && (uint64_t)columns * inner / 2 <= kCachedWeightBytes);
+}
+
 bool launch_ksplit_dense(fh_backend *backend, const KsplitDense &d) {
   int waves = 0, groups = 0;
-  if (d.rows == 0 || d.rows > 32 || !ksplit_shape(d.inner, &waves, &groups)) return false;
-  if (!ksplit_supports(d.inner, d.columns, false, false)) return false;
-  if (d.rows > 16 && groups > 4) return false;   // two row tiles of that many groups do not fit
+  if (!ksplit_dense_supports(d.rows, d.inner, d.columns) || !ksplit_shape(d.inner, &waves, &groups)) return false;
+  const bool wide_tiles = d.rows > 16 && groups <= 4;
   KsplitArgs a{};
   a.x = d.x;
   a.x_row_stride = d.x_row_stride;
@@ -577,9 +591,11 @@ bool launch_ksplit_dense(fh_backend *backend, const KsplitDense &d) {
   a.columns = d.columns;
   const uint32_t batch_cols = 16 * batch_tiles(false, groups);
   a.batches_per_tile = (d.columns + batch_cols - 1) / batch_cols;
+  const uint32_t tile_rows = wide_tiles ? 32 : 16;
+  const uint64_t units = (uint64_t)((d.rows + tile_rows - 1) / tile_rows) * a.batches_per_tile;
   KernelTimer timer(backend, FH_KC_QMM_KERNEL);
-  return d.rows <= 16 ? launch_shape<1, false, false>(backend, a, a.batches_per_tile)
-                      : launch_shape<2, false, false>(backend, a, a.batches_per_tile);
+  return wide_tiles ? launch_shape<2, false, false>(backend, a, units)
+                    : launch_shape<1, false, false>(backend, a, units);
 }
 
 bool launch_ksplit_routed(fh_backend *backend, const KsplitRouted &r) {

@@ -160,7 +160,21 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   constexpr int kTriples = kQuads * 4;       // (column tile, row tile, row) triples of a batch
   constexpr int TPW = (kTriples + WAVES - 1) / WAVES;
   constexpr int kShare = kWide ? QPW * 4 : TPW;         // results per lane this wave finishes per batch
+  // Scales and biases of a batch: kSub blocks of 16 columns x K/64 bf16 (each projection and
+  // column tile, scales then biases), contiguous in memory.  A wave needs 2G bytes of each column
+  // row; read directly, those 8-byte pieces of 64-byte sectors cost a quarter of the weight
+  // bandwidth (measured).  So the workgroup reads each block once, coalesced -- a thread fetches
+  // kShareWords words of every batch -- and passes it through LDS, two batches deep: written
+  // before the exchange barrier of the batch before, read at the start of its own batch.
+  // (Only where the memory requests bound the kernel: with two row tiles the instruction stream
+  // does, and the direct loads, which cost no extra instructions, stay.)
+  constexpr bool kStage = RT == 1;
+  constexpr int kSub = P * CT * 2;
+  constexpr int kPieces = kSub * 16 * WAVES;          // 2G-byte pieces of a batch (one per column and wave)
+  constexpr int PT = kPieces / (64 * WAVES);          // pieces a thread fetches per batch (1 or 2)
+  static_assert(PT * 64 * WAVES == kPieces, "whole pieces per thread");
   extern __shared__ __attribute__((aligned(16))) float exchange[];   // f32x4 [2][WAVES][kSlots][64]
+  uint32_t *scale_lds = (uint32_t *)(exchange + 2 * WAVES * kSlots * 4 * 64);   // [2][kPieces][W2]
   const uint32_t lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t words_per_row = a.inner / 8, groups_per_row = a.inner / kGroup;
@@ -240,7 +254,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   // before it touches a batch counts exactly the younger batches still in flight.
   struct Batch {
     uint4 w[P][CT][W2];         // the lane's 32 nibbles of each pair of groups
-    uint32_t s[P][CT][W2], b[P][CT][W2];   // the column's G scales and biases, two to a word
+    uint32_t s[P][CT][W2], b[P][CT][W2];   // direct form only: the column's G scales and biases, two to a word
     uint32_t residual[kShare];  // dense only: the values added to this wave's share of the results
   };
   // Where a stream of units stands: the loads run a ring ahead of the arithmetic, each with its own
@@ -266,6 +280,45 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   // is the same for the whole wave and stays in scalar registers.
   const uint32_t lane_weight_bytes = (n * words_per_row + wave * (G * 8) + 4 * g) * 4;
   const uint32_t lane_group_bytes = (n * groups_per_row + wave * G) * 2;
+  // This thread's share of a batch's scales and biases: piece threadIdx.x + i * threads of the
+  // kPieces, i.e. block piece / (16 WAVES), and inside the block (contiguous in memory and in
+  // LDS alike) piece % (16 WAVES).  The part of the address that does not change is kept.
+  struct Share {
+    uint32_t words[PT][W2];
+  };
+  const uint16_t *share_from[PT];
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const uint32_t piece = threadIdx.x + i * (64 * WAVES);
+    const uint32_t block = piece / (16 * WAVES), inside = piece % (16 * WAVES);
+    const uint16_t *from = a.scales[0];
+#pragma unroll
+    for (int sub = 0; sub < kSub; ++sub) {
+      const int tp = sub / 2, pj = tp / CT, ct = tp % CT;
+      const uint16_t *base = (sub % 2 ? a.biases[pj] : a.scales[pj]) + (uint64_t)(16 * ct) * groups_per_row;
+      if (block == (uint32_t)sub) from = base;
+    }
+    share_from[i] = from + (uint64_t)inside * G;
+  }
+  auto load_share = [&](Share &r, const Cursor &c) {
+    if constexpr (!kStage) return;
+    const uint64_t groups = c.expert * a.expert_groups + (uint64_t)c.batch * kBatchCols * groups_per_row;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      const uint32_t *from = (const uint32_t *)(share_from[i] + groups);
+#pragma unroll
+      for (int k = 0; k < W2; ++k) r.words[i][k] = from[k];
+    }
+  };
+  auto write_share = [&](const Share &r, uint32_t half) {
+    if constexpr (!kStage) return;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      uint32_t *to = scale_lds + ((uint64_t)half * kPieces + threadIdx.x + i * (64 * WAVES)) * W2;
+#pragma unroll
+      for (int k = 0; k < W2; ++k) to[k] = r.words[i][k];
+    }
+  };
   auto load_batch = [&](Batch &r, const Cursor &c) {
     const uint32_t batch = c.batch;
 #pragma unroll
@@ -274,16 +327,18 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
       for (int ct = 0; ct < CT; ++ct) {
         const uint64_t tile_column = batch * kBatchCols + 16 * ct;   // a multiple of 16 below a.columns
         const uint64_t words = c.expert * a.expert_words + tile_column * words_per_row;
-        const uint64_t groups = c.expert * a.expert_groups + tile_column * groups_per_row;
         const char *wp = (const char *)(a.packed[pj] + words) + lane_weight_bytes;
-        const char *sp = (const char *)(a.scales[pj] + groups) + lane_group_bytes;
-        const char *bp = (const char *)(a.biases[pj] + groups) + lane_group_bytes;
 #pragma unroll
         for (int k = 0; k < W2; ++k) r.w[pj][ct][k] = *(const uint4 *)(wp + 64 * k);
+        if constexpr (!kStage) {
+          const uint64_t groups = c.expert * a.expert_groups + tile_column * groups_per_row;
+          const char *sp = (const char *)(a.scales[pj] + groups) + lane_group_bytes;
+          const char *bp = (const char *)(a.biases[pj] + groups) + lane_group_bytes;
 #pragma unroll
-        for (int i = 0; i < W2; ++i) {
-          r.s[pj][ct][i] = *(const uint32_t *)(sp + 4 * i);
-          r.b[pj][ct][i] = *(const uint32_t *)(bp + 4 * i);
+          for (int i = 0; i < W2; ++i) {
+            r.s[pj][ct][i] = *(const uint32_t *)(sp + 4 * i);
+            r.b[pj][ct][i] = *(const uint32_t *)(bp + 4 * i);
+          }
         }
       }
     if (!kRouted) {
@@ -317,7 +372,19 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
 
   // Contracts the batch against the stationary rows, hands the partial sums to LDS buffer `buf`,
   // and takes this wave's share of the epilogue.
-  auto finish_batch = [&](const Batch &r, uint32_t batch, uint32_t buf) {
+  // ... `pass_on` is this thread's share of the NEXT batch's scales and biases, written to the other
+  // half of their LDS ring before the barrier; this batch's are read from half `buf` first.
+  auto finish_batch = [&](const Batch &r, const Share &pass_on, uint32_t batch, uint32_t buf) {
+    uint32_t scales[P * CT][W2], biases[P * CT][W2];
+#pragma unroll
+    for (int tp = 0; tp < P * CT; ++tp) {
+      const uint32_t *at = scale_lds + ((uint64_t)buf * kPieces + (2 * tp) * (16 * WAVES) + n * WAVES + wave) * W2;
+#pragma unroll
+      for (int k = 0; k < W2; ++k) {
+        scales[tp][k] = kStage ? at[k] : r.s[tp / CT][tp % CT][k];
+        biases[tp][k] = kStage ? at[(16 * WAVES) * W2 + k] : r.b[tp / CT][tp % CT][k];
+      }
+    }
     f32x4 acc[P * CT][RT];
     // bias term sum_j (bias_j - 16 scale_j) * xsum_j[row] first: an f32 matrix step over four
     // groups, lane quarter g supplying group 4q + g of both operands
@@ -328,8 +395,8 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
       for (int rt = 0; rt < RT; ++rt) acc[tp][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int q = 0; q < Q; ++q) {
-        const float shift = packed_bf16_at<W2>(r.b[pj][ct], 4 * q + g) -
-                            16.0f * packed_bf16_at<W2>(r.s[pj][ct], 4 * q + g);
+        const float shift = packed_bf16_at<W2>(biases[tp], 4 * q + g) -
+                            16.0f * packed_bf16_at<W2>(scales[tp], 4 * q + g);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
           acc[tp][rt] = __builtin_amdgcn_mfma_f32_16x16x4f32(xs[rt][q], shift, acc[tp][rt], 0, 0, 0);
@@ -349,7 +416,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
         second_words = __builtin_amdgcn_permlane32_swap(w.y, w.w, false, false);
       }
       const bf16x8 b0 = unpack_word(first_words[j % 2]), b1 = unpack_word(second_words[j % 2]);
-      const uint32_t word = r.s[pj][ct][j / 2];
+      const uint32_t word = scales[tp][j / 2];
       const float scale = __uint_as_float((j & 1) ? (word & 0xffff0000u) : (word << 16));
       f32x4 part[RT];
 #pragma unroll
@@ -390,6 +457,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
       for (int tp = 0; tp < P * CT; ++tp)
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) mine[(tp * RT + rt) * 64] = acc[tp][rt];
+      write_share(pass_on, buf ^ 1u);
       __syncthreads();
       // (column tile, row tile) blocks of 16 x 16 results are dealt round-robin to the waves; the
       // owner adds the waves' sums in wave order (fixed: results do not depend on scheduling), four
@@ -427,6 +495,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) mine[((tp * RT + rt) * 4 + i) * 64] = acc[tp][rt][i];
+      write_share(pass_on, buf ^ 1u);
       __syncthreads();
       // (column tile, row tile, row) triples are dealt round-robin to the waves, one result to a lane
 #pragma unroll
@@ -458,24 +527,39 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   if (first_unit >= last_unit) return;
   Cursor loading{first_unit, first_unit / a.batches_per_tile, first_unit % a.batches_per_tile, 0};
   loading.expert = expert_of(loading.tile);
-  Cursor computing = loading;
+  Cursor computing = loading, sharing = loading;
+  // Scales and biases run one batch further ahead than the weights: the share of the first unit
+  // goes to LDS at once, those of the next two are in flight when the loop starts.
+  Share shares[NS], first_share;
+  load_share(first_share, sharing);
+  advance(sharing);
+#pragma unroll
+  for (int slot = 1; slot <= 2; ++slot) {
+    load_share(shares[slot % NS], sharing);
+    advance(sharing);
+  }
   Batch ring[NS];
 #pragma unroll
   for (int slot = 0; slot < NS; ++slot) {
     load_batch(ring[slot], loading);
     advance(loading);
   }
+  write_share(first_share, 0);
+  if (kStage) __syncthreads();   // the first unit's scales are in LDS
   // Whole rounds of the ring first, in a loop without exits in its body (an exit that rejoins the
   // loop would make every wait assume the shortest path, i.e. drain the ring); the last, partial
-  // round is a copy of the body that requests nothing.
+  // round is a copy of the body that requests nothing.  Unit number i of this workgroup uses ring
+  // slot i % NS; share i + 1 is passed on while unit i is finished, share i + 3 requested after it.
   uint32_t base = first_unit, buf = 0;
   for (; base + NS <= last_unit; base += NS) {
 #pragma unroll
     for (int slot = 0; slot < NS; ++slot) {
       if (computing.tile != current_tile) load_tile(computing.tile);
-      finish_batch(ring[slot], computing.batch, buf);
+      finish_batch(ring[slot], shares[(slot + 1) % NS], computing.batch, buf);
       buf ^= 1u;
+      load_share(shares[(slot + 3) % NS], sharing);
       load_batch(ring[slot], loading);
+      advance(sharing);
       advance(loading);
       advance(computing);
     }
@@ -484,7 +568,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   for (int slot = 0; slot < NS - 1; ++slot) {
     if (base + slot >= last_unit) break;
     if (computing.tile != current_tile) load_tile(computing.tile);
-    finish_batch(ring[slot], computing.batch, buf);
+    finish_batch(ring[slot], shares[(slot + 1) % NS], computing.batch, buf);
     buf ^= 1u;
     advance(computing);
   }
@@ -509,7 +593,8 @@ bool ksplit_shape(uint32_t inner, int *waves, int *groups) {
 template <int WAVES, int G, int RT, bool kPair, bool kRouted>
 void launch_one(fh_backend *backend, const KsplitArgs &a, uint64_t most_units) {
   constexpr int P = kPair ? 2 : 1, CT = batch_tiles(kPair, G);
-  constexpr uint32_t lds = 2u * WAVES * (CT * P * RT * 4) * 64 * sizeof(float);
+  constexpr uint32_t lds = 2u * WAVES * (CT * P * RT * 4) * 64 * sizeof(float) +   // partial sums
+                           (RT == 1 ? 2u * (P * CT * 2 * 16 * WAVES) * (G / 2) * sizeof(uint32_t) : 0u);   // scales and biases
   const void *kernel = reinterpret_cast<const void *>(&qmm_ksplit_kernel<WAVES, G, RT, kPair, kRouted>);
   static int per_unit = 0;   // set once per process: the dynamic LDS limit and the occupancy
   if (per_unit == 0) {

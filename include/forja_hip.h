@@ -88,8 +88,14 @@ typedef enum fh_op_kind {
    *   inputs : q [T,Hq,D], k_new [T,Hkv,D], v_new [T,Hkv,Dv], tables u32 [L,table_pages,2],
    *            generations u32 [P], cu_seqlens u32 [L+1], q_starts u32 [L], activity u32 [L]
    *   outputs: out [T,Hq,Dv], key pool [P,pt,Hkv,D], value pool [P,pt,Hkv,Dv]
-   * Lanes must address pairwise distinct (page,slot) destinations; inactive lanes produce zeros
-   * and leave the pools untouched.  `k` = 1 is the recorder's promise that no lane brings more
+   * Precondition, NOT checked for this op: no lane's destination (page, slot) is another lane's
+   * destination or lies inside another lane's attended range - what the host's copy-on-write
+   * pages guarantee (crates/forja-host/src/lib.rs:5408-5470).  Every append of the batch is
+   * performed before every attention, so a batch that breaks it is not the serial sequence.
+   * (fh_submit does check it, on the device, before it executes a run of per-lane dispatches
+   * this way, and falls back to one dispatch at a time.)  Inactive lanes produce zeros and leave
+   * the pools untouched; a cu_seqlens that decreases or passes T is refused on the device (zero
+   * rows, pools untouched, the lowest offending lane reported).  `k` = 1 is the recorder's promise that no lane brings more
    * than one query row (a decode batch): the library then stores the new rows from inside the
    * attention kernel.  The promise is checked on the device; a lane that breaks it is reported
    * as FH_DEVICE_ERROR_FLAG with the first offending token as value.  `k` = 0: no promise. */

@@ -632,6 +632,9 @@ def main():
                              "profiler run should be given)")
     parser.add_argument("--no-profile", action="store_true",
                         help="skip the HIP-event kernel timing inside the timed region")
+    parser.add_argument("--headline-only", action="store_true",
+                        help="the timed step, its roofline and the per-op breakdown; none of the "
+                             "secondary workloads, no CPU baseline")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only run the config 4 prefill projection measurement and exit")
     parser.add_argument("--gemv-only", action="store_true",
@@ -836,7 +839,7 @@ def main():
                                             "routed_products_reference_bounds": [weights["routed_minimum"] / 1e9,
                                                                                  weights["routed_maximum"] / 1e9]}
     result["step_hbm_fraction_of_peak"] = step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS
-    if not args.no_profile:
+    if not args.no_profile and not args.headline_only:
         if config.moe:
             # The same step with the routing the prescribed weights give by themselves.
             plain = session.encode_variant(None)
@@ -872,7 +875,7 @@ def main():
             if not args.no_lane_by_lane:
                 result["secondary_workloads"]["engine_dtype_step"] = engine_dtype_step(
                     backend, workload, args.seed, ctx_lo, ctx_hi)
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not args.headline_only:
         result["cpu_baseline"] = cpu_baseline(config, args.seed, args.cpu_sample_lanes, ctx_lo, ctx_hi)
     print(json.dumps(result))
 

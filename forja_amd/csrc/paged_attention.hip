@@ -268,7 +268,7 @@ constexpr uint32_t kMinSplitTokens = 128, kMaxSplitTokens = 1024;  // split leng
 // Groups of several query tokens (prefill) are many and each split of theirs costs a merge of
 // `members x heads` partial rows: they are split only beyond this many keys.
 constexpr uint32_t kPrefillSplitTokens = 2048;
-constexpr uint32_t kTargetItems = 1024;  // (token, split) items wanted per launch
+constexpr uint32_t kTargetItems = 1024;  // (token, split) items wanted per launch of grouped tokens
 constexpr uint32_t kTile = 32;          // tokens per inner step
 
 struct TokenPlan {
@@ -294,6 +294,9 @@ struct FastRagged {
   uint64_t q_stride_t, q_stride_h, out_stride_t, out_stride_h;
   uint32_t tokens, lanes, query_heads, kv_heads, group, page_tokens, physical_pages, table_pages,
       max_splits, split_tokens;
+  // Workgroups of the decode kernel the device holds at once (0: not a decode batch).  The plan
+  // sizes the splits so that the items fill these places once.
+  uint32_t item_slots;
   // Query tokens of one lane are processed `group_tokens` at a time (they share the lane's K/V
   // stream): 1 for decode batches (a wave per kv head), kSharedWaves * kSharedTiles * (16 / group)
   // for prefill batches (a workgroup per kv head).
@@ -313,6 +316,18 @@ struct FastRagged {
   uint32_t append_in_kernel, append_error_back;
   uint32_t promised;   // one query row per lane, vouched for by the caller: verified by the plan
 };
+
+// Splits of a group whose longest member attends `longest` keys: as few as keep each within
+// `split_tokens`, of equal length rounded up to whole tiles.
+__device__ inline void split_layout(uint32_t longest, uint32_t members, uint32_t split_tokens,
+                                    uint32_t max_splits, uint32_t *chunk, uint32_t *splits) {
+  if (members > 1 && split_tokens < kPrefillSplitTokens) split_tokens = kPrefillSplitTokens;
+  uint32_t want = (longest + split_tokens - 1) / split_tokens;
+  if (want > max_splits) want = max_splits;
+  const uint32_t even = (longest + want - 1) / want;
+  *chunk = (even + kTile - 1) / kTile * kTile;
+  *splits = (longest + *chunk - 1) / *chunk;
+}
 
 // Work decomposition of one token.  Tokens of a lane are grouped `group_tokens` at a time; a
 // group shares its split layout, sized for its last (longest) member, and every member carries
@@ -350,13 +365,8 @@ __device__ inline TokenPlan plan_token(const FastRagged &p, uint32_t token, uint
   plan.leader = (uint32_t)(first_of_lane + leader);
   plan.members = (uint32_t)(last - leader + 1);
   plan.attended = (uint32_t)attended;
-  const uint32_t longest = (uint32_t)group_attended;
-  if (plan.members > 1 && split_tokens < kPrefillSplitTokens) split_tokens = kPrefillSplitTokens;
-  uint32_t want = (longest + split_tokens - 1) / split_tokens;
-  if (want > p.max_splits) want = p.max_splits;
-  uint32_t chunk = (longest + want - 1) / want;
-  plan.chunk = (chunk + kTile - 1) / kTile * kTile;
-  plan.splits = (longest + plan.chunk - 1) / plan.chunk;
+  split_layout((uint32_t)group_attended, plan.members, split_tokens, p.max_splits, &plan.chunk,
+               &plan.splits);
   return plan;
 }
 
@@ -394,10 +404,13 @@ __global__ __launch_bounds__(256) void ragged_validate_kernel(const uint32_t *cu
 __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlot *error) {
   __shared__ uint32_t class_items[kSizeClasses];   // items per class, then the class's cursor
   __shared__ unsigned long long total_attended;
-  __shared__ uint32_t merge_count, malformed_lane;
+  __shared__ uint32_t merge_count, malformed_lane, longest_keys, trial_items;
+  constexpr uint32_t kKeysHeld = 4096;   // tokens whose key counts the split search keeps in LDS
+  __shared__ uint32_t keys_held[kKeysHeld];
   for (uint32_t c = threadIdx.x; c < kSizeClasses; c += 256) class_items[c] = 0;
   if (threadIdx.x == 0) {
     total_attended = 0;
+    longest_keys = 0;
     merge_count = 0;
     malformed_lane = 0xffffffffu;
   }
@@ -427,19 +440,61 @@ __global__ __launch_bounds__(256) void ragged_plan_kernel(FastRagged p, ErrorSlo
   }
   if (threadIdx.x == 0) p.item_count[2] = 0;
   // Split length: long enough that a wave's fixed start-up cost (plan, table, query) is small
-  // against its stream, short enough that the batch still yields ~kTargetItems work items.
+  // against its stream, short enough that the batch still yields enough work items.
   uint32_t split_tokens = p.split_tokens;
   if (split_tokens == 0) {
     unsigned long long mine = 0;
-    for (uint32_t token = threadIdx.x; token < p.tokens; token += 256)
-      mine += plan_token(p, token, 1u << 30).attended / p.group_tokens;
+    uint32_t mine_longest = 0;
+    for (uint32_t token = threadIdx.x; token < p.tokens; token += 256) {
+      const TokenPlan whole = plan_token(p, token, 1u << 30);
+      // the keys of the token's group in whole tiles, for the search below: a decode batch has
+      // groups of one token
+      const uint32_t keys = whole.splits ? whole.chunk : 0;
+      if (token < kKeysHeld) keys_held[token] = keys;
+      else if (p.item_slots) p.plans[token].chunk = keys;
+      mine += whole.attended / p.group_tokens;
+      mine_longest = max(mine_longest, keys);
+    }
     for (int offset = 32; offset > 0; offset >>= 1) mine += __shfl_xor(mine, offset, 64);
     if ((threadIdx.x & 63) == 0) atomicAdd(&total_attended, mine);
+    atomicMax(&longest_keys, mine_longest);
     __syncthreads();
-    unsigned long long per_item = total_attended / kTargetItems;
-    split_tokens = (uint32_t)((per_item + kTile - 1) / kTile * kTile);
-    if (split_tokens < kMinSplitTokens) split_tokens = kMinSplitTokens;
-    if (split_tokens > kMaxSplitTokens) split_tokens = kMaxSplitTokens;
+    if (p.item_slots == 0) {
+      unsigned long long per_item = total_attended / kTargetItems;
+      split_tokens = (uint32_t)((per_item + kTile - 1) / kTile * kTile);
+      if (split_tokens < kMinSplitTokens) split_tokens = kMinSplitTokens;
+      if (split_tokens > kMaxSplitTokens) split_tokens = kMaxSplitTokens;
+    } else {
+      // Decode batches: the shortest split length whose items all find a place on the device at
+      // once.  One item per place costs each place one start-up and leaves no second, partly
+      // filled round behind (128 lanes of 256 to 32768 keys: 311 us against 330 us for any
+      // length that needs two rounds).  When the lanes alone outnumber the places no length
+      // achieves that, and one far above the even share would leave the longest lanes running
+      // alone at the end: then the even share of a place is the length.
+      const unsigned long long share = (total_attended + p.item_slots - 1) / p.item_slots;
+      uint32_t even = (uint32_t)((share + kTile - 1) / kTile * kTile);
+      if (even < kMinSplitTokens) even = kMinSplitTokens;
+      uint32_t low = even / kTile, high = max(longest_keys, even) / kTile;   // in tiles
+      while (low < high) {   // smallest length in [low, high] with at most item_slots items
+        const uint32_t middle = (low + high) / 2;
+        if (threadIdx.x == 0) trial_items = 0;
+        __syncthreads();
+        uint32_t items = 0;
+        for (uint32_t token = threadIdx.x; token < p.tokens; token += 256) {
+          const uint32_t keys = token < kKeysHeld ? keys_held[token] : p.plans[token].chunk;
+          if (keys == 0) continue;
+          uint32_t chunk, splits;
+          split_layout(keys, 1, middle * kTile, p.max_splits, &chunk, &splits);
+          items += splits;
+        }
+        if (items) atomicAdd(&trial_items, items);
+        __syncthreads();
+        const bool fits = trial_items <= p.item_slots;
+        __syncthreads();
+        if (fits) high = middle; else low = middle + 1;
+      }
+      split_tokens = low * kTile <= 2 * even ? low * kTile : even;
+    }
   }
   auto class_of = [](const TokenPlan &plan) {
     const uint32_t c = plan.chunk / kTile;
@@ -594,11 +649,11 @@ __device__ inline void load_tile(const FastRagged &p, TileRegs &r, uint32_t tile
     const uint16_t *k_base = p.key_pool + row0 * lc.row_elems;
     const uint16_t *v_base = p.value_pool + row0 * lc.row_elems;
     for (int step = 0; step < 4; ++step) {
-      r.k[sub][step] = *(const uint4 *)(k_base + lc.k_offset + 32 * step);
+      r.k[sub][step] = stream_load(k_base + lc.k_offset + 32 * step);
       if (kMasked && tok0 + hl >= end) r.k[sub][step] = make_uint4(0, 0, 0, 0);
     }
     for (int i = 0; i < 4; ++i) {
-      r.v[4 * sub + i] = *(const uint4 *)(v_base + lc.v_offset + i * lc.row_elems);
+      r.v[4 * sub + i] = stream_load(v_base + lc.v_offset + i * lc.row_elems);
       if (kMasked && tok0 + 4 * g + i >= end) r.v[4 * sub + i] = make_uint4(0, 0, 0, 0);
     }
   }
@@ -1204,12 +1259,49 @@ void launch_plan(hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
   ragged_plan_kernel<<<dim3(1), 256, 0, stream>>>(f, error);
 }
 
+// queries or outputs of another dtype than the pools': the kernels choose at run time
+bool mixed_dtypes(const FastRagged &f) {
+  const uint32_t pool_dtype = f.pool_half ? FH_F16 : FH_BF16;
+  return f.q_dtype != pool_dtype || f.out_dtype != pool_dtype;
+}
+
+using DecodeKernel = void (*)(FastRagged, ErrorSlot *);
+
+DecodeKernel decode_kernel(const FastRagged &f) {
+  const bool mixed = mixed_dtypes(f);
+  return f.pool_half ? (mixed ? ragged_attention_mfma_kernel<true, true>
+                              : ragged_attention_mfma_kernel<true, false>)
+                     : (mixed ? ragged_attention_mfma_kernel<false, true>
+                              : ragged_attention_mfma_kernel<false, false>);
+}
+
+uint32_t decode_waves(const FastRagged &f) { return f.kv_heads < 8 ? f.kv_heads : 8; }
+
+// Work items of a decode batch the device runs at once: resident workgroups per compute unit
+// times compute units, over the workgroups an item takes (one per 8 kv heads).  Needs q_dtype,
+// out_dtype, pool_half and kv_heads.
+uint32_t decode_item_slots(fh_backend *backend, const FastRagged &f) {
+  static uint32_t resident[2][2][9];   // [f16 pools][mixed][waves]; every writer stores the same value
+  const uint32_t waves = decode_waves(f);
+  uint32_t &known = resident[f.pool_half ? 1 : 0][mixed_dtypes(f) ? 1 : 0][waves];
+  uint32_t per_unit = known;
+  if (per_unit == 0) {
+    int blocks = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decode_kernel(f), (int)(64 * waves), 0) !=
+            hipSuccess ||
+        blocks < 1)
+      blocks = 1;
+    known = per_unit = (uint32_t)blocks;
+  }
+  const uint32_t per_item = (f.kv_heads + waves - 1) / waves;
+  const uint32_t slots = per_unit * backend_compute_units(backend) / per_item;
+  return slots ? slots : 1;
+}
+
 void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, ErrorSlot *error) {
   uint64_t groups = f.group_tokens > 1 ? f.tokens / f.group_tokens + f.lanes : f.tokens;
   uint64_t blocks = groups * f.max_splits;
-  // queries or outputs of another dtype than the pools': the kernels choose at run time
-  const uint32_t pool_dtype = f.pool_half ? FH_F16 : FH_BF16;
-  const bool mixed = f.q_dtype != pool_dtype || f.out_dtype != pool_dtype;
+  const bool mixed = mixed_dtypes(f);
   {
     KernelTimer timer(backend, FH_KC_ATTENTION_KERNEL);
     // one workgroup per work item, up to 8 (decode) or 4 (prefill) kv heads of it per workgroup
@@ -1221,13 +1313,9 @@ void launch_fast(fh_backend *backend, hipStream_t stream, const FastRagged &f, E
                                           : ragged_attention_prefill_kernel<false, false>);
       kernel<<<grid, 64 * kSharedWaves, 0, stream>>>(f, error);
     } else {
-      const uint32_t waves = f.kv_heads < 8 ? f.kv_heads : 8;
+      const uint32_t waves = decode_waves(f);
       const dim3 grid((unsigned)blocks, (f.kv_heads + waves - 1) / waves);
-      auto *kernel = f.pool_half ? (mixed ? ragged_attention_mfma_kernel<true, true>
-                                          : ragged_attention_mfma_kernel<true, false>)
-                                 : (mixed ? ragged_attention_mfma_kernel<false, true>
-                                          : ragged_attention_mfma_kernel<false, false>);
-      kernel<<<grid, 64 * waves, 0, stream>>>(f, error);
+      decode_kernel(f)<<<grid, 64 * waves, 0, stream>>>(f, error);
     }
   }
   ragged_reduce_kernel<<<dim3(f.query_heads, f.tokens < 1024 ? f.tokens : 1024), 256, 0, stream>>>(f);
@@ -1273,6 +1361,7 @@ bool try_fast_lane_attention(fh_backend *backend, const LaneAttention &lane, Err
   f.starts = nullptr;
   f.activity =
       lane.activity.base ? (const uint32_t *)lane.activity.base + lane.activity.offset : nullptr;
+  f.item_slots = f.group_tokens == 1 ? decode_item_slots(backend, f) : 0;
   // q / out are [Hq, Sq, D] views: the token axis is axis 1.
   f.q_stride_t = lane.q.stride[1];
   f.q_stride_h = lane.q.stride[0];
@@ -1301,6 +1390,10 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     f.table_pages = p.table_pages;
     f.max_splits = splits_for(p.tokens);
     fit_splits(backend, &f, false);
+    f.q_dtype = p.q.dtype;
+    f.out_dtype = p.out.dtype;
+    f.pool_half = p.key_pool.dtype == FH_F16;
+    f.item_slots = f.group_tokens == 1 ? decode_item_slots(backend, f) : 0;
     f.error_stride = p.error_stride;
     f.scale_log2 = p.scale * 1.4426950408889634f;
     f.tables = (const uint32_t *)p.tables.base + p.tables.offset;
@@ -1319,18 +1412,15 @@ bool run_ragged_attention(fh_backend *backend, const RaggedAttention &p, ErrorSl
     key.address[4] = (uint64_t)f.generations;
     f.promised = p.one_row_per_lane;
     f.append_in_kernel = p.one_row_per_lane && append_in_kernel_possible(p);
-    const uint32_t params[12] = {f.tokens, f.lanes, f.group_tokens, f.page_tokens, f.physical_pages,
+    const uint32_t params[13] = {f.tokens, f.lanes, f.group_tokens, f.page_tokens, f.physical_pages,
                                  f.table_pages, f.max_splits, forced_split_tokens(), f.kv_heads,
-                                 f.query_heads, f.append_in_kernel, f.promised};
-    for (int i = 0; i < 12; ++i) key.params[i] = params[i];
+                                 f.query_heads, f.append_in_kernel, f.promised, f.item_slots};
+    for (int i = 0; i < 13; ++i) key.params[i] = params[i];
     bool reuse = false;
     char *plan_storage = backend_attention_plan(backend, key, plan_storage_bytes(f), &reuse);
     if (!plan_storage || !carve_partials(backend, &f, plan_storage)) return false;
     f.q = (const char *)p.q.base + p.q.offset * dtype_size(p.q.dtype);
     f.out = (char *)p.out.base + p.out.offset * dtype_size(p.out.dtype);
-    f.q_dtype = p.q.dtype;
-    f.out_dtype = p.out.dtype;
-    f.pool_half = p.key_pool.dtype == FH_F16;
     f.key_pool = (const uint16_t *)p.key_pool.base + p.key_pool.offset;
     f.value_pool = (const uint16_t *)p.value_pool.base + p.value_pool.offset;
     f.q_stride_t = p.q.stride[0];

@@ -560,13 +560,15 @@ class CpuBackend:
         return entries, gens
 
     def _paged_copy(self, ordinary: Tensor, pool: Tensor, table, generations, activity, direction,
-                    start, page_tokens):
+                    start, page_tokens, held=None):
+        """`held`: the pool's bytes, already gathered by a caller that runs many copies and
+        writes the pool back itself (the ragged op); the copy then lands there."""
         if not self._lane_active(activity):
             return
         entries, gens = self._page_table(table, generations)
         physical_pages, _, elements = pool.shape
         row_bytes = elements * pool.dtype.byte_size
-        pool_raw = self._gather(pool)
+        pool_raw = self._gather(pool) if held is None else held
         tokens = ordinary.shape[0]
         if direction == INTO_PAGES:
             rows = encode(self._floats(ordinary), pool.dtype)
@@ -575,7 +577,8 @@ class CpuBackend:
                                              _p(gens), C.c_uint64(start), C.c_uint64(tokens),
                                              _p(rows))
             _ok(status, Status.INVALID_INPUT)
-            self.write(pool, pool_raw.tobytes())
+            if held is None:
+                self.write(pool, pool_raw.tobytes())
         else:
             rows = np.empty(tokens * row_bytes, dtype=np.uint8)
             status = lib().orc_paged_copy_out(_p(pool_raw), _sz(physical_pages), _sz(page_tokens),
@@ -593,11 +596,12 @@ class CpuBackend:
                          d.op.page_tokens)
 
     def _paged_sdpa(self, q, key_pool, value_pool, table, generations, activity, output, scale,
-                    causal, q_start, key_length, page_tokens):
+                    causal, q_start, key_length, page_tokens, held=None):
+        """`held`: the bytes of both pools, already gathered (see _paged_copy)."""
         if not self._lane_active(activity):
             self._write_output(output, np.zeros(output.layout.element_count, dtype=np.float32))
             return
-        kp, vp = self._gather(key_pool), self._gather(value_pool)
+        kp, vp = (self._gather(key_pool), self._gather(value_pool)) if held is None else held
         entries, gens = self._page_table(table, generations)
         query = self._floats(q)
         hq, sq, width = q.shape
@@ -654,24 +658,35 @@ class CpuBackend:
                 raise BackendError(Status.DEVICE_ERROR_FLAG, index=int(cu_values[lane]))
         p, pt, hkv, width = key_pool.shape
         value_width = value_pool.shape[3]
-        for lane in range(lanes):
-            first, last = int(cu_values[lane]), int(cu_values[lane + 1])
-            count = last - first
-            if count <= 0:
-                continue
-            act = activity.narrow(0, lane, 1) if activity is not None else None
-            table = tables.narrow(0, lane, 1).reshape([tables.shape[1], 2])
-            q_start = int(start_values[lane])
-            key_plane = key_pool.reshape([p, pt, hkv * width])
-            value_plane = value_pool.reshape([p, pt, hkv * value_width])
-            self._paged_copy(k_new.narrow(0, first, count), key_plane, table, generations, act,
-                             INTO_PAGES, q_start, d.op.page_tokens)
-            self._paged_copy(v_new.narrow(0, first, count), value_plane, table, generations, act,
-                             INTO_PAGES, q_start, d.op.page_tokens)
-            lane_q = q.narrow(0, first, count).permute([1, 0, 2])
-            lane_out = out.narrow(0, first, count).permute([1, 0, 2])
-            self._paged_sdpa(lane_q, key_pool, value_pool, table, generations, act, lane_out,
-                             d.op.scale, True, q_start, q_start + count, d.op.page_tokens)
+        # The same sequence of calls per lane, on one copy of each pool's bytes that is written
+        # back when the lanes are through (or a lane has failed): gathering and rewriting both
+        # pools for every lane costs more than the attention itself.
+        whole = (key_pool.layout.is_contiguous() and value_pool.layout.is_contiguous()
+                 and key_pool.writable and value_pool.writable)
+        held = (self._gather(key_pool), self._gather(value_pool)) if whole else None
+        try:
+            for lane in range(lanes):
+                first, last = int(cu_values[lane]), int(cu_values[lane + 1])
+                count = last - first
+                if count <= 0:
+                    continue
+                act = activity.narrow(0, lane, 1) if activity is not None else None
+                table = tables.narrow(0, lane, 1).reshape([tables.shape[1], 2])
+                q_start = int(start_values[lane])
+                key_plane = key_pool.reshape([p, pt, hkv * width])
+                value_plane = value_pool.reshape([p, pt, hkv * value_width])
+                self._paged_copy(k_new.narrow(0, first, count), key_plane, table, generations, act,
+                                 INTO_PAGES, q_start, d.op.page_tokens, held=held and held[0])
+                self._paged_copy(v_new.narrow(0, first, count), value_plane, table, generations, act,
+                                 INTO_PAGES, q_start, d.op.page_tokens, held=held and held[1])
+                lane_q = q.narrow(0, first, count).permute([1, 0, 2])
+                lane_out = out.narrow(0, first, count).permute([1, 0, 2])
+                self._paged_sdpa(lane_q, key_pool, value_pool, table, generations, act, lane_out,
+                                 d.op.scale, True, q_start, q_start + count, d.op.page_tokens, held=held)
+        finally:
+            if held is not None:
+                self.write(key_pool, held[0].tobytes())
+                self.write(value_pool, held[1].tobytes())
 
     def _route_pack(self, d):
         indices = self._u32(d.inputs[0]).reshape(d.inputs[0].shape)

@@ -753,6 +753,12 @@ RAGGED_CASES = [
     ([0, 64], [200, 37], 16, 8, 16),                               # 16 tokens per query group, ragged tails
     ([500], [96], 32, 4, 16),                                      # a chunk continuing a long context
     ([0, 5], [33, 31], 4, 4, 16),                                  # one head per kv head: 32 tokens per group
+    # decode lanes of very different lengths: the split length is the shortest that gives every
+    # work item a place on the device at once
+    ([5000, 100, 2500, 3100, 33, 4000, 777, 1500, 6000, 9000, 7000, 8990], [1] * 12, 8, 8, 16),
+    # more decode lanes than the device holds workgroups, two of them long: split at the even
+    # share of a place, up to the split limit of so many tokens
+    ([3000 if i == 5 else 2000 if i == 200 else (37 * i) % 60 for i in range(300)], [1] * 300, 8, 8, 16),
 ]
 
 

@@ -195,6 +195,10 @@ struct fh_backend {
 
   // Fusion of runs of per-lane attention dispatches: gathered lane metadata followed by the
   // attended rows, kept between the layers of a step (every layer names the same lanes).
+  // The normalisation the dispatch after a weighted sum applies to its rows, offered to the sum
+  // while it is planned, and whether the sum's kernels have produced it.
+  const NormTail *norm_tail = nullptr;
+  bool *norm_tail_taken = nullptr;
   bool lane_fusion = true;
   char *lane_scratch = nullptr;
   uint64_t lane_scratch_bytes = 0;
@@ -718,6 +722,8 @@ fh_status plan_gather(fh_backend *b, const Planned &pl, ErrorSlot *error, bool e
     problem.columns = columns;
     problem.bits = d.bits;
     problem.group = d.group_size;
+    problem.norm_tail = b->norm_tail;
+    problem.norm_tail_taken = b->norm_tail_taken;
     if (!d.epilogue) {
       problem.out = pl.out[0];
       if (try_fast_gather_weighted(b, problem, nullptr, error)) return FH_OK;
@@ -1266,6 +1272,43 @@ fh_status process(fh_backend *b, const fh_dispatch &d, ErrorSlot *error, bool ex
   case FH_OP_FILL_SEEDED: return plan_fill(b, pl, execute);
   default: return FH_UNSUPPORTED_OPERATION;
   }
+}
+
+// ---------------------------------------------------------------- a normalisation after a sum
+//
+// Every decoder layer ends with the MoE weighted sum (+ residual) into the hidden rows and the
+// next layer begins with the RMS normalisation of exactly those rows
+// (engines/qwen3-coder/src/lib.rs records them back to back).  When `next` is that normalisation
+// of what `d` produces, the kernel that forms the rows can write the normalised rows too: same
+// values, one launch less.  Nothing is assumed: `next` is validated as the dispatch it is, reads
+// the produced tensor element for element, and writes nothing that `d` still reads.
+bool find_norm_tail(fh_backend *b, const fh_dispatch &d, const fh_dispatch &next, NormTail *tail) {
+  if (d.op != FH_OP_GATHER_QUANT_MATMUL || next.op != FH_OP_PROGRAM || b->static_mode) return false;
+  if (d.n_outputs != 1 || next.n_inputs != 2 || next.n_outputs != 1) return false;
+  auto program = b->programs.find(next.program);
+  if (program == b->programs.end() || program->second.fast.kind != kProgramRmsNorm) return false;
+  const fh_tensor &made = d.outputs[0], &read = next.inputs[0];
+  if (made.buffer != read.buffer || made.offset != read.offset || made.rank != 2 || read.rank != 2 ||
+      made.dtype != read.dtype)
+    return false;
+  for (uint32_t axis = 0; axis < 2; ++axis)
+    if (made.shape[axis] != read.shape[axis] || made.stride[axis] != read.stride[axis]) return false;
+  // rows of the sum are still being formed while normalised rows are written, and the weights
+  // of the normalisation are read while rows of the sum are written
+  for (uint32_t i = 0; i < d.n_inputs && i < FH_MAX_INPUTS; ++i)
+    if (may_overlap(next.outputs[0], d.inputs[i])) return false;
+  if (may_overlap(next.outputs[0], made) || may_overlap(next.inputs[1], made)) return false;
+  if (process(b, next, nullptr, false) != FH_OK) return false;
+  View in[2], out, produced;
+  if (make_view(b, next.inputs[0], false, &in[0]) != FH_OK ||
+      make_view(b, next.inputs[1], false, &in[1]) != FH_OK ||
+      make_view(b, next.outputs[0], true, &out) != FH_OK || make_view(b, made, true, &produced) != FH_OK)
+    return false;
+  ProgramArgs args;
+  if (bind_program(b, program->second, next.inputs, 2, in, next.outputs, 1, &out, next.outputs[0].shape,
+                   next.outputs[0].rank, &args) != FH_OK)
+    return false;
+  return norm_tail_of(program->second.fast, args, produced, tail);
 }
 
 // ---------------------------------------------------------------- fusion of per-lane attention
@@ -2129,7 +2172,20 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
         }
       }
     } else {
+      NormTail tail;
+      bool tail_taken = false;
+      if (op == FH_OP_GATHER_QUANT_MATMUL && i + 1 < count &&
+          find_norm_tail(b, dispatches[i], dispatches[i + 1], &tail)) {
+        b->norm_tail = &tail;
+        b->norm_tail_taken = &tail_taken;
+      }
       status = process(b, dispatches[i], &s->device_errors[i], true);
+      b->norm_tail = nullptr;
+      b->norm_tail_taken = nullptr;
+      if (tail_taken) {   // the next dispatch has been executed with this one
+        consumed = 2;
+        s->ops[i + 1] = dispatches[i + 1].op;
+      }
     }
     for (uint32_t member = 0; member < consumed; ++member) note_outputs(dispatches[i + member]);
     if (b->profiling >= 2) {

@@ -1383,6 +1383,13 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
     const uint16_t *res = residual ? (const uint16_t *)residual->base + residual->offset : nullptr;
     const uint64_t res_stride = residual ? residual->stride[0] : 0;
     uint16_t *out = (uint16_t *)p.out.base + p.out.offset;
+    if (p.norm_tail && p.k <= 8 && p.columns % 8 == 0 && p.columns <= 2048 && p.out.stride[0] % 8 == 0 &&
+        p.out.offset % 8 == 0 && (!residual || (residual->stride[0] % 8 == 0 && residual->offset % 8 == 0))) {
+      launch_combine_routes_norm(stream, partial, p.indices, p.weights, res, res_stride, out,
+                                 p.out.stride[0], p.rows, p.k, p.columns, p.experts, *p.norm_tail);
+      *p.norm_tail_taken = true;
+      return true;
+    }
     const dim3 grid((unsigned)((work / 4 + 255) / 256));
     if (p.k <= 8)
       combine_routes_rows_kernel<8><<<grid, 256, 0, stream>>>(partial, p.indices, p.weights, res, res_stride,

@@ -348,6 +348,58 @@ def test_gather_projection_pair_and_weighted_sum(cpu, hip, rows, k, experts, n, 
     differential(cpu, hip, build)
 
 
+@pytest.mark.parametrize("form", ["plain", "residual", "norm_into_residual", "norm_of_a_slice",
+                                  "weights_in_the_sum"])
+@pytest.mark.parametrize("rows,k,experts,n,inner", [(128, 8, 128, 768, 2048), (19, 4, 7, 256, 256)])
+def test_weighted_sum_followed_by_the_normalisation_of_its_rows(cpu, hip, rows, k, experts, n, inner, form):
+    """A decoder layer ends with the routed weighted sum and the next begins by normalising those
+    rows (engines/qwen3-coder/src/lib.rs): the backend may run the two as one kernel.  The result
+    must be that of the two dispatches, also where the second is not what the first can absorb: a
+    normalisation that overwrites the sum's residual, one that reads only part of the rows, one
+    whose weights are the rows themselves."""
+    down = Quantised(33, 21, (inner, n), experts=experts)
+    indices = routed_case(33, rows, k, experts, n, inner)
+    activated_values = normal_bf16(33, 40, (rows, k, n))
+    logits = orc.fill_normal_f32(33, 41, rows * k).reshape(rows, k)
+    w_values = np.exp(logits) / np.exp(logits).sum(axis=1, keepdims=True)
+    residual_values = normal_bf16(33, 42, (rows, inner))
+    norm_values = normal_bf16(33, 43, (inner,))
+
+    def build(backend):
+        activated = upload(backend, activated_values, DType.BF16)
+        idx = upload(backend, indices, DType.U32)
+        d = down.upload(backend)
+        weights = upload(backend, w_values, DType.BF16)
+        residual = upload(backend, residual_values, DType.BF16)
+        norm_weight = upload(backend, norm_values, DType.BF16).broadcast((rows, inner))
+        summed = backend.alloc(DType.BF16, (rows, inner))
+        normed = backend.alloc(DType.BF16, (rows, inner))
+        add = backend.prepare_epilogue(programs.add_elements())
+        norm = backend.prepare_program(programs.rms_norm_rows(1e-6))
+        commands = CommandList()
+        outputs = [summed, normed]
+        if form == "plain":
+            commands.dispatch(Op.gather_quant_matmul(4, 64), [activated, *d, idx, weights], summed)
+        else:
+            commands.dispatch_epilogue(Op.gather_quant_matmul(4, 64), [activated, *d, idx, weights], summed,
+                                       add, [residual])
+        if form == "norm_into_residual":
+            commands.dispatch_kernel(norm, [summed, norm_weight], [residual])
+            outputs = [summed, residual]
+        elif form == "norm_of_a_slice":
+            half = rows // 2
+            commands.dispatch_kernel(norm, [summed.narrow(0, 0, half), norm_weight.narrow(0, 0, half)],
+                                     [normed.narrow(0, 0, half)])
+            commands.dispatch(Op.copy(), [summed.narrow(0, half, rows - half)], normed.narrow(0, half, rows - half))
+        elif form == "weights_in_the_sum":
+            commands.dispatch_kernel(norm, [summed, summed], [normed])
+        else:
+            commands.dispatch_kernel(norm, [summed, norm_weight], [normed])
+        return commands, outputs
+    # rows normalised by themselves square the one-ulp differences the sums may have: twice the bar
+    differential(cpu, hip, build, **({"rel": 3e-2} if form == "weights_in_the_sum" else {}))
+
+
 @pytest.mark.parametrize("dtype,bits,group,scale_dtype", [
     (DType.F32, 4, 64, DType.BF16),      # the qwen3-coder engine: f32 activations
     (DType.F16, 8, 32, DType.F16),

@@ -89,24 +89,28 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &problem, const uin
 // 32 per projection of a pair).
 bool ksplit_supports(uint32_t inner, uint32_t columns, bool pair, bool routed);
 struct KsplitDense {
-  const uint16_t *x;
+  const void *x;            // bf16 rows, or f32 rows with `wide`
   uint64_t x_row_stride;
   const uint32_t *packed;
   const uint16_t *scales, *biases;
   void *out;
   uint64_t out_row_stride;
   uint32_t out_f32;
-  const uint16_t *residual;
+  const void *residual;     // rows of the activations' dtype
   uint64_t residual_row_stride;
   uint32_t rows, inner, columns;
+  bool wide;                // f32 activations, residual and result (at most 32 rows)
+  // Non-zero: `inner` is a range of the K of weight rows `weight_inner` long; x, packed, scales and
+  // biases point at the range's first element.
+  uint32_t weight_inner;
 };
 // Whether launch_ksplit_dense takes a product of `rows` rows: at most 128, in row tiles of 16 or
 // 32, and more than one tile only for weights small enough to stay cached between the tiles.
-bool ksplit_dense_supports(uint32_t rows, uint32_t inner, uint32_t columns);
+bool ksplit_dense_supports(uint32_t rows, uint32_t inner, uint32_t columns, bool wide = false);
 // False when ksplit_dense_supports is: nothing was launched.
 bool launch_ksplit_dense(fh_backend *backend, const KsplitDense &problem);
 struct KsplitRouted {
-  const uint16_t *x;
+  const void *x;            // bf16 rows, or f32 rows with `wide`
   uint64_t x_row_stride;
   const uint32_t *packed[2];
   const uint16_t *scales[2], *biases[2];
@@ -116,6 +120,7 @@ struct KsplitRouted {
   uint32_t inner, columns;
   const uint32_t *sorted_routes, *blocks, *n_blocks;
   uint32_t max_blocks, tile_rows, route_div;
+  bool wide;                // f32 activations and results; tiles of 16 routes only
 };
 bool launch_ksplit_routed(fh_backend *backend, const KsplitRouted &problem);
 

@@ -518,28 +518,36 @@ __global__ void argmax_kernel(View in, View out, uint32_t rows, uint32_t width) 
   }
 }
 
-// bf16 rows with a contiguous innermost axis: 16-byte loads, 1024 threads per row.
-__global__ __launch_bounds__(1024) void argmax_bf16_kernel(const uint16_t *in, uint64_t row_stride,
+// bf16 or f32 (kWide) rows with a contiguous innermost axis: 16-byte loads of data read once,
+// 1024 threads per row, eight consecutive elements a thread and step, in ascending order.
+template <bool kWide>
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const void *in, uint64_t row_stride,
                                                            View out, uint32_t width) {
   __shared__ int32_t keys[16];
   __shared__ uint32_t idxs[16];
   const uint32_t row = blockIdx.x;
-  const uint16_t *x = in + (uint64_t)row * row_stride;
   int32_t best_key = (int32_t)0x80000000;
   uint32_t best_index = 0xffffffffu;
   for (uint32_t c = threadIdx.x * 8; c < width; c += 1024 * 8) {
-    uint4 v = *(const uint4 *)(x + c);
-    uint32_t words[4] = {v.x, v.y, v.z, v.w};
-    for (int i = 0; i < 4; ++i) {
-      int32_t lo = total_key(__uint_as_float(words[i] << 16));
-      int32_t hi = total_key(__uint_as_float(words[i] & 0xffff0000u));
-      if (best_index == 0xffffffffu || lo >= best_key) {
-        best_key = lo;
-        best_index = c + 2 * i;
+    float value[8];
+    if constexpr (kWide) {
+      const float *x = (const float *)in + (uint64_t)row * row_stride + c;
+      const uint4 a = stream_load(x), b = stream_load(x + 4);
+      const uint32_t words[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      for (int i = 0; i < 8; ++i) value[i] = __uint_as_float(words[i]);
+    } else {
+      const uint4 v = stream_load((const uint16_t *)in + (uint64_t)row * row_stride + c);
+      const uint32_t words[4] = {v.x, v.y, v.z, v.w};
+      for (int i = 0; i < 4; ++i) {
+        value[2 * i] = __uint_as_float(words[i] << 16);
+        value[2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u);
       }
-      if (hi >= best_key) {
-        best_key = hi;
-        best_index = c + 2 * i + 1;
+    }
+    for (int i = 0; i < 8; ++i) {
+      const int32_t key = total_key(value[i]);
+      if (best_index == 0xffffffffu || key >= best_key) {
+        best_key = key;
+        best_index = c + i;
       }
     }
   }
@@ -948,8 +956,14 @@ void launch_argmax(hipStream_t s, const View &in, const View &out, uint32_t rows
   if (rows == 0) return;
   if (in.dtype == FH_BF16 && in.stride[1] == 1 && width % 8 == 0 && in.offset % 8 == 0 &&
       (rows == 1 || in.stride[0] % 8 == 0)) {
-    argmax_bf16_kernel<<<dim3(rows), 1024, 0, s>>>((const uint16_t *)in.base + in.offset,
-                                                   in.stride[0], out, width);
+    argmax_rows_kernel<false><<<dim3(rows), 1024, 0, s>>>((const uint16_t *)in.base + in.offset,
+                                                          in.stride[0], out, width);
+    return;
+  }
+  if (in.dtype == FH_F32 && in.stride[1] == 1 && width % 8 == 0 && in.offset % 4 == 0 &&
+      (rows == 1 || in.stride[0] % 4 == 0)) {
+    argmax_rows_kernel<true><<<dim3(rows), 1024, 0, s>>>((const float *)in.base + in.offset, in.stride[0],
+                                                         out, width);
     return;
   }
   argmax_kernel<<<dim3(rows), kBlock, 0, s>>>(in, out, rows, width);

@@ -1083,8 +1083,44 @@ const uint16_t *u16_ptr(const View &v) { return (const uint16_t *)v.base + v.off
 
 }  // namespace
 
+namespace {
+
+// f32 activations (the engines' own activation dtype) on the matrix cores: each value goes in as
+// three bf16 pieces that add up to it exactly, so nothing of it is rounded away before the f32
+// accumulation.  Decode batches of at most 32 rows, f32 results.
+bool try_wide_quant_matmul(fh_backend *backend, const QmmProblem &p) {
+  if (p.out.dtype != FH_F32 || p.out.stride[1] != 1) return false;
+  if (!weights_eligible(p.packed, p.scales, p.biases, 2, p.inner, p.bits, p.group)) return false;
+  if (p.x.stride[1] != 1 || p.x.stride[0] % 4 != 0 || p.x.offset % 4 != 0) return false;
+  // K = 4096 (three pieces of so long a slice do not fit the registers): two launches over half
+  // the K each, the second adding to what the first stored
+  const uint32_t ranges = p.inner == 4096 ? 2 : 1, range = p.inner / ranges;
+  if (!ksplit_dense_supports(p.rows, range, p.columns, true)) return false;
+  const float *residual = nullptr;
+  uint64_t residual_row_stride = 0;
+  if (p.residual) {
+    const View &r = *p.residual;
+    if (r.dtype != FH_F32 || r.stride[1] != 1) return false;
+    residual = (const float *)r.base + r.offset;
+    residual_row_stride = r.stride[0];
+  }
+  float *out = (float *)p.out.base + p.out.offset;
+  for (uint32_t i = 0; i < ranges; ++i) {
+    const uint32_t first = i * range;
+    KsplitDense d{(const float *)p.x.base + p.x.offset + first, p.x.stride[0], u32_ptr(p.packed) + first / 8,
+                  u16_ptr(p.scales) + first / kGroup, u16_ptr(p.biases) + first / kGroup, out, p.out.stride[0], 1,
+                  i == 0 ? (const void *)residual : (const void *)out,
+                  i == 0 ? residual_row_stride : p.out.stride[0], p.rows, range, p.columns, true, p.inner};
+    if (!launch_ksplit_dense(backend, d)) return false;   // (refused before anything ran: same answer for every range)
+  }
+  return true;
+}
+
+}  // namespace
+
 bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
   hipStream_t stream = backend_stream(backend);
+  if (p.x.dtype == FH_F32) return try_wide_quant_matmul(backend, p);
   if (p.x.dtype != FH_BF16) return false;
   if (p.out.dtype != FH_BF16 && p.out.dtype != FH_F32) return false;
   if (!weights_eligible(p.packed, p.scales, p.biases, 2, p.inner, p.bits, p.group)) return false;
@@ -1283,8 +1319,88 @@ void launch_combine_routes(hipStream_t stream, const float *partial, const Gathe
       p.k, p.columns, p.experts);
 }
 
+namespace {
+
+// The routed products on f32 activations (three bf16 pieces a value, see try_wide_quant_matmul):
+// tiles of 16 routes, so only while an expert sees few routes on average -- the decode batches of
+// a few lanes the engines run.  `x_rows` input rows of `x_row_stride` elements, `route_div` routes
+// per input row; results are f32 rows of `p.columns`.
+bool launch_wide_routed(fh_backend *backend, const GatherProblem &p, int projections, const float *x,
+                        uint64_t x_row_stride, uint32_t route_div, float *out, const RoutePlan &plan) {
+  KsplitRouted r{};
+  r.x = x;
+  r.x_row_stride = x_row_stride;
+  for (int pj = 0; pj < projections; ++pj) {
+    r.packed[pj] = u32_ptr(p.packed[pj]);
+    r.scales[pj] = u16_ptr(p.scales[pj]);
+    r.biases[pj] = u16_ptr(p.biases[pj]);
+  }
+  r.pair = projections == 2;
+  r.out = out;
+  r.out_f32 = 1;
+  r.inner = p.inner;
+  r.columns = p.columns;
+  r.sorted_routes = plan.sorted_routes;
+  r.blocks = plan.blocks;
+  r.n_blocks = plan.n_blocks;
+  r.max_blocks = plan.max_blocks;
+  r.tile_rows = 16;
+  r.route_div = route_div;
+  r.wide = true;
+  KernelTimer timer(backend, FH_KC_MOE_KERNEL);
+  return launch_ksplit_routed(backend, r);
+}
+
+bool wide_gather_eligible(const GatherProblem &p, int projections) {
+  if (p.x.dtype != FH_F32) return false;
+  for (int pj = 0; pj < projections; ++pj)
+    if (!weights_eligible(p.packed[pj], p.scales[pj], p.biases[pj], 3, p.inner, p.bits, p.group))
+      return false;
+  if ((uint64_t)p.rows * p.k > (1u << 24) || p.experts > 512) return false;
+  return ksplit_route_tile(p, projections == 2) == 16;
+}
+
+bool try_wide_gather_projection(fh_backend *backend, const GatherProblem &p, int projections,
+                                bool swiglu, ErrorSlot *error) {
+  if (!wide_gather_eligible(p, projections) || (projections == 2 && !swiglu)) return false;
+  if (p.out.dtype != FH_F32) return false;
+  if (p.x.stride[1] != 1 || p.x.stride[0] % 4 != 0 || p.x.offset % 4 != 0) return false;
+  if (p.out.stride[2] != 1 || p.out.stride[1] != p.columns ||
+      p.out.stride[0] != (uint64_t)p.k * p.columns)
+    return false;
+  // rows of bad routes read zero: cleared by the packing kernel as it meets them, or all rows
+  // first when an earlier plan is reused (see try_fast_gather_projection)
+  RoutePlan plan;
+  float *out = (float *)p.out.base + p.out.offset;
+  if (!plan_routes(backend, p, 0, error, &plan, (uint32_t *)out, p.columns, 16)) return false;
+  if (plan.reused)
+    launch_fill_u32(backend_stream(backend), (uint32_t *)out, (uint64_t)p.rows * p.k * p.columns, 0);
+  return launch_wide_routed(backend, p, projections, (const float *)p.x.base + p.x.offset, p.x.stride[0],
+                            p.k, out, plan);
+}
+
+bool try_wide_gather_weighted(fh_backend *backend, const GatherProblem &p, const View *residual,
+                              ErrorSlot *error) {
+  if (!wide_gather_eligible(p, 1)) return false;
+  if (p.x.stride[2] != 1 || p.x.stride[1] % 4 != 0 || p.x.offset % 4 != 0 ||
+      p.x.stride[0] != (uint64_t)p.k * p.x.stride[1])
+    return false;
+  const uint64_t partial_bytes = (uint64_t)p.rows * p.k * p.columns * sizeof(float);
+  RoutePlan plan;
+  if (!plan_routes(backend, p, partial_bytes, error, &plan, nullptr, 0, 16)) return false;
+  float *partial = (float *)plan.rest;
+  if (!launch_wide_routed(backend, p, 1, (const float *)p.x.base + p.x.offset, p.x.stride[1], 1, partial,
+                          plan))
+    return false;
+  launch_combine_routes(backend_stream(backend), partial, p, residual);
+  return true;
+}
+
+}  // namespace
+
 bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int projections,
                                 bool swiglu, ErrorSlot *error) {
+  if (p.x.dtype == FH_F32) return try_wide_gather_projection(backend, p, projections, swiglu, error);
   if (!gather_eligible(p, projections)) return false;
   if (projections == 2 && !swiglu) return false;
   if (p.out.dtype != FH_BF16 || ((uint64_t)p.rows * p.k * p.columns) % 2 != 0) return false;
@@ -1339,6 +1455,7 @@ bool try_fast_gather_projection(fh_backend *backend, const GatherProblem &p, int
 
 bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const View *residual,
                               ErrorSlot *error) {
+  if (p.x.dtype == FH_F32) return try_wide_gather_weighted(backend, p, residual, error);
   if (!gather_eligible(p, 1)) return false;
   // x [R,k,K] dense rows so that route r*k+s is row r*k+s of [R*k, K]
   if (p.x.stride[2] != 1 || p.x.stride[1] % 8 != 0 || p.x.offset % 8 != 0 ||

@@ -43,7 +43,7 @@ constexpr int kGroup = 64;
 constexpr uint32_t kNoBlock = 0xffffffffu;
 
 struct KsplitArgs {
-  const uint16_t *x;        // bf16 activations, innermost axis contiguous
+  const void *x;            // bf16 (or, in the three-piece form, f32) activations, innermost axis contiguous
   uint64_t x_row_stride;    // elements between input rows
   const uint32_t *packed[2];
   const uint16_t *scales[2], *biases[2];
@@ -52,9 +52,10 @@ struct KsplitArgs {
   void *out;                // bf16 or f32
   uint64_t out_row_stride;  // elements
   uint32_t out_f32;
-  const uint16_t *residual; // dense only: optional bf16 rows added before the result is rounded
+  const void *residual;     // dense only: optional rows (of the activations' dtype) added before the result is rounded
   uint64_t residual_row_stride;
   uint32_t rows, inner, columns;
+  uint32_t weight_inner;    // K of the weight matrix: the length of its rows (>= inner)
   // routed form: tiles (expert, first, count) over sorted_routes; input row = route / route_div
   const uint32_t *sorted_routes, *blocks, *n_blocks;
   uint32_t route_div;
@@ -138,13 +139,19 @@ typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
 // Waves per SIMD the registers must leave room for: two workgroups per compute unit where the
 // stationary rows are few (one contracts while the other waits at its exchange barrier).
-constexpr int resident_waves(int waves, int row_tiles, int groups, bool routed) {
-  const bool two = row_tiles == 1 ? groups <= 4 : groups <= 2 && waves <= 6 && routed;
+constexpr int resident_waves(int waves, int row_tiles, int groups, bool routed, int pieces) {
+  const bool two = pieces > 1 ? false : row_tiles == 1 ? groups <= 4 : groups <= 2 && waves <= 6 && routed;
   return two ? (2 * waves + 3) / 4 : (waves + 3) / 4;
 }
 
-template <int WAVES, int G, int RT, bool kPair, bool kRouted>
-__global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) void qmm_ksplit_kernel(KsplitArgs a) {
+// XP = bf16 pieces an activation is held in: 1 for bf16 rows; 3 for f32 rows, each value split
+// exactly into the bf16 numbers of its high, middle and low eight significant bits, so that the
+// three products with a weight operand (exact 16+q in bf16) add up, in the f32 accumulator, to
+// the product with the f32 value itself.  The stationary rows then take three times the
+// registers: one 16-row tile, one workgroup per compute unit.
+template <int WAVES, int G, int RT, bool kPair, bool kRouted, int XP>
+__global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted, XP)) void qmm_ksplit_kernel(KsplitArgs a) {
+  static_assert(XP == 1 || (XP == 3 && RT == 1), "f32 rows: one row tile");
   constexpr int P = kPair ? 2 : 1;
   constexpr int NS = ring_slots(RT, G, kRouted);
   constexpr int CT = batch_tiles(kPair, G);
@@ -177,7 +184,8 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   uint32_t *scale_lds = (uint32_t *)(exchange + 2 * WAVES * kSlots * 4 * 64);   // [2][kPieces][W2]
   const uint32_t lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t words_per_row = a.inner / 8, groups_per_row = a.inner / kGroup;
+  // a weight row may be longer than the K this launch contracts (one of several K ranges)
+  const uint32_t words_per_row = a.weight_inner / 8, groups_per_row = a.weight_inner / kGroup;
   const uint32_t tiles = kRouted ? table_word(a.n_blocks, 0) : (a.rows + 16 * RT - 1) / (16 * RT);
   const uint32_t units = tiles * a.batches_per_tile;
   const uint32_t first_unit = (uint32_t)((uint64_t)blockIdx.x * units / gridDim.x);
@@ -188,7 +196,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
   // contiguous bytes of each of 16 weight rows; two half-wave swaps then leave the lane quarters
   // g = 0..3 holding words (0,4,2,6) and (1,5,3,7) of ONE group, and the activations are laid out
   // to match: quarter g holds the group's values [16 g', 16 g' + 16), g' = (0,2,1,3)[g].
-  uint4 xa[RT][G][2];      // A operands: [row tile][group][half of the lane's 16 values]
+  uint4 xa[XP][RT][G][2];  // A operands: [piece][row tile][group][half of the lane's 16 values]
   float xs[RT][Q];         // sum of the row's activations over group 4q + g (bias term operand)
   uint32_t out_rows[RT][4]; // output row of accumulator (row tile, i): tile row 16 rt + 4 g + i
   uint32_t tile_first = 0, tile_count = 0, current_tile = kNoBlock;
@@ -219,17 +227,51 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
       const uint32_t row = 16 * rt + n;
       const uint32_t safe = row < tile_count ? row : 0;
       const uint64_t in_row = kRouted ? a.sorted_routes[tile_first + safe] / a.route_div : tile_first + safe;
-      const uint16_t *xp = a.x + in_row * a.x_row_stride + (uint64_t)wave * (G * kGroup) + 16 * g_perm;
+      const uint64_t x_at = in_row * a.x_row_stride + (uint64_t)wave * (G * kGroup) + 16 * g_perm;
       float sums[G];
 #pragma unroll
       for (int j = 0; j < G; ++j) {
-        const uint4 lo = *(const uint4 *)(xp + kGroup * j), hi = *(const uint4 *)(xp + kGroup * j + 8);
-        float s = sum8(lo) + sum8(hi);
+        float s;
+        if constexpr (XP == 1) {
+          const uint16_t *xp = (const uint16_t *)a.x + x_at;
+          const uint4 lo = *(const uint4 *)(xp + kGroup * j), hi = *(const uint4 *)(xp + kGroup * j + 8);
+          s = sum8(lo) + sum8(hi);
+          xa[0][rt][j][0] = permute_slots(lo);
+          xa[0][rt][j][1] = permute_slots(hi);
+        } else {
+          const float *xp = (const float *)a.x + x_at + kGroup * j;
+          float value[16];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const float4 four = *(const float4 *)(xp + 4 * v);
+            value[4 * v] = four.x, value[4 * v + 1] = four.y, value[4 * v + 2] = four.z, value[4 * v + 3] = four.w;
+          }
+          s = 0.0f;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) s += value[v];
+          // piece 0 = low bits ... piece 2 = high bits: the small products are added first
+#pragma unroll
+          for (int piece = XP - 1; piece >= 0; --piece) {
+            uint32_t top[16];   // the piece's bf16 bits in the upper half of a word
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              top[v] = __float_as_uint(value[v]) & 0xffff0000u;
+              value[v] -= __uint_as_float(top[v]);   // exact: what the lower pieces hold
+            }
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+              uint4 packed;   // eight consecutive values, two to a word, as bf16 rows hold them
+              packed.x = __builtin_amdgcn_perm(top[8 * half + 1], top[8 * half + 0], 0x07060302u);
+              packed.y = __builtin_amdgcn_perm(top[8 * half + 3], top[8 * half + 2], 0x07060302u);
+              packed.z = __builtin_amdgcn_perm(top[8 * half + 5], top[8 * half + 4], 0x07060302u);
+              packed.w = __builtin_amdgcn_perm(top[8 * half + 7], top[8 * half + 6], 0x07060302u);
+              xa[piece][rt][j][half] = permute_slots(packed);
+            }
+          }
+        }
         s += __shfl_xor(s, 16, 64);      // the four quarters of the group
         s += __shfl_xor(s, 32, 64);
         sums[j] = s;
-        xa[rt][j][0] = permute_slots(lo);
-        xa[rt][j][1] = permute_slots(hi);
       }
 #pragma unroll
       for (int q = 0; q < Q; ++q) {
@@ -298,7 +340,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
       const uint16_t *base = (sub % 2 ? a.biases[pj] : a.scales[pj]) + (uint64_t)(16 * ct) * groups_per_row;
       if (block == (uint32_t)sub) from = base;
     }
-    share_from[i] = from + (uint64_t)inside * G;
+    share_from[i] = from + (uint64_t)(inside / WAVES) * groups_per_row + (inside % WAVES) * G;
   }
   auto load_share = [&](Share &r, const Cursor &c) {
     if constexpr (!kStage) return;
@@ -318,6 +360,13 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
 #pragma unroll
       for (int k = 0; k < W2; ++k) to[k] = r.words[i][k];
     }
+  };
+  // The value added to result (row, column), as the bits of its dtype (any readable word when
+  // there is no residual: the load is unconditional).
+  auto residual_at = [&](uint32_t row, uint32_t column) -> uint32_t {
+    const uint64_t at = (uint64_t)row * a.residual_row_stride + column;
+    if constexpr (XP == 1) return *(a.residual ? (const uint16_t *)a.residual + at : (const uint16_t *)a.x);
+    return *(a.residual ? (const uint32_t *)a.residual + at : (const uint32_t *)a.x);
   };
   auto load_batch = [&](Batch &r, const Cursor &c) {
     const uint32_t batch = c.batch;
@@ -352,8 +401,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const uint32_t row = min(c.tile * (16 * RT) + 16 * rt + 4 * g + i, a.rows - 1);
-            const uint16_t *rp = a.residual ? a.residual + (uint64_t)row * a.residual_row_stride + column : a.x;
-            r.residual[4 * qq + i] = *rp;
+            r.residual[4 * qq + i] = residual_at(row, column);
           }
         }
       } else {
@@ -363,8 +411,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
           const uint32_t ct = t / (RT * 4), rt = (t / 4) % RT, i = t % 4;
           const uint32_t row = min(c.tile * (16 * RT) + 16 * rt + 4 * g + i, a.rows - 1);
           const uint32_t column = min(batch * kBatchCols + 16 * ct + n, a.columns - 1);
-          const uint16_t *rp = a.residual ? a.residual + (uint64_t)row * a.residual_row_stride + column : a.x;
-          r.residual[tt] = *rp;
+          r.residual[tt] = residual_at(row, column);
         }
       }
     }
@@ -422,8 +469,11 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         part[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        part[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[rt][j][0]), b0, part[rt], 0, 0, 0);
-        part[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[rt][j][1]), b1, part[rt], 0, 0, 0);
+#pragma unroll
+        for (int piece = 0; piece < XP; ++piece) {
+          part[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[piece][rt][j][0]), b0, part[rt], 0, 0, 0);
+          part[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[piece][rt][j][1]), b1, part[rt], 0, 0, 0);
+        }
       }
       if (s > 0) {
         const int before = (s - 1) / G;
@@ -444,7 +494,7 @@ __global__ __launch_bounds__(64 * WAVES, resident_waves(WAVES, RT, G, kRouted)) 
     // One result: activation of a pair, residual of a dense product, rounding, store.
     auto store_result = [&](float value, float up, uint32_t out_row, uint32_t column, uint32_t residual_bits) {
       if (kPair) value = value * (1.0f / (1.0f + __expf(-value))) * up;
-      if (!kRouted && a.residual) value += bf16_bits(residual_bits & 0xffffu);
+      if (!kRouted && a.residual) value += XP == 1 ? bf16_bits(residual_bits & 0xffffu) : __uint_as_float(residual_bits);
       const uint64_t at = (uint64_t)out_row * a.out_row_stride + column;
       if (a.out_f32)
         ((float *)a.out)[at] = value;
@@ -590,12 +640,12 @@ bool ksplit_shape(uint32_t inner, int *waves, int *groups) {
 
 // One launch: as many workgroups as stay resident at once (the runtime's own occupancy figure for
 // this instantiation), never more than there are units of work.
-template <int WAVES, int G, int RT, bool kPair, bool kRouted>
+template <int WAVES, int G, int RT, bool kPair, bool kRouted, int XP>
 void launch_one(fh_backend *backend, const KsplitArgs &a, uint64_t most_units) {
   constexpr int P = kPair ? 2 : 1, CT = batch_tiles(kPair, G);
   constexpr uint32_t lds = 2u * WAVES * (CT * P * RT * 4) * 64 * sizeof(float) +   // partial sums
                            (RT == 1 ? 2u * (P * CT * 2 * 16 * WAVES) * (G / 2) * sizeof(uint32_t) : 0u);   // scales and biases
-  const void *kernel = reinterpret_cast<const void *>(&qmm_ksplit_kernel<WAVES, G, RT, kPair, kRouted>);
+  const void *kernel = reinterpret_cast<const void *>(&qmm_ksplit_kernel<WAVES, G, RT, kPair, kRouted, XP>);
   static int per_unit = 0;   // set once per process: the dynamic LDS limit and the occupancy
   if (per_unit == 0) {
     (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -606,28 +656,28 @@ void launch_one(fh_backend *backend, const KsplitArgs &a, uint64_t most_units) {
   }
   const uint64_t resident = (uint64_t)backend_compute_units(backend) * (uint32_t)per_unit;
   const uint32_t grid = (uint32_t)(most_units < resident ? most_units : resident);
-  qmm_ksplit_kernel<WAVES, G, RT, kPair, kRouted><<<dim3(grid), 64 * WAVES, lds, backend_stream(backend)>>>(a);
+  qmm_ksplit_kernel<WAVES, G, RT, kPair, kRouted, XP><<<dim3(grid), 64 * WAVES, lds, backend_stream(backend)>>>(a);
 }
 
-template <int RT, bool kPair, bool kRouted>
+template <int RT, bool kPair, bool kRouted, int XP>
 bool launch_shape(fh_backend *backend, const KsplitArgs &a, uint64_t most_units) {
   int waves = 0, groups = 0;
   if (!ksplit_shape(a.inner, &waves, &groups)) return false;
   switch (waves * 16 + groups) {
-  case 4 * 16 + 2: launch_one<4, 2, RT, kPair, kRouted>(backend, a, most_units); return true;
-  case 6 * 16 + 2: launch_one<6, 2, RT, kPair, kRouted>(backend, a, most_units); return true;
-  case 8 * 16 + 2: launch_one<8, 2, RT, kPair, kRouted>(backend, a, most_units); return true;
-  case 6 * 16 + 4: launch_one<6, 4, RT, kPair, kRouted>(backend, a, most_units); return true;
-  case 8 * 16 + 4: launch_one<8, 4, RT, kPair, kRouted>(backend, a, most_units); return true;
+  case 4 * 16 + 2: launch_one<4, 2, RT, kPair, kRouted, XP>(backend, a, most_units); return true;
+  case 6 * 16 + 2: launch_one<6, 2, RT, kPair, kRouted, XP>(backend, a, most_units); return true;
+  case 8 * 16 + 2: launch_one<8, 2, RT, kPair, kRouted, XP>(backend, a, most_units); return true;
+  case 6 * 16 + 4: launch_one<6, 4, RT, kPair, kRouted, XP>(backend, a, most_units); return true;
+  case 8 * 16 + 4: launch_one<8, 4, RT, kPair, kRouted, XP>(backend, a, most_units); return true;
   default: break;
   }
-  if constexpr (RT == 1 && !kRouted) {   // the long rows of dense decode products
+  if constexpr (RT == 1 && !kRouted && XP == 1) {   // the long rows of dense decode products
     if (waves == 8 && groups == 6) {
-      launch_one<8, 6, 1, false, false>(backend, a, most_units);
+      launch_one<8, 6, 1, false, false, 1>(backend, a, most_units);
       return true;
     }
     if (waves == 8 && groups == 8) {
-      launch_one<8, 8, 1, false, false>(backend, a, most_units);
+      launch_one<8, 8, 1, false, false, 1>(backend, a, most_units);
       return true;
     }
   }
@@ -647,10 +697,12 @@ bool ksplit_supports(uint32_t inner, uint32_t columns, bool pair, bool routed) {
 // first find the weights in the caches in front of HBM.
 constexpr uint64_t kCachedWeightBytes = 32ull << 20;
 
-bool ksplit_dense_supports(uint32_t rows, uint32_t inner, uint32_t columns) {
+bool ksplit_dense_supports(uint32_t rows, uint32_t inner, uint32_t columns, bool wide) {
   int waves = 0, groups = 0;
   if (rows == 0 || rows > 128 || !ksplit_shape(inner, &waves, &groups)) return false;
   if (!ksplit_supports(inner, columns, false, false)) return false;
+  // f32 rows: 16-row tiles of K slices of at most four groups, two passes at most
+  if (wide) return groups <= 4 && rows <= 32 && (rows <= 16 || (uint64_t)columns * inner / 2 <= kCachedWeightBytes);
   const uint32_t tile_rows = rows > 16 && groups <= 4 ? 32 : 16;
   // (row tiles of 16, which the long K slices are held to, would take eight passes for 128 rows)
   return rows <= tile_rows || (groups <= 4 && (uint64_t)columns * inner / 2 <= kCachedWeightBytes);
@@ -658,8 +710,9 @@ bool ksplit_dense_supports(uint32_t rows, uint32_t inner, uint32_t columns) {
 
 bool launch_ksplit_dense(fh_backend *backend, const KsplitDense &d) {
   int waves = 0, groups = 0;
-  if (!ksplit_dense_supports(d.rows, d.inner, d.columns) || !ksplit_shape(d.inner, &waves, &groups)) return false;
-  const bool wide_tiles = d.rows > 16 && groups <= 4;
+  if (!ksplit_dense_supports(d.rows, d.inner, d.columns, d.wide) || !ksplit_shape(d.inner, &waves, &groups)) return false;
+  if (d.wide && !d.out_f32) return false;
+  const bool wide_tiles = d.rows > 16 && groups <= 4 && !d.wide;
   KsplitArgs a{};
   a.x = d.x;
   a.x_row_stride = d.x_row_stride;
@@ -673,14 +726,16 @@ bool launch_ksplit_dense(fh_backend *backend, const KsplitDense &d) {
   a.residual_row_stride = d.residual_row_stride;
   a.rows = d.rows;
   a.inner = d.inner;
+  a.weight_inner = d.weight_inner ? d.weight_inner : d.inner;
   a.columns = d.columns;
   const uint32_t batch_cols = 16 * batch_tiles(false, groups);
   a.batches_per_tile = (d.columns + batch_cols - 1) / batch_cols;
   const uint32_t tile_rows = wide_tiles ? 32 : 16;
   const uint64_t units = (uint64_t)((d.rows + tile_rows - 1) / tile_rows) * a.batches_per_tile;
   KernelTimer timer(backend, FH_KC_QMM_KERNEL);
-  return wide_tiles ? launch_shape<2, false, false>(backend, a, units)
-                    : launch_shape<1, false, false>(backend, a, units);
+  if (d.wide) return launch_shape<1, false, false, 3>(backend, a, units);
+  return wide_tiles ? launch_shape<2, false, false, 1>(backend, a, units)
+                    : launch_shape<1, false, false, 1>(backend, a, units);
 }
 
 bool launch_ksplit_routed(fh_backend *backend, const KsplitRouted &r) {
@@ -702,6 +757,7 @@ bool launch_ksplit_routed(fh_backend *backend, const KsplitRouted &r) {
   a.out_row_stride = r.columns;
   a.out_f32 = r.out_f32;
   a.inner = r.inner;
+  a.weight_inner = r.inner;
   a.columns = r.columns;
   a.sorted_routes = r.sorted_routes;
   a.blocks = r.blocks;
@@ -710,11 +766,15 @@ bool launch_ksplit_routed(fh_backend *backend, const KsplitRouted &r) {
   const uint32_t batch_cols = 16 * batch_tiles(r.pair, groups);
   a.batches_per_tile = (r.columns + batch_cols - 1) / batch_cols;
   const uint64_t most = (uint64_t)r.max_blocks * a.batches_per_tile;
+  if (r.wide) {   // f32 rows: 16-row tiles, f32 results
+    if (r.tile_rows != 16 || !r.out_f32) return false;
+    return r.pair ? launch_shape<1, true, true, 3>(backend, a, most) : launch_shape<1, false, true, 3>(backend, a, most);
+  }
   if (r.pair)
-    return r.tile_rows == 16 ? launch_shape<1, true, true>(backend, a, most)
-                             : launch_shape<2, true, true>(backend, a, most);
-  return r.tile_rows == 16 ? launch_shape<1, false, true>(backend, a, most)
-                           : launch_shape<2, false, true>(backend, a, most);
+    return r.tile_rows == 16 ? launch_shape<1, true, true, 1>(backend, a, most)
+                             : launch_shape<2, true, true, 1>(backend, a, most);
+  return r.tile_rows == 16 ? launch_shape<1, false, true, 1>(backend, a, most)
+                           : launch_shape<2, false, true, 1>(backend, a, most);
 }
 
 }  // namespace fh

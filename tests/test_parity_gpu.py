@@ -190,6 +190,64 @@ def test_quant_matmul(cpu, hip, rows, n, k, bits, group, dtype):
     differential(cpu, hip, build)
 
 
+@pytest.mark.parametrize("rows,n,k,residual", [(8, 5120, 2048, False), (1, 2048, 768, False), (16, 768, 2048, True),
+                                               (20, 2048, 1024, True), (31, 96, 512, False),
+                                               (8, 2048, 4096, True), (24, 512, 4096, False)])   # o_proj: two K ranges
+def test_quant_matmul_on_f32_activations_that_use_their_whole_mantissa(cpu, hip, rows, n, k, residual):
+    """The engines' activations are f32 (engines/qwen3-coder/src/lib.rs:296-437) and carry 24
+    significant bits, unlike the bf16-valued inputs of the cases above: a kernel that rounded them
+    to bf16, or to two bf16 pieces, on its way to the matrix cores would miss the f32 bar."""
+    weights = Quantised(25, n + k, (n, k))
+    x_values = orc.fill_normal_f32(25, 1, rows * k).reshape(rows, k)
+    extra_values = orc.fill_normal_f32(25, 2, rows * n).reshape(rows, n)
+
+    def build(backend):
+        x = upload(backend, x_values, DType.F32)
+        out = backend.alloc(DType.F32, (rows, n))
+        commands = CommandList()
+        if residual:
+            extra = upload(backend, extra_values, DType.F32)
+            add = backend.prepare_epilogue(programs.add_elements())
+            commands.dispatch_epilogue(Op.quant_matmul(4, 64), [x, *weights.upload(backend)], out, add, [extra])
+        else:
+            commands.dispatch(Op.quant_matmul(4, 64), [x, *weights.upload(backend)], out)
+        return commands, [out]
+    differential(cpu, hip, build)
+
+
+@pytest.mark.parametrize("rows,k,experts,n,inner", [(8, 8, 128, 768, 2048), (3, 4, 16, 512, 1024), (40, 2, 64, 256, 512)])
+def test_routed_products_on_f32_activations_that_use_their_whole_mantissa(cpu, hip, rows, k, experts, n, inner):
+    """The MoE block of a small decode batch in the engine's dtypes: gate/up pair with SwiGLU, the
+    down projection as a weighted sum with the residual, all f32."""
+    gate = Quantised(26, 1, (n, inner), experts=experts)
+    up = Quantised(26, 11, (n, inner), experts=experts)
+    down = Quantised(26, 21, (inner, n), experts=experts)
+    indices = routed_case(26, rows, k, experts, n, inner)
+    x_values = orc.fill_normal_f32(26, 40, rows * inner).reshape(rows, inner)
+    logits = orc.fill_normal_f32(26, 41, rows * k).reshape(rows, k)
+    w_values = np.exp(logits) / np.exp(logits).sum(axis=1, keepdims=True)
+    residual_values = orc.fill_normal_f32(26, 42, rows * inner).reshape(rows, inner)
+
+    def build(backend):
+        x = upload(backend, x_values, DType.F32)
+        idx = upload(backend, indices, DType.U32)
+        g, u, d = gate.upload(backend), up.upload(backend), down.upload(backend)
+        plain = backend.alloc(DType.F32, (rows, k, n))
+        activated = backend.alloc(DType.F32, (rows, k, n))
+        combined = backend.alloc(DType.F32, (rows, inner))
+        weights = upload(backend, w_values, DType.F32)
+        residual = upload(backend, residual_values, DType.F32)
+        swiglu = backend.prepare_epilogue(programs.silu_mul_elements())
+        add = backend.prepare_epilogue(programs.add_elements())
+        commands = CommandList()
+        commands.dispatch(Op.gather_quant_matmul(4, 64), [x, *g, idx], plain)
+        commands.dispatch_epilogue(Op.gather_quant_matmul(4, 64), [x, *g, *u, idx], activated, swiglu, [])
+        commands.dispatch_epilogue(Op.gather_quant_matmul(4, 64), [activated, *d, idx, weights], combined,
+                                   add, [residual])
+        return commands, [plain, activated, combined]
+    differential(cpu, hip, build)
+
+
 @pytest.mark.parametrize("dtype,bits,group", [(DType.F32, 4, 64), (DType.F16, 8, 32), (DType.BF16, 4, 128)])
 def test_quant_matmul_with_f16_scales_and_a_residual_in_other_dtypes(cpu, hip, dtype, bits, group):
     """f16 affine parameters (the reference allows f16 or bf16, quantized.rs:78-121) and the
@@ -584,10 +642,12 @@ def test_argmax_ties_and_vocabulary_width(cpu, hip):
 
     def build(backend):
         a, b = upload(backend, logits, DType.BF16), upload(backend, small, DType.F32)
-        outs = [backend.alloc(DType.U32, (4,)), backend.alloc(DType.U32, (1,))]
+        c = upload(backend, logits, DType.F32)             # the engine's f32 logits
+        outs = [backend.alloc(DType.U32, (4,)), backend.alloc(DType.U32, (1,)), backend.alloc(DType.U32, (4,))]
         commands = CommandList()
         commands.dispatch(Op.argmax(), [a], outs[0])
         commands.dispatch(Op.argmax(), [b], outs[1])
+        commands.dispatch(Op.argmax(), [c], outs[2])
         return commands, outs
     (_, _), (hip_out, _) = differential(cpu, hip, build)
     assert np.frombuffer(hip.read(hip_out[1]), np.uint32).tolist() == [3]

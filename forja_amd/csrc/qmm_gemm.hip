@@ -49,10 +49,15 @@ constexpr int kPadK = 64;   // operand rows are padded to a multiple of this (ev
 // K step and LDS stages of the GEMM.  Steps of 32 with three or four stages measured the same
 // (the kernel is bound by what the matrix cores and the L2 -> LDS path sustain, not by latency).
 constexpr int kGemmK = 64, kGemmStages = 2;
-constexpr int kOutPitch = 2 * 128 + 16;           // bytes per row of a wave's staged output quadrant
-constexpr int kGemmPipelineLds = kGemmStages * 2 * kBM * 2 * kGemmK;   // both operand tiles of every stage
-constexpr int kGemmOutputLds = 4 * (128 * kOutPitch + 512);            // four quadrants of bf16 rows + row factors
-constexpr int kGemmLds = kGemmPipelineLds > kGemmOutputLds ? kGemmPipelineLds : kGemmOutputLds;
+// A tile is 2 x 2 quadrants of kQ x kQ, one per wave: kQ = 128 (256 x 256 tiles) wherever that
+// gives every compute unit work, kQ = 64 (128 x 128 tiles, four times as many) for the small
+// products of small models, which would otherwise leave most of the device idle.
+constexpr int out_pitch(int quadrant) { return 2 * quadrant + 16; }   // bytes per row of a wave's staged output quadrant
+constexpr int gemm_lds_bytes(int quadrant) {
+  const int pipeline = kGemmStages * 2 * (2 * quadrant) * 2 * kGemmK;   // both operand tiles of every stage
+  const int output = 4 * (quadrant * out_pitch(quadrant) + 4 * quadrant);   // four quadrants of bf16 rows + row factors
+  return pipeline > output ? pipeline : output;
+}
 constexpr int kBand = 8;   // column tiles per band of the tile numbering
 constexpr uint32_t kMaxGroups = 512;              // quantisation groups per row the row kernel holds
 
@@ -225,15 +230,19 @@ constexpr uint32_t wait_vmcnt(uint32_t n) {   // s_waitcnt immediate: vmcnt(n) o
   return (n & 15u) | ((n >> 4) << 14) | 0x0f70u;
 }
 
-template <int kBK, int kStages>
+template <int kBK, int kStages, int kQ>
 __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   if (a.refused[0] != 0) return;
+  constexpr int kSide = 2 * kQ;                  // rows (and columns) of a tile
+  constexpr int kMI = kQ / 32;                   // 32 x 32 blocks along a quadrant's side
+  constexpr int kOutPitch = out_pitch(kQ);
   constexpr int kSub = kBK / 16;                 // MFMA sub-steps per K step
   constexpr int kRowBytes = 2 * kBK;             // one tile row in LDS
-  constexpr int kTile = kBM * kRowBytes;         // one operand tile of one stage
+  constexpr int kTile = kSide * kRowBytes;       // one operand tile of one stage
   constexpr int kSlots = kRowBytes / 16;         // 16-byte pieces per row
   constexpr int kRowsPerLoad = 64 / kSlots;      // rows one wave-wide load instruction covers
-  constexpr int kLoads = 64 / kRowsPerLoad;      // instructions per wave, operand and stage
+  constexpr int kStaged = kSide / 4;             // rows of each operand tile a wave stages
+  constexpr int kLoads = kStaged / kRowsPerLoad; // instructions per wave, operand and stage
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
   unsigned char *a_tiles = gemm_lds;                      // [kStages][kBM][kRowBytes], pieces swizzled
   unsigned char *b_tiles = gemm_lds + kStages * kTile;    // [kStages][kBN][kRowBytes]
@@ -258,7 +267,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   const uint32_t band_width = min((uint32_t)kBand, a.column_tiles - band * kBand);
   const uint32_t in_band = tile - band * a.row_tiles * kBand;
   const uint32_t bm = in_band / band_width, bn = band * kBand + in_band % band_width;
-  const uint32_t row0 = bm * kBM, col0 = bn * kBN;
+  const uint32_t row0 = bm * kSide, col0 = bn * kSide;
 
   // Staging: a wave owns 64 rows of each operand tile; one instruction moves kRowsPerLoad rows
   // (lane -> row lane / kSlots, LDS slot lane % kSlots) and the piece a lane fetches is its slot
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   uint32_t a_off[kLoads], b_off[kLoads];
 #pragma unroll
   for (int i = 0; i < kLoads; ++i) {
-    const uint32_t in_tile = 64 * wave + kRowsPerLoad * i + lane / kSlots;
+    const uint32_t in_tile = kStaged * wave + kRowsPerLoad * i + lane / kSlots;
     const uint32_t piece = (lane % kSlots) ^ swizzle_of(in_tile);
     a_off[i] = (min(row0 + in_tile, a.rows - 1) * a.kt + 8 * piece) * 2;
     b_off[i] = (min(col0 + in_tile, a.columns - 1) * a.kt + 8 * piece) * 2;
@@ -279,31 +288,31 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
     const uint32_t st = min(step, steps - 1);   // past the end: reload the last step, never used
     const unsigned char *from_a = (const unsigned char *)a.a + (uint64_t)st * (kBK * 2);
     const unsigned char *from_b = (const unsigned char *)a.b + (uint64_t)st * (kBK * 2);
-    unsigned char *to_a = a_tiles + buffer * kTile + (64 * wave + kRowsPerLoad * i) * kRowBytes;
-    unsigned char *to_b = b_tiles + buffer * kTile + (64 * wave + kRowsPerLoad * i) * kRowBytes;
+    unsigned char *to_a = a_tiles + buffer * kTile + (kStaged * wave + kRowsPerLoad * i) * kRowBytes;
+    unsigned char *to_b = b_tiles + buffer * kTile + (kStaged * wave + kRowsPerLoad * i) * kRowBytes;
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from_a + a_off[i]),
                                      (__attribute__((address_space(3))) void *)to_a, 16, 0, 0);
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from_b + b_off[i]),
                                      (__attribute__((address_space(3))) void *)to_b, 16, 0, 0);
   };
 
-  f32x16 acc[4][4];
+  f32x16 acc[kMI][kMI];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < kMI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < kMI; ++j)
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   // Operand registers, two sets: the set for the next sub-step is read from LDS while the matrix
   // pipe works on the current one.
-  f16x8 a_op[2][4], b_op[2][4];
+  f16x8 a_op[2][kMI], b_op[2][kMI];
   const uint32_t swizzle = swizzle_of(l32);
   auto read_operands = [&](uint32_t buffer, int s, int set) {
-    const unsigned char *at = a_tiles + buffer * kTile + (128 * wm + l32) * kRowBytes;
-    const unsigned char *bt = b_tiles + buffer * kTile + (128 * wn + l32) * kRowBytes;
+    const unsigned char *at = a_tiles + buffer * kTile + (kQ * wm + l32) * kRowBytes;
+    const unsigned char *bt = b_tiles + buffer * kTile + (kQ * wn + l32) * kRowBytes;
     const uint32_t piece = 16 * ((2 * s + kh) ^ swizzle);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kMI; ++i) {
       a_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * kRowBytes + piece));
       b_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kRowBytes + piece));
     }
@@ -329,9 +338,9 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
       if (s + 1 < kSub) read_operands(buffer, s + 1, (s + 1) & 1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < kMI; ++i) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < kMI; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
         if (issued < kLoads) {
           __builtin_amdgcn_sched_barrier(0);
@@ -341,7 +350,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
         }
       }
     }
-    static_assert(kLoads <= 4 * kSub, "one load pair per MFMA row at most");
+    static_assert(kLoads <= kMI * kSub, "one load pair per MFMA row at most");
     __builtin_amdgcn_s_waitcnt(0xc07f);                                   // lgkmcnt(0): reads done
     __builtin_amdgcn_s_waitcnt(wait_vmcnt((kStages - 2) * 2 * kLoads));   // step + 1 has landed
     __syncthreads();
@@ -357,16 +366,18 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   // result (f32 sum, one rounding), and the rows leave with one 16-byte store per lane, 256
   // contiguous bytes per row.  Only wave-local ordering is needed: nobody else touches the piece.
   if (a.row_stores) {
-    unsigned char *mine = gemm_lds + wave * (128 * kOutPitch + 512);
-    float *unscale_of = (float *)(mine + 128 * kOutPitch);   // the quadrant's 128 row factors
-    const uint32_t quad_row0 = row0 + 128 * wm, quad_col0 = col0 + 128 * wn;
-    const uint32_t piece_row = lane >> 4, piece_col = 8 * (lane & 15);
+    constexpr int kPieces = kQ / 8;            // 16-byte pieces of a quadrant's row
+    constexpr int kRowsAtOnce = 64 / kPieces;  // rows one wave-wide 16-byte access covers
+    unsigned char *mine = gemm_lds + wave * (kQ * kOutPitch + 4 * kQ);
+    float *unscale_of = (float *)(mine + kQ * kOutPitch);   // the quadrant's row factors
+    const uint32_t quad_row0 = row0 + kQ * wm, quad_col0 = col0 + kQ * wn;
+    const uint32_t piece_row = lane / kPieces, piece_col = 8 * (lane % kPieces);
     unscale_of[lane] = a.row_unscale[min(quad_row0 + lane, a.rows - 1)];
-    unscale_of[64 + lane] = a.row_unscale[min(quad_row0 + 64 + lane, a.rows - 1)];
+    if (kQ > 64) unscale_of[64 + lane] = a.row_unscale[min(quad_row0 + 64 + lane, a.rows - 1)];
     if (a.residual) {
 #pragma unroll 4
-      for (int it = 0; it < 32; ++it) {
-        const uint32_t row = 4 * it + piece_row;
+      for (int it = 0; it < kQ / kRowsAtOnce; ++it) {
+        const uint32_t row = kRowsAtOnce * it + piece_row;
         uint4 v = make_uint4(0, 0, 0, 0);
         if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
           v = *(const uint4 *)(a.residual + (uint64_t)(quad_row0 + row) * a.residual_row_stride +
@@ -378,13 +389,13 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kMI; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const uint32_t row = 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
         const float unscale = unscale_of[row];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kMI; ++j) {
           uint16_t *slot = (uint16_t *)(mine + row * kOutPitch) + 32 * j + l32;
           float value = acc[i][j][r] * unscale;
           if (a.residual) value += bf16_bits_to_f32(*slot);
@@ -396,8 +407,8 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     uint16_t *out = (uint16_t *)a.out;
 #pragma unroll 4
-    for (int it = 0; it < 32; ++it) {
-      const uint32_t row = 4 * it + piece_row;
+    for (int it = 0; it < kQ / kRowsAtOnce; ++it) {
+      const uint32_t row = kRowsAtOnce * it + piece_row;
       const uint4 v = *(const uint4 *)(mine + row * kOutPitch + 2 * piece_col);
       if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
         *(uint4 *)(out + (uint64_t)(quad_row0 + row) * a.out_row_stride + quad_col0 + piece_col) = v;
@@ -406,13 +417,13 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   }
   // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < kMI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t column = col0 + 128 * wn + 32 * j + l32;
+    for (int j = 0; j < kMI; ++j) {
+      const uint32_t column = col0 + kQ * wn + 32 * j + l32;
       if (column >= a.columns) continue;
       for (int r = 0; r < 16; ++r) {
-        const uint32_t row = row0 + 128 * wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+        const uint32_t row = row0 + kQ * wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
         if (row >= a.rows) continue;
         const uint64_t at_out = (uint64_t)row * a.out_row_stride + column;
         float value = acc[i][j][r] * a.row_unscale[row];
@@ -458,13 +469,19 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
                  (!p.residual || (p.residual->stride[0] % 8 == 0 && p.residual->offset % 8 == 0));
   a.rows = p.rows;
   a.columns = p.columns;
-  a.row_tiles = (p.rows + kBM - 1) / kBM;
-  a.column_tiles = (p.columns + kBN - 1) / kBN;
+  // 256 x 256 tiles unless they are fewer than three quarters of the compute units
+  const uint64_t large_tiles = (uint64_t)((p.rows + kBM - 1) / kBM) * ((p.columns + kBN - 1) / kBN);
+  const bool small_tiles = large_tiles * 4 < 3ull * backend_compute_units(backend);
+  const uint32_t side = small_tiles ? 128 : 256;
+  a.row_tiles = (p.rows + side - 1) / side;
+  a.column_tiles = (p.columns + side - 1) / side;
   a.refused = flag;
   static bool configured = false;   // raise the dynamic LDS limit once per process
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds) != hipSuccess)
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages, 128>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, gemm_lds_bytes(128)) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages, 64>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, gemm_lds_bytes(64)) != hipSuccess)
       return false;
     configured = true;
   }
@@ -478,7 +495,10 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
       (const uint16_t *)p.scales.base + p.scales.offset,
       (const uint16_t *)p.biases.base + p.biases.offset, p.columns, p.inner, kt,
       (uint16_t *)(ws + a_bytes), flag);
-  gemm_f16_kernel<kGemmK, kGemmStages><<<grid, 256, kGemmLds, stream>>>(a);
+  if (small_tiles)
+    gemm_f16_kernel<kGemmK, kGemmStages, 64><<<grid, 256, gemm_lds_bytes(64), stream>>>(a);
+  else
+    gemm_f16_kernel<kGemmK, kGemmStages, 128><<<grid, 256, gemm_lds_bytes(128), stream>>>(a);
   *refused = flag;
   return true;
 }

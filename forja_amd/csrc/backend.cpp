@@ -193,12 +193,49 @@ struct fh_backend {
   uint64_t class_ns[FH_KC_COUNT] = {};
   uint64_t class_launches[FH_KC_COUNT] = {};
 
-  // Fusion of runs of per-lane attention dispatches: gathered lane metadata followed by the
-  // attended rows, kept between the layers of a step (every layer names the same lanes).
+  // Prepared (fp16) forms of weight matrices kept for the prefill GEMM, see
+  // backend_prepared_weights; `prepared_watch` counts, per allocation, the entries built from it.
+  struct Prepared {
+    PreparedKey key;
+    char *operand;
+    uint64_t bytes;
+    int verdict;
+  };
+  std::vector<Prepared> prepared;
+  std::unordered_map<uint64_t, uint32_t> prepared_watch;
+  uint64_t prepared_bytes = 0, prepared_limit = 0;
+  void drop_prepared(uint64_t buffer) {   // the allocation is written or released
+    if (prepared_watch.find(buffer) == prepared_watch.end()) return;
+    if (static_mode) {
+      // nothing may be freed (or waited for) now: the entries stop matching and go with the backend
+      for (Prepared &e : prepared)
+        if (e.key.buffers[0] == buffer || e.key.buffers[1] == buffer || e.key.buffers[2] == buffer)
+          e.key.columns = 0;
+      return;
+    }
+    (void)hipStreamSynchronize(stream);   // kernels in flight may still read an operand
+    for (size_t i = 0; i < prepared.size();) {
+      const Prepared &e = prepared[i];
+      if (e.key.buffers[0] != buffer && e.key.buffers[1] != buffer && e.key.buffers[2] != buffer) {
+        ++i;
+        continue;
+      }
+      (void)hipFree(e.operand);
+      prepared_bytes -= e.bytes;
+      for (uint64_t watched : e.key.buffers) {
+        auto it = prepared_watch.find(watched);
+        if (it != prepared_watch.end() && --it->second == 0) prepared_watch.erase(it);
+      }
+      prepared[i] = prepared.back();
+      prepared.pop_back();
+    }
+  }
   // The normalisation the dispatch after a weighted sum applies to its rows, offered to the sum
   // while it is planned, and whether the sum's kernels have produced it.
   const NormTail *norm_tail = nullptr;
   bool *norm_tail_taken = nullptr;
+  // Fusion of runs of per-lane attention dispatches: gathered lane metadata followed by the
+  // attended rows, kept between the layers of a step (every layer names the same lanes).
   bool lane_fusion = true;
   char *lane_scratch = nullptr;
   uint64_t lane_scratch_bytes = 0;
@@ -656,6 +693,7 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
   if (!d.epilogue) {
     QmmProblem problem{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows, inner, columns,
                        d.bits, d.group_size};
+    for (int i = 0; i < 3; ++i) problem.weight_buffers[i] = d.inputs[1 + i].buffer;
     if (try_fast_quant_matmul(b, problem) || try_valu_quant_matmul(b, problem)) return FH_OK;
     launch_quant_matmul_generic(b->stream, pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows,
                                 inner, columns, d.bits, d.group_size);
@@ -668,6 +706,7 @@ fh_status plan_quant_matmul(fh_backend *b, const Planned &pl, ErrorSlot *, bool 
       prog->second.add_epilogue && shape_is(d.inputs[primitive], {rows, columns})) {
     QmmProblem fused{pl.in[0], pl.in[1], pl.in[2], pl.in[3], pl.out[0], rows, inner, columns,
                      d.bits, d.group_size, &pl.in[primitive]};
+    for (int i = 0; i < 3; ++i) fused.weight_buffers[i] = d.inputs[1 + i].buffer;
     if (try_fast_quant_matmul(b, fused) || try_valu_quant_matmul(b, fused)) return FH_OK;
   }
   // The accumulators live apart from the workspace, which the product kernels use themselves.
@@ -1835,6 +1874,7 @@ void fh_destroy(fh_backend *b) {
     if (b->lane_scratch) (void)hipFree(b->lane_scratch);
     if (b->route_plan) (void)hipFree(b->route_plan);
     if (b->attention_plan) (void)hipFree(b->attention_plan);
+    for (auto &e : b->prepared) (void)hipFree(e.operand);
     for (auto &e : b->error_pool) {
       (void)hipFree(e.device);
       (void)hipHostFree(e.host);
@@ -1883,6 +1923,7 @@ fh_status fh_release(fh_backend *b, fh_buffer buffer) {
   if (it == b->allocations.end()) return FH_INVALID_INPUT;
   (void)hipSetDevice(b->device);
   (void)hipStreamSynchronize(b->stream);
+  b->drop_prepared(buffer);
   (void)hipFree(it->second.ptr);
   b->used_bytes -= it->second.bytes;
   b->allocations.erase(it);
@@ -1912,6 +1953,7 @@ fh_status fh_write(fh_backend *b, fh_buffer buffer, uint64_t byte_offset, const 
     return FH_INVALID_INPUT;
   if (len == 0) return FH_OK;
   (void)hipSetDevice(b->device);
+  b->drop_prepared(buffer);
   // Small writes are staged through a pinned ring and ordered on the stream without waiting for
   // it; the caller's bytes may be reused as soon as this returns either way.
   constexpr uint64_t kRingBytes = 32ull << 20, kRingPiece = 4ull << 20;
@@ -2134,6 +2176,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   auto note_outputs = [b](const fh_dispatch &d) {
     for (uint32_t o = 0; o < d.n_outputs && o < FH_MAX_OUTPUTS; ++o) {
       uint64_t written = d.outputs[o].buffer;
+      b->drop_prepared(written);
       if (b->route_plan_valid && written == b->route_plan_key.buffer) b->route_plan_valid = false;
       if (b->attention_plan_valid)
         for (uint64_t watched : b->attention_plan_key.buffers)
@@ -2298,6 +2341,7 @@ fh_status fh_submit_static(fh_backend *b, const fh_dispatch *dispatches, uint32_
     if (status != FH_OK) break;
     for (uint32_t o = 0; o < d.n_outputs && o < FH_MAX_OUTPUTS; ++o) {
       const uint64_t written = d.outputs[o].buffer;
+      b->drop_prepared(written);
       if (b->route_plan_valid && written == b->route_plan_key.buffer) b->route_plan_valid = false;
       if (b->attention_plan_valid)
         for (uint64_t watched : b->attention_plan_key.buffers)
@@ -2533,6 +2577,55 @@ char *backend_attention_plan(fh_backend *b, const AttentionPlanKey &key, uint64_
   b->attention_plan_valid = true;
   return b->attention_plan;
 }
+namespace {
+bool same_weights(const PreparedKey &l, const PreparedKey &r) {
+  for (int i = 0; i < 3; ++i)
+    if (l.buffers[i] != r.buffers[i] || l.address[i] != r.address[i]) return false;
+  return l.columns == r.columns && l.inner == r.inner;
+}
+}  // namespace
+
+char *backend_prepared_weights(fh_backend *b, const PreparedKey &key, uint64_t bytes, bool *fresh,
+                               int *verdict) {
+  *fresh = false;
+  *verdict = -1;
+  if (b->static_mode) return nullptr;
+  for (const auto &e : b->prepared)
+    if (same_weights(e.key, key) && e.bytes == bytes) {
+      *verdict = e.verdict;
+      return e.operand;
+    }
+  if (b->prepared_limit == 0) {
+    // a quarter of the device's memory unless FORJA_HIP_PREPARED_MB says otherwise (0: keep nothing)
+    const char *env = getenv("FORJA_HIP_PREPARED_MB");
+    b->prepared_limit = env ? (uint64_t)strtoull(env, nullptr, 10) << 20 : (uint64_t)b->props.totalGlobalMem / 4;
+    if (b->prepared_limit == 0) b->prepared_limit = 1;   // asked for nothing: nothing fits
+  }
+  if (b->prepared_bytes + bytes + 256 > b->prepared_limit) return nullptr;
+  void *ptr = nullptr;
+  if (hipMalloc(&ptr, bytes + 256) != hipSuccess) {
+    (void)hipGetLastError();   // no room: the workspace serves
+    return nullptr;
+  }
+  b->prepared.push_back({key, (char *)ptr, bytes, -1});
+  b->prepared_bytes += bytes + 256;
+  for (uint64_t watched : key.buffers) ++b->prepared_watch[watched];
+  *fresh = true;
+  return (char *)ptr;
+}
+
+void backend_prepared_verdict(fh_backend *b, const PreparedKey &key) {
+  for (auto &e : b->prepared)
+    if (same_weights(e.key, key)) {
+      uint32_t flag = 1;
+      if (hipMemcpyAsync(&flag, e.operand + e.bytes, sizeof(flag), hipMemcpyDeviceToHost, b->stream) != hipSuccess ||
+          hipStreamSynchronize(b->stream) != hipSuccess)
+        return;   // stays unknown: products keep their conditioned second kernel
+      e.verdict = flag ? 1 : 0;
+      return;
+    }
+}
+
 hipStream_t backend_stream(fh_backend *backend) { return backend->stream; }
 uint32_t backend_compute_units(fh_backend *backend) {
   return (uint32_t)backend->props.multiProcessorCount;

@@ -60,6 +60,9 @@ struct QmmProblem {
   // Optional [rows, columns] bf16 rows added to the f32 result before it is rounded (the dense
   // residual-add epilogue); only honoured together with a bf16 `out`.
   const View *residual = nullptr;
+  // Allocation identities of packed, scales and biases (0: not known): what a kept copy of the
+  // prepared weights is watched by.
+  uint64_t weight_buffers[3] = {0, 0, 0};
 };
 bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &problem);
 // The f32 vector-ALU kernel for what the matrix-core kernels do not take: any float activation and
@@ -78,7 +81,28 @@ bool try_valu_gather(fh_backend *backend, const View &x, const View &packed, con
 // when the launch could not be configured.  On success `*refused` points at a device word the
 // launched kernels leave non-zero when some scale or bias is outside their fp16 scheme; they
 // have then written nothing and the caller must run a kernel conditioned on that word.
+// `*refused` is null when the weights are known to be inside the scheme (their prepared form is
+// kept, see backend_prepared_weights): nothing else need run.  False also when they are known to
+// be outside it.
 bool launch_quant_gemm(fh_backend *backend, const QmmProblem &problem, const uint32_t **refused);
+
+// The prepared (dequantised, fp16) form of a weight matrix, kept from the first prefill product
+// that needs it until one of its three allocations is written or released: a prompt is many
+// chunks and a server many prompts, and preparing 2 bytes per weight again for each is a twentieth
+// of a large layer's time and a tenth of a small model's.  `bytes` of device memory followed by a
+// flag word; *fresh says the caller must fill them (and then report the flag through
+// backend_prepared_verdict).  *verdict: -1 not known yet, 0 inside the fp16 scheme, 1 outside it
+// (nothing is kept then but the verdict).  Null when nothing can be kept (allocation identities
+// unknown, the memory set aside for it used up, a caller that may not allocate).
+struct PreparedKey {
+  uint64_t buffers[3];
+  const void *address[3];
+  uint32_t columns, inner;
+};
+char *backend_prepared_weights(fh_backend *backend, const PreparedKey &key, uint64_t bytes, bool *fresh,
+                               int *verdict);
+// Waits for the stream and reads the flag word behind the operand the caller has just filled.
+void backend_prepared_verdict(fh_backend *backend, const PreparedKey &key);
 
 // ---- qmm_ksplit.hip: products over at most 32 activation rows per weight (decode GEMV, routed
 // MoE tiles), K split over the waves of a workgroup with the rows stationary in registers.

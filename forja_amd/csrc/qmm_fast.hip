@@ -1174,7 +1174,10 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
   if (p.rows > 128) {
     // the tiled GEMM, followed by the any-range kernel conditioned on the GEMM's refusal
     const uint32_t *refused = nullptr;
-    if (launch_quant_gemm(backend, p, &refused)) a.run_if_set = refused;
+    if (launch_quant_gemm(backend, p, &refused)) {
+      if (!refused) return true;   // weights known to be in range: the GEMM has done the product
+      a.run_if_set = refused;
+    }
   }
   int mt = p.rows <= 32 ? 1 : 2;
   uint32_t row_blocks = (p.rows + 32 * mt - 1) / (32 * mt);

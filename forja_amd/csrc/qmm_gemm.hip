@@ -448,14 +448,33 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
   const uint64_t a_bytes = ((uint64_t)p.rows * kt * 2 + 255) / 256 * 256;
   const uint64_t b_bytes = ((uint64_t)p.columns * kt * 2 + 255) / 256 * 256;
   const uint64_t unscale_bytes = ((uint64_t)p.rows * sizeof(float) + 255) / 256 * 256;
-  char *ws = backend_workspace(backend, a_bytes + b_bytes + unscale_bytes + 256);
+  // the weights' operand: a kept copy when there is one (or room for one), else workspace
+  PreparedKey key{};
+  bool keepable = p.weight_buffers[0] && p.weight_buffers[1] && p.weight_buffers[2];
+  bool fresh = true;
+  int verdict = -1;
+  char *kept = nullptr;
+  if (keepable) {
+    for (int i = 0; i < 3; ++i) key.buffers[i] = p.weight_buffers[i];
+    key.address[0] = (const uint32_t *)p.packed.base + p.packed.offset;
+    key.address[1] = (const uint16_t *)p.scales.base + p.scales.offset;
+    key.address[2] = (const uint16_t *)p.biases.base + p.biases.offset;
+    key.columns = p.columns;
+    key.inner = p.inner;
+    kept = backend_prepared_weights(backend, key, b_bytes, &fresh, &verdict);
+    if (verdict == 1) return false;   // outside the fp16 scheme: the caller's any-range kernel
+  }
+  char *ws = backend_workspace(backend, a_bytes + (kept ? 0 : b_bytes) + unscale_bytes + 256);
   if (!ws) return false;
   hipStream_t stream = backend_stream(backend);
-  uint32_t *flag = (uint32_t *)(ws + a_bytes + b_bytes + unscale_bytes);
+  char *b_operand = kept ? kept : ws + a_bytes;
+  char *after = ws + a_bytes + (kept ? 0 : b_bytes);
+  // the flag of a kept operand lives behind it (and reads zero once the verdict is in)
+  uint32_t *flag = kept ? (uint32_t *)(kept + b_bytes) : (uint32_t *)(after + unscale_bytes);
   GemmArgs a{};
   a.a = (const uint16_t *)ws;
-  a.b = (const uint16_t *)(ws + a_bytes);
-  a.row_unscale = (const float *)(ws + a_bytes + b_bytes);
+  a.b = (const uint16_t *)b_operand;
+  a.row_unscale = (const float *)after;
   a.kt = kt;
   a.out = p.out.dtype == FH_F32 ? (void *)((float *)p.out.base + p.out.offset)
                                 : (void *)((uint16_t *)p.out.base + p.out.offset);
@@ -488,18 +507,22 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
   const uint32_t grid = (a.row_tiles * a.column_tiles + 255) / 256 * 256;
   prepare_rows_kernel<<<(p.rows + 3) / 4, 256, 0, stream>>>(
       (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, kt, (uint16_t *)ws,
-      (float *)(ws + a_bytes + b_bytes), flag);
-  const uint64_t weight_threads = (uint64_t)p.columns * (kt / 64) * 8;
-  prepare_weights_kernel<<<(uint32_t)((weight_threads + 255) / 256), 256, 0, stream>>>(
-      (const uint32_t *)p.packed.base + p.packed.offset,
-      (const uint16_t *)p.scales.base + p.scales.offset,
-      (const uint16_t *)p.biases.base + p.biases.offset, p.columns, p.inner, kt,
-      (uint16_t *)(ws + a_bytes), flag);
+      (float *)after, flag);
+  if (!kept || fresh) {
+    const uint64_t weight_threads = (uint64_t)p.columns * (kt / 64) * 8;
+    prepare_weights_kernel<<<(uint32_t)((weight_threads + 255) / 256), 256, 0, stream>>>(
+        (const uint32_t *)p.packed.base + p.packed.offset,
+        (const uint16_t *)p.scales.base + p.scales.offset,
+        (const uint16_t *)p.biases.base + p.biases.offset, p.columns, p.inner, kt,
+        (uint16_t *)b_operand, flag);
+  }
   if (small_tiles)
     gemm_f16_kernel<kGemmK, kGemmStages, 64><<<grid, 256, gemm_lds_bytes(64), stream>>>(a);
   else
     gemm_f16_kernel<kGemmK, kGemmStages, 128><<<grid, 256, gemm_lds_bytes(128), stream>>>(a);
-  *refused = flag;
+  *refused = (kept && verdict == 0) ? nullptr : flag;
+  // the first product over kept weights learns, once, whether they fit the scheme
+  if (kept && fresh) backend_prepared_verdict(backend, key);
   return true;
 }
 

@@ -327,6 +327,39 @@ def test_quant_matmul_on_strided_views_with_bias_epilogue(cpu, hip):
     differential(cpu, hip, build)
 
 
+def test_prefill_products_follow_weights_that_are_rewritten(cpu, hip):
+    """Products of more than 128 rows keep a prepared copy of their weights from one product to the
+    next.  The copy must go when any of the three tensors is written: by the host, by a dispatch,
+    or when the allocation is released and its memory taken by other weights."""
+    rows, n, k = 200, 320, 512
+    first, second, third = (Quantised(27, seed, (n, k)) for seed in (1, 2, 3))
+    x_values = normal_bf16(27, 9, (rows, k))
+
+    def build(backend):
+        x = upload(backend, x_values, DType.BF16)
+        packed, scales, biases = first.upload(backend)
+        outs = [backend.alloc(DType.BF16, (rows, n)) for _ in range(5)]
+        op = Op.quant_matmul(4, 64)
+
+        def product(out, triple):
+            commands = CommandList()
+            commands.dispatch(op, [x, *triple], out)
+            run(backend, commands)
+        product(outs[0], (packed, scales, biases))
+        product(outs[1], (packed, scales, biases))                      # the kept copy serves
+        backend.write(scales, np.ascontiguousarray(second.scales).tobytes())   # written by the host
+        product(outs[2], (packed, scales, biases))
+        commands = CommandList()                                        # written by a dispatch
+        commands.dispatch(Op.copy(), [upload_raw(backend, third.packed, DType.U32, third.packed.shape)], packed)
+        commands.dispatch(op, [x, packed, scales, biases], outs[3])
+        run(backend, commands)
+        for tensor in (packed, scales, biases):                         # released: the memory may come back
+            backend.release(tensor)
+        product(outs[4], second.upload(backend))
+        return CommandList(), outs
+    differential(cpu, hip, build)
+
+
 @pytest.mark.parametrize("rows,n,k,kind", [
     (128, 256, 1024, "add"),    # decode rows: the add joins the slab sum
     (8, 64, 256, "add"),        # a single K slab: accumulators + epilogue program

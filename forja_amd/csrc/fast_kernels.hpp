@@ -149,13 +149,14 @@ struct KsplitRouted {
 bool launch_ksplit_routed(fh_backend *backend, const KsplitRouted &problem);
 
 // A row-wise RMS normalisation the next dispatch applies to the rows a weighted sum produces:
-// out[r,:] = rows[r,:] * rsqrt(mean(rows[r,:]^2) + eps) * weight[r,:], everything bf16.  The
-// kernel that writes the rows can produce this too and save the launch.
+// out[r,:] = rows[r,:] * rsqrt(mean(rows[r,:]^2) + eps) * weight[r,:], everything bf16 or
+// everything f32 (`wide`).  The kernel that writes the rows can produce this too and save the launch.
 struct NormTail {
-  const uint16_t *weight;
-  uint16_t *out;
+  const void *weight;
+  void *out;
   uint64_t weight_stride, out_stride;   // elements per row
   float eps;
+  bool wide;
 };
 
 struct GatherProblem {
@@ -243,16 +244,16 @@ ProgramClass classify_program(uint32_t kind, const fh_inst *insts, uint32_t n_in
                               const uint32_t *pairs, uint32_t n_pairs);
 bool try_fast_program(hipStream_t stream, const ProgramClass &cls, const ProgramArgs &args,
                       uint64_t elements);
-// Whether the program is the plain RMS normalisation of bf16 rows of at most 2048 columns that
-// norm_rows_kernel would run, reading exactly `produced`; fills `tail` if so.
+// Whether the program is the plain RMS normalisation of bf16 or f32 rows of at most 2048 columns
+// that norm_rows_kernel would run, reading exactly `produced`; fills `tail` if so.
 bool norm_tail_of(const ProgramClass &cls, const ProgramArgs &args, const View &produced,
                   NormTail *tail);
 // combine_routes_rows_kernel followed by that normalisation, one workgroup per row: `out` gets
 // the sums (+ residual), `tail.out` their normalisation.  columns <= 2048, a multiple of 8;
-// routes <= 8; bf16 rows with 16-byte aligned pieces.
+// routes <= 8; rows of the tail's dtype with 16-byte aligned pieces of 8 elements.
 void launch_combine_routes_norm(hipStream_t stream, const float *partial, const View &indices,
-                                const View &weights, const uint16_t *residual,
-                                uint64_t residual_row_stride, uint16_t *out, uint64_t out_row_stride,
+                                const View &weights, const void *residual,
+                                uint64_t residual_row_stride, void *out, uint64_t out_row_stride,
                                 uint32_t rows, uint32_t routes, uint32_t columns, uint32_t experts,
                                 const NormTail &tail);
 

@@ -107,9 +107,10 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(RowArgs a) {
 // The weighted sum of a row's routed partial rows (+ residual), as combine_routes_rows_kernel
 // forms it, and the RMS normalisation of the stored (bf16) result, as norm_rows_kernel forms it:
 // thread t owns columns 8t .. 8t+7 in both, so the sums and the reduction add in the same order.
+template <bool kWide>
 __global__ __launch_bounds__(256) void combine_routes_norm_kernel(
-    const float *partial, View indices, View weights, const uint16_t *residual,
-    uint64_t residual_row_stride, uint16_t *out, uint64_t out_row_stride, uint32_t routes,
+    const float *partial, View indices, View weights, const void *residual,
+    uint64_t residual_row_stride, void *out, uint64_t out_row_stride, uint32_t routes,
     uint32_t columns, uint32_t experts, NormTail tail) {
   __shared__ float scratch[4];
   const uint32_t row = blockIdx.x, column = 8 * threadIdx.x;
@@ -147,12 +148,13 @@ __global__ __launch_bounds__(256) void combine_routes_norm_kernel(
     }
     if (residual) {
       float r[8];
-      load8<false>(residual, (uint64_t)row * residual_row_stride + column, r);
+      load8<kWide>(residual, (uint64_t)row * residual_row_stride + column, r);
       for (int i = 0; i < 8; ++i) value[i] += r[i];
     }
-    store8<false>(out, (uint64_t)row * out_row_stride + column, value);
+    store8<kWide>(out, (uint64_t)row * out_row_stride + column, value);
     // the normalisation reads what was stored
-    for (int i = 0; i < 8; ++i) value[i] = lo_f32(pack2(value[i], 0.0f));
+    if (!kWide)
+      for (int i = 0; i < 8; ++i) value[i] = lo_f32(pack2(value[i], 0.0f));
   }
   float acc = 0.0f;
   for (int i = 0; i < 8; ++i) acc += value[i] * value[i];
@@ -160,9 +162,9 @@ __global__ __launch_bounds__(256) void combine_routes_norm_kernel(
   const float inverse = 1.0f / sqrtf(total / (float)columns + tail.eps);
   if (live) {
     float w[8], normed[8];
-    load8<false>(tail.weight, (uint64_t)row * tail.weight_stride + column, w);
+    load8<kWide>(tail.weight, (uint64_t)row * tail.weight_stride + column, w);
     for (int i = 0; i < 8; ++i) normed[i] = value[i] * inverse * w[i];
-    store8<false>(tail.out, (uint64_t)row * tail.out_stride + column, normed);
+    store8<kWide>(tail.out, (uint64_t)row * tail.out_stride + column, normed);
   }
 }
 
@@ -517,30 +519,34 @@ bool norm_tail_of(const ProgramClass &cls, const ProgramArgs &p, const View &pro
   if (cls.kind != kProgramRmsNorm || p.rank != 2 || cls.axis != 1 || p.n_inputs != 2) return false;
   const View &x = p.inputs[0], &w = p.inputs[1], &out = p.outputs[0];
   if (p.shape[1] % 8 != 0 || p.shape[1] > 2048 || p.shape[0] == 0) return false;
+  const uint32_t dtype = x.dtype;
+  if (dtype != FH_BF16 && dtype != FH_F32) return false;
   for (const View *v : {&x, &w, &out}) {
-    if (!typed_rows(*v, 2, FH_BF16) || v->offset % 8 || v->stride[0] % 8) return false;
+    if (!typed_rows(*v, 2, dtype) || v->offset % 8 || v->stride[0] % 8) return false;
   }
   // the rows it reads are the rows just produced, element for element
-  if (x.base != produced.base || x.offset != produced.offset || produced.dtype != FH_BF16 ||
+  if (x.base != produced.base || x.offset != produced.offset || produced.dtype != dtype ||
       produced.rank != 2 || produced.shape[0] != p.shape[0] || produced.shape[1] != p.shape[1] ||
       x.stride[0] != produced.stride[0] || x.stride[1] != produced.stride[1])
     return false;
-  tail->weight = (const uint16_t *)w.base + w.offset;
+  const uint64_t size = dtype_size(dtype);
+  tail->weight = w.base + w.offset * size;
   tail->weight_stride = w.stride[0];
-  tail->out = (uint16_t *)out.base + out.offset;
+  tail->out = out.base + out.offset * size;
   tail->out_stride = out.stride[0];
   tail->eps = cls.c[0];
+  tail->wide = dtype == FH_F32;
   return true;
 }
 
 void launch_combine_routes_norm(hipStream_t stream, const float *partial, const View &indices,
-                                const View &weights, const uint16_t *residual,
-                                uint64_t residual_row_stride, uint16_t *out, uint64_t out_row_stride,
+                                const View &weights, const void *residual,
+                                uint64_t residual_row_stride, void *out, uint64_t out_row_stride,
                                 uint32_t rows, uint32_t routes, uint32_t columns, uint32_t experts,
                                 const NormTail &tail) {
-  combine_routes_norm_kernel<<<dim3(rows), 256, 0, stream>>>(partial, indices, weights, residual,
-                                                             residual_row_stride, out, out_row_stride,
-                                                             routes, columns, experts, tail);
+  auto *kernel = tail.wide ? combine_routes_norm_kernel<true> : combine_routes_norm_kernel<false>;
+  kernel<<<dim3(rows), 256, 0, stream>>>(partial, indices, weights, residual, residual_row_stride, out,
+                                         out_row_stride, routes, columns, experts, tail);
 }
 
 }  // namespace fh

@@ -1395,6 +1395,18 @@ bool try_wide_gather_weighted(fh_backend *backend, const GatherProblem &p, const
   if (!launch_wide_routed(backend, p, 1, (const float *)p.x.base + p.x.offset, p.x.stride[1], 1, partial,
                           plan))
     return false;
+  auto rows_of_eight = [](const View &v) {   // f32 [rows, columns] in 16-byte aligned pieces of 8
+    return v.dtype == FH_F32 && v.stride[1] == 1 && v.stride[0] % 8 == 0 && v.offset % 8 == 0;
+  };
+  if (p.norm_tail && p.norm_tail->wide && p.k <= 8 && p.columns % 8 == 0 && p.columns <= 2048 &&
+      rows_of_eight(p.out) && (!residual || rows_of_eight(*residual))) {
+    launch_combine_routes_norm(backend_stream(backend), partial, p.indices, p.weights,
+                               residual ? (const float *)residual->base + residual->offset : nullptr,
+                               residual ? residual->stride[0] : 0, (float *)p.out.base + p.out.offset,
+                               p.out.stride[0], p.rows, p.k, p.columns, p.experts, *p.norm_tail);
+    *p.norm_tail_taken = true;
+    return true;
+  }
   launch_combine_routes(backend_stream(backend), partial, p, residual);
   return true;
 }
@@ -1503,7 +1515,7 @@ bool try_fast_gather_weighted(fh_backend *backend, const GatherProblem &p, const
     const uint16_t *res = residual ? (const uint16_t *)residual->base + residual->offset : nullptr;
     const uint64_t res_stride = residual ? residual->stride[0] : 0;
     uint16_t *out = (uint16_t *)p.out.base + p.out.offset;
-    if (p.norm_tail && p.k <= 8 && p.columns % 8 == 0 && p.columns <= 2048 && p.out.stride[0] % 8 == 0 &&
+    if (p.norm_tail && !p.norm_tail->wide && p.k <= 8 && p.columns % 8 == 0 && p.columns <= 2048 && p.out.stride[0] % 8 == 0 &&
         p.out.offset % 8 == 0 && (!residual || (residual->stride[0] % 8 == 0 && residual->offset % 8 == 0))) {
       launch_combine_routes_norm(stream, partial, p.indices, p.weights, res, res_stride, out,
                                  p.out.stride[0], p.rows, p.k, p.columns, p.experts, *p.norm_tail);

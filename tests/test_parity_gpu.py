@@ -491,6 +491,38 @@ def test_weighted_sum_followed_by_the_normalisation_of_its_rows(cpu, hip, rows, 
     differential(cpu, hip, build, **({"rel": 3e-2} if form == "weights_in_the_sum" else {}))
 
 
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_f32_weighted_sum_followed_by_the_normalisation_of_its_rows(cpu, hip, with_residual):
+    """The same pair in the engine's dtypes: an 8-row decode batch, everything f32."""
+    rows, k, experts, n, inner = 8, 8, 128, 768, 2048
+    down = Quantised(34, 21, (inner, n), experts=experts)
+    indices = routed_case(34, rows, k, experts, n, inner)
+    activated_values = orc.fill_normal_f32(34, 40, rows * k * n).reshape(rows, k, n)
+    logits = orc.fill_normal_f32(34, 41, rows * k).reshape(rows, k)
+    w_values = np.exp(logits) / np.exp(logits).sum(axis=1, keepdims=True)
+    residual_values = orc.fill_normal_f32(34, 42, rows * inner).reshape(rows, inner)
+    norm_values = orc.fill_normal_f32(34, 43, inner)
+
+    def build(backend):
+        activated = upload(backend, activated_values, DType.F32)
+        idx = upload(backend, indices, DType.U32)
+        weights = upload(backend, w_values, DType.F32)
+        residual = upload(backend, residual_values, DType.F32)
+        norm_weight = upload(backend, norm_values, DType.F32).broadcast((rows, inner))
+        summed = backend.alloc(DType.F32, (rows, inner))
+        normed = backend.alloc(DType.F32, (rows, inner))
+        commands = CommandList()
+        if with_residual:
+            add = backend.prepare_epilogue(programs.add_elements())
+            commands.dispatch_epilogue(Op.gather_quant_matmul(4, 64), [activated, *down.upload(backend), idx, weights],
+                                       summed, add, [residual])
+        else:
+            commands.dispatch(Op.gather_quant_matmul(4, 64), [activated, *down.upload(backend), idx, weights], summed)
+        commands.dispatch_kernel(backend.prepare_program(programs.rms_norm_rows(1e-6)), [summed, norm_weight], [normed])
+        return commands, [summed, normed]
+    differential(cpu, hip, build)
+
+
 @pytest.mark.parametrize("dtype,bits,group,scale_dtype", [
     (DType.F32, 4, 64, DType.BF16),      # the qwen3-coder engine: f32 activations
     (DType.F16, 8, 32, DType.F16),

@@ -293,6 +293,23 @@ class StepBuffers:
         self.next_tokens = backend.alloc(DType.U32, (tokens,))
 
 
+def seeded_router_logits(model: Model, buffers: StepBuffers, seed: int) -> Tensor:
+    """[layers, tokens, experts] N(0,1) values, stream 7000 + layer of `seed`, filled on first use
+    and kept with the step's buffers."""
+    kept = getattr(buffers, "seeded_logits", None)
+    if kept is not None and kept[0] == seed:
+        return kept[1]
+    c, backend = model.config, model.backend
+    noise = backend.alloc(c.activation_dtype, (model.n_layers, buffers.tokens, c.experts))
+    fill = CommandList()
+    for layer in range(model.n_layers):
+        fill.dispatch(Op.fill_seeded(2, seed, 7000 + layer), [],
+                      noise.narrow(0, layer, 1).reshape((buffers.tokens, c.experts)))
+    backend.submit(fill).wait()
+    buffers.seeded_logits = (seed, noise)
+    return noise
+
+
 def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: CommandList,
                 feed_back: bool = False, route_trace: Optional[Tensor] = None,
                 head: bool = True, lane_starts=None, lane_sites: Optional[list] = None,
@@ -310,10 +327,11 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
     dispatch so that a replay can patch it.  `one_row_per_lane` passes the packed op the promise
     that the batch is a decode batch (every lane at most one row).
 
-    `router_noise_seed`: every layer's router logits are overwritten, after the router product has
-    run, with seeded N(0,1) values (a stream per layer): the routing law of the single-block
-    configuration ("top-8 of softmax of N(0,1) router logits"), under which nearly every expert is
-    touched; under the prescribed weight law alone all tokens choose the same few experts."""
+    `router_noise_seed`: every layer's top-k reads seeded N(0,1) logits (a stream per layer, filled
+    once into a tensor of their own when the step is recorded) instead of what the router product,
+    which still runs, has written: the routing law of the single-block configuration ("top-8 of
+    softmax of N(0,1) router logits"), under which nearly every expert is touched; under the
+    prescribed weight law alone all tokens choose the same few experts."""
     c, b = model.config, buffers
     tokens = b.tokens
     heads = c.q_heads + c.kv_heads
@@ -376,9 +394,11 @@ def record_step(model: Model, cache: KvCache, buffers: StepBuffers, commands: Co
         if c.moe:
             commands.dispatch(Op.quant_matmul(c.router_bits, GROUP), [normalized, *layer.router.triple],
                               b.router_logits)
+            logits = b.router_logits
             if router_noise_seed is not None:
-                commands.dispatch(Op.fill_seeded(2, router_noise_seed, 7000 + index), [], b.router_logits)
-            commands.dispatch_many(Op.top_k(c.top_k, True), [b.router_logits],
+                logits = seeded_router_logits(model, b, router_noise_seed).narrow(0, index, 1).reshape(
+                    (tokens, c.experts))
+            commands.dispatch_many(Op.top_k(c.top_k, True), [logits],
                                    [b.route_weights, b.route_indices])
             if route_trace is not None:
                 commands.dispatch(Op.copy(), [b.route_indices],

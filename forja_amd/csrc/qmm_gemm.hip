@@ -463,6 +463,9 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
     key.inner = p.inner;
     kept = backend_prepared_weights(backend, key, b_bytes, &fresh, &verdict);
     if (verdict == 1) return false;   // outside the fp16 scheme: the caller's any-range kernel
+    // a kept operand whose verdict could not be read is prepared again: the flag is only raised
+    // by the preparation
+    if (kept && verdict < 0) fresh = true;
   }
   char *ws = backend_workspace(backend, a_bytes + (kept ? 0 : b_bytes) + unscale_bytes + 256);
   if (!ws) return false;

@@ -360,6 +360,31 @@ def test_prefill_products_follow_weights_that_are_rewritten(cpu, hip):
     differential(cpu, hip, build)
 
 
+def test_prefill_products_without_kept_weights(cpu, monkeypatch):
+    """FORJA_HIP_PREPARED_MB=0: nothing is kept, every product prepares its weights into the
+    workspace and stands by with the conditioned second kernel, as it does when the memory set
+    aside for kept weights is used up."""
+    from forja_amd.hip_backend import HipBackend
+    monkeypatch.setenv("FORJA_HIP_PREPARED_MB", "0")
+    frugal = HipBackend(0)
+    try:
+        rows, n, k = 300, 520, 512
+        weights = Quantised(28, 1, (n, k))
+        x_values = normal_bf16(28, 2, (rows, k))
+
+        def build(backend):
+            x = upload(backend, x_values, DType.BF16)
+            triple = weights.upload(backend)
+            outs = [backend.alloc(DType.BF16, (rows, n)) for _ in range(2)]
+            commands = CommandList()
+            for out in outs:
+                commands.dispatch(Op.quant_matmul(4, 64), [x, *triple], out)
+            return commands, outs
+        differential(cpu, frugal, build)
+    finally:
+        frugal.close()
+
+
 @pytest.mark.parametrize("rows,n,k,kind", [
     (128, 256, 1024, "add"),    # decode rows: the add joins the slab sum
     (8, 64, 256, "add"),        # a single K slab: accumulators + epilogue program

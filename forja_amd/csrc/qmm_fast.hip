@@ -70,15 +70,14 @@ __device__ inline float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_flo
 // constants are literals (a VOP3 instruction reads one scalar operand at most); with the mask in a
 // scalar register and the other constant in a vector register it is a single v_and_or_b32.
 __device__ inline uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
-  return r;
+  return (x & mask) | magic;
 }
 
 // Eight nibbles of `w` as bf16 (16+q), in slot order (0,4)(1,5)(2,6)(3,7): two instructions per
 // pair of nibbles.
 __device__ inline bf16x8 unpack_word(uint32_t w) {
-  const uint32_t mask = 0x00780078u, magic = 0x41804180u;
+  uint32_t mask = 0x00780078u, magic = 0x41804180u;
+  asm("" : "+s"(mask), "+v"(magic));   // no instruction: keeps the two constants in registers
   uint4 r;
   r.x = and_or(w << 3, mask, magic);
   r.y = and_or(w >> 1, mask, magic);

@@ -78,16 +78,15 @@ __device__ inline uint32_t pack_bf16_pair(float lo, float hi) {
 
 __device__ inline float bf16_bits(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
-// (x & mask) | magic in one instruction (mask in a scalar register, magic in a vector register).
+// (x & mask) | magic: one v_and_or_b32 when neither constant is a literal (see unpack_word).
 __device__ inline uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
-  return r;
+  return (x & mask) | magic;
 }
 
 // Eight nibbles of `w` as bf16 (16+q) in slot order (0,4)(1,5)(2,6)(3,7).
 __device__ inline bf16x8 unpack_word(uint32_t w) {
-  const uint32_t mask = 0x00780078u, magic = 0x41804180u;
+  uint32_t mask = 0x00780078u, magic = 0x41804180u;
+  asm("" : "+s"(mask), "+v"(magic));   // no instruction: keeps the two constants in registers
   uint4 r;
   r.x = and_or(w << 3, mask, magic);
   r.y = and_or(w >> 1, mask, magic);

@@ -259,7 +259,7 @@ def prefill_gemm_c4(backend, rows=8256, seed=91, repeats=3):
                      f"64 decode rows), hidden {c.hidden}, intermediate {c.intermediate}, MLX-4bit"),
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "kernel": "gemm_f16_kernel, with prepare_rows_kernel and prepare_weights_kernel"},
+                     "kernel": "gemm_q4_kernel, with prepare_rows_kernel (and prepare_extras_kernel on a weight's first use)"},
         "ms_per_layer_projections": total_ns / 1e6, "products": products,
     }
 

@@ -1,5 +1,7 @@
-// MLX-4bit quantised matmul for many activation rows (prefill chunks): the weights are
-// dequantised to fp16 once per product and a plain tiled f16 MFMA GEMM does the rest.
+// MLX-4bit quantised matmul for many activation rows (prefill chunks): a tiled f16 MFMA GEMM
+// whose weight operand is dequantised on its way from LDS into the operand registers
+// (gemm_q4_kernel: the packed words travel, 0.5 byte per weight), or, for the shapes that kernel
+// does not take, once per product into an fp16 matrix (gemm_f16_kernel).
 //
 // y[m,n] = sum_k x[m,k] * (scale[n,k/64] * q[n,k] + bias[n,k/64])   (affine_quant_dot,
 // crates/forja-cpu/src/lib.rs:1277-1310).  With thousands of rows per weight the work is bound
@@ -33,6 +35,8 @@
 //     about 4 row tiles x 8 column tiles, so that its L2 serves each activation tile to 8
 //     workgroups and each weight tile to 4, instead of every workgroup streaming its own.
 // Accumulation is f32.
+#include <type_traits>
+
 #include "fast_kernels.hpp"
 
 namespace fh {
@@ -58,6 +62,10 @@ constexpr int gemm_lds_bytes(int quadrant) {
   const int output = 4 * (quadrant * out_pitch(quadrant) + 4 * quadrant);   // four quadrants of bf16 rows + row factors
   return pipeline > output ? pipeline : output;
 }
+constexpr int gemm_q4_lds_bytes(int quadrant) {   // the same plus the packed words of two pairs of K steps
+  const int pipeline = kGemmStages * 2 * (2 * quadrant) * 2 * kGemmK + 2 * (2 * quadrant) * 64;
+  return pipeline > gemm_lds_bytes(quadrant) ? pipeline : gemm_lds_bytes(quadrant);
+}
 constexpr int kBand = 8;   // column tiles per band of the tile numbering
 constexpr uint32_t kMaxGroups = 512;              // quantisation groups per row the row kernel holds
 
@@ -69,6 +77,12 @@ inline uint32_t padded_inner(uint32_t inner) {
 
 struct GemmArgs {
   const uint16_t *a, *b;    // fp16 operand matrices [rows, kt] and [columns, kt]
+  // gemm_q4_kernel instead of b: the weights as they are, and the fp16 columns [columns, kt - inner]
+  // that follow the inner values in a row of b
+  const uint32_t *packed;
+  const uint16_t *scales;
+  const uint16_t *extras;
+  uint32_t inner;
   const float *row_unscale; // per row: multiply the result by this
   uint32_t kt;
   void *out;
@@ -230,12 +244,100 @@ constexpr uint32_t wait_vmcnt(uint32_t n) {   // s_waitcnt immediate: vmcnt(n) o
   return (n & 15u) | ((n >> 4) << 14) | 0x0f70u;
 }
 
+// Stores a workgroup's finished tile: acc[i][j] is the 32 x 32 block (i, j) of wave (wm, wn)'s
+// quadrant, rows scaled back by row_unscale, the residual rows added, one rounding.
+template <int kQ>
+__device__ inline void store_tile(const GemmArgs &a, f32x16 (&acc)[kQ / 32][kQ / 32], unsigned char *gemm_lds,
+                                  uint32_t row0, uint32_t col0) {
+  constexpr int kMI = kQ / 32;
+  constexpr int kOutPitch = out_pitch(kQ);
+  const uint32_t tid = threadIdx.x, lane = tid & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t wm = wave >> 1, wn = wave & 1;
+  const uint32_t l32 = lane & 31, kh = lane >> 5;
+  // Lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile: a column
+  // per lane, the wrong way round for memory.  When the output rows allow 16-byte stores, every
+  // wave turns its 128 x 128 quadrant round through its own piece of LDS: the residual rows (if
+  // any) are staged there first, every lane then replaces "its" elements by the finished bf16
+  // result (f32 sum, one rounding), and the rows leave with one 16-byte store per lane, 256
+  // contiguous bytes per row.  Only wave-local ordering is needed: nobody else touches the piece.
+  if (a.row_stores) {
+    constexpr int kPieces = kQ / 8;            // 16-byte pieces of a quadrant's row
+    constexpr int kRowsAtOnce = 64 / kPieces;  // rows one wave-wide 16-byte access covers
+    unsigned char *mine = gemm_lds + wave * (kQ * kOutPitch + 4 * kQ);
+    float *unscale_of = (float *)(mine + kQ * kOutPitch);   // the quadrant's row factors
+    const uint32_t quad_row0 = row0 + kQ * wm, quad_col0 = col0 + kQ * wn;
+    const uint32_t piece_row = lane / kPieces, piece_col = 8 * (lane % kPieces);
+    unscale_of[lane] = a.row_unscale[min(quad_row0 + lane, a.rows - 1)];
+    if (kQ > 64) unscale_of[64 + lane] = a.row_unscale[min(quad_row0 + 64 + lane, a.rows - 1)];
+    if (a.residual) {
+#pragma unroll 4
+      for (int it = 0; it < kQ / kRowsAtOnce; ++it) {
+        const uint32_t row = kRowsAtOnce * it + piece_row;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
+          v = *(const uint4 *)(a.residual + (uint64_t)(quad_row0 + row) * a.residual_row_stride +
+                               quad_col0 + piece_col);
+        *(uint4 *)(mine + row * kOutPitch + 2 * piece_col) = v;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int i = 0; i < kMI; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+        const float unscale = unscale_of[row];
+#pragma unroll
+        for (int j = 0; j < kMI; ++j) {
+          uint16_t *slot = (uint16_t *)(mine + row * kOutPitch) + 32 * j + l32;
+          float value = acc[i][j][r] * unscale;
+          if (a.residual) value += bf16_bits_to_f32(*slot);
+          *slot = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+        }
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    uint16_t *out = (uint16_t *)a.out;
+#pragma unroll 4
+    for (int it = 0; it < kQ / kRowsAtOnce; ++it) {
+      const uint32_t row = kRowsAtOnce * it + piece_row;
+      const uint4 v = *(const uint4 *)(mine + row * kOutPitch + 2 * piece_col);
+      if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
+        *(uint4 *)(out + (uint64_t)(quad_row0 + row) * a.out_row_stride + quad_col0 + piece_col) = v;
+    }
+    return;
+  }
+  // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile
+#pragma unroll
+  for (int i = 0; i < kMI; ++i)
+#pragma unroll
+    for (int j = 0; j < kMI; ++j) {
+      const uint32_t column = col0 + kQ * wn + 32 * j + l32;
+      if (column >= a.columns) continue;
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row = row0 + kQ * wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+        if (row >= a.rows) continue;
+        const uint64_t at_out = (uint64_t)row * a.out_row_stride + column;
+        float value = acc[i][j][r] * a.row_unscale[row];
+        if (a.residual)
+          value += __uint_as_float((uint32_t)a.residual[(uint64_t)row * a.residual_row_stride + column] << 16);
+        if (a.out_f32)
+          ((float *)a.out)[at_out] = value;
+        else
+          ((uint16_t *)a.out)[at_out] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+      }
+    }
+}
+
 template <int kBK, int kStages, int kQ>
 __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   if (a.refused[0] != 0) return;
   constexpr int kSide = 2 * kQ;                  // rows (and columns) of a tile
   constexpr int kMI = kQ / 32;                   // 32 x 32 blocks along a quadrant's side
-  constexpr int kOutPitch = out_pitch(kQ);
   constexpr int kSub = kBK / 16;                 // MFMA sub-steps per K step
   constexpr int kRowBytes = 2 * kBK;             // one tile row in LDS
   constexpr int kTile = kSide * kRowBytes;       // one operand tile of one stage
@@ -359,85 +461,355 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   }
   __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));   // nothing is on its way into LDS any more
   __syncthreads();
-  // Lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile: a column
-  // per lane, the wrong way round for memory.  When the output rows allow 16-byte stores, every
-  // wave turns its 128 x 128 quadrant round through its own piece of LDS: the residual rows (if
-  // any) are staged there first, every lane then replaces "its" elements by the finished bf16
-  // result (f32 sum, one rounding), and the rows leave with one 16-byte store per lane, 256
-  // contiguous bytes per row.  Only wave-local ordering is needed: nobody else touches the piece.
-  if (a.row_stores) {
-    constexpr int kPieces = kQ / 8;            // 16-byte pieces of a quadrant's row
-    constexpr int kRowsAtOnce = 64 / kPieces;  // rows one wave-wide 16-byte access covers
-    unsigned char *mine = gemm_lds + wave * (kQ * kOutPitch + 4 * kQ);
-    float *unscale_of = (float *)(mine + kQ * kOutPitch);   // the quadrant's row factors
-    const uint32_t quad_row0 = row0 + kQ * wm, quad_col0 = col0 + kQ * wn;
-    const uint32_t piece_row = lane / kPieces, piece_col = 8 * (lane % kPieces);
-    unscale_of[lane] = a.row_unscale[min(quad_row0 + lane, a.rows - 1)];
-    if (kQ > 64) unscale_of[64 + lane] = a.row_unscale[min(quad_row0 + 64 + lane, a.rows - 1)];
-    if (a.residual) {
-#pragma unroll 4
-      for (int it = 0; it < kQ / kRowsAtOnce; ++it) {
-        const uint32_t row = kRowsAtOnce * it + piece_row;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
-          v = *(const uint4 *)(a.residual + (uint64_t)(quad_row0 + row) * a.residual_row_stride +
-                               quad_col0 + piece_col);
-        *(uint4 *)(mine + row * kOutPitch + 2 * piece_col) = v;
-      }
+  store_tile<kQ>(a, acc, gemm_lds, row0, col0);
+}
+
+
+// packed/scales/biases [columns, inner] -> the columns an operand row holds after its inner
+// values, fp16 [columns, kt - inner]: per group (head, head, tail) of 64 * (bias + 7.5 * scale),
+// then zeros.  One thread per 8 values; refused[0] is set when a group is out of range.
+__global__ __launch_bounds__(256) void prepare_extras_kernel(const uint16_t *scales, const uint16_t *biases,
+                                                             uint32_t columns, uint32_t inner, uint32_t kt,
+                                                             uint16_t *out, uint32_t *refused) {
+  const uint64_t flat = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t width = kt - inner, chunks = width / 8, groups = inner / 64;
+  if (flat >= (uint64_t)columns * chunks) return;
+  const uint32_t column = (uint32_t)(flat / chunks), chunk = (uint32_t)(flat % chunks);
+  const uint16_t *s_row = scales + (uint64_t)column * groups, *b_row = biases + (uint64_t)column * groups;
+  uint16_t values[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t extra = 8 * chunk + i;
+    const uint32_t group = extra / 3, kind = extra % 3;
+    float value = 0.0f;
+    if (group < groups) {
+      const float scale = bf16_bits_to_f32(s_row[group]), bias = bf16_bits_to_f32(b_row[group]);
+      // the GEMM multiplies by the scale as an fp16 number: it must be one exactly
+      if (kind == 0 && (!f16_safe(scale, bias) || (scale != 0.0f && fabsf(scale) < 6.103515625e-5f))) refused[0] = 1;
+      float head, tail;
+      split_f16(64.0f * (bias + 7.5f * scale), &head, &tail);
+      value = kind == 2 ? tail : head;
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int i = 0; i < kMI; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const uint32_t row = 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
-        const float unscale = unscale_of[row];
-#pragma unroll
-        for (int j = 0; j < kMI; ++j) {
-          uint16_t *slot = (uint16_t *)(mine + row * kOutPitch) + 32 * j + l32;
-          float value = acc[i][j][r] * unscale;
-          if (a.residual) value += bf16_bits_to_f32(*slot);
-          *slot = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
-        }
-      }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    uint16_t *out = (uint16_t *)a.out;
-#pragma unroll 4
-    for (int it = 0; it < kQ / kRowsAtOnce; ++it) {
-      const uint32_t row = kRowsAtOnce * it + piece_row;
-      const uint4 v = *(const uint4 *)(mine + row * kOutPitch + 2 * piece_col);
-      if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
-        *(uint4 *)(out + (uint64_t)(quad_row0 + row) * a.out_row_stride + quad_col0 + piece_col) = v;
-    }
-    return;
+    values[i] = f16_bits(value);
   }
-  // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile
+  *(uint4 *)(out + (uint64_t)column * width + 8 * chunk) =
+      make_uint4(values[0] | ((uint32_t)values[1] << 16), values[2] | ((uint32_t)values[3] << 16),
+                 values[4] | ((uint32_t)values[5] << 16), values[6] | ((uint32_t)values[7] << 16));
+}
+
+// Eight nibbles of `w` as the centred weights scale * (q - 7.5) in fp16, in the order
+// (0,4)(1,5)(2,6)(3,7).  A nibble lands in mantissa bits 1..4 of 512.0 (whose unit in the last
+// place is 0.5), giving 512 + q exactly; 519.5 is taken off exactly and the product with the
+// scale is rounded once, like a weight formed in f32 and rounded.  scale2 = (scale, scale).
+__device__ inline f16x8 dequantise_word(uint32_t w, f16x2 scale2, uint32_t mask, uint32_t magic) {
+  const f16x2 centre = {(_Float16)519.5f, (_Float16)519.5f};
+  uint32_t bits[4] = {((w << 1) & mask) | magic, ((w >> 3) & mask) | magic, ((w >> 7) & mask) | magic,
+                      ((w >> 11) & mask) | magic};
+  uint4 r;
+  r.x = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(f16x2, bits[0]) - centre) * scale2);
+  r.y = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(f16x2, bits[1]) - centre) * scale2);
+  r.z = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(f16x2, bits[2]) - centre) * scale2);
+  r.w = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(f16x2, bits[3]) - centre) * scale2);
+  return __builtin_bit_cast(f16x8, r);
+}
+
+// A 16-byte store to LDS the compiler does not see as one.  Before a store to LDS it can see, the
+// compiler waits for every global_load_lds in flight (any of them might write the same bytes),
+// which would stall each store of a weight tile behind the loads of the step's activation tile.
+// Those write other buffers; the stores are ordered by the kernel's own waits and barriers.
+__device__ inline void lds_store_16(unsigned char *to, f16x8 value) {
+  typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+  const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)to;
+  asm volatile("ds_write_b128 %0, %1" : : "v"(at), "v"(__builtin_bit_cast(u32x4, value)) : "memory");
+}
+
+// The GEMM with the weights dequantised on their way into LDS.
+//   * Activations: the fp16 rows prepare_rows_kernel writes, staged exactly as in gemm_f16_kernel.
+//   * Weights: the packed words themselves go from memory into LDS (global_load_lds; 64 bytes =
+//     two K steps of a column per request, half a byte per weight instead of two).  While the
+//     matrix instructions of step t run, thread c of the workgroup turns the 32 bytes of column c
+//     and step t + 1 into that column's 64 fp16 weights (per nibble pair two integer and two packed
+//     fp16 instructions, spread over the step behind the matrix instructions) and writes them
+//     into the fp16 tile of step t + 1, in the layout gemm_f16_kernel's tiles have.  Per K step a
+//     workgroup moves 40 KB from memory instead of 64.
+//   * The columns after the inner values (the bias term, see the head of this file) are plain fp16
+//     on both sides: for the last few K steps the weights' tile is loaded from `extras`.
+//   * Scales: a thread keeps the bf16 scales of eight groups of its column in registers (one
+//     16-byte load per eight K steps).
+// LDS: activations [2][tile rows][128 B], weights [2][tile columns][128 B], packed words of two
+// pairs of K steps [2][tile columns][64 B].  A column's four 16-byte quarters of a pair sit in
+// slots quarter ^ ((column >> 2) & 3), which spreads the 16 lanes a read serves at once over all
+// banks.  Tiles of 128 x 128 (kQ = 64) give two threads to a column: each takes half a group.
+template <int kQ>
+__global__ __launch_bounds__(256) void gemm_q4_kernel(GemmArgs a) {
+  if (a.refused[0] != 0) return;
+  constexpr int kBK = 64;
+  constexpr int kSide = 2 * kQ;
+  constexpr int kMI = kQ / 32;
+  constexpr int kSub = 4;
+  constexpr int kRowBytes = 2 * kBK;
+  constexpr int kTile = kSide * kRowBytes;       // one fp16 operand tile
+  constexpr int kPair = kSide * 64;              // the packed words of two K steps of a tile's columns
+  constexpr int kStaged = kSide / 4;             // rows of an fp16 tile a wave stages
+  constexpr int kLoads = kStaged / 8;            // instructions per wave and fp16 tile (8 rows each)
+  constexpr int kPairLoads = kSide / 64;         // instructions per wave and pair (16 columns each)
+  constexpr int kShare = 256 / kSide;            // threads per column: 1 or 2
+  constexpr int kWords = 8 / kShare;             // words of a K step a thread dequantises
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
+  unsigned char *a_tiles = gemm_lds;                 // [2][kSide][128]
+  unsigned char *b_tiles = gemm_lds + 2 * kTile;     // [2][kSide][128]
+  unsigned char *pairs = gemm_lds + 4 * kTile;       // [2][kSide][64]
+  const uint32_t tid = threadIdx.x, lane = tid & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t wm = wave >> 1, wn = wave & 1;
+  const uint32_t l32 = lane & 31, kh = lane >> 5;
+  auto swizzle_of = [](uint32_t row) { return (row >> 1) & 7u; };
+
+  const uint32_t xcd = blockIdx.x % 8, nth = blockIdx.x / 8;
+  const uint32_t tile = (nth / 32) * 256 + xcd * 32 + nth % 32;
+  if (tile >= a.row_tiles * a.column_tiles) return;
+  const uint32_t band = tile / (a.row_tiles * kBand);
+  const uint32_t band_width = min((uint32_t)kBand, a.column_tiles - band * kBand);
+  const uint32_t in_band = tile - band * a.row_tiles * kBand;
+  const uint32_t bm = in_band / band_width, bn = band * kBand + in_band % band_width;
+  const uint32_t row0 = bm * kSide, col0 = bn * kSide;
+
+  const uint32_t main_steps = a.inner / kBK, steps = a.kt / kBK;
+  const uint32_t extras_width = a.kt - a.inner;
+  // ---- staging addresses: a wave-uniform base that advances with K plus a per-lane offset
+  uint32_t a_off[kLoads], e_off[kLoads], p_off[kPairLoads];
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) {
+    const uint32_t in_tile = kStaged * wave + 8 * i + lane / 8;
+    const uint32_t piece = (lane % 8) ^ swizzle_of(in_tile);
+    a_off[i] = (min(row0 + in_tile, a.rows - 1) * a.kt + 8 * piece) * 2;
+    e_off[i] = (min(col0 + in_tile, a.columns - 1) * extras_width + 8 * piece) * 2;
+  }
+#pragma unroll
+  for (int i = 0; i < kPairLoads; ++i) {
+    const uint32_t column = 16 * (kPairLoads * wave + i) + lane / 4;
+    const uint32_t quarter = (lane % 4) ^ ((column >> 2) & 3u);
+    p_off[i] = min(col0 + column, a.columns - 1) * (a.inner / 2) + 16 * quarter;
+  }
+  auto stage_a = [&](uint32_t buffer, uint32_t step, int i) {
+    const uint32_t st = min(step, steps - 1);
+    const unsigned char *from = (const unsigned char *)a.a + (uint64_t)st * (kBK * 2);
+    unsigned char *to = a_tiles + buffer * kTile + (kStaged * wave + 8 * i) * kRowBytes;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from + a_off[i]),
+                                     (__attribute__((address_space(3))) void *)to, 16, 0, 0);
+  };
+  // the weights' fp16 tile of step `step`, one of the steps after the inner ones
+  auto stage_extras = [&](uint32_t buffer, uint32_t step, int i) {
+    const uint32_t st = min(step, steps - 1) - main_steps;
+    const unsigned char *from = (const unsigned char *)a.extras + (uint64_t)st * (kBK * 2);
+    unsigned char *to = b_tiles + buffer * kTile + (kStaged * wave + 8 * i) * kRowBytes;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from + e_off[i]),
+                                     (__attribute__((address_space(3))) void *)to, 16, 0, 0);
+  };
+  auto stage_pair = [&](uint32_t pair, int i) {
+    const uint32_t pr = min(pair, main_steps / 2 - 1);
+    const unsigned char *from = (const unsigned char *)a.packed + (uint64_t)pr * 64;
+    unsigned char *to = pairs + (pair & 1u) * kPair + 16 * (kPairLoads * wave + i) * 64;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from + p_off[i]),
+                                     (__attribute__((address_space(3))) void *)to, 16, 0, 0);
+  };
+
+  f32x16 acc[kMI][kMI];
 #pragma unroll
   for (int i = 0; i < kMI; ++i)
 #pragma unroll
-    for (int j = 0; j < kMI; ++j) {
-      const uint32_t column = col0 + kQ * wn + 32 * j + l32;
-      if (column >= a.columns) continue;
-      for (int r = 0; r < 16; ++r) {
-        const uint32_t row = row0 + kQ * wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
-        if (row >= a.rows) continue;
-        const uint64_t at_out = (uint64_t)row * a.out_row_stride + column;
-        float value = acc[i][j][r] * a.row_unscale[row];
-        if (a.residual)
-          value += __uint_as_float((uint32_t)a.residual[(uint64_t)row * a.residual_row_stride + column] << 16);
-        if (a.out_f32)
-          ((float *)a.out)[at_out] = value;
-        else
-          ((uint16_t *)a.out)[at_out] = (uint16_t)(pack2(value, 0.0f) & 0xffffu);
+    for (int j = 0; j < kMI; ++j)
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  f16x8 a_op[2][kMI], b_op[2][kMI];
+  const uint32_t swizzle = swizzle_of(l32);
+  auto read_operands = [&](uint32_t buffer, int s, int set) {
+    const unsigned char *at = a_tiles + buffer * kTile + (kQ * wm + l32) * kRowBytes;
+    const unsigned char *bt = b_tiles + buffer * kTile + (kQ * wn + l32) * kRowBytes;
+    const uint32_t piece = 16 * ((2 * s + kh) ^ swizzle);
+#pragma unroll
+    for (int i = 0; i < kMI; ++i) {
+      a_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * kRowBytes + piece));
+      b_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kRowBytes + piece));
+    }
+  };
+  // ---- this thread's share of the dequantisation: column `mine`, words [kWords part, + kWords)
+  const uint32_t mine = tid / kShare, part = tid % kShare;
+  const uint32_t mine_swizzle = swizzle_of(mine), quarter_swizzle = (mine >> 2) & 3u;
+  uint32_t words[kWords];
+  auto read_words = [&](uint32_t step) {   // the packed words of step `step`
+    const unsigned char *from = pairs + ((step >> 1) & 1u) * kPair + mine * 64;
+#pragma unroll
+    for (int q = 0; q < kWords / 4; ++q) {
+      const uint32_t quarter = 2 * (step & 1u) + (kShare == 1 ? q : part);
+      const uint4 v = *(const uint4 *)(from + 16 * (quarter ^ quarter_swizzle));
+      words[4 * q] = v.x, words[4 * q + 1] = v.y, words[4 * q + 2] = v.z, words[4 * q + 3] = v.w;
+    }
+  };
+  auto write_weights = [&](uint32_t buffer, int nth, f16x2 scale2, uint32_t mask, uint32_t magic) {
+    const uint32_t piece = kWords * part + nth;   // word `piece` of the group = piece `piece` of the row
+    unsigned char *to = b_tiles + buffer * kTile + mine * kRowBytes + 16 * (piece ^ mine_swizzle);
+    lds_store_16(to, dequantise_word(words[nth], scale2, mask, magic));
+  };
+  const uint32_t groups = a.inner / 64;
+  const uint32_t scale_off = min(col0 + mine, a.columns - 1) * groups * 2;
+  uint4 scale_block, next_block;   // bf16 scales of eight groups of the column
+  auto load_scales = [&](uint4 &to, uint32_t block) {
+    const uint32_t bl = min(block, groups / 8 - 1);
+    to = *(const uint4 *)((const unsigned char *)a.scales + (uint64_t)bl * 16 + scale_off);
+  };
+  auto pick_scale = [&](uint32_t step) -> f16x2 {
+    const uint32_t e = step & 7u;   // uniform
+    const uint4 v = scale_block;
+    const uint32_t word = e < 4 ? (e < 2 ? v.x : v.y) : (e < 6 ? v.z : v.w);
+    const float scale = __uint_as_float((e & 1u) ? (word & 0xffff0000u) : (word << 16));
+    const _Float16 h = (_Float16)scale;
+    return f16x2{h, h};
+  };
+  uint32_t mask = 0x001e001eu, magic = 0x60006000u;
+  asm("" : "+s"(mask), "+v"(magic));   // no instruction: keeps the two constants in registers
+
+  // ---- prologue: activations of step 0, packed words of steps 0..1, scales of groups 0..15;
+  // then the weights' tile of step 0
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) stage_a(0, 0, i);
+#pragma unroll
+  for (int i = 0; i < kPairLoads; ++i) stage_pair(0, i);
+  load_scales(scale_block, 0);
+  load_scales(next_block, 1);
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+  __syncthreads();
+  {
+    read_words(0);
+    const f16x2 scale2 = pick_scale(0);
+#pragma unroll
+    for (int nth = 0; nth < kWords; ++nth) write_weights(0, nth, scale2, mask, magic);
+  }
+  __syncthreads();
+  read_operands(0, 0, 0);
+  // One inner step.  On entry the operands of its first sub-step are in registers (set 0).  kOdd:
+  // the step's parity (= the LDS buffers its tiles are in); kLast: the last inner step, which
+  // requests the first fp16 tile of the weights' side instead of dequantising one.  Even steps
+  // request the packed words of the two steps after the next (past the end: the last pair again,
+  // into the buffer nobody reads).  Every request of the step is made at its start, so that it has
+  // the whole step to land; the matrix instructions of the last sub-step run behind the barrier,
+  // covering the latency of the next step's first operand reads.
+  auto inner_step = [&](auto odd_tag, auto last_tag, uint32_t step) {
+    constexpr bool kOdd = decltype(odd_tag)::value, kLast = decltype(last_tag)::value;
+    constexpr uint32_t buffer = kOdd ? 1u : 0u;
+    f16x2 scale2 = {0, 0};
+    if (!kLast) {
+      if (kOdd && ((step + 1) & 7u) == 0) {   // the next step opens a block of eight groups
+        scale_block = next_block;
+        load_scales(next_block, (step + 1) / 8 + 1);
+      }
+      scale2 = pick_scale(step + 1);
+      read_words(step + 1);
+    }
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      stage_a(buffer ^ 1u, step + 1, i);
+    }
+    if (kLast) {
+#pragma unroll
+      for (int i = 0; i < kLoads; ++i) stage_extras(buffer ^ 1u, main_steps, i);
+    } else if (!kOdd) {
+#pragma unroll
+      for (int i = 0; i < kPairLoads; ++i) stage_pair(step / 2 + 1, i);
+    }
+    int written = 0;
+#pragma unroll
+    for (int s = 0; s < kSub - 1; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      read_operands(buffer, s + 1, (s + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < kMI; ++i) {
+#pragma unroll
+        for (int j = 0; j < kMI; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
+        // behind two rows of matrix instructions in three: one word of the next step's weights
+        if (!kLast && written < kWords && (s * kMI + i) % 3 != 2) {
+          write_weights(buffer ^ 1u, written, scale2, mask, magic);
+          ++written;
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+    static_assert(kWords <= 2 * kMI, "the words fit the rows of three sub-steps");
+    __builtin_amdgcn_s_waitcnt(0xc07f);            // lgkmcnt(0): operand reads and tile stores done
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));     // step + 1 has landed
+    __syncthreads();
+    read_operands(buffer ^ 1u, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < kMI; ++i)
+#pragma unroll
+      for (int j = 0; j < kMI; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[1][i], b_op[1][j], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  typedef std::integral_constant<bool, false> no;
+  typedef std::integral_constant<bool, true> yes;
+  uint32_t step = 0;
+  for (; step + 2 < main_steps; step += 2) {   // main_steps is even
+    inner_step(no{}, no{}, step);
+    inner_step(yes{}, no{}, step + 1);
+  }
+  inner_step(no{}, no{}, step);
+  inner_step(yes{}, yes{}, step + 1);
+  // ---- the columns after the inner values: both operands fp16 tiles loaded from memory
+  uint32_t buffer = 0;
+  for (step = main_steps; step < steps; ++step) {
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      stage_a(buffer ^ 1u, step + 1, i);
+      stage_extras(buffer ^ 1u, step + 1, i);
+    }
+#pragma unroll
+    for (int s = 0; s < kSub - 1; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      read_operands(buffer, s + 1, (s + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < kMI; ++i)
+#pragma unroll
+        for (int j = 0; j < kMI; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+    __syncthreads();
+    buffer ^= 1u;
+    read_operands(buffer, 0, 0);   // (after the last step: a tile nobody uses)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < kMI; ++i)
+#pragma unroll
+      for (int j = 0; j < kMI; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[1][i], b_op[1][j], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __syncthreads();   // the last reads are done before the tile's stores reuse LDS
+  store_tile<kQ>(a, acc, gemm_lds, row0, col0);
 }
 
 }  // namespace
+
+// Whether gemm_q4_kernel takes the product: whole blocks of eight groups per weight row (a lane
+// reads eight scales at a time), packed rows and scale rows 16-byte aligned, 32-bit offsets.
+static bool packed_form_fits(const QmmProblem &p, uint32_t kt) {
+  static const bool disabled = [] {
+    const char *env = getenv("FORJA_HIP_GEMM_PREPARED");   // 1: dequantise to fp16 in memory first
+    return env && env[0] == '1';
+  }();
+  if (disabled) return false;
+  if (p.inner % 512 != 0 || p.packed.offset % 4 != 0 || p.scales.offset % 8 != 0) return false;
+  if ((uint64_t)p.columns * (p.inner / 2) >= (1ull << 32)) return false;
+  if ((uint64_t)p.columns * (kt - p.inner) * 2 >= (1ull << 32)) return false;
+  return true;
+}
 
 bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t **refused) {
   if (p.inner / 64 > kMaxGroups) return false;
@@ -445,8 +817,10 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
   // the GEMM addresses its operand matrices with 32-bit byte offsets
   if ((uint64_t)p.rows * kt * 2 >= (1ull << 32) || (uint64_t)p.columns * kt * 2 >= (1ull << 32))
     return false;
+  const bool packed_form = packed_form_fits(p, kt);
   const uint64_t a_bytes = ((uint64_t)p.rows * kt * 2 + 255) / 256 * 256;
-  const uint64_t b_bytes = ((uint64_t)p.columns * kt * 2 + 255) / 256 * 256;
+  // the weights' side: every column of the operand matrix, or only those after the inner values
+  const uint64_t b_bytes = ((uint64_t)p.columns * (packed_form ? kt - p.inner : kt) * 2 + 255) / 256 * 256;
   const uint64_t unscale_bytes = ((uint64_t)p.rows * sizeof(float) + 255) / 256 * 256;
   // the weights' operand: a kept copy when there is one (or room for one), else workspace
   PreparedKey key{};
@@ -477,6 +851,10 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
   GemmArgs a{};
   a.a = (const uint16_t *)ws;
   a.b = (const uint16_t *)b_operand;
+  a.packed = (const uint32_t *)p.packed.base + p.packed.offset;
+  a.scales = (const uint16_t *)p.scales.base + p.scales.offset;
+  a.extras = (const uint16_t *)b_operand;
+  a.inner = p.inner;
   a.row_unscale = (const float *)after;
   a.kt = kt;
   a.out = p.out.dtype == FH_F32 ? (void *)((float *)p.out.base + p.out.offset)
@@ -500,11 +878,15 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
   a.refused = flag;
   static bool configured = false;   // raise the dynamic LDS limit once per process
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages, 128>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, gemm_lds_bytes(128)) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages, 64>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, gemm_lds_bytes(64)) != hipSuccess)
-      return false;
+    const struct { const void *kernel; int bytes; } limits[] = {
+        {reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages, 128>), gemm_lds_bytes(128)},
+        {reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages, 64>), gemm_lds_bytes(64)},
+        {reinterpret_cast<const void *>(&gemm_q4_kernel<128>), gemm_q4_lds_bytes(128)},
+        {reinterpret_cast<const void *>(&gemm_q4_kernel<64>), gemm_q4_lds_bytes(64)}};
+    for (const auto &limit : limits) {
+      if (hipFuncSetAttribute(limit.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, limit.bytes) != hipSuccess)
+        return false;
+    }
     configured = true;
   }
   const uint32_t grid = (a.row_tiles * a.column_tiles + 255) / 256 * 256;
@@ -512,17 +894,30 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
       (const uint16_t *)p.x.base + p.x.offset, p.x.stride[0], p.rows, p.inner, kt, (uint16_t *)ws,
       (float *)after, flag);
   if (!kept || fresh) {
-    const uint64_t weight_threads = (uint64_t)p.columns * (kt / 64) * 8;
-    prepare_weights_kernel<<<(uint32_t)((weight_threads + 255) / 256), 256, 0, stream>>>(
-        (const uint32_t *)p.packed.base + p.packed.offset,
-        (const uint16_t *)p.scales.base + p.scales.offset,
-        (const uint16_t *)p.biases.base + p.biases.offset, p.columns, p.inner, kt,
-        (uint16_t *)b_operand, flag);
+    if (packed_form) {
+      const uint64_t threads = (uint64_t)p.columns * ((kt - p.inner) / 8);
+      prepare_extras_kernel<<<(uint32_t)((threads + 255) / 256), 256, 0, stream>>>(
+          (const uint16_t *)p.scales.base + p.scales.offset, (const uint16_t *)p.biases.base + p.biases.offset,
+          p.columns, p.inner, kt, (uint16_t *)b_operand, flag);
+    } else {
+      const uint64_t weight_threads = (uint64_t)p.columns * (kt / 64) * 8;
+      prepare_weights_kernel<<<(uint32_t)((weight_threads + 255) / 256), 256, 0, stream>>>(
+          (const uint32_t *)p.packed.base + p.packed.offset,
+          (const uint16_t *)p.scales.base + p.scales.offset,
+          (const uint16_t *)p.biases.base + p.biases.offset, p.columns, p.inner, kt,
+          (uint16_t *)b_operand, flag);
+    }
   }
-  if (small_tiles)
+  if (packed_form) {
+    if (small_tiles)
+      gemm_q4_kernel<64><<<grid, 256, gemm_q4_lds_bytes(64), stream>>>(a);
+    else
+      gemm_q4_kernel<128><<<grid, 256, gemm_q4_lds_bytes(128), stream>>>(a);
+  } else if (small_tiles) {
     gemm_f16_kernel<kGemmK, kGemmStages, 64><<<grid, 256, gemm_lds_bytes(64), stream>>>(a);
-  else
+  } else {
     gemm_f16_kernel<kGemmK, kGemmStages, 128><<<grid, 256, gemm_lds_bytes(128), stream>>>(a);
+  }
   *refused = (kept && verdict == 0) ? nullptr : flag;
   // the first product over kept weights learns, once, whether they fit the scheme
   if (kept && fresh) backend_prepared_verdict(backend, key);

@@ -60,7 +60,8 @@ def release(hip, *tensors):
     (128, 151936, 2048, "config 3 lm_head"),
     (2048, 4096, 1024, "config 1 stacked qkv over the packed 2048-token batch"),
     (8256, 512, 5120, "config 4 prefill rows, a 512-column slice of a projection"),
-    (8256, 256, 17408, "config 4 down projection depth, a 256-column slice"),
+    (8256, 256, 17408, "config 4 down projection depth, a 256-column slice (128 x 128 tiles)"),
+    (8256, 1536, 17408, "config 4 down projection depth in 256 x 256 tiles (33 x 6 of them)"),
 ])
 def test_quantised_projection_fast_and_generic_paths_agree(hip, rows, n, k, note):
     weights = quantised(hip, n, k, seed=101)
@@ -102,6 +103,30 @@ def test_config4_gate_up_projection_at_full_width(hip):
     rows, n, k = 8256, 34816, 5120
     weights = quantised(hip, n, k, seed=131)
     x = seeded(hip, DType.BF16, (rows, k), 131, 4)
+    fast = hip.alloc(DType.BF16, (rows, n))
+    commands = CommandList()
+    commands.dispatch(Op.quant_matmul(4, 64), [x, *weights], fast)
+    run(hip, commands)
+    for first in (0, 4096, rows - 64):
+        block = as_f32(hip, x.narrow(0, first, 64))
+        generic = hip.alloc(DType.F32, (64, n))
+        commands = CommandList()
+        commands.dispatch(Op.quant_matmul(4, 64), [block, *weights], generic)
+        run(hip, commands)
+        assert_close(to_f32(hip.read(fast.narrow(0, first, 64)), DType.BF16),
+                     to_f32(hip.read(generic), DType.F32), DType.BF16)
+        release(hip, block, generic)
+    release(hip, x, fast, *weights)
+
+
+def test_config4_down_projection_at_full_depth(hip):
+    """Config 4's down projection at its real shape, 8256 rows x 5120 columns x 17408, the deepest
+    contraction of the configurations (the case the centred weights and the scaled rows of the
+    tiled GEMM exist for): one product on the matrix cores over all rows, and the f32 kernels over
+    three 64-row blocks of the same rows (first, middle, last), every column."""
+    rows, n, k = 8256, 5120, 17408
+    weights = quantised(hip, n, k, seed=133)
+    x = seeded(hip, DType.BF16, (rows, k), 133, 4)
     fast = hip.alloc(DType.BF16, (rows, n))
     commands = CommandList()
     commands.dispatch(Op.quant_matmul(4, 64), [x, *weights], fast)

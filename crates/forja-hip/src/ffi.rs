@@ -136,7 +136,20 @@ pub struct fh_device_info {
     pub wavefront: u32,
 }
 
-unsafe extern "C" {
+unsafe /// `fh_dispatch_timing`: device time from the start of a submission to the start and end of one
+/// executed dispatch (or group of dispatches executed together).
+#[repr(C)]
+#[derive(Clone, Copy, Debug, Default)]
+pub struct fh_dispatch_timing {
+    pub dispatch: u32,
+    pub dispatches: u32,
+    pub op: u32,
+    pub reserved: u32,
+    pub start_ns: u64,
+    pub end_ns: u64,
+}
+
+extern "C" {
     pub fn fh_create(device: c_int, out: *mut *mut fh_backend) -> u32;
     pub fn fh_destroy(backend: *mut fh_backend);
     pub fn fh_alloc(backend: *mut fh_backend, bytes: u64, out: *mut fh_buffer) -> u32;
@@ -162,6 +175,9 @@ unsafe extern "C" {
     pub fn fh_submission_free(submission: *mut fh_submission);
     pub fn fh_device_info_get(backend: *mut fh_backend, out: *mut fh_device_info) -> u32;
     pub fn fh_memory_usage(backend: *mut fh_backend, bytes: *mut u64) -> u32;
+    pub fn fh_set_memory_limit(backend: *mut fh_backend, bytes: u64) -> u32;
+    pub fn fh_submit_profiled(backend: *mut fh_backend, dispatches: *const fh_dispatch, count: u32, out: *mut *mut fh_submission) -> u32;
+    pub fn fh_submission_profile(submission: *mut fh_submission, out: *mut fh_dispatch_timing, capacity: u32, n: *mut u32) -> u32;
     pub fn fh_synchronize(backend: *mut fh_backend) -> u32;
     pub fn fh_profile_enable(backend: *mut fh_backend, enabled: c_int) -> u32;
     pub fn fh_profile_select(backend: *mut fh_backend, class_mask: u32) -> u32;

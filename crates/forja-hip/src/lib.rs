@@ -21,9 +21,9 @@ use std::time::Duration;
 
 use forja_core::{
     AllocationRegistry, Backend, BackendError, BinOp, BufferId, CommandList, CompletionResource,
-    DType, DeviceInfo, Dispatch, Inst, KernelSignature, Layout, MemoryUsage, Op,
-    PagedCopyDirection, ProgramKind, ReadonlyImport, RedOp, Submission, Tensor, UnOp,
-    ValidatedProgram, ValueType, ViewOp,
+    DType, DeviceInfo, Dispatch, DispatchProfile, Inst, KernelCost, KernelSignature, Layout,
+    MemoryUsage, Op, PagedCopyDirection, ProfileTensor, ProgramKind, ReadonlyImport, RedOp,
+    Submission, SubmissionProfile, Tensor, UnOp, ValidatedProgram, ValueType, ViewOp,
 };
 use forja_mmap::MappedRegion;
 
@@ -432,6 +432,7 @@ impl HipBackend {
         &self,
         commands: CommandList,
         owners: Vec<CompletionResource>,
+        profiled: bool,
     ) -> Result<HipSubmission, BackendError> {
         let dispatches = commands.into_dispatches();
         let mut keep = Vec::new();
@@ -442,19 +443,20 @@ impl HipBackend {
                 .map(|dispatch| self.lower_dispatch(&registry, dispatch, &mut keep))
                 .collect::<Result<Vec<_>, _>>()?
         };
+        let count = u32::try_from(lowered.len()).map_err(|_| BackendError::InvalidInput)?;
         let mut raw = std::ptr::null_mut();
         check(unsafe {
-            ffi::fh_submit(
-                self.raw.ptr(),
-                lowered.as_ptr(),
-                u32::try_from(lowered.len()).map_err(|_| BackendError::InvalidInput)?,
-                &mut raw,
-            )
+            if profiled {
+                ffi::fh_submit_profiled(self.raw.ptr(), lowered.as_ptr(), count, &mut raw)
+            } else {
+                ffi::fh_submit(self.raw.ptr(), lowered.as_ptr(), count, &mut raw)
+            }
         })?;
         Ok(HipSubmission {
             raw: NonNull::new(raw).ok_or(BackendError::ExecutionFailed)?,
             _backend: Arc::clone(&self.raw),
-            _dispatches: dispatches,
+            dispatches,
+            profiled,
             _programs: keep,
             _owners: owners,
         })
@@ -467,7 +469,8 @@ impl HipBackend {
 pub struct HipSubmission {
     raw: NonNull<ffi::fh_submission>,
     _backend: Arc<RawBackend>,
-    _dispatches: Vec<Dispatch>,
+    dispatches: Vec<Dispatch>,
+    profiled: bool,
     _programs: Vec<Arc<HipProgram>>,
     _owners: Vec<CompletionResource>,
 }
@@ -499,6 +502,75 @@ impl Submission for HipSubmission {
             nanoseconds => Some(Duration::from_nanos(nanoseconds)),
         }
     }
+
+    /// Per-dispatch device timeline of a submission made by `submit_profiled_retained`, after a
+    /// successful wait (crates/forja-core/src/backend.rs:455-579).  The library times every
+    /// dispatch it executes; dispatches it executed as one group (per-lane attention fused into
+    /// one ragged launch) share the group's interval, the first member carrying `gap_before`.
+    /// Costs are the logical ones of `KernelCost::of`; this backend has no variant catalog, no
+    /// admission forecast and no padded-flop accounting, so those fields stay empty.
+    fn profile(&self) -> Option<SubmissionProfile> {
+        if !self.profiled {
+            return None;
+        }
+        let mut count = 0_u32;
+        let status = unsafe {
+            ffi::fh_submission_profile(self.raw.as_ptr(), std::ptr::null_mut(), 0, &mut count)
+        };
+        if status != ffi::FH_OK {
+            return None; // not waited for yet
+        }
+        let mut timings = vec![ffi::fh_dispatch_timing::default(); count as usize];
+        let status = unsafe {
+            ffi::fh_submission_profile(self.raw.as_ptr(), timings.as_mut_ptr(), count, &mut count)
+        };
+        if status != ffi::FH_OK {
+            return None;
+        }
+        let mut per_dispatch = Vec::with_capacity(self.dispatches.len());
+        let mut previous_end = Duration::ZERO;
+        for timing in &timings {
+            let start = Duration::from_nanos(timing.start_ns);
+            let end = Duration::from_nanos(timing.end_ns);
+            let first = timing.dispatch as usize;
+            let members = self.dispatches.get(first..first + timing.dispatches as usize)?;
+            for (nth, dispatch) in members.iter().enumerate() {
+                let cost = KernelCost::of(dispatch).unwrap_or_default();
+                per_dispatch.push(DispatchProfile {
+                    scope: dispatch.profile_scope().map(|scope| (**scope).clone()),
+                    op: dispatch.op(),
+                    kernel: operation_name(timing.op),
+                    variant: None,
+                    alternatives: Vec::new(),
+                    physical_dispatches: u64::from(nth == 0),
+                    physical_threadgroups: 0,
+                    predicted_gpu: Duration::ZERO,
+                    compute_dtype: DType::F32,
+                    cost,
+                    scheduled_cost: cost,
+                    critical_path_cost: KernelCost::default(),
+                    padded_flops: [cost.flops, cost.flops],
+                    inputs: dispatch.inputs().iter().map(ProfileTensor::from).collect(),
+                    outputs: dispatch.outputs().iter().map(ProfileTensor::from).collect(),
+                    barrier: true, // one in-order stream: every dispatch follows the one before
+                    gpu_start: start,
+                    gpu_end: end,
+                    gap_before: if nth == 0 { start.saturating_sub(previous_end) } else { Duration::ZERO },
+                    gpu_time: if nth == 0 { end.saturating_sub(start) } else { Duration::ZERO },
+                    internal: Vec::new(),
+                });
+            }
+            previous_end = end;
+        }
+        Some(SubmissionProfile {
+            command_buffers: 1,
+            gpu_time: self.gpu_time().unwrap_or_default(),
+            dispatches: self.dispatches.len() as u64,
+            barriers: self.dispatches.len().saturating_sub(1) as u64,
+            per_dispatch,
+            ..SubmissionProfile::default()
+        })
+    }
 }
 
 impl Drop for HipSubmission {
@@ -518,7 +590,14 @@ impl Backend for HipBackend {
         if status != ffi::FH_OK {
             return MemoryUsage::default();
         }
+        // every device byte the library holds for this backend, kept operands of the prefill
+        // products and workspaces included
         MemoryUsage { charged_bytes: bytes, device_bytes: Some(bytes), ..MemoryUsage::default() }
+    }
+
+    fn set_memory_limit(&self, bytes: u64) {
+        // the quota covers allocations and kept operands; the library evicts the latter first
+        let _ = unsafe { ffi::fh_set_memory_limit(self.raw.ptr(), bytes) };
     }
 
     fn device_info(&self) -> Result<DeviceInfo, BackendError> {
@@ -661,7 +740,7 @@ impl Backend for HipBackend {
     }
 
     fn submit(&self, commands: CommandList) -> Result<Self::Submission, BackendError> {
-        self.submit_owned(commands, Vec::new())
+        self.submit_owned(commands, Vec::new(), false)
     }
 
     fn submit_retained(
@@ -669,7 +748,7 @@ impl Backend for HipBackend {
         commands: CommandList,
         owners: Vec<CompletionResource>,
     ) -> Result<Self::Submission, BackendError> {
-        self.submit_owned(commands, owners)
+        self.submit_owned(commands, owners, false)
     }
 
     fn submit_profiled_retained(
@@ -677,9 +756,8 @@ impl Backend for HipBackend {
         commands: CommandList,
         owners: Vec<CompletionResource>,
     ) -> Result<Self::Submission, BackendError> {
-        // Per-dispatch device timelines are read with rocprofv3; the submission reports its
-        // device time through `gpu_time`.
-        self.submit_owned(commands, owners)
+        // one device timer per executed dispatch; read back by `Submission::profile`
+        self.submit_owned(commands, owners, true)
     }
 }
 

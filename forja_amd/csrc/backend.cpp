@@ -145,6 +145,15 @@ struct fh_submission {
   fh_status result = FH_OK;
   fh_error error{};
   uint64_t gpu_ns = 0;
+  // fh_submit_profiled: one pair of events per executed dispatch (or fused group of dispatches),
+  // turned into offsets from `start` once the submission has been waited for
+  bool profiled = false;
+  struct Span {
+    uint32_t first, dispatches, op;
+    hipEvent_t begin, finish;
+  };
+  std::vector<Span> spans;
+  std::vector<fh_dispatch_timing> timings;
 };
 
 struct fh_backend {
@@ -204,28 +213,67 @@ struct fh_backend {
   std::vector<Prepared> prepared;
   std::unordered_map<uint64_t, uint32_t> prepared_watch;
   uint64_t prepared_bytes = 0, prepared_limit = 0;
+  // operands whose weights were rewritten while nothing could be freed (fh_submit_static): freed
+  // by the next call that may wait for the stream
+  std::vector<Prepared> dead_prepared;
+  // Backend::set_memory_limit: the most `used_bytes` plus the kept operands may reach (0: no limit)
+  uint64_t memory_limit = 0;
+  static constexpr uint64_t kPreparedTail = 256;   // the flag word behind an operand, padded
+  void unwatch(const Prepared &e) {
+    for (uint64_t watched : e.key.buffers) {
+      auto it = prepared_watch.find(watched);
+      if (it != prepared_watch.end() && --it->second == 0) prepared_watch.erase(it);
+    }
+  }
+  void free_operand(Prepared &e) {   // the stream must be idle
+    if (!e.operand) return;
+    (void)hipFree(e.operand);
+    e.operand = nullptr;
+    prepared_bytes -= e.bytes + kPreparedTail;
+  }
+  void reap_dead_prepared() {   // from entry points that may wait for the stream
+    if (dead_prepared.empty() || static_mode) return;
+    (void)hipStreamSynchronize(stream);
+    for (Prepared &e : dead_prepared) free_operand(e);
+    dead_prepared.clear();
+  }
+  // Frees every kept operand (an allocation failed, or the memory limit is reached): products
+  // prepare into the workspace again, or keep a fresh copy later.
+  bool evict_prepared() {
+    if (static_mode || (prepared.empty() && dead_prepared.empty())) return false;
+    (void)hipStreamSynchronize(stream);
+    bool freed = false;
+    for (Prepared &e : dead_prepared) freed |= e.operand != nullptr, free_operand(e);
+    dead_prepared.clear();
+    for (size_t i = 0; i < prepared.size();) {
+      Prepared &e = prepared[i];
+      if (!e.operand) {   // a verdict only: costs nothing, stays
+        ++i;
+        continue;
+      }
+      freed = true;
+      free_operand(e);
+      unwatch(e);
+      prepared[i] = prepared.back();
+      prepared.pop_back();
+    }
+    return freed;
+  }
   void drop_prepared(uint64_t buffer) {   // the allocation is written or released
     if (prepared_watch.find(buffer) == prepared_watch.end()) return;
-    if (static_mode) {
-      // nothing may be freed (or waited for) now: the entries stop matching and go with the backend
-      for (Prepared &e : prepared)
-        if (e.key.buffers[0] == buffer || e.key.buffers[1] == buffer || e.key.buffers[2] == buffer)
-          e.key.columns = 0;
-      return;
-    }
-    (void)hipStreamSynchronize(stream);   // kernels in flight may still read an operand
+    const bool can_wait = !static_mode;
+    if (can_wait) (void)hipStreamSynchronize(stream);   // kernels in flight may still read an operand
     for (size_t i = 0; i < prepared.size();) {
-      const Prepared &e = prepared[i];
+      Prepared &e = prepared[i];
       if (e.key.buffers[0] != buffer && e.key.buffers[1] != buffer && e.key.buffers[2] != buffer) {
         ++i;
         continue;
       }
-      (void)hipFree(e.operand);
-      prepared_bytes -= e.bytes;
-      for (uint64_t watched : e.key.buffers) {
-        auto it = prepared_watch.find(watched);
-        if (it != prepared_watch.end() && --it->second == 0) prepared_watch.erase(it);
-      }
+      if (can_wait)
+        free_operand(e);
+      else if (e.operand)
+        dead_prepared.push_back(e);   // still allocated and still counted, until it is reaped
+      unwatch(e);
       prepared[i] = prepared.back();
       prepared.pop_back();
     }
@@ -268,7 +316,14 @@ struct fh_backend {
     have = 0;
     uint64_t want = std::max<uint64_t>(bytes, floor);
     void *fresh = nullptr;
-    if (hipMalloc(&fresh, want) != hipSuccess) return false;
+    if (hipMalloc(&fresh, want) != hipSuccess) {
+      (void)hipGetLastError();
+      // out of memory: the kept operands of the prefill products go first, then once more
+      if (!evict_prepared() || hipMalloc(&fresh, want) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
+    }
     ptr = (char *)fresh;
     have = want;
     return true;
@@ -1779,6 +1834,11 @@ void recycle_submission(fh_backend *b, fh_submission *s) {
   if (s->start) b->event_pool.push_back(s->start);
   if (s->end) b->event_pool.push_back(s->end);
   if (s->done) b->event_pool.push_back(s->done);
+  for (auto &span : s->spans) {
+    b->event_pool.push_back(span.begin);
+    b->event_pool.push_back(span.finish);
+  }
+  s->spans.clear();
   s->device_errors = nullptr;
   s->host_errors = nullptr;
   s->start = s->end = s->done = nullptr;
@@ -1875,6 +1935,7 @@ void fh_destroy(fh_backend *b) {
     if (b->route_plan) (void)hipFree(b->route_plan);
     if (b->attention_plan) (void)hipFree(b->attention_plan);
     for (auto &e : b->prepared) (void)hipFree(e.operand);
+    for (auto &e : b->dead_prepared) (void)hipFree(e.operand);
     for (auto &e : b->error_pool) {
       (void)hipFree(e.device);
       (void)hipHostFree(e.host);
@@ -1897,7 +1958,18 @@ void fh_destroy(fh_backend *b) {
 static fh_status alloc_locked(fh_backend *b, uint64_t bytes, bool readonly, fh_buffer *out) {
   void *ptr = nullptr;
   uint64_t want = bytes == 0 ? 256 : bytes;
-  if (hipMalloc(&ptr, want) != hipSuccess) return FH_ALLOCATION_FAILED;
+  b->reap_dead_prepared();
+  // the quota covers the caller's allocations and what the library keeps for them; what it keeps
+  // goes before an allocation is refused
+  if (b->memory_limit && b->used_bytes + b->prepared_bytes + bytes > b->memory_limit) b->evict_prepared();
+  if (b->memory_limit && b->used_bytes + b->prepared_bytes + bytes > b->memory_limit) return FH_QUOTA_EXCEEDED;
+  if (hipMalloc(&ptr, want) != hipSuccess) {
+    (void)hipGetLastError();
+    if (!b->evict_prepared() || hipMalloc(&ptr, want) != hipSuccess) {
+      (void)hipGetLastError();
+      return FH_ALLOCATION_FAILED;
+    }
+  }
   if (hipMemsetAsync(ptr, 0, want, b->stream) != hipSuccess) {
     (void)hipFree(ptr);
     return FH_DEVICE_EXECUTION_FAILED;
@@ -1923,6 +1995,7 @@ fh_status fh_release(fh_backend *b, fh_buffer buffer) {
   if (it == b->allocations.end()) return FH_INVALID_INPUT;
   (void)hipSetDevice(b->device);
   (void)hipStreamSynchronize(b->stream);
+  b->reap_dead_prepared();
   b->drop_prepared(buffer);
   (void)hipFree(it->second.ptr);
   b->used_bytes -= it->second.bytes;
@@ -1953,6 +2026,7 @@ fh_status fh_write(fh_backend *b, fh_buffer buffer, uint64_t byte_offset, const 
     return FH_INVALID_INPUT;
   if (len == 0) return FH_OK;
   (void)hipSetDevice(b->device);
+  b->reap_dead_prepared();
   b->drop_prepared(buffer);
   // Small writes are staged through a pinned ring and ordered on the stream without waiting for
   // it; the caller's bytes may be reused as soon as this returns either way.
@@ -2121,12 +2195,38 @@ fh_status fh_release_program(fh_backend *b, fh_program program) {
   return FH_OK;
 }
 
+static fh_status submit_locked(fh_backend *b, const fh_dispatch *dispatches, uint32_t count, bool profiled,
+                               fh_submission **out);
+
 fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count,
                     fh_submission **out) {
   if (!b || !out || (!dispatches && count)) return FH_INVALID_INPUT;
   *out = nullptr;
   std::lock_guard<std::mutex> lock(b->mutex);
   (void)hipSetDevice(b->device);
+  return submit_locked(b, dispatches, count, false, out);
+}
+
+fh_status fh_submit_profiled(fh_backend *b, const fh_dispatch *dispatches, uint32_t count,
+                             fh_submission **out) {
+  if (!b || !out || (!dispatches && count)) return FH_INVALID_INPUT;
+  *out = nullptr;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  return submit_locked(b, dispatches, count, true, out);
+}
+
+fh_status fh_submission_profile(fh_submission *s, fh_dispatch_timing *out, uint32_t capacity, uint32_t *n) {
+  if (!s || !n || (!out && capacity)) return FH_INVALID_INPUT;
+  if (!s->waited) return FH_INVALID_INPUT;   // the timeline exists once the submission has been waited for
+  *n = (uint32_t)s->timings.size();
+  for (uint32_t i = 0; i < *n && i < capacity; ++i) out[i] = s->timings[i];
+  return FH_OK;
+}
+
+static fh_status submit_locked(fh_backend *b, const fh_dispatch *dispatches, uint32_t count, bool profiled,
+                               fh_submission **out) {
+  b->reap_dead_prepared();
   // Validate the whole list before anything is enqueued (lib.rs:1423-1432).
   for (uint32_t i = 0; i < count; ++i) {
     fh_status status = process(b, dispatches[i], nullptr, false);
@@ -2137,6 +2237,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
   s->backend = b;
   s->serial = b->next_serial++;
   s->count = count;
+  s->profiled = profiled;
   s->ops.resize(count);
   uint32_t slots = count == 0 ? 1 : count;
   bool pooled = false;
@@ -2199,7 +2300,7 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
       no_run_before = i + run.dispatches;
     for (uint32_t member = 0; member < consumed; ++member) s->ops[i + member] = dispatches[i + member].op;
     hipEvent_t t0 = nullptr, t1 = nullptr;
-    if (b->profiling >= 2) {
+    if (b->profiling >= 2 || profiled) {
       t0 = take_event(b);
       t1 = take_event(b);
       (void)hipEventRecord(t0, b->stream);
@@ -2231,9 +2332,12 @@ fh_status fh_submit(fh_backend *b, const fh_dispatch *dispatches, uint32_t count
       }
     }
     for (uint32_t member = 0; member < consumed; ++member) note_outputs(dispatches[i + member]);
-    if (b->profiling >= 2) {
+    if (t1) {
       (void)hipEventRecord(t1, b->stream);
-      b->timed.push_back({t0, t1, fused ? (uint32_t)FH_KC_ATTENTION : kernel_class_of(dispatches[i].op)});
+      if (profiled)
+        s->spans.push_back({i, consumed, dispatches[i].op, t0, t1});
+      else
+        b->timed.push_back({t0, t1, fused ? (uint32_t)FH_KC_ATTENTION : kernel_class_of(dispatches[i].op)});
     }
     i += consumed;
   }
@@ -2419,6 +2523,19 @@ fh_status fh_wait(fh_submission *s, uint64_t timeout_ns, fh_error *error) {
       float ms = 0.0f;
       if (hipEventElapsedTime(&ms, s->start, s->end) == hipSuccess)
         s->gpu_ns = (uint64_t)((double)ms * 1e6);
+      for (const auto &span : s->spans) {
+        float begin_ms = 0.0f, finish_ms = 0.0f;
+        if (hipEventElapsedTime(&begin_ms, s->start, span.begin) != hipSuccess ||
+            hipEventElapsedTime(&finish_ms, s->start, span.finish) != hipSuccess)
+          continue;
+        fh_dispatch_timing timing{};
+        timing.dispatch = span.first;
+        timing.dispatches = span.dispatches;
+        timing.op = span.op;
+        timing.start_ns = (uint64_t)((double)begin_ms * 1e6);
+        timing.end_ns = (uint64_t)((double)finish_ms * 1e6);
+        s->timings.push_back(timing);
+      }
       for (uint32_t i = 0; i < s->count; ++i) {
         if (!s->host_errors[i].flag) continue;
         s->result = failure_of(s->ops[i], i, s->serial, s->host_errors[i], &s->error);
@@ -2473,7 +2590,17 @@ fh_status fh_device_info_get(fh_backend *b, fh_device_info *out) {
 fh_status fh_memory_usage(fh_backend *b, uint64_t *bytes) {
   if (!b || !bytes) return FH_INVALID_INPUT;
   std::lock_guard<std::mutex> lock(b->mutex);
-  *bytes = b->used_bytes + b->workspace_bytes;
+  *bytes = b->used_bytes + b->prepared_bytes + b->workspace_bytes + b->accumulator_bytes + b->route_plan_bytes +
+           b->attention_plan_bytes + b->lane_scratch_bytes;
+  return FH_OK;
+}
+
+fh_status fh_set_memory_limit(fh_backend *b, uint64_t bytes) {
+  if (!b) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  b->memory_limit = bytes;
+  if (bytes && b->used_bytes + b->prepared_bytes > bytes) b->evict_prepared();
   return FH_OK;
 }
 
@@ -2591,9 +2718,9 @@ char *backend_prepared_weights(fh_backend *b, const PreparedKey &key, uint64_t b
   *verdict = -1;
   if (b->static_mode) return nullptr;
   for (const auto &e : b->prepared)
-    if (same_weights(e.key, key) && e.bytes == bytes) {
+    if (same_weights(e.key, key) && (e.bytes == bytes || !e.operand)) {
       *verdict = e.verdict;
-      return e.operand;
+      return e.operand;   // null for weights known to be outside the scheme: the verdict is all that is kept
     }
   if (b->prepared_limit == 0) {
     // a quarter of the device's memory unless FORJA_HIP_PREPARED_MB says otherwise (0: keep nothing)
@@ -2601,14 +2728,16 @@ char *backend_prepared_weights(fh_backend *b, const PreparedKey &key, uint64_t b
     b->prepared_limit = env ? (uint64_t)strtoull(env, nullptr, 10) << 20 : (uint64_t)b->props.totalGlobalMem / 4;
     if (b->prepared_limit == 0) b->prepared_limit = 1;   // asked for nothing: nothing fits
   }
-  if (b->prepared_bytes + bytes + 256 > b->prepared_limit) return nullptr;
+  const uint64_t cost = bytes + fh_backend::kPreparedTail;
+  if (b->prepared_bytes + cost > b->prepared_limit) return nullptr;
+  if (b->memory_limit && b->used_bytes + b->prepared_bytes + cost > b->memory_limit) return nullptr;
   void *ptr = nullptr;
-  if (hipMalloc(&ptr, bytes + 256) != hipSuccess) {
+  if (hipMalloc(&ptr, cost) != hipSuccess) {
     (void)hipGetLastError();   // no room: the workspace serves
     return nullptr;
   }
   b->prepared.push_back({key, (char *)ptr, bytes, -1});
-  b->prepared_bytes += bytes + 256;
+  b->prepared_bytes += cost;
   for (uint64_t watched : key.buffers) ++b->prepared_watch[watched];
   *fresh = true;
   return (char *)ptr;
@@ -2616,12 +2745,14 @@ char *backend_prepared_weights(fh_backend *b, const PreparedKey &key, uint64_t b
 
 void backend_prepared_verdict(fh_backend *b, const PreparedKey &key) {
   for (auto &e : b->prepared)
-    if (same_weights(e.key, key)) {
+    if (same_weights(e.key, key) && e.operand) {
       uint32_t flag = 1;
       if (hipMemcpyAsync(&flag, e.operand + e.bytes, sizeof(flag), hipMemcpyDeviceToHost, b->stream) != hipSuccess ||
           hipStreamSynchronize(b->stream) != hipSuccess)
         return;   // stays unknown: products keep their conditioned second kernel
       e.verdict = flag ? 1 : 0;
+      // outside the scheme: the operand is never read again (the stream has just been waited for)
+      if (e.verdict == 1) b->free_operand(e);
       return;
     }
 }

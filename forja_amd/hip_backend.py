@@ -51,6 +51,11 @@ class FhError(C.Structure):
                 ("reserved", C.c_uint32)]
 
 
+class FhDispatchTiming(C.Structure):
+    _fields_ = [("dispatch", C.c_uint32), ("dispatches", C.c_uint32), ("op", C.c_uint32),
+                ("reserved", C.c_uint32), ("start_ns", C.c_uint64), ("end_ns", C.c_uint64)]
+
+
 class FhDeviceInfo(C.Structure):
     _fields_ = [("family", C.c_char * 64), ("total_memory", C.c_uint64), ("lds_bytes", C.c_uint64),
                 ("compute_units", C.c_uint32), ("wavefront", C.c_uint32)]
@@ -59,7 +64,8 @@ class FhDeviceInfo(C.Structure):
 EXPORTS = [
     "fh_create", "fh_destroy", "fh_alloc", "fh_release", "fh_import", "fh_write", "fh_read",
     "fh_read_tensor", "fh_prepare_program", "fh_release_program", "fh_submit", "fh_submit_static", "fh_wait",
-    "fh_gpu_time_ns", "fh_submission_free", "fh_device_info_get", "fh_memory_usage",
+    "fh_gpu_time_ns", "fh_submission_free", "fh_device_info_get", "fh_memory_usage", "fh_set_memory_limit",
+    "fh_submit_profiled", "fh_submission_profile",
     "fh_synchronize", "fh_profile_enable", "fh_profile_select", "fh_profile_reset", "fh_profile_read",
     "fh_fusion_enable", "fh_fusion_stats", "fh_version",
 ]
@@ -98,6 +104,8 @@ def load_library():
     lib.fh_submission_free.restype = None
     lib.fh_device_info_get.argtypes = [vp, C.POINTER(FhDeviceInfo)]
     lib.fh_memory_usage.argtypes = [vp, C.POINTER(u64)]
+    lib.fh_set_memory_limit.argtypes = [vp, u64]
+    lib.fh_submission_profile.argtypes = [vp, C.POINTER(FhDispatchTiming), u32, C.POINTER(u32)]
     lib.fh_synchronize.argtypes = [vp]
     lib.fh_profile_enable.argtypes = [vp, C.c_int]
     lib.fh_profile_reset.argtypes = [vp]
@@ -149,6 +157,15 @@ class HipSubmission:
 
     def gpu_time_ns(self) -> int:
         return int(self._lib.fh_gpu_time_ns(self._handle))
+
+    def profile(self) -> list:
+        """`Submission::profile`: per-dispatch device timeline of a submission made by
+        `submit_profiled`, as (first dispatch, dispatches covered, op, start_ns, end_ns)."""
+        count = C.c_uint32()
+        _check(self._lib.fh_submission_profile(self._handle, None, 0, C.byref(count)))
+        entries = (FhDispatchTiming * max(count.value, 1))()
+        _check(self._lib.fh_submission_profile(self._handle, entries, count.value, C.byref(count)))
+        return [(e.dispatch, e.dispatches, e.op, e.start_ns, e.end_ns) for e in entries[:count.value]]
 
     def free(self):
         if self._handle is not None:
@@ -309,6 +326,13 @@ class HipBackend:
         _check(self._lib.fh_submit(self._handle, encoded.array, encoded.count, C.byref(handle)))
         return HipSubmission(self, handle)
 
+    def submit_profiled(self, commands) -> HipSubmission:
+        """`Backend::submit_profiled_retained`: a device timer around every dispatch."""
+        encoded = commands if isinstance(commands, EncodedCommands) else self.encode(commands)
+        handle = C.c_void_p()
+        _check(self._lib.fh_submit_profiled(self._handle, encoded.array, encoded.count, C.byref(handle)))
+        return HipSubmission(self, handle)
+
     def submit_static(self, commands, wait: bool = True) -> None:
         """fh_submit_static: the same dispatches executed without any allocation, all device
         scratch taken from the library's fixed array.  `wait` false only enqueues."""
@@ -331,9 +355,14 @@ class HipBackend:
                 "wavefront": info.wavefront}
 
     def memory_usage(self) -> int:
+        """MemoryUsage::charged_bytes: every device byte the backend holds."""
         value = C.c_uint64()
         _check(self._lib.fh_memory_usage(self._handle, C.byref(value)))
         return value.value
+
+    def set_memory_limit(self, limit: int):
+        """Backend::set_memory_limit: quota over allocations plus kept operands; 0 lifts it."""
+        _check(self._lib.fh_set_memory_limit(self._handle, int(limit)))
 
     # ---- profiling aid
     def profile_enable(self, level: int):

@@ -248,6 +248,25 @@ void write_and_release_contract(HipBackend &backend) {
   check(!backend.read(t).ok(), "released tensor is rejected");
 }
 
+// Backend::submit_profiled_retained / Submission::profile (crates/forja-core/src/backend.rs:455-579)
+// and Backend::set_memory_limit (:683-686).
+void profile_and_quota_contract(HipBackend &backend) {
+  Tensor a = backend.alloc(DType::F32, {64, 64}).value, b = backend.alloc(DType::F32, {64, 64}).value;
+  CommandList commands;
+  commands.dispatch(Op::copy(), {a}, {b});
+  commands.dispatch(Op::copy(), {b}, {a});
+  Result<Submission> submitted = backend.submit_profiled(commands);
+  check(submitted.ok() && submitted.value.wait().ok(), "profiled submission runs");
+  std::vector<fh_dispatch_timing> timeline = submitted.value.profile();
+  check(timeline.size() == 2 && timeline[0].dispatch == 0 && timeline[1].dispatch == 1 &&
+            timeline[0].start_ns <= timeline[0].end_ns && timeline[0].end_ns <= timeline[1].start_ns,
+        "one ordered timeline entry per dispatch");
+  const uint64_t held = backend.memory_usage().value;
+  check(backend.set_memory_limit(held).ok(), "set_memory_limit");
+  check(backend.alloc(DType::F32, {1u << 20, 64}).error.code == FH_QUOTA_EXCEEDED, "allocation beyond the limit refused");
+  check(backend.set_memory_limit(0).ok() && backend.alloc(DType::F32, {1024}).ok(), "limit lifted");
+}
+
 }  // namespace
 
 int main() {
@@ -264,6 +283,7 @@ int main() {
   paged_append_stores_both_planes(backend);
   paged_attention_hand_checked(backend);
   write_and_release_contract(backend);
+  profile_and_quota_contract(backend);
   delete created.value;
   if (failures == 0) std::printf("conformance: all checks passed\n");
   return failures == 0 ? 0 : 1;

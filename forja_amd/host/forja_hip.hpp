@@ -301,6 +301,16 @@ class Submission {
     return r;
   }
   uint64_t gpu_time_ns() const { return raw_ ? fh_gpu_time_ns(raw_) : 0; }
+  // Submission::profile: the per-dispatch device timeline of a submission made by
+  // submit_profiled, once it has been waited for (empty otherwise).
+  std::vector<fh_dispatch_timing> profile() const {
+    std::vector<fh_dispatch_timing> timings;
+    uint32_t n = 0;
+    if (!raw_ || fh_submission_profile(raw_, nullptr, 0, &n) != FH_OK || n == 0) return timings;
+    timings.resize(n);
+    if (fh_submission_profile(raw_, timings.data(), n, &n) != FH_OK) timings.clear();
+    return timings;
+  }
 
  private:
   void reset() {
@@ -406,6 +416,14 @@ class HipBackend {
     if (r.ok()) r.value = Submission(raw);
     return r;
   }
+  // Backend::submit_profiled_retained: submit with a device timer around every dispatch.
+  Result<Submission> submit_profiled(const CommandList &commands) {
+    Result<Submission> r;
+    fh_submission *raw = nullptr;
+    r.error.code = fh_submit_profiled(raw_, commands.dispatches().data(), (uint32_t)commands.dispatches().size(), &raw);
+    if (r.ok()) r.value = Submission(raw);
+    return r;
+  }
   Result<fh_device_info> device_info() {
     Result<fh_device_info> r;
     r.error.code = fh_device_info_get(raw_, &r.value);
@@ -414,6 +432,12 @@ class HipBackend {
   Result<uint64_t> memory_usage() {
     Result<uint64_t> r;
     r.error.code = fh_memory_usage(raw_, &r.value);
+    return r;
+  }
+  // Backend::set_memory_limit: quota over allocations plus the operands the library keeps.
+  Result<Unit> set_memory_limit(uint64_t bytes) {
+    Result<Unit> r;
+    r.error.code = fh_set_memory_limit(raw_, bytes);
     return r;
   }
   Result<Unit> synchronize() {

@@ -233,9 +233,40 @@ FH_API fh_status fh_wait(fh_submission *submission, uint64_t timeout_ns, fh_erro
 FH_API uint64_t fh_gpu_time_ns(fh_submission *submission);
 FH_API void fh_submission_free(fh_submission *submission);
 
+/* Backend::submit_profiled_retained (backend.rs:813-857): fh_submit with one device timer
+ * around every dispatch it executes.  A run of dispatches executed together (per-lane attention
+ * fused into one ragged launch, a weighted sum with the normalisation that follows it) gets one
+ * timer.  The timers cost two event records per dispatch on the stream. */
+FH_API fh_status fh_submit_profiled(fh_backend *backend, const fh_dispatch *dispatches, uint32_t count,
+                             fh_submission **out);
+/* One entry of SubmissionProfile::per_dispatch (backend.rs:455-500): device time from the start
+ * of the submission to the start and to the end of dispatch `dispatch` (gpu_start, gpu_end); the
+ * entry covers `dispatches` consecutive dispatches, more than one when they ran as one group. */
+typedef struct fh_dispatch_timing {
+  uint32_t dispatch, dispatches;
+  uint32_t op; /* fh_op_kind of the first dispatch */
+  uint32_t reserved;
+  uint64_t start_ns, end_ns;
+} fh_dispatch_timing;
+/* Submission::profile (backend.rs:609-647).  After fh_wait on a submission made by
+ * fh_submit_profiled: copies up to `capacity` entries, in dispatch order, and stores the number
+ * there are in *n (0 for a submission made by fh_submit).  FH_INVALID_INPUT before fh_wait. */
+FH_API fh_status fh_submission_profile(fh_submission *submission, fh_dispatch_timing *out, uint32_t capacity,
+                                uint32_t *n);
+
 /* Backend::device_info / memory_usage. */
 FH_API fh_status fh_device_info_get(fh_backend *backend, fh_device_info *out);
+/* MemoryUsage::charged_bytes (backend.rs:30-39): every device byte the backend holds - the
+ * caller's allocations, the operands kept for prefill products (the fp16 bias columns of weight
+ * matrices, kept from a weight's first product of more than 128 rows until the weight is written
+ * or released), workspace, epilogue accumulators, route and attention plans, lane scratch. */
 FH_API fh_status fh_memory_usage(fh_backend *backend, uint64_t *bytes);
+/* Backend::set_memory_limit (backend.rs:683-686): the most the caller's allocations plus the kept
+ * operands may take; 0 lifts the limit.  An fh_alloc or fh_import that would pass it first drops
+ * the kept operands (products then prepare into workspace again) and fails with
+ * FH_QUOTA_EXCEEDED if that is not enough.  The same eviction happens, once, when the device
+ * itself runs out of memory. */
+FH_API fh_status fh_set_memory_limit(fh_backend *backend, uint64_t bytes);
 /* Blocks until all submitted work has finished. */
 FH_API fh_status fh_synchronize(fh_backend *backend);
 

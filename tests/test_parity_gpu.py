@@ -385,6 +385,88 @@ def test_prefill_products_without_kept_weights(cpu, monkeypatch):
         frugal.close()
 
 
+def test_memory_limit_counts_and_evicts_what_the_library_keeps(cpu):
+    """`Backend::set_memory_limit` (crates/forja-core/src/backend.rs:683-686) covers the caller's
+    allocations and the operands the library keeps for prefill products; `memory_usage` counts
+    both.  An allocation that would pass the limit drops the kept operands first and succeeds;
+    one that cannot fit is refused with QuotaExceeded; results do not depend on any of it."""
+    from forja_amd.hip_backend import HipBackend
+    own = HipBackend(0)     # its own backend: the shared one holds other tests' allocations
+    try:
+        rows, n, k = 200, 2048, 512
+        weights = Quantised(29, 1, (n, k))
+        x_values = normal_bf16(29, 2, (rows, k))
+        kept = n * 64 * 2 + 256     # fp16 bias columns (3 per group of 64, padded to 64 a row) + flag
+        names = ("kept", "served by the kept operand", "prepared into workspace", "kept again")
+        x = upload(own, x_values, DType.BF16)
+        triple = weights.upload(own)
+        outs = {name: own.alloc(DType.BF16, (rows, n)) for name in names}
+        allocated = sum(t.layout.buffer_len for t in (x, *triple, *outs.values()))
+
+        def product(backend, x, triple, out):
+            commands = CommandList()
+            commands.dispatch(Op.quant_matmul(4, 64), [x, *triple], out)
+            run(backend, commands)
+        before = own.memory_usage()
+        assert before >= allocated
+        product(own, x, triple, outs["kept"])
+        held = own.memory_usage()
+        assert held >= before + kept                       # the kept operand is counted (and the workspace)
+        product(own, x, triple, outs["served by the kept operand"])
+        assert own.memory_usage() == held
+        # room for half the kept operand more: an allocation of its size fits only once it is dropped
+        own.set_memory_limit(allocated + kept + kept // 2)
+        extra = own.alloc(DType.U32, ((kept - 256) // 4,))
+        assert own.memory_usage() == held - kept + (kept - 256)
+        product(own, x, triple, outs["prepared into workspace"])     # no room to keep anything
+        assert own.memory_usage() <= held + (kept - 256)
+        with pytest.raises(BackendError) as refused:
+            own.alloc(DType.U32, (kept,))
+        assert refused.value.status == Status.QUOTA_EXCEEDED
+        own.set_memory_limit(0)
+        own.release(extra)
+        product(own, x, triple, outs["kept again"])
+        assert own.memory_usage() >= held
+        expected = cpu.alloc(DType.BF16, (rows, n))
+        product(cpu, upload(cpu, x_values, DType.BF16), weights.upload(cpu), expected)
+        for name in names:
+            compare(cpu, own, expected, outs[name])
+    finally:
+        own.close()
+
+
+def test_profiled_submission_reports_an_ordered_timeline(hip):
+    """`submit_profiled_retained` / `Submission::profile` (crates/forja-core/src/backend.rs:455-579):
+    one entry per executed dispatch, in order, intervals that do not overlap, inside the
+    submission's device time."""
+    weights = Quantised(30, 1, (512, 1024))
+    x = upload(hip, normal_bf16(30, 2, (8, 1024)), DType.BF16)
+    triple = weights.upload(hip)
+    outs = [hip.alloc(DType.BF16, (8, 512)) for _ in range(3)]
+    total = hip.alloc(DType.BF16, (8, 512))
+    commands = CommandList()
+    for out in outs:
+        commands.dispatch(Op.quant_matmul(4, 64), [x, *triple], out)
+    commands.dispatch(Op.copy(), [outs[0]], total)
+    plain = hip.submit(commands)
+    plain.wait()
+    assert plain.profile() == []                       # not asked for: nothing recorded
+    submission = hip.submit_profiled(commands)
+    with pytest.raises(BackendError):
+        submission.profile()                           # the timeline exists after the wait
+    submission.wait()
+    timeline = submission.profile()
+    assert [entry[0] for entry in timeline] == [0, 1, 2, 3]
+    assert [entry[1] for entry in timeline] == [1, 1, 1, 1]
+    assert [entry[2] for entry in timeline] == [int(d.op.kind) for d in commands.dispatches]
+    previous_end = 0
+    for _, _, _, start, end in timeline:
+        assert previous_end <= start <= end
+        previous_end = end
+    assert sum(end - start for _, _, _, start, end in timeline) <= submission.gpu_time_ns() * 1.05 + 2000
+    assert previous_end <= submission.gpu_time_ns() * 1.05 + 2000
+
+
 @pytest.mark.parametrize("rows,n,k,kind", [
     (128, 256, 1024, "add"),    # decode rows: the add joins the slab sum
     (8, 64, 256, "add"),        # a single K slab: accumulators + epilogue program

@@ -637,6 +637,8 @@ def main():
                              "secondary workloads, no CPU baseline")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only run the config 4 prefill projection measurement and exit")
+    parser.add_argument("--gemm-only", action="store_true",
+                        help="only the projections of one config 4 layer (the prefill GEMM), for counter runs")
     parser.add_argument("--gemv-only", action="store_true",
                         help="only run the small-batch GEMV measurement (on --layers layers, default 8) "
                              "and exit")
@@ -658,6 +660,9 @@ def main():
             backend.submit(commands).wait()
         print(json.dumps({"copy_bytes_read": elements * 4, "copy_bytes_written": elements * 4,
                           "kernel": "copy_flat_kernel", "launches": 8}))
+        return
+    if args.gemm_only:
+        print(json.dumps({"prefill_gemm_c4": prefill_gemm_c4(HipBackend(0))}))
         return
     if args.gemv_only:
         backend = HipBackend(0)

@@ -216,47 +216,62 @@ def moe_block_c2(backend, model, tokens=256, seed=77):
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
-def prefill_gemm_c4(backend, rows=8256, seed=91, repeats=3):
-    """The quantised projections of one BASELINE config 4 layer (dense 27B-class shape) over the
-    8192-token prefill chunk plus its 64 decode rows: stacked qkv, o, stacked gate/up, down.
-    Each product runs `repeats` times after one warm-up; device time from HIP events around the
-    kernels."""
+def prefill_gemm_c4(backend, rows=8256, seed=91, layers=4, repeats=5):
+    """The quantised projections of BASELINE config 4 layers (dense 27B-class shape) over the
+    8192-token prefill chunk plus its 64 decode rows: stacked qkv, o, stacked gate/up, down, in the
+    order and rhythm of a prefill: the four products of a layer one after the other, `layers`
+    layers with weights of their own (no product finds its weights in a cache), the whole sequence
+    `repeats` times back to back after one warm-up pass, with no host wait in between.  (The device
+    is power-limited under this load: its clock settles near 1.5-1.7 GHz a few milliseconds into a
+    stream of such products, and isolated launches with the host waiting in between measure 10 %
+    lower.)  Device time per product from the per-dispatch timeline of the profiled submissions."""
     from forja_amd.model import DENSE_27B, QuantLinear
     c = DENSE_27B
     qkv_width = (c.q_heads + 2 * c.kv_heads) * c.head_dim
     shapes = [("qkv", qkv_width, c.hidden), ("o_proj", c.hidden, c.q_heads * c.head_dim),
               ("gate_up", 2 * c.intermediate, c.hidden), ("down", c.hidden, c.intermediate)]
+    inputs = {k: backend.alloc(DType.BF16, (rows, k)) for k in sorted({k for _, _, k in shapes})}
+    outputs = {n: backend.alloc(DType.BF16, (rows, n)) for n in sorted({n for _, n, _ in shapes})}
+    fill = CommandList()
+    for index, x in enumerate(inputs.values()):
+        fill.dispatch(Op.fill_seeded(2, seed, 5 + index), [], x)
+    weights = []
+    for layer in range(layers):
+        for index, (name, n, k) in enumerate(shapes):
+            linear = QuantLinear(backend, n, k)
+            linear.fill(fill, seed, 100 * layer + 10 * index)
+            weights.append((name, n, k, linear))
+    backend.submit(fill).wait()
+    commands = CommandList()
+    for name, n, k, linear in weights:
+        commands.dispatch(Op.quant_matmul(4, 64), [inputs[k], *linear.triple], outputs[n])
+    encoded = backend.encode(commands)
+    backend.submit(encoded).wait()     # warm-up: every weight's kept operand exists
+    submissions = [backend.submit_profiled(encoded) for _ in range(repeats)]
+    for submission in submissions:
+        submission.wait()
+    spans = {}
+    for submission in submissions:
+        for first, _, _, start, end in submission.profile():
+            spans.setdefault(weights[first][0], []).append(end - start)
     products, total_flops, total_ns = {}, 0.0, 0.0
-    for index, (name, n, k) in enumerate(shapes):
-        linear = QuantLinear(backend, n, k)
-        x = backend.alloc(DType.BF16, (rows, k))
-        out = backend.alloc(DType.BF16, (rows, n))
-        fill = CommandList()
-        linear.fill(fill, seed, 10 * index)
-        fill.dispatch(Op.fill_seeded(2, seed, 10 * index + 5), [], x)
-        backend.submit(fill).wait()
-        commands = CommandList()
-        commands.dispatch(Op.quant_matmul(4, 64), [x, *linear.triple], out)
-        encoded = backend.encode(commands)
-        backend.submit(encoded).wait()
-        backend.profile_enable(1)
-        backend.profile_reset()
-        for _ in range(repeats):
-            backend.submit(encoded).wait()
-        ns, launches = backend.profile_read(KC_QMM_KERNEL)
-        backend.profile_enable(0)
+    for name, n, k in shapes:
+        per_launch = float(np.mean(spans[name]))
         flops = 2.0 * rows * n * k
-        per_launch = ns / max(launches, 1)
-        products[name] = {"n": n, "k": k, "us": per_launch / 1e3,
-                          "tflops": flops / (per_launch * 1e-9) / 1e12 if per_launch else 0.0}
+        products[name] = {"n": n, "k": k, "us": per_launch / 1e3, "launches": len(spans[name]),
+                          "tflops": flops / (per_launch * 1e-9) / 1e12}
         total_flops += flops
         total_ns += per_launch
-        for tensor in (x, out, *linear.triple):
+    for tensor in (*inputs.values(), *outputs.values()):
+        backend.release(tensor)
+    for _, _, _, linear in weights:
+        for tensor in linear.triple:
             backend.release(tensor)
     achieved = total_flops / (total_ns * 1e-9) / 1e12 if total_ns else 0.0
     return {
         "workload": (f"BASELINE config 4 layer projections: {rows} rows (8192-token prefill chunk + "
-                     f"64 decode rows), hidden {c.hidden}, intermediate {c.intermediate}, MLX-4bit"),
+                     f"64 decode rows), hidden {c.hidden}, intermediate {c.intermediate}, MLX-4bit; "
+                     f"the products of {layers} layers back to back, {repeats} times"),
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "kernel": "gemm_q4_kernel, with prepare_rows_kernel (and prepare_extras_kernel on a weight's first use)"},
@@ -264,7 +279,7 @@ def prefill_gemm_c4(backend, rows=8256, seed=91, repeats=3):
     }
 
 
-def prefill_layer_c4(backend, seed=95, repeats=2):
+def prefill_layer_c4(backend, seed=95, repeats=8):
     """One whole BASELINE config 4 decoder layer over the packed batch (6 prompts of 512..3072
     tokens summing to 8192, plus 64 decode rows): norms, stacked qkv, qk-norm + rope, paged
     attention, o, gate/up, SwiGLU, down with residual.  Device time of the step from the
@@ -278,10 +293,11 @@ def prefill_layer_c4(backend, seed=95, repeats=2):
     model = Model(backend, c, seed=seed, layers=1)
     step = PackedStep(model, contexts, counts, seed=seed, head=False)
     step.run()
-    nanoseconds = 0
-    for _ in range(repeats):
-        nanoseconds += step.run().gpu_time_ns()
-    seconds = nanoseconds / repeats * 1e-9
+    # the layer `repeats` times back to back, as the layers of a prefill follow each other
+    submissions = [backend.submit(step.encoded) for _ in range(repeats)]
+    for submission in submissions:
+        submission.wait()
+    seconds = sum(submission.gpu_time_ns() for submission in submissions) / repeats * 1e-9
     rows = step.tokens
     qkv_width = (c.q_heads + 2 * c.kv_heads) * c.head_dim
     weights = qkv_width * c.hidden + c.hidden * c.q_heads * c.head_dim + 3 * c.intermediate * c.hidden
@@ -307,10 +323,11 @@ def packed_step_c1(backend, seed=97, repeats=3):
     model = Model(backend, c, seed=seed)
     step = PackedStep(model, contexts, counts, seed=seed, head=True)
     step.run()
-    nanoseconds = 0
-    for _ in range(repeats):
-        nanoseconds += step.run().gpu_time_ns()
-    seconds = nanoseconds / repeats * 1e-9
+    # the step `repeats` times back to back, as the steps of a server follow each other
+    submissions = [backend.submit(step.encoded) for _ in range(repeats)]
+    for submission in submissions:
+        submission.wait()
+    seconds = sum(submission.gpu_time_ns() for submission in submissions) / repeats * 1e-9
     return {"workload": "BASELINE config 1: 28 layers, 48 decode rows + prefill chunks 256/384/512/848 "
                         "packed into 2048 tokens, lm_head and argmax on every row",
             "tokens": step.tokens, "ms_per_step": seconds * 1e3, "tok_per_s": step.tokens / seconds}

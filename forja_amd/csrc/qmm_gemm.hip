@@ -62,10 +62,14 @@ constexpr int gemm_lds_bytes(int quadrant) {
   const int output = 4 * (quadrant * out_pitch(quadrant) + 4 * quadrant);   // four quadrants of bf16 rows + row factors
   return pipeline > output ? pipeline : output;
 }
-constexpr int gemm_q4_lds_bytes(int quadrant) {   // the same plus the packed words of two pairs of K steps
-  const int pipeline = kGemmStages * 2 * (2 * quadrant) * 2 * kGemmK + 2 * (2 * quadrant) * 64;
-  return pipeline > gemm_lds_bytes(quadrant) ? pipeline : gemm_lds_bytes(quadrant);
+constexpr int gemm_q4_lds_bytes(int side, int waves, int part_rows, int part_columns) {
+  const int pipeline = 4 * side * 2 * kGemmK + 2 * side * 64;   // two tiles a side + packed words of two pairs of K steps
+  const int output = waves * (part_rows * out_pitch(part_columns) + 4 * part_rows);
+  return pipeline > output ? pipeline : output;
 }
+constexpr int kLargeLds = gemm_q4_lds_bytes(256, 8, 128, 64), kSmallLds = gemm_q4_lds_bytes(128, 4, 64, 64);
+constexpr int kWideLds = 8 * (128 * out_pitch(64) + 4 * 128) > 4 * 256 * 2 * kGemmK ? 8 * (128 * out_pitch(64) + 4 * 128)
+                                                                                      : 4 * 256 * 2 * kGemmK;
 constexpr int kBand = 8;   // column tiles per band of the tile numbering
 constexpr uint32_t kMaxGroups = 512;              // quantisation groups per row the row kernel holds
 
@@ -246,14 +250,15 @@ constexpr uint32_t wait_vmcnt(uint32_t n) {   // s_waitcnt immediate: vmcnt(n) o
 
 // Stores a workgroup's finished tile: acc[i][j] is the 32 x 32 block (i, j) of wave (wm, wn)'s
 // quadrant, rows scaled back by row_unscale, the residual rows added, one rounding.
-template <int kQ>
-__device__ inline void store_tile(const GemmArgs &a, f32x16 (&acc)[kQ / 32][kQ / 32], unsigned char *gemm_lds,
+// A wave's part of the tile is kQM rows x kQN columns; the waves are arranged kWN to a row.
+template <int kQM, int kQN, int kWN>
+__device__ inline void store_tile(const GemmArgs &a, f32x16 (&acc)[kQM / 32][kQN / 32], unsigned char *gemm_lds,
                                   uint32_t row0, uint32_t col0) {
-  constexpr int kMI = kQ / 32;
-  constexpr int kOutPitch = out_pitch(kQ);
+  constexpr int kMIR = kQM / 32, kMIC = kQN / 32;
+  constexpr int kOutPitch = out_pitch(kQN);
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t wm = wave >> 1, wn = wave & 1;
+  const uint32_t wm = wave / kWN, wn = wave % kWN;
   const uint32_t l32 = lane & 31, kh = lane >> 5;
   // Lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile: a column
   // per lane, the wrong way round for memory.  When the output rows allow 16-byte stores, every
@@ -262,17 +267,17 @@ __device__ inline void store_tile(const GemmArgs &a, f32x16 (&acc)[kQ / 32][kQ /
   // result (f32 sum, one rounding), and the rows leave with one 16-byte store per lane, 256
   // contiguous bytes per row.  Only wave-local ordering is needed: nobody else touches the piece.
   if (a.row_stores) {
-    constexpr int kPieces = kQ / 8;            // 16-byte pieces of a quadrant's row
+    constexpr int kPieces = kQN / 8;           // 16-byte pieces of a quadrant's row
     constexpr int kRowsAtOnce = 64 / kPieces;  // rows one wave-wide 16-byte access covers
-    unsigned char *mine = gemm_lds + wave * (kQ * kOutPitch + 4 * kQ);
-    float *unscale_of = (float *)(mine + kQ * kOutPitch);   // the quadrant's row factors
-    const uint32_t quad_row0 = row0 + kQ * wm, quad_col0 = col0 + kQ * wn;
+    unsigned char *mine = gemm_lds + wave * (kQM * kOutPitch + 4 * kQM);
+    float *unscale_of = (float *)(mine + kQM * kOutPitch);   // the quadrant's row factors
+    const uint32_t quad_row0 = row0 + kQM * wm, quad_col0 = col0 + kQN * wn;
     const uint32_t piece_row = lane / kPieces, piece_col = 8 * (lane % kPieces);
     unscale_of[lane] = a.row_unscale[min(quad_row0 + lane, a.rows - 1)];
-    if (kQ > 64) unscale_of[64 + lane] = a.row_unscale[min(quad_row0 + 64 + lane, a.rows - 1)];
+    if (kQM > 64) unscale_of[64 + lane] = a.row_unscale[min(quad_row0 + 64 + lane, a.rows - 1)];
     if (a.residual) {
 #pragma unroll 4
-      for (int it = 0; it < kQ / kRowsAtOnce; ++it) {
+      for (int it = 0; it < kQM / kRowsAtOnce; ++it) {
         const uint32_t row = kRowsAtOnce * it + piece_row;
         uint4 v = make_uint4(0, 0, 0, 0);
         if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
@@ -285,13 +290,13 @@ __device__ inline void store_tile(const GemmArgs &a, f32x16 (&acc)[kQ / 32][kQ /
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-    for (int i = 0; i < kMI; ++i)
+    for (int i = 0; i < kMIR; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const uint32_t row = 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
         const float unscale = unscale_of[row];
 #pragma unroll
-        for (int j = 0; j < kMI; ++j) {
+        for (int j = 0; j < kMIC; ++j) {
           uint16_t *slot = (uint16_t *)(mine + row * kOutPitch) + 32 * j + l32;
           float value = acc[i][j][r] * unscale;
           if (a.residual) value += bf16_bits_to_f32(*slot);
@@ -303,7 +308,7 @@ __device__ inline void store_tile(const GemmArgs &a, f32x16 (&acc)[kQ / 32][kQ /
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     uint16_t *out = (uint16_t *)a.out;
 #pragma unroll 4
-    for (int it = 0; it < kQ / kRowsAtOnce; ++it) {
+    for (int it = 0; it < kQM / kRowsAtOnce; ++it) {
       const uint32_t row = kRowsAtOnce * it + piece_row;
       const uint4 v = *(const uint4 *)(mine + row * kOutPitch + 2 * piece_col);
       if (quad_row0 + row < a.rows && quad_col0 + piece_col < a.columns)
@@ -313,13 +318,13 @@ __device__ inline void store_tile(const GemmArgs &a, f32x16 (&acc)[kQ / 32][kQ /
   }
   // store: lane (column l32, half kh) holds rows 8*(r/4) + 4*kh + r%4 of each 32 x 32 tile
 #pragma unroll
-  for (int i = 0; i < kMI; ++i)
+  for (int i = 0; i < kMIR; ++i)
 #pragma unroll
-    for (int j = 0; j < kMI; ++j) {
-      const uint32_t column = col0 + kQ * wn + 32 * j + l32;
+    for (int j = 0; j < kMIC; ++j) {
+      const uint32_t column = col0 + kQN * wn + 32 * j + l32;
       if (column >= a.columns) continue;
       for (int r = 0; r < 16; ++r) {
-        const uint32_t row = row0 + kQ * wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+        const uint32_t row = row0 + kQM * wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
         if (row >= a.rows) continue;
         const uint64_t at_out = (uint64_t)row * a.out_row_stride + column;
         float value = acc[i][j][r] * a.row_unscale[row];
@@ -461,9 +466,125 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(GemmArgs a) {
   }
   __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));   // nothing is on its way into LDS any more
   __syncthreads();
-  store_tile<kQ>(a, acc, gemm_lds, row0, col0);
+  store_tile<kQ, kQ, 2>(a, acc, gemm_lds, row0, col0);
 }
 
+
+// 64 lanes x 16 bytes from memory straight into LDS at `lds_base` + 16 * lane, issued as an
+// instruction the compiler does not see: while it knows of such a load in flight it waits for ALL
+// outstanding LDS reads wherever it has to wait for one (it cannot tell the load's LDS write from
+// the wave's own LDS traffic), i.e. also for the operand reads just issued for the next sub-step,
+// and it drains every such load at a __syncthreads().  Callers order these loads by hand (vmcnt).
+__device__ inline void load_to_lds_16(const void *from, unsigned char *lds_base) {
+  // (uniform by construction; the intrinsic tells the compiler so)
+  const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(from), "s"(at) : "memory");   // (m0 is the compiler's only for its own such loads: kernels that use this have none)
+}
+
+__device__ inline void lds_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// The same GEMM with eight waves to a 256 x 256 tile (two per SIMD), each owning 128 rows x 64
+// columns (128 accumulator registers): while one wave of a SIMD waits for its operands or at the
+// barrier the other one feeds the matrix pipe.
+template <int kBK>
+__global__ __launch_bounds__(512) void gemm_f16_wide_kernel(GemmArgs a) {
+  if (a.refused[0] != 0) return;
+  constexpr int kSide = 256, kQM = 128, kQN = 64, kWN = 4;
+  constexpr int kMIR = kQM / 32, kMIC = kQN / 32;
+  constexpr int kSub = kBK / 16;
+  constexpr int kRowBytes = 2 * kBK;
+  constexpr int kTile = kSide * kRowBytes;
+  constexpr int kSlots = kRowBytes / 16;
+  constexpr int kRowsPerLoad = 64 / kSlots;
+  constexpr int kStaged = kSide / 8;             // rows of each operand tile a wave stages
+  constexpr int kLoads = kStaged / kRowsPerLoad;
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
+  unsigned char *a_tiles = gemm_lds;
+  unsigned char *b_tiles = gemm_lds + 2 * kTile;
+  const uint32_t tid = threadIdx.x, lane = tid & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t wm = wave / kWN, wn = wave % kWN;
+  const uint32_t l32 = lane & 31, kh = lane >> 5;
+  auto swizzle_of = [](uint32_t row) { return kBK == 64 ? (row >> 1) & 7u : (row >> 2) & 3u; };
+  const uint32_t xcd = blockIdx.x % 8, nth = blockIdx.x / 8;
+  const uint32_t tile = (nth / 32) * 256 + xcd * 32 + nth % 32;
+  if (tile >= a.row_tiles * a.column_tiles) return;
+  const uint32_t band = tile / (a.row_tiles * kBand);
+  const uint32_t band_width = min((uint32_t)kBand, a.column_tiles - band * kBand);
+  const uint32_t in_band = tile - band * a.row_tiles * kBand;
+  const uint32_t bm = in_band / band_width, bn = band * kBand + in_band % band_width;
+  const uint32_t row0 = bm * kSide, col0 = bn * kSide;
+  uint32_t a_off[kLoads], b_off[kLoads];
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) {
+    const uint32_t in_tile = kStaged * wave + kRowsPerLoad * i + lane / kSlots;
+    const uint32_t piece = (lane % kSlots) ^ swizzle_of(in_tile);
+    a_off[i] = (min(row0 + in_tile, a.rows - 1) * a.kt + 8 * piece) * 2;
+    b_off[i] = (min(col0 + in_tile, a.columns - 1) * a.kt + 8 * piece) * 2;
+  }
+  const uint32_t steps = a.kt / kBK;
+  auto stage_pair = [&](uint32_t buffer, uint32_t step, int i) {
+    const uint32_t st = min(step, steps - 1);
+    const unsigned char *from_a = (const unsigned char *)a.a + (uint64_t)st * (kBK * 2);
+    const unsigned char *from_b = (const unsigned char *)a.b + (uint64_t)st * (kBK * 2);
+    unsigned char *to_a = a_tiles + buffer * kTile + (kStaged * wave + kRowsPerLoad * i) * kRowBytes;
+    unsigned char *to_b = b_tiles + buffer * kTile + (kStaged * wave + kRowsPerLoad * i) * kRowBytes;
+    load_to_lds_16(from_a + a_off[i], to_a);
+    load_to_lds_16(from_b + b_off[i], to_b);
+  };
+  f32x16 acc[kMIR][kMIC];
+#pragma unroll
+  for (int i = 0; i < kMIR; ++i)
+#pragma unroll
+    for (int j = 0; j < kMIC; ++j)
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  f16x8 a_op[2][kMIR], b_op[2][kMIC];
+  const uint32_t swizzle = swizzle_of(l32);
+  auto read_operands = [&](uint32_t buffer, int s, int set) {
+    const unsigned char *at = a_tiles + buffer * kTile + (kQM * wm + l32) * kRowBytes;
+    const unsigned char *bt = b_tiles + buffer * kTile + (kQN * wn + l32) * kRowBytes;
+    const uint32_t piece = 16 * ((2 * s + kh) ^ swizzle);
+#pragma unroll
+    for (int i = 0; i < kMIR; ++i)
+      a_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * kRowBytes + piece));
+#pragma unroll
+    for (int j = 0; j < kMIC; ++j)
+      b_op[set][j] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * j * kRowBytes + piece));
+  };
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) stage_pair(0, 0, i);
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+  lds_barrier();
+  uint32_t buffer = 0;
+  for (uint32_t step = 0; step < steps; ++step) {
+    read_operands(buffer, 0, 0);
+    int issued = 0;
+#pragma unroll
+    for (int s = 0; s < kSub; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 1 < kSub) read_operands(buffer, s + 1, (s + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < kMIR; ++i) {
+#pragma unroll
+        for (int j = 0; j < kMIC; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
+        if (issued < kLoads) {
+          __builtin_amdgcn_sched_barrier(0);
+          stage_pair(buffer ^ 1u, step + 1, issued);
+          ++issued;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+    lds_barrier();
+    buffer ^= 1u;
+  }
+  lds_barrier();
+  store_tile<kQM, kQN, kWN>(a, acc, gemm_lds, row0, col0);
+}
 
 // packed/scales/biases [columns, inner] -> the columns an operand row holds after its inner
 // values, fp16 [columns, kt - inner]: per group (head, head, tail) of 64 * (bias + 7.5 * scale),
@@ -513,10 +634,7 @@ __device__ inline f16x8 dequantise_word(uint32_t w, f16x2 scale2, uint32_t mask,
   return __builtin_bit_cast(f16x8, r);
 }
 
-// A 16-byte store to LDS the compiler does not see as one.  Before a store to LDS it can see, the
-// compiler waits for every global_load_lds in flight (any of them might write the same bytes),
-// which would stall each store of a weight tile behind the loads of the step's activation tile.
-// Those write other buffers; the stores are ordered by the kernel's own waits and barriers.
+// A 16-byte store to LDS the compiler does not see as one (ordered by the kernel's own waits).
 __device__ inline void lds_store_16(unsigned char *to, f16x8 value) {
   typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
   const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)to;
@@ -524,44 +642,52 @@ __device__ inline void lds_store_16(unsigned char *to, f16x8 value) {
 }
 
 // The GEMM with the weights dequantised on their way into LDS.
-//   * Activations: the fp16 rows prepare_rows_kernel writes, staged exactly as in gemm_f16_kernel.
-//   * Weights: the packed words themselves go from memory into LDS (global_load_lds; 64 bytes =
-//     two K steps of a column per request, half a byte per weight instead of two).  While the
-//     matrix instructions of step t run, thread c of the workgroup turns the 32 bytes of column c
-//     and step t + 1 into that column's 64 fp16 weights (per nibble pair two integer and two packed
-//     fp16 instructions, spread over the step behind the matrix instructions) and writes them
-//     into the fp16 tile of step t + 1, in the layout gemm_f16_kernel's tiles have.  Per K step a
-//     workgroup moves 40 KB from memory instead of 64.
+//   * Waves: kWM x kWN of them share a square tile, each owning kQM rows x kQN columns of it:
+//     2 x 4 waves of 128 x 64 for 256 x 256 tiles (two waves per SIMD: while one waits for its
+//     operands or at the barrier the other feeds the matrix pipe; with one wave per SIMD owning
+//     128 x 128 the pipe sat idle 45 % of the time), 2 x 2 waves of 64 x 64 for 128 x 128 tiles (two
+//     workgroups per compute unit).
+//   * Activations: the fp16 rows prepare_rows_kernel writes, from memory straight into LDS
+//     (load_to_lds_16), double buffered.
+//   * Weights: the packed words themselves go from memory into LDS the same way (64 bytes = two K
+//     steps of a column per request, half a byte per weight instead of two), and from there into
+//     the operand registers: a lane reads the 16 bytes that hold its 32 weights of a K step (a
+//     column, half a group) and turns one word into one matrix operand per sub-step (per nibble
+//     pair two integer and two packed fp16 instructions).  The dequantised weights never exist in
+//     LDS: per K step a workgroup moves 40 KB from memory instead of 64 and reads 150 KB of LDS
+//     instead of 190.
 //   * The columns after the inner values (the bias term, see the head of this file) are plain fp16
 //     on both sides: for the last few K steps the weights' tile is loaded from `extras`.
 //   * Scales: a thread keeps the bf16 scales of eight groups of its column in registers (one
 //     16-byte load per eight K steps).
-// LDS: activations [2][tile rows][128 B], weights [2][tile columns][128 B], packed words of two
-// pairs of K steps [2][tile columns][64 B].  A column's four 16-byte quarters of a pair sit in
-// slots quarter ^ ((column >> 2) & 3), which spreads the 16 lanes a read serves at once over all
-// banks.  Tiles of 128 x 128 (kQ = 64) give two threads to a column: each takes half a group.
-template <int kQ>
-__global__ __launch_bounds__(256) void gemm_q4_kernel(GemmArgs a) {
+//   * Every load into LDS and every store of a dequantised piece is issued as inline assembly and
+//     ordered by the waits written here (see load_to_lds_16, lds_barrier): what the compiler
+//     knows of are the operand reads, whose waits it then counts exactly.
+// LDS: activations [2][side][128 B], weights [2][side][128 B], packed words of two pairs of K
+// steps [2][side][64 B].  A column's four 16-byte quarters of a pair sit in slots
+// quarter ^ ((column >> 2) & 3), which spreads the 16 lanes a read serves at once over all banks.
+template <int kWM, int kWN, int kQM, int kQN>
+__global__ __launch_bounds__(64 * kWM * kWN) void gemm_q4_kernel(GemmArgs a) {
   if (a.refused[0] != 0) return;
+  constexpr int kWaves = kWM * kWN, kThreads = 64 * kWaves;
   constexpr int kBK = 64;
-  constexpr int kSide = 2 * kQ;
-  constexpr int kMI = kQ / 32;
+  constexpr int kSide = kQM * kWM;
+  static_assert(kSide == kQN * kWN, "square tiles");
+  constexpr int kMIR = kQM / 32, kMIC = kQN / 32;
   constexpr int kSub = 4;
   constexpr int kRowBytes = 2 * kBK;
   constexpr int kTile = kSide * kRowBytes;       // one fp16 operand tile
   constexpr int kPair = kSide * 64;              // the packed words of two K steps of a tile's columns
-  constexpr int kStaged = kSide / 4;             // rows of an fp16 tile a wave stages
+  constexpr int kStaged = kSide / kWaves;        // rows of an fp16 tile a wave stages
   constexpr int kLoads = kStaged / 8;            // instructions per wave and fp16 tile (8 rows each)
-  constexpr int kPairLoads = kSide / 64;         // instructions per wave and pair (16 columns each)
-  constexpr int kShare = 256 / kSide;            // threads per column: 1 or 2
-  constexpr int kWords = 8 / kShare;             // words of a K step a thread dequantises
+  constexpr int kPairLoads = kSide / 16 / kWaves;   // instructions per wave and pair (16 columns each)
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
   unsigned char *a_tiles = gemm_lds;                 // [2][kSide][128]
   unsigned char *b_tiles = gemm_lds + 2 * kTile;     // [2][kSide][128]
   unsigned char *pairs = gemm_lds + 4 * kTile;       // [2][kSide][64]
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t wm = wave >> 1, wn = wave & 1;
+  const uint32_t wm = wave / kWN, wn = wave % kWN;
   const uint32_t l32 = lane & 31, kh = lane >> 5;
   auto swizzle_of = [](uint32_t row) { return (row >> 1) & 7u; };
 
@@ -574,7 +700,7 @@ __global__ __launch_bounds__(256) void gemm_q4_kernel(GemmArgs a) {
   const uint32_t bm = in_band / band_width, bn = band * kBand + in_band % band_width;
   const uint32_t row0 = bm * kSide, col0 = bn * kSide;
 
-  const uint32_t main_steps = a.inner / kBK, steps = a.kt / kBK;
+  const uint32_t main_steps = a.inner / kBK, steps = a.kt / kBK;   // main_steps is even
   const uint32_t extras_width = a.kt - a.inner;
   // ---- staging addresses: a wave-uniform base that advances with K plus a per-lane offset
   uint32_t a_off[kLoads], e_off[kLoads], p_off[kPairLoads];
@@ -592,88 +718,86 @@ __global__ __launch_bounds__(256) void gemm_q4_kernel(GemmArgs a) {
     p_off[i] = min(col0 + column, a.columns - 1) * (a.inner / 2) + 16 * quarter;
   }
   auto stage_a = [&](uint32_t buffer, uint32_t step, int i) {
-    const uint32_t st = min(step, steps - 1);
+    const uint32_t st = min(step, steps - 1);   // past the end: the last tile again, never used
     const unsigned char *from = (const unsigned char *)a.a + (uint64_t)st * (kBK * 2);
-    unsigned char *to = a_tiles + buffer * kTile + (kStaged * wave + 8 * i) * kRowBytes;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from + a_off[i]),
-                                     (__attribute__((address_space(3))) void *)to, 16, 0, 0);
+    load_to_lds_16(from + a_off[i], a_tiles + buffer * kTile + (kStaged * wave + 8 * i) * kRowBytes);
   };
   // the weights' fp16 tile of step `step`, one of the steps after the inner ones
   auto stage_extras = [&](uint32_t buffer, uint32_t step, int i) {
     const uint32_t st = min(step, steps - 1) - main_steps;
     const unsigned char *from = (const unsigned char *)a.extras + (uint64_t)st * (kBK * 2);
-    unsigned char *to = b_tiles + buffer * kTile + (kStaged * wave + 8 * i) * kRowBytes;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from + e_off[i]),
-                                     (__attribute__((address_space(3))) void *)to, 16, 0, 0);
+    load_to_lds_16(from + e_off[i], b_tiles + buffer * kTile + (kStaged * wave + 8 * i) * kRowBytes);
   };
   auto stage_pair = [&](uint32_t pair, int i) {
-    const uint32_t pr = min(pair, main_steps / 2 - 1);
+    const uint32_t pr = min(pair, main_steps / 2 - 1);   // past the end: into the buffer nobody reads
     const unsigned char *from = (const unsigned char *)a.packed + (uint64_t)pr * 64;
-    unsigned char *to = pairs + (pair & 1u) * kPair + 16 * (kPairLoads * wave + i) * 64;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(from + p_off[i]),
-                                     (__attribute__((address_space(3))) void *)to, 16, 0, 0);
+    load_to_lds_16(from + p_off[i], pairs + (pair & 1u) * kPair + 16 * (kPairLoads * wave + i) * 64);
   };
 
-  f32x16 acc[kMI][kMI];
+  f32x16 acc[kMIR][kMIC];
 #pragma unroll
-  for (int i = 0; i < kMI; ++i)
+  for (int i = 0; i < kMIR; ++i)
 #pragma unroll
-    for (int j = 0; j < kMI; ++j)
+    for (int j = 0; j < kMIC; ++j)
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  f16x8 a_op[2][kMI], b_op[2][kMI];
+  f16x8 a_op[2][kMIR], b_op[2][kMIC];
   const uint32_t swizzle = swizzle_of(l32);
-  auto read_operands = [&](uint32_t buffer, int s, int set) {
-    const unsigned char *at = a_tiles + buffer * kTile + (kQ * wm + l32) * kRowBytes;
-    const unsigned char *bt = b_tiles + buffer * kTile + (kQ * wn + l32) * kRowBytes;
-    const uint32_t piece = 16 * ((2 * s + kh) ^ swizzle);
+  // Lane half kh contracts K values [32 kh + 8 s, + 8) of a step in sub-step s (the order in which
+  // its 16 bytes of packed words unpack), i.e. piece 4 kh + s of a tile row.
+  auto read_a = [&](uint32_t buffer, int s, int set) {
+    const unsigned char *at = a_tiles + buffer * kTile + (kQM * wm + l32) * kRowBytes;
+    const uint32_t piece = 16 * ((4 * kh + s) ^ swizzle);
 #pragma unroll
-    for (int i = 0; i < kMI; ++i) {
+    for (int i = 0; i < kMIR; ++i)
       a_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(at + 32 * i * kRowBytes + piece));
-      b_op[set][i] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * i * kRowBytes + piece));
-    }
   };
-  // ---- this thread's share of the dequantisation: column `mine`, words [kWords part, + kWords)
-  const uint32_t mine = tid / kShare, part = tid % kShare;
-  const uint32_t mine_swizzle = swizzle_of(mine), quarter_swizzle = (mine >> 2) & 3u;
-  uint32_t words[kWords];
-  auto read_words = [&](uint32_t step) {   // the packed words of step `step`
-    const unsigned char *from = pairs + ((step >> 1) & 1u) * kPair + mine * 64;
+  auto read_b = [&](uint32_t buffer, int s, int set) {
+    const unsigned char *bt = b_tiles + buffer * kTile + (kQN * wn + l32) * kRowBytes;
+    const uint32_t piece = 16 * ((4 * kh + s) ^ swizzle);
 #pragma unroll
-    for (int q = 0; q < kWords / 4; ++q) {
-      const uint32_t quarter = 2 * (step & 1u) + (kShare == 1 ? q : part);
-      const uint4 v = *(const uint4 *)(from + 16 * (quarter ^ quarter_swizzle));
-      words[4 * q] = v.x, words[4 * q + 1] = v.y, words[4 * q + 2] = v.z, words[4 * q + 3] = v.w;
-    }
+    for (int j = 0; j < kMIC; ++j)
+      b_op[set][j] = __builtin_bit_cast(f16x8, *(const uint4 *)(bt + 32 * j * kRowBytes + piece));
   };
-  // (Neighbouring columns' rows share a swizzle, so these stores meet some bank conflicts; giving
-  // odd columns a rotated word order removes them and measured 6 % slower, for the select it adds
-  // in front of every word.)
-  auto write_weights = [&](uint32_t buffer, int nth, f16x2 scale2, uint32_t mask, uint32_t magic) {
-    const uint32_t piece = kWords * part + nth;   // word `piece` of the group = piece `piece` of the row
-    unsigned char *to = b_tiles + buffer * kTile + mine * kRowBytes + 16 * (piece ^ mine_swizzle);
-    lds_store_16(to, dequantise_word(words[nth], scale2, mask, magic));
+  // ---- the weights of this lane's columns kQN wn + 32 j + l32: 16 bytes of packed words per
+  // column and K step (the half kh of the step's group), one word per sub-step, and the columns'
+  // scales
+  const uint32_t quarter_swizzle = (l32 >> 2) & 3u;
+  uint4 words[kMIC], next_words[kMIC];
+  auto read_words = [&](uint4 (&to)[kMIC], uint32_t step) {
+    const unsigned char *from = pairs + ((step >> 1) & 1u) * kPair + (kQN * wn + l32) * 64 +
+                                16 * ((2 * (step & 1u) + kh) ^ quarter_swizzle);
+#pragma unroll
+    for (int j = 0; j < kMIC; ++j) to[j] = *(const uint4 *)(from + 32 * j * 64);
   };
   const uint32_t groups = a.inner / 64;
-  const uint32_t scale_off = min(col0 + mine, a.columns - 1) * groups * 2;
-  uint4 scale_block, next_block;   // bf16 scales of eight groups of the column
-  auto load_scales = [&](uint4 &to, uint32_t block) {
+  uint32_t scale_off[kMIC];
+#pragma unroll
+  for (int j = 0; j < kMIC; ++j) scale_off[j] = min(col0 + kQN * wn + 32 * j + l32, a.columns - 1) * groups * 2;
+  uint4 scale_block[kMIC], next_block[kMIC];   // bf16 scales of eight groups per column
+  auto load_scales = [&](uint4 (&to)[kMIC], uint32_t block) {
     const uint32_t bl = min(block, groups / 8 - 1);
-    to = *(const uint4 *)((const unsigned char *)a.scales + (uint64_t)bl * 16 + scale_off);
+    const unsigned char *from = (const unsigned char *)a.scales + (uint64_t)bl * 16;
+#pragma unroll
+    for (int j = 0; j < kMIC; ++j) to[j] = *(const uint4 *)(from + scale_off[j]);
   };
-  auto pick_scale = [&](uint32_t step) -> f16x2 {
+  f16x2 scale2[kMIC], next_scale2[kMIC];
+  auto pick_scales = [&](f16x2 (&to)[kMIC], uint32_t step) {
     const uint32_t e = step & 7u;   // uniform
-    const uint4 v = scale_block;
-    const uint32_t word = e < 4 ? (e < 2 ? v.x : v.y) : (e < 6 ? v.z : v.w);
-    const float scale = __uint_as_float((e & 1u) ? (word & 0xffff0000u) : (word << 16));
-    const _Float16 h = (_Float16)scale;
-    return f16x2{h, h};
+#pragma unroll
+    for (int j = 0; j < kMIC; ++j) {
+      const uint4 v = scale_block[j];
+      const uint32_t word = e < 4 ? (e < 2 ? v.x : v.y) : (e < 6 ? v.z : v.w);
+      const float scale = __uint_as_float((e & 1u) ? (word & 0xffff0000u) : (word << 16));
+      const _Float16 h = (_Float16)scale;
+      to[j] = f16x2{h, h};
+    }
   };
   uint32_t mask = 0x001e001eu, magic = 0x60006000u;
   asm("" : "+s"(mask), "+v"(magic));   // no instruction: keeps the two constants in registers
 
   // ---- prologue: activations of step 0, packed words of steps 0..1, scales of groups 0..15;
-  // then the weights' tile of step 0
+  // then the operands of the first sub-step
 #pragma unroll
   for (int i = 0; i < kLoads; ++i) stage_a(0, 0, i);
 #pragma unroll
@@ -681,81 +805,86 @@ __global__ __launch_bounds__(256) void gemm_q4_kernel(GemmArgs a) {
   load_scales(scale_block, 0);
   load_scales(next_block, 1);
   __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
-  __syncthreads();
-  {
-    read_words(0);
-    const f16x2 scale2 = pick_scale(0);
+  lds_barrier();
+  read_words(words, 0);
+  pick_scales(scale2, 0);
+  read_a(0, 0, 0);
 #pragma unroll
-    for (int nth = 0; nth < kWords; ++nth) write_weights(0, nth, scale2, mask, magic);
-  }
-  __syncthreads();
-  read_operands(0, 0, 0);
+  for (int j = 0; j < kMIC; ++j) b_op[0][j] = dequantise_word(words[j].x, scale2[j], mask, magic);
   // One inner step.  On entry the operands of its first sub-step are in registers (set 0).  kOdd:
-  // the step's parity (= the LDS buffers its tiles are in); kLast: the last inner step, which
-  // requests the first fp16 tile of the weights' side instead of dequantising one.  Even steps
-  // request the packed words of the two steps after the next (past the end: the last pair again,
-  // into the buffer nobody reads).  Every request of the step is made at its start, so that it has
-  // the whole step to land; the matrix instructions of the last sub-step run behind the barrier,
-  // covering the latency of the next step's first operand reads.
+  // the step's parity (= the LDS buffer its activations are in); kLast: the last inner step, which
+  // requests the first fp16 tile of the weights' side and prepares no weights for a next step.
+  // Even steps request the packed words of the two steps after the next.  Every request of the
+  // step is made at its start; behind the first rows of matrix instructions of a sub-step the
+  // lane unpacks the word of the next sub-step of each of its columns (a wave's unpacking runs
+  // beside the matrix instructions of the other wave on its SIMD); the matrix instructions of the
+  // last sub-step run behind the barrier, covering the latency of the next step's first reads.
   auto inner_step = [&](auto odd_tag, auto last_tag, uint32_t step) {
     constexpr bool kOdd = decltype(odd_tag)::value, kLast = decltype(last_tag)::value;
     constexpr uint32_t buffer = kOdd ? 1u : 0u;
-    f16x2 scale2 = {0, 0};
     if (!kLast) {
       if (kOdd && ((step + 1) & 7u) == 0) {   // the next step opens a block of eight groups
-        scale_block = next_block;
+#pragma unroll
+        for (int j = 0; j < kMIC; ++j) scale_block[j] = next_block[j];
         load_scales(next_block, (step + 1) / 8 + 1);
       }
-      scale2 = pick_scale(step + 1);
-      read_words(step + 1);
+      pick_scales(next_scale2, step + 1);
+      read_words(next_words, step + 1);
     }
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-      stage_a(buffer ^ 1u, step + 1, i);
-    }
+    for (int i = 0; i < kLoads; ++i) stage_a(buffer ^ 1u, step + 1, i);
     if (kLast) {
 #pragma unroll
-      for (int i = 0; i < kLoads; ++i) stage_extras(buffer ^ 1u, main_steps, i);
+      for (int i = 0; i < kLoads; ++i) stage_extras(0, main_steps, i);
     } else if (!kOdd) {
 #pragma unroll
       for (int i = 0; i < kPairLoads; ++i) stage_pair(step / 2 + 1, i);
     }
-    int written = 0;
 #pragma unroll
     for (int s = 0; s < kSub - 1; ++s) {
       __builtin_amdgcn_sched_barrier(0);
-      read_operands(buffer, s + 1, (s + 1) & 1);
+      read_a(buffer, s + 1, (s + 1) & 1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < kMI; ++i) {
+      for (int i = 0; i < kMIR; ++i) {
 #pragma unroll
-        for (int j = 0; j < kMI; ++j)
+        for (int j = 0; j < kMIC; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
-        // behind two rows of matrix instructions in three: one word of the next step's weights
-        if (!kLast && written < kWords && (s * kMI + i) % 3 != 2) {
-          write_weights(buffer ^ 1u, written, scale2, mask, magic);
-          ++written;
+        if (i < kMIC) {   // behind row i: the operand of column block i for the next sub-step
+          const uint4 v = words[i];
+          const uint32_t w = s == 0 ? v.y : s == 1 ? v.z : v.w;
+          b_op[(s + 1) & 1][i] = dequantise_word(w, scale2[i], mask, magic);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    static_assert(kWords <= 2 * kMI, "the words fit the rows of three sub-steps");
-    __builtin_amdgcn_s_waitcnt(0xc07f);            // lgkmcnt(0): operand reads and tile stores done
+    static_assert(kMIC <= kMIR, "a row of matrix instructions for every column block");
+    __builtin_amdgcn_s_waitcnt(0xc07f);            // lgkmcnt(0): operand reads done
     __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));     // step + 1 has landed
-    __syncthreads();
-    read_operands(buffer ^ 1u, 0, 0);
+    lds_barrier();
+    read_a(buffer ^ 1u, 0, 0);
+    if (kLast) read_b(0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < kMI; ++i)
+    for (int i = 0; i < kMIR; ++i) {
 #pragma unroll
-      for (int j = 0; j < kMI; ++j)
+      for (int j = 0; j < kMIC; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[1][i], b_op[1][j], acc[i][j], 0, 0, 0);
+      if (!kLast && i < kMIC) b_op[0][i] = dequantise_word(next_words[i].x, next_scale2[i], mask, magic);
+    }
     __builtin_amdgcn_sched_barrier(0);
+    if (!kLast) {
+#pragma unroll
+      for (int j = 0; j < kMIC; ++j) {
+        words[j] = next_words[j];
+        scale2[j] = next_scale2[j];
+      }
+    }
   };
   typedef std::integral_constant<bool, false> no;
   typedef std::integral_constant<bool, true> yes;
   uint32_t step = 0;
-  for (; step + 2 < main_steps; step += 2) {   // main_steps is even
+  for (; step + 2 < main_steps; step += 2) {
     inner_step(no{}, no{}, step);
     inner_step(yes{}, no{}, step + 1);
   }
@@ -772,30 +901,32 @@ __global__ __launch_bounds__(256) void gemm_q4_kernel(GemmArgs a) {
 #pragma unroll
     for (int s = 0; s < kSub - 1; ++s) {
       __builtin_amdgcn_sched_barrier(0);
-      read_operands(buffer, s + 1, (s + 1) & 1);
+      read_a(buffer, s + 1, (s + 1) & 1);
+      read_b(buffer, s + 1, (s + 1) & 1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < kMI; ++i)
+      for (int i = 0; i < kMIR; ++i)
 #pragma unroll
-        for (int j = 0; j < kMI; ++j)
+        for (int j = 0; j < kMIC; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[s & 1][i], b_op[s & 1][j], acc[i][j], 0, 0, 0);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
-    __syncthreads();
+    lds_barrier();
     buffer ^= 1u;
-    read_operands(buffer, 0, 0);   // (after the last step: a tile nobody uses)
+    read_a(buffer, 0, 0);   // (after the last step: tiles nobody uses)
+    read_b(buffer, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < kMI; ++i)
+    for (int i = 0; i < kMIR; ++i)
 #pragma unroll
-      for (int j = 0; j < kMI; ++j)
+      for (int j = 0; j < kMIC; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_op[1][i], b_op[1][j], acc[i][j], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
   }
   __builtin_amdgcn_s_waitcnt(0xc07f);
-  __syncthreads();   // the last reads are done before the tile's stores reuse LDS
-  store_tile<kQ>(a, acc, gemm_lds, row0, col0);
+  lds_barrier();   // the last reads are done before the tile's stores reuse LDS
+  store_tile<kQM, kQN, kWN>(a, acc, gemm_lds, row0, col0);
 }
 
 }  // namespace
@@ -882,10 +1013,10 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
   static bool configured = false;   // raise the dynamic LDS limit once per process
   if (!configured) {
     const struct { const void *kernel; int bytes; } limits[] = {
-        {reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages, 128>), gemm_lds_bytes(128)},
+        {reinterpret_cast<const void *>(&gemm_f16_wide_kernel<kGemmK>), kWideLds},
         {reinterpret_cast<const void *>(&gemm_f16_kernel<kGemmK, kGemmStages, 64>), gemm_lds_bytes(64)},
-        {reinterpret_cast<const void *>(&gemm_q4_kernel<128>), gemm_q4_lds_bytes(128)},
-        {reinterpret_cast<const void *>(&gemm_q4_kernel<64>), gemm_q4_lds_bytes(64)}};
+        {reinterpret_cast<const void *>(&gemm_q4_kernel<2, 4, 128, 64>), kLargeLds},
+        {reinterpret_cast<const void *>(&gemm_q4_kernel<2, 2, 64, 64>), kSmallLds}};
     for (const auto &limit : limits) {
       if (hipFuncSetAttribute(limit.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, limit.bytes) != hipSuccess)
         return false;
@@ -913,13 +1044,13 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
   }
   if (packed_form) {
     if (small_tiles)
-      gemm_q4_kernel<64><<<grid, 256, gemm_q4_lds_bytes(64), stream>>>(a);
+      gemm_q4_kernel<2, 2, 64, 64><<<grid, 256, kSmallLds, stream>>>(a);
     else
-      gemm_q4_kernel<128><<<grid, 256, gemm_q4_lds_bytes(128), stream>>>(a);
+      gemm_q4_kernel<2, 4, 128, 64><<<grid, 512, kLargeLds, stream>>>(a);
   } else if (small_tiles) {
     gemm_f16_kernel<kGemmK, kGemmStages, 64><<<grid, 256, gemm_lds_bytes(64), stream>>>(a);
   } else {
-    gemm_f16_kernel<kGemmK, kGemmStages, 128><<<grid, 256, gemm_lds_bytes(128), stream>>>(a);
+    gemm_f16_wide_kernel<kGemmK><<<grid, 512, kWideLds, stream>>>(a);
   }
   *refused = (kept && verdict == 0) ? nullptr : flag;
   // the first product over kept weights learns, once, whether they fit the scheme

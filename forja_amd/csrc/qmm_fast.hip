@@ -1170,7 +1170,10 @@ bool try_fast_quant_matmul(fh_backend *backend, const QmmProblem &p) {
   a.residual = residual;
   a.residual_row_stride = residual_row_stride;
   KernelTimer timer(backend, FH_KC_QMM_KERNEL);
-  if (p.rows > 128) {
+  // (also a full decode batch against a vocabulary-sized matrix: 128 x 151936 x 2048 takes 132 us
+  // through the GEMM's 128 x 128 tiles and 224 us through the streaming kernel, which reads the
+  // weights once per 64 rows)
+  if (p.rows > 128 || (p.rows > 64 && p.columns >= 32768)) {
     // the tiled GEMM, followed by the any-range kernel conditioned on the GEMM's refusal
     const uint32_t *refused = nullptr;
     if (launch_quant_gemm(backend, p, &refused)) {

@@ -1005,7 +1005,8 @@ bool launch_quant_gemm(fh_backend *backend, const QmmProblem &p, const uint32_t 
   a.columns = p.columns;
   // 256 x 256 tiles unless they are fewer than three quarters of the compute units
   const uint64_t large_tiles = (uint64_t)((p.rows + kBM - 1) / kBM) * ((p.columns + kBN - 1) / kBN);
-  const bool small_tiles = large_tiles * 4 < 3ull * backend_compute_units(backend);
+  // (and for at most 128 rows, which would leave half of every large tile empty)
+  const bool small_tiles = large_tiles * 4 < 3ull * backend_compute_units(backend) || p.rows <= 128;
   const uint32_t side = small_tiles ? 128 : 256;
   a.row_tiles = (p.rows + side - 1) / side;
   a.column_tiles = (p.columns + side - 1) / side;

@@ -1,13 +1,12 @@
 // MLX-4bit quantised matmul for many activation rows (prefill chunks): a tiled f16 MFMA GEMM
 // whose weight operand is dequantised on its way from LDS into the operand registers
 // (gemm_q4_kernel: the packed words travel, 0.5 byte per weight), or, for the shapes that kernel
-// does not take, once per product into an fp16 matrix (gemm_f16_kernel).
+// does not take, read from an fp16 matrix written once per weight (gemm_f16_wide_kernel,
+// gemm_f16_kernel).
 //
 // y[m,n] = sum_k x[m,k] * (scale[n,k/64] * q[n,k] + bias[n,k/64])   (affine_quant_dot,
 // crates/forja-cpu/src/lib.rs:1277-1310).  With thousands of rows per weight the work is bound
-// by the matrix cores, not by HBM: writing the dequantised matrix (4 bytes per weight, written and
-// read back) costs a few percent of the product's time and takes every unpacking instruction,
-// strided weight load and register-staged tile out of the GEMM loop.
+// by the matrix cores, not by HBM.
 //   * Operands are fp16, not bf16: a dequantised weight rounded to bf16 (8 significant bits) is
 //     too coarse for the stated tolerance on outputs that cancel, fp16 (11 bits) is not, and the
 //     matrix cores run both at the same rate.  bf16 activations convert to fp16 exactly once a row
@@ -15,22 +14,24 @@
 //   * Weights are centred: w = scale * q - c with c = 7.5 * scale, which halves their magnitude
 //     and so their rounding error; at the deepest contraction (K = 17408) the uncentred form does
 //     not meet the tolerance.  What centring takes out, (bias + c) * sum of the group's
-//     activations, is put back through the same GEMM: both operand matrices get three more
-//     columns per quantisation group, holding S/64 and 64 * (bias + c) each split in an fp16
-//     head and tail (head*head + tail*head + head*tail, about 22 significant bits), so the
-//     kernel needs no side channel for it.  The contraction grows by 3/64.
-//   * prepare_rows_kernel and prepare_weights_kernel write the two operand matrices
-//     [rows, Kt] and [N, Kt], Kt = K + 3K/64 rounded up to the K step, every 8 values in the
-//     order (0,4,1,5,2,6,3,7) in which nibbles unpack pairwise.  prepare_weights_kernel also
-//     raises a flag when some scale or bias does not fit this scheme's fp16 range; the GEMM
-//     kernel then returns at once and the caller runs its any-range kernel instead.
-//   * GEMM: workgroup tile 256 rows x 256 columns, K step 64; four waves in a 2 x 2
-//     arrangement, each owning 128 x 128 outputs = 16 accumulator tiles of
-//     v_mfma_f32_32x32x16_f16 (256 accumulator registers).  Both operand tiles go from memory
-//     straight into LDS (global_load_lds, no registers), double buffered, their 16-byte pieces
-//     XOR-swizzled inside each 128-byte row so that operand reads are bank-conflict free
-//     without padding; one barrier per step.  Operand registers are double buffered too: the
-//     reads of a sub-step are issued before the previous sub-step's MFMAs.
+//     activations, is put back through the same GEMM: both operands get three more K columns per
+//     quantisation group, holding S/64 and 64 * (bias + c) each split in an fp16 head and tail
+//     (head*head + tail*head + head*tail, about 22 significant bits), so the kernel needs no
+//     side channel for it.  The contraction grows by 3/64.
+//   * prepare_rows_kernel writes the activation operand [rows, Kt], Kt = K + 3K/64 rounded up to
+//     the K step, every 8 values in the order (0,4,1,5,2,6,3,7) in which nibbles unpack pairwise.
+//     prepare_extras_kernel writes the weights' extra columns [N, Kt - K] (kept per weight matrix
+//     by the backend: 3/64 of a value per weight), prepare_weights_kernel the whole fp16 operand
+//     [N, Kt] for the kernels that read one.  Both raise a flag when some scale or bias does not
+//     fit this scheme's fp16 range; the GEMM kernel then returns at once and the caller runs its
+//     any-range kernel instead.
+//   * GEMM: workgroup tile 256 rows x 256 columns, K step 64, eight waves in a 2 x 4 arrangement
+//     (two per SIMD), each owning 128 x 64 outputs = 8 accumulator tiles of
+//     v_mfma_f32_32x32x16_f16; 128 x 128 tiles of four waves where the large tiles would leave
+//     compute units idle.  What comes from memory goes straight into LDS (no registers), double
+//     buffered, 16-byte pieces XOR-swizzled inside each row so that operand reads are
+//     bank-conflict free without padding; one barrier per step.  Operand registers are double
+//     buffered too: the reads of a sub-step are issued before the previous sub-step's MFMAs.
 //   * The workgroup -> tile map gives the 32 workgroups that run together on one XCD a patch of
 //     about 4 row tiles x 8 column tiles, so that its L2 serves each activation tile to 8
 //     workgroups and each weight tile to 4, instead of every workgroup streaming its own.
@@ -634,13 +635,6 @@ __device__ inline f16x8 dequantise_word(uint32_t w, f16x2 scale2, uint32_t mask,
   return __builtin_bit_cast(f16x8, r);
 }
 
-// A 16-byte store to LDS the compiler does not see as one (ordered by the kernel's own waits).
-__device__ inline void lds_store_16(unsigned char *to, f16x8 value) {
-  typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-  const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)to;
-  asm volatile("ds_write_b128 %0, %1" : : "v"(at), "v"(__builtin_bit_cast(u32x4, value)) : "memory");
-}
-
 // The GEMM with the weights dequantised on their way into LDS.
 //   * Waves: kWM x kWN of them share a square tile, each owning kQM rows x kQN columns of it:
 //     2 x 4 waves of 128 x 64 for 256 x 256 tiles (two waves per SIMD: while one waits for its
@@ -660,10 +654,10 @@ __device__ inline void lds_store_16(unsigned char *to, f16x8 value) {
 //     on both sides: for the last few K steps the weights' tile is loaded from `extras`.
 //   * Scales: a thread keeps the bf16 scales of eight groups of its column in registers (one
 //     16-byte load per eight K steps).
-//   * Every load into LDS and every store of a dequantised piece is issued as inline assembly and
-//     ordered by the waits written here (see load_to_lds_16, lds_barrier): what the compiler
-//     knows of are the operand reads, whose waits it then counts exactly.
-// LDS: activations [2][side][128 B], weights [2][side][128 B], packed words of two pairs of K
+//   * Every load into LDS is issued as inline assembly and ordered by the waits written here
+//     (see load_to_lds_16, lds_barrier): what the compiler knows of are the operand reads, whose
+//     waits it then counts exactly.
+// LDS: activations [2][side][128 B], fp16 weights of the extra columns [2][side][128 B], packed words of two pairs of K
 // steps [2][side][64 B].  A column's four 16-byte quarters of a pair sit in slots
 // quarter ^ ((column >> 2) & 3), which spreads the 16 lanes a read serves at once over all banks.
 template <int kWM, int kWN, int kQM, int kQN>

@@ -1430,6 +1430,7 @@ struct LaneMember {
   bool has_copy = false;      // an Op::Copy of the output row follows
   fh_tensor copy_target{};
   uint32_t q_start = 0, page_tokens = 0;
+  uint32_t tokens = 1;        // query rows (more than one: a prefill chunk, see chunk_member_at)
   float scale = 0.0f;
   uint32_t dispatches = 0;    // dispatches of the member, the copy included
   uint32_t attention_at = 0;  // which of them is the attention (its failures are recorded there)
@@ -1792,6 +1793,441 @@ fh_status run_lane_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors, b
       }
     }
     launch_scatter_lane_rows(b->stream, targets, rows, base, chunk, (uint32_t)row_bytes);
+  }
+  b->fused_runs += 1;
+  b->fused_dispatches += run.dispatches;
+  return FH_OK;
+}
+
+// ---- runs that bring prefill chunks ----
+// A sequence's chunk of n > 1 rows recorded on its own (the multi-row branch of
+// paged_cache_attention, engines/qwen3-coder/src/lib.rs:685-707: cache.append, then
+// cache.attention): two Op::PagedCopy{IntoPages} of the chunk's key and value rows and one causal
+// Op::PagedSdpa over its n query rows, optionally followed by the Op::Copy that moves the
+// attended rows, token-major, into the packed activation.  Such members, and one-row members in
+// either idiom, next to each other are one ragged launch over the packed rows.
+
+// rows [n, ...] whose inner axes are packed, as [n, heads, width] with its own row stride.
+bool as_chunk_rows(const fh_tensor &rows, uint32_t n, uint32_t heads, uint32_t width, fh_tensor *out) {
+  if (rows.rank < 2 || rows.shape[0] != n) return false;
+  uint64_t inner = 1;
+  for (uint32_t axis = rows.rank; axis-- > 1;) {
+    if (rows.stride[axis] != inner) return false;
+    inner *= rows.shape[axis];
+  }
+  if (inner != (uint64_t)heads * width) return false;
+  *out = rows;
+  out->rank = 3;
+  out->shape[0] = n;
+  out->shape[1] = heads;
+  out->shape[2] = width;
+  out->stride[1] = width;
+  out->stride[2] = 1;
+  return true;
+}
+
+// `copy` moves the attended rows of `out` [heads, n, width], token by token, into a destination
+// [n, heads, width] whose head rows are dense.
+bool copies_attended_chunk(const fh_tensor &out, const fh_dispatch &copy) {
+  if (copy.op != FH_OP_COPY || copy.n_inputs != 1 || copy.n_outputs != 1) return false;
+  const fh_tensor &in = copy.inputs[0], &to = copy.outputs[0];
+  if (in.buffer != out.buffer || in.offset != out.offset || in.dtype != out.dtype || to.dtype != out.dtype)
+    return false;
+  if (in.rank != 3 || to.rank != 3) return false;
+  const uint32_t shape[3] = {out.shape[1], out.shape[0], out.shape[2]};
+  for (uint32_t axis = 0; axis < 3; ++axis)
+    if (in.shape[axis] != shape[axis] || to.shape[axis] != shape[axis]) return false;
+  if (in.stride[0] != out.stride[1] || in.stride[1] != out.stride[0] || in.stride[2] != 1) return false;
+  return to.stride[2] == 1 && to.stride[1] == to.shape[2];
+}
+
+bool chunk_member_at(const fh_dispatch *d, uint32_t count, uint32_t at, LaneMember *m) {
+  *m = LaneMember{};
+  if (at + 2 >= count) return false;
+  const fh_dispatch &first = d[at], &second = d[at + 1], &attention = d[at + 2];
+  if (first.op != FH_OP_PAGED_COPY || second.op != FH_OP_PAGED_COPY || attention.op != FH_OP_PAGED_SDPA)
+    return false;
+  if (first.direction != 0 || second.direction != 0 || attention.causal == 0) return false;
+  if (first.n_inputs != second.n_inputs || attention.n_inputs != first.n_inputs + 2) return false;
+  if (attention.n_outputs != 1) return false;
+  const fh_tensor &q = attention.inputs[0], &kp = attention.inputs[1], &vp = attention.inputs[2];
+  const uint32_t n = q.shape[1];
+  if (n < 2 || q.stride[2] != 1) return false;
+  if (first.outputs[0].buffer != kp.buffer || first.outputs[0].offset != kp.offset ||
+      first.outputs[0].dtype != kp.dtype || second.outputs[0].buffer != vp.buffer ||
+      second.outputs[0].offset != vp.offset || second.outputs[0].dtype != vp.dtype)
+    return false;
+  if (first.start != attention.q_start || second.start != attention.q_start ||
+      (uint64_t)attention.key_length != (uint64_t)attention.q_start + n ||
+      first.page_tokens != attention.page_tokens || second.page_tokens != attention.page_tokens)
+    return false;
+  for (const fh_dispatch *copy : {&first, &second}) {
+    if (!same_tensor(copy->inputs[1], attention.inputs[3]) || !same_tensor(copy->inputs[2], attention.inputs[4]))
+      return false;
+    if (copy->n_inputs == 4 && !same_tensor(copy->inputs[3], attention.inputs[5])) return false;
+  }
+  if (!as_chunk_rows(first.inputs[0], n, kp.shape[2], kp.shape[3], &m->k_new) ||
+      !as_chunk_rows(second.inputs[0], n, vp.shape[2], vp.shape[3], &m->v_new))
+    return false;
+  m->q = q;
+  m->table = attention.inputs[3];
+  m->generations = attention.inputs[4];
+  m->has_activity = attention.n_inputs == 6;
+  if (m->has_activity) m->activity = attention.inputs[5];
+  m->out = attention.outputs[0];
+  m->key_pool = kp;
+  m->value_pool = vp;
+  m->q_start = attention.q_start;
+  m->page_tokens = attention.page_tokens;
+  m->tokens = n;
+  m->scale = attention.scale;
+  m->dispatches = 3;
+  m->attention_at = 2;
+  if (m->k_new.dtype != q.dtype || m->v_new.dtype != q.dtype) return false;
+  if (m->out.stride[2] != 1 || !is_contiguous(m->table)) return false;
+  if (m->has_activity && element_count(m->activity) != 1) return false;
+  if (at + 3 < count && copies_attended_chunk(m->out, d[at + 3])) {
+    m->has_copy = true;
+    m->copy_target = d[at + 3].outputs[0];
+    m->dispatches = 4;
+  }
+  return true;
+}
+
+// Whether `b` can follow `a` in a run with chunks: everything but the per-member row count, the
+// outputs' layouts and the presence of a copy agrees.
+bool same_chunk_shape(const LaneMember &a, const LaneMember &b) {
+  if (a.has_activity != b.has_activity) return false;
+  if (memcmp(&a.scale, &b.scale, sizeof(float)) != 0 || a.page_tokens != b.page_tokens) return false;
+  const fh_tensor *left[3] = {&a.q, &a.k_new, &a.v_new}, *right[3] = {&b.q, &b.k_new, &b.v_new};
+  for (uint32_t i = 0; i < 3; ++i)
+    if (left[i]->buffer != right[i]->buffer || left[i]->dtype != right[i]->dtype) return false;
+  // heads, widths and the distance between a row's heads
+  if (a.q.shape[0] != b.q.shape[0] || a.q.shape[2] != b.q.shape[2] || a.q.stride[0] != b.q.stride[0] ||
+      a.q.stride[2] != b.q.stride[2])
+    return false;
+  for (uint32_t i = 1; i < 3; ++i)
+    if (left[i]->shape[1] != right[i]->shape[1] || left[i]->shape[2] != right[i]->shape[2] ||
+        left[i]->stride[1] != right[i]->stride[1] || left[i]->stride[2] != right[i]->stride[2])
+      return false;
+  if (!same_layout(a.table, b.table) || !same_tensor(a.generations, b.generations)) return false;
+  if (a.has_activity && !same_layout(a.activity, b.activity)) return false;
+  if (a.out.dtype != b.out.dtype || a.out.shape[0] != b.out.shape[0] || a.out.shape[2] != b.out.shape[2]) return false;
+  return same_tensor(a.key_pool, b.key_pool) && same_tensor(a.value_pool, b.value_pool);
+}
+
+// The elements [lo, hi) of its buffer a strided tensor touches at most.
+void extent_of(const fh_tensor &t, uint64_t *lo, uint64_t *hi) {
+  uint64_t last = 0;
+  for (uint32_t axis = 0; axis < t.rank; ++axis)
+    if (t.shape[axis] > 0) last += (uint64_t)(t.shape[axis] - 1) * t.stride[axis];
+  *lo = t.offset;
+  *hi = t.offset + last + 1;
+}
+
+// Most rows of attended output a run with chunks may stage, and most work of its overlap check.
+constexpr uint64_t kChunkRowsBytes = 256ull << 20;
+constexpr uint64_t kChunkCheckWork = 1ull << 27;
+
+// Longest run starting at `first` that has at least two members, at least one of them a chunk, and
+// whose packed rows follow each other at one row stride per tensor.  `run->delta` holds the row
+// strides of q and the new key and value rows.
+bool find_chunk_run(const fh_dispatch *d, uint32_t count, uint32_t first, LaneRun *run) {
+  *run = LaneRun{};
+  {   // nothing to look for unless the stretch of per-lane dispatches ahead holds a multi-row attention
+    bool chunk_ahead = false;
+    for (uint32_t at = first; at < count && !chunk_ahead; ++at) {
+      const uint32_t op = d[at].op;
+      if (op == FH_OP_PAGED_SDPA)
+        chunk_ahead = d[at].n_inputs >= 1 && d[at].inputs[0].rank == 3 && d[at].inputs[0].shape[1] > 1;
+      else if (op != FH_OP_PAGED_COPY && op != FH_OP_PAGED_SDPA_APPEND && op != FH_OP_COPY)
+        break;
+    }
+    if (!chunk_ahead) return false;
+  }
+  auto member_at = [&](uint32_t at, LaneMember *m) {
+    return chunk_member_at(d, count, at, m) || lane_member_at(d, count, at, m);
+  };
+  // row strides: known from a chunk member's own tensors, else from the first two members
+  auto strides_of = [](const LaneMember &m, int64_t out[3]) {
+    out[0] = (int64_t)m.q.stride[1];
+    out[1] = (int64_t)m.k_new.stride[0];
+    out[2] = (int64_t)m.v_new.stride[0];
+  };
+  LaneMember member;
+  if (!member_at(first, &member)) return false;
+  bool known = member.tokens > 1, any_chunk = member.tokens > 1;
+  if (known) strides_of(member, run->delta);
+  run->members.push_back(member);
+  run->dispatches = member.dispatches;
+  uint64_t tokens = member.tokens;
+  for (;;) {
+    const uint32_t at = first + run->dispatches;
+    if (at >= count || !member_at(at, &member)) break;
+    const LaneMember &head = run->members[0];
+    if (!same_chunk_shape(head, member)) break;
+    const fh_tensor *mine[3] = {&member.q, &member.k_new, &member.v_new};
+    const fh_tensor *heads[3] = {&head.q, &head.k_new, &head.v_new};
+    int64_t delta[3] = {run->delta[0], run->delta[1], run->delta[2]};
+    bool regular = true;
+    for (uint32_t i = 0; i < 3 && regular; ++i) {
+      const int64_t distance = (int64_t)mine[i]->offset - (int64_t)heads[i]->offset;
+      if (distance <= 0) regular = false;
+      else if (!known) {
+        if (distance % (int64_t)tokens != 0) regular = false;
+        delta[i] = distance / (int64_t)tokens;
+      } else if (distance != delta[i] * (int64_t)tokens) {
+        regular = false;
+      }
+    }
+    if (regular && member.tokens > 1) {
+      int64_t own[3];
+      strides_of(member, own);
+      for (uint32_t i = 0; i < 3; ++i)
+        if (own[i] != delta[i]) regular = false;
+    }
+    if (!regular) break;
+    for (uint32_t i = 0; i < 3; ++i) run->delta[i] = delta[i];
+    known = true;
+    any_chunk = any_chunk || member.tokens > 1;
+    tokens += member.tokens;
+    run->members.push_back(member);
+    run->dispatches += member.dispatches;
+  }
+  if (run->members.size() < 2 || !any_chunk) return false;
+  const LaneMember &head = run->members[0];
+  for (uint32_t i = 0; i < 3; ++i)
+    if (run->delta[i] <= 0) return false;
+  if (tokens * head.q.shape[0] * head.out.shape[2] * dtype_size(head.out.dtype) > kChunkRowsBytes) return false;
+  // the overlap check walks every reader's pages against every writer's: bounded here
+  {
+    uint64_t read_pages = 0, written_pages = 0;
+    for (const LaneMember &m : run->members) {
+      read_pages += ((uint64_t)m.q_start + m.tokens) / m.page_tokens + 1;
+      written_pages += (uint64_t)m.tokens / m.page_tokens + 2;
+    }
+    if (read_pages * written_pages > kChunkCheckWork) return false;
+  }
+  // Nothing a member writes may be something another member reads or writes.
+  std::unordered_set<uint64_t> read;
+  for (const fh_tensor *t : {&head.q, &head.k_new, &head.v_new, &head.generations, &head.key_pool,
+                             &head.value_pool})
+    read.insert(t->buffer);
+  struct Span {
+    uint64_t buffer, lo, hi;
+  };
+  std::vector<Span> written;
+  written.reserve(run->members.size() * 2);
+  std::vector<std::pair<uint64_t, uint64_t>> tables;
+  tables.reserve(run->members.size());
+  for (const LaneMember &m : run->members) {
+    read.insert(m.table.buffer);
+    if (m.has_activity) read.insert(m.activity.buffer);
+    uint64_t lo, hi;
+    extent_of(m.out, &lo, &hi);
+    written.push_back({m.out.buffer, lo, hi});
+    if (m.has_copy) {
+      extent_of(m.copy_target, &lo, &hi);
+      written.push_back({m.copy_target.buffer, lo, hi});
+    }
+    tables.push_back({m.table.buffer, m.table.offset});
+  }
+  for (const Span &span : written)
+    if (read.count(span.buffer)) return false;
+  // Two members on one table would store into the same slots: order matters, so no fusion.
+  std::sort(tables.begin(), tables.end());
+  if (std::adjacent_find(tables.begin(), tables.end()) != tables.end()) return false;
+  std::sort(written.begin(), written.end(), [](const Span &a, const Span &b) {
+    return a.buffer != b.buffer ? a.buffer < b.buffer : a.lo < b.lo;
+  });
+  for (size_t i = 1; i < written.size(); ++i)
+    if (written[i].buffer == written[i - 1].buffer && written[i].lo < written[i - 1].hi) return false;
+  return true;
+}
+
+// Executes the run found by find_chunk_run; same contract as run_lane_group.  A member's failures
+// go to the records of its own dispatches: storing a row to the first copy's (or the append's),
+// attending to the attention's.
+fh_status run_chunk_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors, bool *executed) {
+  *executed = true;
+  const LaneMember &head = run.members[0];
+  const fh_tensor &q0 = head.q, &kp = head.key_pool, &vp = head.value_pool;
+  const uint32_t lanes = (uint32_t)run.members.size(), heads = q0.shape[0];
+  const uint32_t table_pages = head.table.shape[0], table_words = table_pages * 2;
+  const uint32_t out_dtype = head.out.dtype, value_width = head.out.shape[2];
+  const uint64_t head_bytes = (uint64_t)value_width * dtype_size(out_dtype);
+  uint64_t tokens64 = 0;
+  for (const LaneMember &m : run.members) tokens64 += m.tokens;
+  FH_REQUIRE(tokens64 < (1ull << 31) && head_bytes * heads < (1ull << 31));
+  const uint32_t tokens = (uint32_t)tokens64;
+  // tables, activity, starts, cu (+ the overlap flag), the members' record indices; staged
+  // failure records of every row; the attended rows
+  const uint64_t metadata_words = (uint64_t)lanes * table_words + 5ull * lanes + 2;
+  const uint64_t staged_at = (metadata_words * 4 + 255) / 256 * 256;
+  const uint64_t rows_at = (staged_at + 2ull * tokens * sizeof(ErrorSlot) + 255) / 256 * 256;
+  char *scratch = b->ensure_lane_scratch(rows_at + (uint64_t)tokens * heads * head_bytes);
+  if (!scratch) {   // no room to stage the run (a caller that may not allocate): one by one
+    *executed = false;
+    return FH_OK;
+  }
+  uint32_t *tables = (uint32_t *)scratch;
+  uint32_t *activity = tables + (uint64_t)lanes * table_words;
+  uint32_t *starts = activity + lanes;
+  uint32_t *cu = starts + lanes;
+  uint32_t *records = cu + lanes + 2;
+  ErrorSlot *staged = (ErrorSlot *)(scratch + staged_at);
+  char *rows = scratch + rows_at;
+
+  std::vector<uint64_t> key;
+  key.reserve(6ull * lanes + 3);
+  key.push_back(~0ull);   // (a run of one-row members never has this first word: its lane count)
+  key.push_back(lanes);
+  key.push_back(table_words);
+  for (const LaneMember &m : run.members) {
+    key.push_back(m.table.buffer);
+    key.push_back(m.table.offset);
+    key.push_back(m.has_activity ? m.activity.buffer : 0);
+    key.push_back(m.has_activity ? m.activity.offset : 0);
+    key.push_back(m.q_start);
+    key.push_back(((uint64_t)m.tokens << 32) | ((uint64_t)m.dispatches << 8) | m.attention_at);
+  }
+  fh_status status;
+  if (!(b->lane_metadata_valid && key == b->lane_metadata_key)) {
+    b->lane_metadata_valid = false;
+    b->attention_plan_valid = false;  // the plan was built from the metadata replaced here
+    b->lane_metadata_watch.clear();
+    uint32_t first_token = 0, record = 0;
+    for (uint32_t base = 0; base < lanes; base += kChunkMembers) {
+      const uint32_t chunk = std::min<uint32_t>(kChunkMembers, lanes - base);
+      ChunkSources sources{};
+      for (uint32_t local = 0; local < chunk; ++local) {
+        const LaneMember &m = run.members[base + local];
+        View table, flag;
+        if ((status = make_view(b, m.table, false, &table)) != FH_OK) return status;
+        sources.table[local] = (const uint32_t *)table.base + table.offset;
+        b->lane_metadata_watch.insert(m.table.buffer);
+        if (m.has_activity) {
+          if ((status = make_view(b, m.activity, false, &flag)) != FH_OK) return status;
+          sources.activity[local] = (const uint32_t *)flag.base + flag.offset;
+          b->lane_metadata_watch.insert(m.activity.buffer);
+        }
+        sources.start[local] = m.q_start;
+        sources.first_token[local] = first_token;
+        sources.append_record[local] = record;
+        sources.attention_record[local] = record + m.attention_at;
+        first_token += m.tokens;
+        record += m.dispatches;
+      }
+      launch_gather_chunk_metadata(b->stream, sources, base, chunk, lanes, tokens, table_words, tables,
+                                   activity, starts, cu, records);
+    }
+    launch_init_errors(b->stream, staged, 2 * tokens);
+    // The one thing the tensors cannot show: a row stored into a slot another member attends.
+    uint32_t *flag = cu + lanes + 1;
+    launch_chunk_conflict_check(b->stream, tables, activity, starts, cu, lanes, table_pages,
+                                head.page_tokens, flag);
+    if (hipMemcpyAsync(b->host_flag, flag, sizeof(uint32_t), hipMemcpyDeviceToHost, b->stream) != hipSuccess ||
+        hipStreamSynchronize(b->stream) != hipSuccess)
+      return FH_DEVICE_EXECUTION_FAILED;
+    b->lane_conflict = *b->host_flag != 0;
+    b->lane_metadata_key = std::move(key);
+    b->lane_metadata_valid = true;
+  }
+  if (b->lane_conflict) {
+    *executed = false;
+    return FH_OK;
+  }
+
+  auto device_view = [](char *base, uint32_t dtype, std::initializer_list<uint32_t> shape) {
+    View v{};
+    v.base = base;
+    v.dtype = dtype;
+    v.rank = (uint32_t)shape.size();
+    for (uint32_t axis = 0; axis < FH_MAX_RANK; ++axis) {
+      v.shape[axis] = 1;
+      v.stride[axis] = 0;
+    }
+    uint32_t axis = 0;
+    for (uint32_t extent : shape) v.shape[axis++] = extent;
+    uint64_t stride = 1;
+    for (int at = (int)v.rank - 1; at >= 0; --at) {
+      v.stride[at] = stride;
+      stride *= v.shape[at];
+    }
+    return v;
+  };
+  RaggedAttention problem{};
+  // q [heads, n, D] per member -> [tokens, heads, D]; new rows [n, Hkv, D] -> [tokens, Hkv, D]
+  if ((status = make_view(b, q0, false, &problem.q)) != FH_OK) return status;
+  problem.q.shape[0] = tokens;
+  problem.q.shape[1] = heads;
+  problem.q.stride[0] = (uint64_t)run.delta[0];
+  problem.q.stride[1] = q0.stride[0];
+  View *appended[2] = {&problem.k_new, &problem.v_new};
+  const fh_tensor *appended_from[2] = {&head.k_new, &head.v_new};
+  for (uint32_t i = 0; i < 2; ++i) {
+    if ((status = make_view(b, *appended_from[i], false, appended[i])) != FH_OK) return status;
+    appended[i]->shape[0] = tokens;
+    appended[i]->stride[0] = (uint64_t)run.delta[1 + i];
+  }
+  if ((status = make_view(b, head.generations, false, &problem.generations)) != FH_OK) return status;
+  if ((status = make_view(b, kp, true, &problem.key_pool)) != FH_OK) return status;
+  if ((status = make_view(b, vp, true, &problem.value_pool)) != FH_OK) return status;
+  problem.tables = device_view((char *)tables, FH_U32, {lanes, table_pages, 2});
+  problem.activity = device_view((char *)activity, FH_U32, {lanes});
+  problem.q_starts = device_view((char *)starts, FH_U32, {lanes});
+  problem.cu_seqlens = device_view((char *)cu, FH_U32, {lanes + 1});
+  problem.out = device_view(rows, out_dtype, {tokens, heads, value_width});
+  problem.tokens = tokens;
+  problem.lanes = lanes;
+  problem.query_heads = heads;
+  problem.kv_heads = kp.shape[2];
+  problem.width = q0.shape[2];
+  problem.value_width = value_width;
+  problem.page_tokens = head.page_tokens;
+  problem.physical_pages = kp.shape[0];
+  problem.table_pages = table_pages;
+  problem.scale = head.scale;
+  problem.metadata_buffers[4] = head.generations.buffer;  // the rest is watched through the gather
+  problem.error_stride = 2;             // staged records: (storing, attending) per row
+  problem.attention_error_offset = 1;
+  problem.one_row_per_lane = 0;
+  if (!run_ragged_attention(b, problem, staged)) {
+    b->lane_metadata_valid = false;
+    return FH_ALLOCATION_FAILED;
+  }
+  launch_fold_chunk_errors(b->stream, staged, errors, cu, records, lanes, tokens);
+
+  const uint32_t element = dtype_size(out_dtype);
+  uint32_t first_token = 0;
+  for (uint32_t base = 0; base < lanes; base += kChunkMembers) {
+    const uint32_t chunk = std::min<uint32_t>(kChunkMembers, lanes - base);
+    ChunkTargets targets{};
+    for (uint32_t local = 0; local < chunk; ++local) {
+      const LaneMember &m = run.members[base + local];
+      View rows_view;
+      if ((status = make_view(b, m.out, true, &rows_view)) != FH_OK) return status;
+      FH_REQUIRE(m.out.stride[0] * element < (1ull << 32));
+      if (m.tokens > 1) FH_REQUIRE(m.out.stride[1] * element < (1ull << 32));
+      targets.target[0][local] = rows_view.base + rows_view.offset * element;
+      targets.token_stride[0][local] = m.tokens > 1 ? (uint32_t)(m.out.stride[1] * element) : 0;   // out is [heads, n, width]
+      targets.head_stride[0][local] = (uint32_t)(m.out.stride[0] * element);
+      if (m.has_copy) {
+        if ((status = make_view(b, m.copy_target, true, &rows_view)) != FH_OK) return status;
+        targets.target[1][local] = rows_view.base + rows_view.offset * element;
+        if (m.tokens > 1) {   // [n, heads, width], head rows dense
+          FH_REQUIRE(m.copy_target.stride[0] * element < (1ull << 32));
+          targets.token_stride[1][local] = (uint32_t)(m.copy_target.stride[0] * element);
+        } else {              // one dense row of heads * width elements
+          targets.token_stride[1][local] = 0;
+        }
+        targets.head_stride[1][local] = (uint32_t)head_bytes;
+      }
+      targets.first_token[local] = first_token;
+      first_token += m.tokens;
+    }
+    targets.first_token[chunk] = first_token;
+    launch_scatter_chunk_rows(b->stream, targets, rows, chunk, heads, (uint32_t)head_bytes);
   }
   b->fused_runs += 1;
   b->fused_dispatches += run.dispatches;
@@ -2292,8 +2728,11 @@ static fh_status submit_locked(fh_backend *b, const fh_dispatch *dispatches, uin
     uint32_t consumed = 1;
     LaneRun run;
     const uint32_t op = dispatches[i].op;
-    bool fused = b->lane_fusion && (op == FH_OP_PAGED_SDPA_APPEND || op == FH_OP_PAGED_COPY) &&
-                 i >= no_run_before && find_lane_run(dispatches, count, i, &run);
+    const bool candidate = b->lane_fusion && (op == FH_OP_PAGED_SDPA_APPEND || op == FH_OP_PAGED_COPY) &&
+                           i >= no_run_before;
+    // a run that brings prefill chunks first (it takes one-row members too), else one of one-row members
+    const bool with_chunks = candidate && find_chunk_run(dispatches, count, i, &run);
+    bool fused = with_chunks || (candidate && find_lane_run(dispatches, count, i, &run));
     if (fused)
       consumed = run.dispatches;
     else if (run.members.size() > 1)
@@ -2307,7 +2746,8 @@ static fh_status submit_locked(fh_backend *b, const fh_dispatch *dispatches, uin
     }
     if (fused) {
       bool executed = true;
-      status = run_lane_group(b, run, &s->device_errors[i], &executed);
+      status = with_chunks ? run_chunk_group(b, run, &s->device_errors[i], &executed)
+                           : run_lane_group(b, run, &s->device_errors[i], &executed);
       if (!executed) {
         fused = false;
         for (uint32_t member = 0; member < consumed && status == FH_OK; ++member) {

@@ -131,4 +131,42 @@ bool launch_lane_conflict_check(hipStream_t s, const uint32_t *tables, const uin
 void launch_scatter_lane_rows(hipStream_t s, const LaneRows &targets, const void *rows,
                               uint32_t first, uint32_t count, uint32_t row_bytes);
 
+// The same glue for runs whose members bring several query rows (prefill chunks recorded per
+// sequence next to decode rows).  Up to kChunkMembers members per launch.
+constexpr uint32_t kChunkMembers = 64;
+struct ChunkSources {
+  const uint32_t *table[kChunkMembers];
+  const uint32_t *activity[kChunkMembers];   // null: always active
+  uint32_t start[kChunkMembers];             // position of the member's first query row
+  uint32_t first_token[kChunkMembers];       // query rows of the members before it
+  uint32_t append_record[kChunkMembers];     // error record of the dispatch that stores its rows ...
+  uint32_t attention_record[kChunkMembers];  // ... and of the one that attends, from the run's first
+};
+struct ChunkTargets {
+  void *target[2][kChunkMembers];            // where the member's rows go (second: null or a copy)
+  uint32_t token_stride[2][kChunkMembers];   // bytes between a member's rows, and between the
+  uint32_t head_stride[2][kChunkMembers];    // heads of a row, in each destination
+  uint32_t first_token[kChunkMembers + 1];
+};
+// Members [first, first + count) of `lanes`: as launch_gather_lane_metadata, with cu from the
+// members' row counts (cu[lanes] = tokens) and the members' record indices in records[2][lanes].
+void launch_gather_chunk_metadata(hipStream_t s, const ChunkSources &sources, uint32_t first,
+                                  uint32_t count, uint32_t lanes, uint32_t tokens,
+                                  uint32_t table_words, uint32_t *tables, uint32_t *activity,
+                                  uint32_t *starts, uint32_t *cu, uint32_t *records);
+// Sets *conflict to 1 when an active member stores a row into a slot another active member
+// attends.
+void launch_chunk_conflict_check(hipStream_t s, const uint32_t *tables, const uint32_t *activity,
+                                 const uint32_t *starts, const uint32_t *cu, uint32_t lanes,
+                                 uint32_t table_pages, uint32_t page_tokens, uint32_t *conflict);
+// rows: [tokens, heads, row_bytes] contiguous; moves the rows of `count` members.
+void launch_scatter_chunk_rows(hipStream_t s, const ChunkTargets &targets, const void *rows,
+                               uint32_t count, uint32_t heads, uint32_t row_bytes);
+// Failures the fused launch recorded per query row (staged[2 * token]: storing the row,
+// staged[2 * token + 1]: attending) go to the records of the dispatches they belong to; the
+// staged records are cleared for the next run.
+void launch_fold_chunk_errors(hipStream_t s, ErrorSlot *staged, ErrorSlot *records_of_run,
+                              const uint32_t *cu, const uint32_t *records, uint32_t lanes,
+                              uint32_t tokens);
+
 }  // namespace fh

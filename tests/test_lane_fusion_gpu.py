@@ -369,3 +369,224 @@ def test_random_recordings_give_the_same_result_fused_and_dispatch_by_dispatch(c
     check(hip, hip, results["serial"], results["fused"], exact=(1, 2), bar=DType.BF16)
     if "cpu" in results:
         check(cpu, hip, results["cpu"], results["fused"], exact=(1, 2), bar=DType.BF16)
+
+
+# ---- runs that bring prefill chunks (a sequence's chunk recorded on its own: cache.append, then
+# cache.attention over its rows, engines/qwen3-coder/src/lib.rs:685-707) ----
+
+class ChunkBatch:
+    """A packed batch of members (start, rows): rows > 1 is a prefill chunk, rows == 1 a decode row.
+    `share` = (a, b, pages): member b's first `pages` table entries name member a's physical pages
+    (a common prompt prefix, read only)."""
+
+    def __init__(self, backend, members, hq, hkv, pt, seed, layers=1, share=None, corrupt=None,
+                 activity=None):
+        self.backend, self.members, self.hq, self.hkv, self.pt = backend, list(members), hq, hkv, pt
+        pages_needed = [(start + rows + pt - 1) // pt for start, rows in members]
+        self.table_pages = max(pages_needed) + 2
+        physical = sum(pages_needed) + 3
+        rng = np.random.default_rng(seed)
+        free = list(rng.permutation(physical))
+        self.tables, self.host_tables = [], []
+        for index, need in enumerate(pages_needed):
+            table = np.zeros((self.table_pages, 2), np.uint32)
+            table[:, 1] = 0xffffffff
+            for logical in range(need):
+                page = free.pop()
+                table[logical] = (page, 11 + page)
+            self.host_tables.append(table)
+        if share is not None:
+            a, b, pages = share
+            self.host_tables[b][:pages] = self.host_tables[a][:pages]
+        if corrupt is not None:
+            self.host_tables[corrupt[0]][corrupt[1], 1] += 1
+        self.tables = [upload(backend, table, DType.U32) for table in self.host_tables]
+        self.generations = upload(backend, 11 + np.arange(physical), DType.U32)
+        self.activity = None if activity is None else upload(backend, np.array(activity), DType.U32)
+        self.tokens = sum(rows for _, rows in members)
+        self.q = upload(backend, normal_bf16(seed, 3, (self.tokens, hq, WIDTH)), DType.BF16)
+        self.k = upload(backend, normal_bf16(seed, 4, (self.tokens, hkv, WIDTH)), DType.BF16)
+        self.v = upload(backend, normal_bf16(seed, 5, (self.tokens, hkv, WIDTH)), DType.BF16)
+        self.pools = []
+        for layer in range(layers):
+            keys = upload(backend, normal_bf16(seed, 10 + 2 * layer, (physical, pt, hkv, WIDTH)), DType.BF16)
+            values = upload(backend, normal_bf16(seed, 11 + 2 * layer, (physical, pt, hkv, WIDTH)), DType.BF16)
+            self.pools.append((keys, values))
+
+    def record_layer(self, commands, layer, copy_rows=True, decode_idiom="append"):
+        backend, hq, hkv, pt = self.backend, self.hq, self.hkv, self.pt
+        scale = 1.0 / math.sqrt(WIDTH)
+        attended = backend.alloc(DType.BF16, (self.tokens, hq * WIDTH))
+        keys, values = self.pools[layer]
+        physical, elements = keys.shape[0], hkv * WIDTH
+        outs, first = [], 0
+        for index, (start, rows) in enumerate(self.members):
+            paging = [self.tables[index], self.generations]
+            if self.activity is not None:
+                paging.append(self.activity.narrow(0, index, 1))
+            q = self.q.narrow(0, first, rows).permute([1, 0, 2])
+            k_rows, v_rows = self.k.narrow(0, first, rows), self.v.narrow(0, first, rows)
+            if rows == 1 and decode_idiom == "append":
+                out = backend.alloc(DType.BF16, (1, hq, WIDTH))
+                commands.dispatch_many(Op.paged_sdpa_append(scale, start, pt), [q, k_rows, v_rows, *paging],
+                                       [out.permute([1, 0, 2]), keys, values])
+                if copy_rows:
+                    commands.dispatch(Op.copy(), [out.reshape((1, hq * WIDTH))], attended.narrow(0, first, 1))
+            else:
+                out = backend.alloc(DType.BF16, (hq, rows, WIDTH))
+                for new_rows, pool in ((k_rows, keys), (v_rows, values)):
+                    commands.dispatch(Op.paged_copy(INTO_PAGES, start, pt),
+                                      [new_rows.reshape((rows, elements)), *paging],
+                                      pool.reshape((physical, pt, elements)))
+                commands.dispatch(Op.paged_sdpa(scale, True, start, start + rows, pt),
+                                  [q, keys, values, *paging], out)
+                if copy_rows:
+                    commands.dispatch(Op.copy(), [out.permute([1, 0, 2])],
+                                      attended.narrow(0, first, rows).reshape((rows, hq, WIDTH)))
+            outs.append(out)
+            first += rows
+        return attended, outs
+
+
+CHUNK_CASES = [
+    # members (start, rows), hq, hkv, page_tokens, share (a, b, pages), dispatches per layer when copies follow
+    ([(48, 37), (130, 1), (0, 20), (77, 1)], 8, 4, 16, (0, 1, 3), "append"),
+    ([(48, 37), (130, 1), (0, 20), (77, 1)], 8, 4, 16, (0, 1, 3), "copies"),
+    ([(0, 300), (64, 129)], 32, 4, 64, None, "append"),                      # chunks only, engine page size
+    ([(5, 1), (9, 1), (16, 16), (31, 2), (200, 1)], 16, 2, 16, (2, 4, 1), "append"),
+]
+
+
+@pytest.mark.parametrize("copy_rows", [True, False])
+@pytest.mark.parametrize("members,hq,hkv,pt,share,decode_idiom", CHUNK_CASES)
+def test_chunks_recorded_per_sequence_run_as_one_ragged_launch(cpu, hip, members, hq, hkv, pt, share,
+                                                                decode_idiom, copy_rows):
+    """Prefill chunks and decode rows of different sequences, each recorded on its own, two layers
+    on the same members: one fused launch per layer on the device, serial on the oracle and in the
+    library's own dispatch-by-dispatch execution; pools bit for bit, rows to the float bar."""
+    outputs = {}
+    for name, backend in (("cpu", cpu), ("fused", hip), ("serial", hip)):
+        if backend is hip:
+            hip.fusion_enable(name == "fused")
+        before = hip.fusion_stats()
+        batch = ChunkBatch(backend, members, hq, hkv, pt, seed=171, layers=2, share=share)
+        commands = CommandList()
+        kept, pools = [], []
+        for layer in range(2):
+            attended, outs = batch.record_layer(commands, layer, copy_rows=copy_rows, decode_idiom=decode_idiom)
+            kept += [attended, *outs] if copy_rows else list(outs)
+            pools += [len(kept), len(kept) + 1]
+            kept += list(batch.pools[layer])
+        recorded = len(commands.dispatches)
+        run(backend, commands)
+        outputs[name] = kept
+        runs, dispatches = (after - start for after, start in zip(hip.fusion_stats(), before))
+        assert (runs, dispatches) == ((2, recorded) if name == "fused" else (0, 0))
+    hip.fusion_enable(True)
+    check(cpu, hip, outputs["cpu"], outputs["fused"], exact=pools)
+    check(cpu, hip, outputs["cpu"], outputs["serial"], exact=pools)
+    check(hip, hip, outputs["serial"], outputs["fused"], exact=pools)
+
+
+@pytest.mark.parametrize("case", ["chunk_into_attended_page", "row_into_chunk_page"])
+def test_a_chunk_stored_into_a_page_another_member_attends_runs_dispatch_by_dispatch(cpu, hip, case):
+    """Two members whose tables name one physical page where one stores rows and the other attends:
+    found on the device, executed one dispatch at a time, equal to the oracle's serial result."""
+    pt = 16
+    members = {"chunk_into_attended_page": [(16, 20), (40, 1)],     # the chunk stores into logical page 1, which the row attends
+               "row_into_chunk_page": [(40, 1), (30, 12)]}[case]    # the row's slot lies in a page the chunk attends
+    results = []
+    for backend in (cpu, hip):
+        batch = ChunkBatch(backend, members, 8, 4, pt, seed=173)
+        if case == "chunk_into_attended_page":
+            batch.host_tables[1][1] = batch.host_tables[0][1]
+            backend.write(batch.tables[1], batch.host_tables[1].tobytes())
+        else:
+            batch.host_tables[1][2] = batch.host_tables[0][2]
+            backend.write(batch.tables[1], batch.host_tables[1].tobytes())
+        before = hip.fusion_stats()
+        commands = CommandList()
+        attended, outs = batch.record_layer(commands, 0)
+        run(backend, commands)
+        if backend is hip:
+            assert hip.fusion_stats() == before
+        results.append([attended, *outs, *batch.pools[0]])
+    pools = (len(results[0]) - 2, len(results[0]) - 1)
+    check(cpu, hip, results[0], results[1], exact=pools)
+
+
+@pytest.mark.parametrize("corrupt,expected", [
+    ((0, 1), (2, 1)),     # stale history page of the first chunk: its attention dispatch, page 1
+    ((2, 0), (6, 0)),     # stale page under the second chunk's rows: that chunk's first copy
+    ((1, 2), (4, 2)),     # stale page under the decode row: its append
+])
+def test_a_chunk_run_reports_a_stale_page_for_the_dispatch_that_meets_it(hip, corrupt, expected):
+    indices = []
+    for fused in (True, False):
+        hip.fusion_enable(fused)
+        batch = ChunkBatch(hip, [(32, 9), (40, 1), (0, 14)], 8, 4, 16, seed=174, corrupt=corrupt)
+        commands = CommandList()
+        batch.record_layer(commands, 0)
+        with pytest.raises(BackendError) as info:
+            run(hip, commands)
+        assert info.value.status == Status.DEVICE_ERROR_FLAG
+        indices.append((info.value.dispatch, info.value.index))
+    hip.fusion_enable(True)
+    assert indices[0] == indices[1] == expected
+
+
+def test_chunk_runs_with_inactive_members(cpu, hip):
+    results = []
+    for backend in (cpu, hip):
+        before = hip.fusion_stats()
+        batch = ChunkBatch(backend, [(20, 18), (33, 1), (0, 7), (64, 5)], 8, 4, 16, seed=175,
+                           activity=[1, 0, 0, 1])
+        commands = CommandList()
+        attended, outs = batch.record_layer(commands, 0, decode_idiom="copies")
+        run(backend, commands)
+        results.append([attended, *outs, *batch.pools[0]])
+        if backend is hip:
+            assert hip.fusion_stats()[0] - before[0] == 1
+    pools = (len(results[0]) - 2, len(results[0]) - 1)
+    check(cpu, hip, results[0], results[1], exact=pools)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_chunk_recordings_give_the_same_result_fused_and_dispatch_by_dispatch(cpu, hip, seed):
+    """Random mixes of chunks and decode rows, with and without the row copies, inactive members and
+    shared prefix pages: pools bit for bit what serial execution leaves, rows to the float bar; the
+    first four seeds are also held to the oracle."""
+    rng = np.random.default_rng(3000 + seed)
+    count = int(rng.integers(2, 7))
+    members = []
+    for _ in range(count):
+        rows = 1 if rng.integers(0, 2) else int(rng.integers(2, 50))
+        members.append((int(rng.integers(0, 150)), rows))
+    if all(rows == 1 for _, rows in members):
+        members[0] = (members[0][0], 9)
+    options = dict(hq=int(rng.choice([4, 8, 16])), hkv=int(rng.choice([2, 4])),
+                   activity=[int(a) for a in (rng.random(count) > 0.25)] if rng.integers(0, 2) else None,
+                   copy_rows=bool(rng.integers(0, 2)), idiom=str(rng.choice(["append", "copies"])))
+    share = None
+    if count >= 2 and rng.integers(0, 2):
+        a, b = (int(v) for v in rng.choice(count, 2, replace=False))
+        pages = min(members[a][0], members[b][0]) // 16     # whole pages of history both have
+        share = (a, b, pages) if pages else None
+    results = {}
+    for name, backend in (("fused", hip), ("serial", hip)) + ((("cpu", cpu),) if seed < 4 else ()):
+        if backend is hip:
+            hip.fusion_enable(name == "fused")
+        batch = ChunkBatch(backend, members, options["hq"], options["hkv"], 16, seed=300 + seed,
+                           share=share, activity=options["activity"])
+        commands = CommandList()
+        before = hip.fusion_stats()[0]
+        attended, outs = batch.record_layer(commands, 0, copy_rows=options["copy_rows"],
+                                            decode_idiom=options["idiom"])
+        run(backend, commands)
+        results[name] = [*batch.pools[0], attended, *outs] if options["copy_rows"] else [*batch.pools[0], *outs]
+        if name == "fused":
+            assert hip.fusion_stats()[0] == before + 1
+    hip.fusion_enable(True)
+    check(hip, hip, results["serial"], results["fused"], exact=(0, 1))
+    if "cpu" in results:
+        check(cpu, hip, results["cpu"], results["fused"], exact=(0, 1))

@@ -237,8 +237,9 @@ __global__ void ragged_attention_generic_kernel(RaggedAttention p, ErrorSlot *er
 // ------------------------------------------------- 2-byte pools (bf16 or f16), D = Dv = 128
 //
 // The pools' dtype is the matrix cores' operand type (kHalf: f16, else bf16).  Queries are of that
-// dtype, or f32 against f16 pools (rounded to f16 once, as they enter the operand registers: an
-// 11-bit significand on one factor of a 128-term dot product moves a score by ~1e-4); outputs are
+// dtype, or f32 (rounded to the pools' dtype once, as they enter the operand registers: an 11-bit
+// significand on one factor of a 128-term dot product moves a score by ~1e-4, the 8 bits of bf16
+// by ~1e-3, within the bar the reference holds outputs attended from such pools to); outputs are
 // written in any float dtype.
 //
 // Split-KV decode-style attention on the matrix cores, registers only.  One wave owns
@@ -564,14 +565,15 @@ __device__ inline f32x4 mfma_16x16x32(const uint4 &a, const uint4 &b, const f32x
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// Eight query elements from `element` as operand words.  An f32 query beyond the f16 range is
-// held at the largest finite f16 (a NaN stays a NaN): the scores stay finite, as the reference's.
+// Eight query elements from `element` as operand words.  An f32 query is rounded to the pools'
+// dtype; against f16 pools an element beyond the f16 range is held at the largest finite f16 (a
+// NaN stays a NaN): the scores stay finite, as the reference's.
 template <bool kHalf, bool kMixed>
 __device__ inline uint4 load_query(const FastRagged &p, uint64_t element) {
   if (!kMixed || p.q_dtype != FH_F32) return *(const uint4 *)((const uint16_t *)p.q + element);
   const float4 lo = *(const float4 *)((const float *)p.q + element);
   const float4 hi = *(const float4 *)((const float *)p.q + element + 4);
-  auto held = [](float v) { return fabsf(v) > 65504.0f ? copysignf(65504.0f, v) : v; };
+  auto held = [](float v) { return kHalf && fabsf(v) > 65504.0f ? copysignf(65504.0f, v) : v; };
   return make_uint4(pack_operand<kHalf>(held(lo.x), held(lo.y)), pack_operand<kHalf>(held(lo.z), held(lo.w)),
                     pack_operand<kHalf>(held(hi.x), held(hi.y)), pack_operand<kHalf>(held(hi.z), held(hi.w)));
 }
@@ -1147,11 +1149,11 @@ __global__ __launch_bounds__(256) void ragged_reduce_kernel(FastRagged p) {
   }
 }
 
-// Pools of one 2-byte dtype; queries of the same dtype, or f32 against f16 pools; any float output.
+// Pools of one 2-byte dtype; queries of the same dtype or f32; any float output.
 bool fast_dtypes(const View &q, const View &out, const View &key_pool, const View &value_pool) {
   const uint32_t pool = key_pool.dtype;
   if ((pool != FH_BF16 && pool != FH_F16) || value_pool.dtype != pool) return false;
-  if (q.dtype != pool && !(pool == FH_F16 && q.dtype == FH_F32)) return false;
+  if (q.dtype != pool && q.dtype != FH_F32) return false;
   return out.dtype == FH_F32 || out.dtype == FH_F16 || out.dtype == FH_BF16;
 }
 

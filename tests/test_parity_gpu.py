@@ -1066,6 +1066,8 @@ DTYPE_MIXES = [
     (DType.F16, DType.F16, DType.F16),
     (DType.F16, DType.F16, DType.BF16),
     (DType.BF16, DType.BF16, DType.F32),
+    (DType.F32, DType.BF16, DType.F32),     # f32 activations against a bf16 cache
+    (DType.F32, DType.BF16, DType.BF16),
 ]
 
 
@@ -1077,7 +1079,7 @@ DTYPE_MIXES = [
     (list(range(0, 520, 13)), [1] * 40, 16, 8, 16, True)])
 def test_ragged_attention_across_activation_and_pool_dtypes(cpu, hip, dtype, pool_dtype, out_dtype, contexts,
                                                             counts, hq, hkv, pt, promise):
-    """f16 or bf16 pools fed by rows of their own dtype or (f16) by f32 rows, any float output: the
+    """f16 or bf16 pools fed by rows of their own dtype or by f32 rows, any float output: the
     stored rows are rounded once, exactly as the oracle rounds them, so the pools match bit for
     bit; a second layer reuses the work plan on other pools."""
     scale = 1.0 / math.sqrt(128)

@@ -328,9 +328,25 @@ def packed_step_c1(backend, seed=97, repeats=3):
     for submission in submissions:
         submission.wait()
     seconds = sum(submission.gpu_time_ns() for submission in submissions) / repeats * 1e-9
+    # what bounds it: the matrix work of 2048 rows (projections, lm_head, attention pairs), and the
+    # bytes that must move whatever the rows (weights once, the KV the decode rows and chunks read)
+    rows = step.tokens
+    qkv_width = (c.q_heads + 2 * c.kv_heads) * c.head_dim
+    per_layer = qkv_width * c.hidden + c.hidden * c.q_heads * c.head_dim + 3 * c.intermediate * c.hidden
+    pairs = sum(n * ctx + n * (n + 1) // 2 for ctx, n in zip(contexts, counts))
+    flops = 2.0 * rows * (c.layers * per_layer + c.vocab * c.hidden) + c.layers * 2.0 * c.q_heads * pairs * 2 * c.head_dim
+    weight_bytes = (c.layers * per_layer + c.vocab * c.hidden) * 0.5625
+    kv_bytes = sum(ctx + n for ctx, n in zip(contexts, counts)) * c.kv_bytes_per_token   # (all layers)
     return {"workload": "BASELINE config 1: 28 layers, 48 decode rows + prefill chunks 256/384/512/848 "
                         "packed into 2048 tokens, lm_head and argmax on every row",
-            "tokens": step.tokens, "ms_per_step": seconds * 1e3, "tok_per_s": step.tokens / seconds}
+            "tokens": step.tokens, "ms_per_step": seconds * 1e3, "tok_per_s": step.tokens / seconds,
+            "roofline": {"bound": "mfma", "achieved": flops / seconds / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": flops / seconds / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                         "flops_per_step": flops,
+                         "hbm_floor_ms": (weight_bytes + kv_bytes) / (HBM_PEAK_GBPS * 1e9) * 1e3,
+                         "mfma_floor_ms": flops / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e3,
+                         "note": "a 0.6B model at 2048 rows: 161 kernels of 20-120 us each, none long "
+                                 "enough to fill the device; neither floor is near"}}
 
 
 def lane_by_lane_step(workload, backend, steps=8, warmup=2):

@@ -181,6 +181,7 @@ extern "C" {
     pub fn fh_synchronize(backend: *mut fh_backend) -> u32;
     pub fn fh_profile_enable(backend: *mut fh_backend, enabled: c_int) -> u32;
     pub fn fh_profile_select(backend: *mut fh_backend, class_mask: u32) -> u32;
+    pub fn fh_profile_sample(backend: *mut fh_backend, every: u32) -> u32;
     pub fn fh_profile_reset(backend: *mut fh_backend) -> u32;
     pub fn fh_profile_read(backend: *mut fh_backend, kernel_class: u32, nanoseconds: *mut u64, launches: *mut u64) -> u32;
     pub fn fh_fusion_enable(backend: *mut fh_backend, enabled: c_int) -> u32;

@@ -181,6 +181,8 @@ struct fh_backend {
   // profiling
   int profiling = 0;  // 0 off, 1 kernel-level timers, 2 also one timer per dispatch
   uint32_t profile_mask = 0xffffffffu;  // kernel classes the kernel-level timers cover
+  uint32_t profile_every = 1;              // kernel-level timers take one launch in this many of a class
+  uint32_t profile_seen[FH_KC_COUNT] = {};
   struct Timed {
     hipEvent_t start, end;
     uint32_t kernel_class;
@@ -1999,6 +2001,13 @@ bool find_chunk_run(const fh_dispatch *d, uint32_t count, uint32_t first, LaneRu
   for (uint32_t i = 0; i < 3; ++i)
     if (run->delta[i] <= 0) return false;
   if (tokens * head.q.shape[0] * head.out.shape[2] * dtype_size(head.out.dtype) > kChunkRowsBytes) return false;
+  // the scatter of the attended rows addresses each destination with 32-bit byte strides
+  for (const LaneMember &m : run->members) {
+    const uint64_t element = dtype_size(m.out.dtype);
+    if (m.out.stride[0] * element >= (1ull << 32)) return false;
+    if (m.tokens > 1 && m.out.stride[1] * element >= (1ull << 32)) return false;
+    if (m.has_copy && m.tokens > 1 && m.copy_target.stride[0] * element >= (1ull << 32)) return false;
+  }
   // the overlap check walks every reader's pages against every writer's: bounded here
   {
     uint64_t read_pages = 0, written_pages = 0;
@@ -2207,8 +2216,6 @@ fh_status run_chunk_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors, 
       const LaneMember &m = run.members[base + local];
       View rows_view;
       if ((status = make_view(b, m.out, true, &rows_view)) != FH_OK) return status;
-      FH_REQUIRE(m.out.stride[0] * element < (1ull << 32));
-      if (m.tokens > 1) FH_REQUIRE(m.out.stride[1] * element < (1ull << 32));
       targets.target[0][local] = rows_view.base + rows_view.offset * element;
       targets.token_stride[0][local] = m.tokens > 1 ? (uint32_t)(m.out.stride[1] * element) : 0;   // out is [heads, n, width]
       targets.head_stride[0][local] = (uint32_t)(m.out.stride[0] * element);
@@ -2216,7 +2223,6 @@ fh_status run_chunk_group(fh_backend *b, const LaneRun &run, ErrorSlot *errors, 
         if ((status = make_view(b, m.copy_target, true, &rows_view)) != FH_OK) return status;
         targets.target[1][local] = rows_view.base + rows_view.offset * element;
         if (m.tokens > 1) {   // [n, heads, width], head rows dense
-          FH_REQUIRE(m.copy_target.stride[0] * element < (1ull << 32));
           targets.token_stride[1][local] = (uint32_t)(m.copy_target.stride[0] * element);
         } else {              // one dense row of heads * width elements
           targets.token_stride[1][local] = 0;
@@ -3073,6 +3079,17 @@ fh_status fh_profile_select(fh_backend *b, uint32_t class_mask) {
   return FH_OK;
 }
 
+fh_status fh_profile_sample(fh_backend *b, uint32_t every) {
+  if (!b || every == 0) return FH_INVALID_INPUT;
+  std::lock_guard<std::mutex> lock(b->mutex);
+  (void)hipSetDevice(b->device);
+  (void)hipStreamSynchronize(b->stream);
+  drain_profile(b);
+  b->profile_every = every;
+  for (uint32_t &seen : b->profile_seen) seen = 0;
+  return FH_OK;
+}
+
 fh_status fh_fusion_enable(fh_backend *b, int enabled) {
   if (!b) return FH_INVALID_INPUT;
   std::lock_guard<std::mutex> lock(b->mutex);
@@ -3204,6 +3221,9 @@ uint32_t backend_compute_units(fh_backend *backend) {
 void backend_profile_begin(fh_backend *backend, uint32_t kernel_class) {
   if (!backend->profiling || kernel_class >= FH_KC_COUNT) return;
   if (!((backend->profile_mask >> kernel_class) & 1u)) return;
+  // one launch in `profile_every` of the class is timed (backend_profile_end finds no open timer
+  // for the others)
+  if (backend->profile_every > 1 && backend->profile_seen[kernel_class]++ % backend->profile_every != 0) return;
   hipEvent_t event = nullptr;
   if (!backend->event_pool.empty()) {
     event = backend->event_pool.back();

@@ -66,7 +66,7 @@ EXPORTS = [
     "fh_read_tensor", "fh_prepare_program", "fh_release_program", "fh_submit", "fh_submit_static", "fh_wait",
     "fh_gpu_time_ns", "fh_submission_free", "fh_device_info_get", "fh_memory_usage", "fh_set_memory_limit",
     "fh_submit_profiled", "fh_submission_profile",
-    "fh_synchronize", "fh_profile_enable", "fh_profile_select", "fh_profile_reset", "fh_profile_read",
+    "fh_synchronize", "fh_profile_enable", "fh_profile_select", "fh_profile_sample", "fh_profile_reset", "fh_profile_read",
     "fh_fusion_enable", "fh_fusion_stats", "fh_version",
 ]
 
@@ -110,6 +110,7 @@ def load_library():
     lib.fh_profile_enable.argtypes = [vp, C.c_int]
     lib.fh_profile_reset.argtypes = [vp]
     lib.fh_profile_select.argtypes = [vp, u32]
+    lib.fh_profile_sample.argtypes = [vp, u32]
     lib.fh_profile_read.argtypes = [vp, u32, C.POINTER(u64), C.POINTER(u64)]
     lib.fh_fusion_enable.argtypes = [vp, C.c_int]
     lib.fh_fusion_stats.argtypes = [vp, C.POINTER(u64), C.POINTER(u64)]
@@ -372,6 +373,10 @@ class HipBackend:
     def profile_select(self, class_mask: int):
         """Kernel classes (bit i = class i) the kernel-level timers cover; all by default."""
         _check(self._lib.fh_profile_select(self._handle, int(class_mask) & 0xffffffff))
+
+    def profile_sample(self, every: int):
+        """The kernel-level timers take one launch in `every` of each selected class."""
+        _check(self._lib.fh_profile_sample(self._handle, int(every)))
 
     def fusion_enable(self, enabled: bool):
         """Whether runs of per-lane attention dispatches are executed as one ragged launch."""

@@ -292,6 +292,10 @@ FH_API fh_status fh_profile_enable(fh_backend *backend, int enabled);
  * all classes by default): every timed launch costs two event records on the stream, so a
  * throughput measurement times only the kernel it reports on. */
 FH_API fh_status fh_profile_select(fh_backend *backend, uint32_t class_mask);
+/* The kernel-level timers take one launch in `every` of each selected class (1: every launch, the
+ * default): the launches of a class do the same work layer after layer, and every timed one
+ * costs the stream about 6 us between kernels. */
+FH_API fh_status fh_profile_sample(fh_backend *backend, uint32_t every);
 FH_API fh_status fh_profile_reset(fh_backend *backend);
 FH_API fh_status fh_profile_read(fh_backend *backend, uint32_t kernel_class, uint64_t *nanoseconds,
                           uint64_t *launches);

@@ -132,7 +132,14 @@ def test_kernel_timers_follow_the_selected_classes(hip):
             run(hip, commands)
             nanoseconds, launches = hip.profile_read(6)
             assert launches == expected and (nanoseconds > 0) == (expected > 0)
+        # fh_profile_sample: one launch in three is timed
+        hip.profile_sample(3)
+        hip.profile_reset()
+        for _ in range(7):
+            run(hip, commands)
+        assert hip.profile_read(6)[1] == 3
     finally:
+        hip.profile_sample(1)
         hip.profile_select(0xffffffff)
         hip.profile_enable(0)
 

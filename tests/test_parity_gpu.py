@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from forja_amd import programs
-from forja_amd.core import (BackendError, BinOp, CommandList, DType, Inst, Op, Program,
+from forja_amd.core import (BackendError, BinOp, CommandList, DType, Inst, Layout, Op, Program,
                             ProgramBuilder, ProgramKind, RedOp, Slice, Status, UnOp, ValueType,
                             INTO_PAGES, OUT_OF_PAGES)
 from oracle import cpu_backend as orc
@@ -808,6 +808,49 @@ def test_router_top_k_is_bit_exact_in_order_and_close_in_weight(cpu, hip, dtype)
         commands = CommandList()
         commands.dispatch_many(Op.top_k(8, True), [x], outs)
         return commands, outs
+    differential(cpu, hip, build)
+
+
+@pytest.mark.parametrize("case", ["chain", "indices_rewritten", "fewer_logits_than_experts", "one_allocation"])
+@pytest.mark.parametrize("rows,dtype", [(1, DType.BF16), (8, DType.BF16), (16, DType.F32), (17, DType.BF16)])
+def test_top_k_of_a_small_batch_feeds_the_routed_products(cpu, hip, rows, dtype, case):
+    """A small decode batch: router logits -> top-k -> routed gate/up + SwiGLU -> routed down with
+    the weighted sum, the two products sharing the route plan packed from the selected indices.
+    The result is the oracle's, also where the indices are overwritten before the products read
+    them, the products know more experts than there were logits, or values and indices live in
+    one allocation."""
+    k, experts, n, inner = 8, 128, 128, 256
+    width = 64 if case == "fewer_logits_than_experts" else experts
+    gate = Quantised(47, 1, (n, inner), experts=experts)
+    up = Quantised(47, 11, (n, inner), experts=experts)
+    down = Quantised(47, 21, (inner, n), experts=experts)
+    logits = orc.fill_normal_f32(47, 31, rows * width).reshape(rows, width)
+    other = routed_case(47, rows, k, experts, n, inner)
+    x_values = normal_bf16(47, 40, (rows, inner))
+
+    def build(backend):
+        x = upload(backend, x_values, DType.BF16)
+        g, u, d = gate.upload(backend), up.upload(backend), down.upload(backend)
+        router = upload(backend, logits, dtype)
+        if case == "one_allocation":      # u32 indices behind the weights in the same allocation
+            both = backend.alloc(DType.U32, (2 * rows, k))
+            span = both.layout.buffer_len
+            weights = both.with_layout(Layout.contiguous(dtype, 0, (rows, k), span))
+            idx = both.with_layout(Layout.contiguous(DType.U32, rows * k, (rows, k), span))
+        else:
+            weights, idx = backend.alloc(dtype, (rows, k)), backend.alloc(DType.U32, (rows, k))
+        activated = backend.alloc(DType.BF16, (rows, k, n))
+        summed = backend.alloc(DType.BF16, (rows, inner))
+        bf16_weights = backend.alloc(DType.BF16, (rows, k))
+        swiglu = backend.prepare_epilogue(programs.silu_mul_elements())
+        commands = CommandList()
+        commands.dispatch_many(Op.top_k(k, True), [router], [weights, idx])
+        if case == "indices_rewritten":
+            commands.dispatch(Op.copy(), [upload(backend, other, DType.U32)], idx)
+        commands.dispatch(Op.copy(), [weights], bf16_weights)
+        commands.dispatch_epilogue(Op.gather_quant_matmul(4, 64), [x, *g, *u, idx], activated, swiglu, [])
+        commands.dispatch(Op.gather_quant_matmul(4, 64), [activated, *d, idx, bf16_weights], summed)
+        return commands, [weights, idx, activated, summed]
     differential(cpu, hip, build)
 
 
